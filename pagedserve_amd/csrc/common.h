@@ -1,0 +1,134 @@
+// Shared device helpers for the gfx950 kernels: storage types, conversions,
+// wave64 reductions and the error channel of the C interface.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#define PS_WAVE 64
+
+// Storage dtypes of the C interface.
+enum PsDtype { PS_F32 = 0, PS_BF16 = 1 };
+
+// Epilogues of the matrix products.
+enum PsEpilogue {
+  PS_EPI_NONE = 0,       // C = A W^T + b
+  PS_EPI_GELU_TANH = 1,  // C = gelu_tanh(A W^T + b)
+  PS_EPI_GELU_ERF = 2,   // C = gelu_erf(A W^T + b)
+  PS_EPI_RESIDUAL = 3,   // C(float) += A W^T + b   (C holds the residual stream)
+};
+
+struct bf16_t {
+  uint16_t bits;
+};
+
+__host__ __device__ inline float bf16_to_float(bf16_t v) {
+  union {
+    uint32_t u;
+    float f;
+  } c;
+  c.u = ((uint32_t)v.bits) << 16;
+  return c.f;
+}
+
+// Round to nearest, ties to even; NaN stays NaN.
+__host__ __device__ inline bf16_t float_to_bf16(float f) {
+  union {
+    uint32_t u;
+    float f;
+  } c;
+  c.f = f;
+  bf16_t out;
+  if ((c.u & 0x7fffffffu) > 0x7f800000u) {
+    out.bits = (uint16_t)((c.u >> 16) | 0x0040u);
+    return out;
+  }
+  uint32_t rounding = 0x7fffu + ((c.u >> 16) & 1u);
+  out.bits = (uint16_t)((c.u + rounding) >> 16);
+  return out;
+}
+
+template <typename T>
+__device__ inline float to_float(T v);
+template <>
+__device__ inline float to_float<float>(float v) {
+  return v;
+}
+template <>
+__device__ inline float to_float<bf16_t>(bf16_t v) {
+  return bf16_to_float(v);
+}
+
+template <typename T>
+__device__ inline T from_float(float v);
+template <>
+__device__ inline float from_float<float>(float v) {
+  return v;
+}
+template <>
+__device__ inline bf16_t from_float<bf16_t>(float v) {
+  return float_to_bf16(v);
+}
+
+__device__ inline float wave_sum(float v) {
+#pragma unroll
+  for (int offset = PS_WAVE / 2; offset > 0; offset >>= 1) v += __shfl_xor(v, offset, PS_WAVE);
+  return v;
+}
+
+__device__ inline float wave_max(float v) {
+#pragma unroll
+  for (int offset = PS_WAVE / 2; offset > 0; offset >>= 1) v = fmaxf(v, __shfl_xor(v, offset, PS_WAVE));
+  return v;
+}
+
+// Sum over a block of up to 1024 threads; every thread receives the total.
+// `scratch` holds at least 16 floats of shared memory.
+__device__ inline float block_sum(float v, float* scratch) {
+  const int lane = threadIdx.x & (PS_WAVE - 1);
+  const int wave = threadIdx.x / PS_WAVE;
+  const int waves = (blockDim.x + PS_WAVE - 1) / PS_WAVE;
+  v = wave_sum(v);
+  __syncthreads();
+  if (lane == 0) scratch[wave] = v;
+  __syncthreads();
+  float total = 0.f;
+  for (int i = 0; i < waves; ++i) total += scratch[i];
+  return total;
+}
+
+__device__ inline float gelu_tanh_f(float u) {
+  const float k = 0.7978845608028654f;  // sqrt(2/pi)
+  return 0.5f * u * (1.0f + tanhf(k * (u + 0.044715f * u * u * u)));
+}
+
+__device__ inline float gelu_erf_f(float u) {
+  return 0.5f * u * (1.0f + erff(u * 0.7071067811865476f));
+}
+
+template <int EPI>
+__device__ inline float apply_activation(float v) {
+  if (EPI == PS_EPI_GELU_TANH) return gelu_tanh_f(v);
+  if (EPI == PS_EPI_GELU_ERF) return gelu_erf_f(v);
+  return v;
+}
+
+// ---- error channel -------------------------------------------------------
+void ps_set_error(const char* fmt, ...);
+
+#define PS_REQUIRE(cond, ...)   \
+  do {                          \
+    if (!(cond)) {              \
+      ps_set_error(__VA_ARGS__); \
+      return 1;                 \
+    }                           \
+  } while (0)
+
+#define PS_CHECK_LAUNCH(name)                                              \
+  do {                                                                     \
+    hipError_t launch_error_ = hipGetLastError();                          \
+    if (launch_error_ != hipSuccess) {                                     \
+      ps_set_error("%s: launch failed: %s", name, hipGetErrorString(launch_error_)); \
+      return 2;                                                            \
+    }                                                                      \
+  } while (0)

@@ -1,0 +1,180 @@
+// Embedding(+position table) add, LayerNorm / RMS norm with row gather, and the scatter of
+// new keys and values into cache pages.  All arithmetic is float; storage may be bfloat16.
+#include <stdarg.h>
+#include <stdio.h>
+#include <string.h>
+
+#include "common.h"
+#include "pagedserve_hip.h"
+
+// ---------------------------------------------------------------- error channel
+static thread_local char g_error[512] = "";
+
+void ps_set_error(const char* fmt, ...) {
+  va_list args;
+  va_start(args, fmt);
+  vsnprintf(g_error, sizeof(g_error), fmt, args);
+  va_end(args);
+}
+
+extern "C" const char* ps_last_error(void) { return g_error; }
+
+extern "C" int ps_device_info(int* compute_units, int* lds_bytes, char* arch, int arch_len) {
+  int device = 0;
+  hipError_t status = hipGetDevice(&device);
+  PS_REQUIRE(status == hipSuccess, "ps_device_info: %s", hipGetErrorString(status));
+  hipDeviceProp_t prop;
+  status = hipGetDeviceProperties(&prop, device);
+  PS_REQUIRE(status == hipSuccess, "ps_device_info: %s", hipGetErrorString(status));
+  if (compute_units) *compute_units = prop.multiProcessorCount;
+  if (lds_bytes) *lds_bytes = (int)prop.sharedMemPerBlock;
+  if (arch && arch_len > 0) {
+    strncpy(arch, prop.gcnArchName, arch_len - 1);
+    arch[arch_len - 1] = 0;
+  }
+  return 0;
+}
+
+// ---------------------------------------------------------------- embedding
+// h0[t] = wte[id[t]] + wpe[pos[t]]  (reference: src/model/paged_decoder.py:306-314).
+template <typename T>
+__global__ void embed_kernel(const T* __restrict__ table, const T* __restrict__ pos_table,
+                             const int* __restrict__ ids, const int* __restrict__ positions,
+                             float* __restrict__ out, int width) {
+  const int t = blockIdx.x;
+  const T* row = table + (int64_t)ids[t] * width;
+  float* dst = out + (int64_t)t * width;
+  if (pos_table != nullptr) {
+    const T* prow = pos_table + (int64_t)positions[t] * width;
+    for (int i = threadIdx.x; i < width; i += blockDim.x)
+      dst[i] = to_float<T>(row[i]) + to_float<T>(prow[i]);
+  } else {
+    for (int i = threadIdx.x; i < width; i += blockDim.x) dst[i] = to_float<T>(row[i]);
+  }
+}
+
+extern "C" int ps_embed(const void* table, const void* pos_table, const int* ids,
+                        const int* positions, float* out, int tokens, int width, int vocab,
+                        int max_positions, int dtype, void* stream) {
+  PS_REQUIRE(tokens >= 0 && width > 0 && vocab > 0, "ps_embed: bad sizes (tokens %d, width %d)",
+             tokens, width);
+  PS_REQUIRE(dtype == PS_F32 || dtype == PS_BF16, "ps_embed: unknown dtype %d", dtype);
+  PS_REQUIRE(pos_table == nullptr || max_positions > 0, "ps_embed: position table without rows");
+  if (tokens == 0) return 0;
+  const int threads = width >= 256 ? 256 : 64;
+  hipStream_t s = (hipStream_t)stream;
+  if (dtype == PS_F32)
+    hipLaunchKernelGGL(embed_kernel<float>, dim3(tokens), dim3(threads), 0, s, (const float*)table,
+                       (const float*)pos_table, ids, positions, out, width);
+  else
+    hipLaunchKernelGGL(embed_kernel<bf16_t>, dim3(tokens), dim3(threads), 0, s,
+                       (const bf16_t*)table, (const bf16_t*)pos_table, ids, positions, out, width);
+  PS_CHECK_LAUNCH("ps_embed");
+  return 0;
+}
+
+// ---------------------------------------------------------------- norms
+// mean, centred values, biased variance of the centred values, rsqrt(var + eps), scale and
+// shift (reference: src/kernels/triton_residual_layernorm.py:25-39).  One block per row; the
+// row is read three times (it stays in cache), so any width works.
+template <typename T, bool RMS>
+__global__ void norm_kernel(const float* __restrict__ x, const int* __restrict__ rows,
+                            const float* __restrict__ gamma, const float* __restrict__ beta,
+                            T* __restrict__ out, int width, float eps) {
+  __shared__ float scratch[16];
+  const int r = blockIdx.x;
+  const float* src = x + (int64_t)(rows ? rows[r] : r) * width;
+  T* dst = out + (int64_t)r * width;
+  float mean = 0.f;
+  if (!RMS) {
+    float partial = 0.f;
+    for (int i = threadIdx.x; i < width; i += blockDim.x) partial += src[i];
+    mean = block_sum(partial, scratch) / (float)width;
+  }
+  float partial = 0.f;
+  for (int i = threadIdx.x; i < width; i += blockDim.x) {
+    const float c = src[i] - mean;
+    partial += c * c;
+  }
+  const float variance = block_sum(partial, scratch) / (float)width;
+  const float inv_std = 1.0f / sqrtf(variance + eps);
+  for (int i = threadIdx.x; i < width; i += blockDim.x) {
+    float v = (src[i] - mean) * inv_std * gamma[i];
+    if (!RMS && beta != nullptr) v += beta[i];
+    dst[i] = from_float<T>(v);
+  }
+}
+
+extern "C" int ps_norm(const float* x, const int* rows, const float* gamma, const float* beta,
+                       void* out, int n_rows, int width, float eps, int rms, int out_dtype,
+                       void* stream) {
+  PS_REQUIRE(n_rows >= 0 && width > 0, "ps_norm: bad sizes (rows %d, width %d)", n_rows, width);
+  PS_REQUIRE(out_dtype == PS_F32 || out_dtype == PS_BF16, "ps_norm: unknown dtype %d", out_dtype);
+  PS_REQUIRE(eps > 0.f, "ps_norm: eps must be positive");
+  if (n_rows == 0) return 0;
+  const int threads = width >= 1024 ? 256 : (width >= 256 ? 128 : 64);
+  hipStream_t s = (hipStream_t)stream;
+#define PS_LAUNCH_NORM(T, RMS)                                                              \
+  hipLaunchKernelGGL((norm_kernel<T, RMS>), dim3(n_rows), dim3(threads), 0, s, x, rows, gamma, \
+                     beta, (T*)out, width, eps)
+  if (out_dtype == PS_F32) {
+    if (rms) PS_LAUNCH_NORM(float, true); else PS_LAUNCH_NORM(float, false);
+  } else {
+    if (rms) PS_LAUNCH_NORM(bf16_t, true); else PS_LAUNCH_NORM(bf16_t, false);
+  }
+#undef PS_LAUNCH_NORM
+  PS_CHECK_LAUNCH("ps_norm");
+  return 0;
+}
+
+// ---------------------------------------------------------------- key/value scatter
+// Token t of request r at position p is stored at (page = table[r][p / page], offset =
+// p % page) (reference: src/model/kv_manager.py:303-308,403-404).
+template <typename T>
+__global__ void kv_write_kernel(const T* __restrict__ k, const T* __restrict__ v, int64_t stride,
+                                T* __restrict__ k_pool, T* __restrict__ v_pool,
+                                const int* __restrict__ tok_item, const int* __restrict__ tok_pos,
+                                const int* __restrict__ tables, int table_width, int kv_heads,
+                                int head_dim, int page_size, int num_pages) {
+  const int t = blockIdx.x;
+  const int pos = tok_pos[t];
+  const int logical = pos / page_size;
+  if (logical >= table_width) return;
+  const int page = tables[(int64_t)tok_item[t] * table_width + logical];
+  if (page < 0 || page >= num_pages) return;
+  const int offset = pos - logical * page_size;
+  const int row = kv_heads * head_dim;
+  for (int i = threadIdx.x; i < row; i += blockDim.x) {
+    const int head = i / head_dim;
+    const int dim = i - head * head_dim;
+    const int64_t dst = (((int64_t)page * kv_heads + head) * page_size + offset) * head_dim + dim;
+    k_pool[dst] = k[(int64_t)t * stride + i];
+    v_pool[dst] = v[(int64_t)t * stride + i];
+  }
+}
+
+extern "C" int ps_kv_write(const void* k, const void* v, int64_t stride, void* k_pool,
+                           void* v_pool, const int* tok_item, const int* tok_pos,
+                           const int* tables, int table_width, int tokens, int kv_heads,
+                           int head_dim, int page_size, int num_pages, int dtype, void* stream) {
+  PS_REQUIRE(tokens >= 0 && kv_heads > 0 && head_dim > 0 && page_size > 0 && num_pages > 0 &&
+                 table_width > 0,
+             "ps_kv_write: bad sizes");
+  PS_REQUIRE(stride >= (int64_t)kv_heads * head_dim, "ps_kv_write: row stride too small");
+  PS_REQUIRE(dtype == PS_F32 || dtype == PS_BF16, "ps_kv_write: unknown dtype %d", dtype);
+  if (tokens == 0) return 0;
+  const int row = kv_heads * head_dim;
+  const int threads = row >= 256 ? 256 : 64;
+  hipStream_t s = (hipStream_t)stream;
+  if (dtype == PS_F32)
+    hipLaunchKernelGGL(kv_write_kernel<float>, dim3(tokens), dim3(threads), 0, s, (const float*)k,
+                       (const float*)v, stride, (float*)k_pool, (float*)v_pool, tok_item, tok_pos,
+                       tables, table_width, kv_heads, head_dim, page_size, num_pages);
+  else
+    hipLaunchKernelGGL(kv_write_kernel<bf16_t>, dim3(tokens), dim3(threads), 0, s,
+                       (const bf16_t*)k, (const bf16_t*)v, stride, (bf16_t*)k_pool,
+                       (bf16_t*)v_pool, tok_item, tok_pos, tables, table_width, kv_heads, head_dim,
+                       page_size, num_pages);
+  PS_CHECK_LAUNCH("ps_kv_write");
+  return 0;
+}

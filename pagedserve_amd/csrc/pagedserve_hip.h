@@ -1,0 +1,61 @@
+// C interface of libpagedserve_hip.so: the gfx950 kernels of the engine.
+//
+// Conventions
+//   * every function returns 0 on success; otherwise ps_last_error() names the fault
+//     (a rejected size, an alignment that a kernel needs, a failed launch);
+//   * pointers are device pointers; `stream` is a hipStream_t;
+//   * `dtype` is PS_F32 (0) or PS_BF16 (1) and names the storage type of activations,
+//     matrices and the cache; norm scales, biases, the residual stream and logits are
+//     always float;
+//   * matrices are stored [out, in] (row n holds the weights of output n), so a product
+//     is C[m, n] = sum_k A[m, k] * W[n, k].
+#pragma once
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+const char* ps_last_error(void);
+int ps_device_info(int* compute_units, int* lds_bytes, char* arch, int arch_len);
+
+// out[t, :] = table[ids[t], :] + (pos_table ? pos_table[positions[t], :] : 0), in float.
+int ps_embed(const void* table, const void* pos_table, const int* ids, const int* positions,
+             float* out, int tokens, int width, int vocab, int max_positions, int dtype,
+             void* stream);
+
+// out[r, :] = norm(x[rows ? rows[r] : r, :]) * gamma (+ beta).  rms != 0: no mean, no beta.
+int ps_norm(const float* x, const int* rows, const float* gamma, const float* beta, void* out,
+            int n_rows, int width, float eps, int rms, int out_dtype, void* stream);
+
+// C[m, n] = epilogue(sum_k A[m, k] W[n, k] + bias[n]).
+//   c_dtype is the storage type of C; PS_EPI_RESIDUAL needs float C and adds into it.
+int ps_gemm_nt(const void* a, const void* w, const float* bias, void* c, int m, int n, int k,
+               int lda, int ldc, int dtype, int c_dtype, int epilogue, void* stream);
+
+// Store keys and values of the step's tokens into their pages.
+//   k, v: [tokens, kv_heads * head_dim] with row stride `stride`;
+//   pools: [pages, kv_heads, page_size, head_dim].
+int ps_kv_write(const void* k, const void* v, int64_t stride, void* k_pool, void* v_pool,
+                const int* tok_item, const int* tok_pos, const int* tables, int table_width,
+                int tokens, int kv_heads, int head_dim, int page_size, int num_pages, int dtype,
+                void* stream);
+
+// Attention of every token of the step over its request's cached keys 0..position
+// (or the last `window` of them), one wave per (token, head).  Any head_dim that is a
+// multiple of 16 up to 256; heads must be a multiple of kv_heads.
+int ps_attention_rowwise(const void* q, int64_t q_stride, const void* k_pool, const void* v_pool,
+                         void* out, int64_t out_stride, const int* tok_item, const int* tok_pos,
+                         const int* tables, int table_width, int tokens, int heads, int kv_heads,
+                         int head_dim, int page_size, int num_pages, float scale, int window,
+                         int dtype, void* stream);
+
+// tokens[r] = argmax (inv_temperature[r] == 0) or a draw from softmax(logits * inv_temperature[r])
+// by inverse CDF at uniform[r] in [0, 1).
+int ps_sample(const float* logits, int64_t ld, const float* inv_temperature, const float* uniform,
+              int* tokens, int rows, int vocab, void* stream);
+
+#ifdef __cplusplus
+}
+#endif

@@ -1,0 +1,66 @@
+"""From a model folder to a bound model, and the random-weights mode."""
+
+import json
+import os
+
+import torch
+
+from ..config.gpt2 import read_config_json
+from ..config.registry import resolve_architecture
+from ..weights.loader import load_parameters
+from ..weights.safetensors_io import write_safetensors
+from .decoder import DecoderModel
+
+DTYPES = {"float32": torch.float32, "bfloat16": torch.bfloat16}
+
+
+def resolve_dtype(dtype):
+    if isinstance(dtype, torch.dtype):
+        if dtype not in DTYPES.values():
+            raise ValueError(f"dtype {dtype} is not supported; choose float32 or bfloat16")
+        return dtype
+    if dtype not in DTYPES:
+        raise ValueError(f"Unknown dtype '{dtype}'. Choose one of: {', '.join(DTYPES)}")
+    return DTYPES[dtype]
+
+
+def load_model(folder, dtype="float32", device="cuda"):
+    """(model, typed config) of the folder's ``config.json`` + ``model.safetensors``."""
+    raw = read_config_json(folder)
+    architecture = resolve_architecture(raw)
+    config = architecture.config_class.from_dict(raw)
+    spec = architecture.build_spec(config)
+    engine_dtype = resolve_dtype(dtype)
+    model = DecoderModel(spec, engine_dtype, device)
+    tensors = load_parameters(
+        folder, model.parameters(), architecture.weight_sources(config, spec), engine_dtype,
+        device, ignorable=lambda name: architecture.ignorable(config, name))
+    model.bind(tensors)
+    return model, config
+
+
+def write_random_model(folder, config, seed=0, store_dtype=torch.float32, prefix="transformer."):
+    """Write ``config.json`` and ``model.safetensors`` of a random model of ``config``.
+
+    ``config`` is a typed configuration of a registered architecture or a raw dict
+    with that architecture's config.json keys."""
+    if isinstance(config, dict):
+        raw = dict(config)
+        architecture = resolve_architecture(
+            raw if raw.get("architectures") or raw.get("model_type")
+            else {**raw, "architectures": ["GPT2LMHeadModel"]})
+        raw.setdefault("architectures", [architecture.name])
+        config = architecture.config_class.from_dict(raw)
+    else:
+        architecture = resolve_architecture({"architectures": [config.architecture]})
+    os.makedirs(folder, exist_ok=True)
+    tensors = architecture.random_tensors(config, seed)
+    stored = {}
+    for name, tensor in tensors.items():
+        key = name if name.startswith("lm_head.") else prefix + name
+        stored[key] = tensor.to(store_dtype).contiguous()
+    write_safetensors(os.path.join(folder, "model.safetensors"), stored,
+                      metadata={"format": "pt", "seed": seed})
+    with open(os.path.join(folder, "config.json"), "w") as handle:
+        json.dump(config.to_dict(), handle, indent=2)
+    return config

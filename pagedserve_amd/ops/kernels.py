@@ -1,0 +1,256 @@
+"""Python faces of the HIP kernels: shape checks on the host, then one C call.
+
+Every function takes torch tensors that live on the GPU, checks what the kernel and
+its grid assume (devices, dtypes, contiguity, extents) and launches on torch's
+current stream.  There is no other implementation behind these functions.
+"""
+
+import ctypes
+from ctypes import c_float, c_int, c_int64, c_void_p
+
+import torch
+
+from .library import load_library
+
+F32 = 0
+BF16 = 1
+
+EPILOGUES = {"none": 0, "gelu_tanh": 1, "gelu_erf": 2, "residual": 3}
+
+_DTYPE_CODE = {torch.float32: F32, torch.bfloat16: BF16}
+
+_SIGNATURES = {
+    "ps_embed": [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int,
+                 c_int, c_void_p],
+    "ps_norm": [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_float, c_int,
+                c_int, c_void_p],
+    "ps_gemm_nt": [c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int,
+                   c_int, c_int, c_int, c_void_p],
+    "ps_kv_write": [c_void_p, c_void_p, c_int64, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
+                    c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_void_p],
+    "ps_attention_rowwise": [c_void_p, c_int64, c_void_p, c_void_p, c_void_p, c_int64, c_void_p,
+                             c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_int,
+                             c_float, c_int, c_int, c_void_p],
+    "ps_sample": [c_void_p, c_int64, c_void_p, c_void_p, c_void_p, c_int, c_int, c_void_p],
+}
+
+_BOUND = {}
+
+
+def _fn(name):
+    fn = _BOUND.get(name)
+    if fn is None:
+        fn = getattr(load_library(), name)
+        fn.argtypes = _SIGNATURES[name]
+        fn.restype = c_int
+        _BOUND[name] = fn
+    return fn
+
+
+class KernelError(RuntimeError):
+    pass
+
+
+def _call(name, *args):
+    status = _fn(name)(*args)
+    if status != 0:
+        message = load_library().ps_last_error().decode("utf-8", "replace")
+        raise KernelError(f"{name} failed ({status}): {message}")
+
+
+def _stream():
+    return torch.cuda.current_stream().cuda_stream
+
+
+def dtype_code(dtype: torch.dtype) -> int:
+    try:
+        return _DTYPE_CODE[dtype]
+    except KeyError:
+        raise KernelError(f"dtype {dtype} is not supported by the kernels "
+                          "(float32 and bfloat16 are)") from None
+
+
+def _check(tensor, name, dtype=None, ndim=None):
+    if not isinstance(tensor, torch.Tensor):
+        raise KernelError(f"{name} must be a tensor")
+    if not tensor.is_cuda:
+        raise KernelError(f"{name} must live on the GPU; the engine has no CPU path")
+    if dtype is not None and tensor.dtype != dtype:
+        raise KernelError(f"{name} must be {dtype}, got {tensor.dtype}")
+    if ndim is not None and tensor.ndim != ndim:
+        raise KernelError(f"{name} must have {ndim} dimensions, got shape {tuple(tensor.shape)}")
+    return tensor
+
+
+def _rows(tensor, name):
+    """2-D tensor with unit stride in its last dimension; returns the row stride."""
+    if tensor.ndim != 2 or (tensor.shape[1] > 1 and tensor.stride(1) != 1):
+        raise KernelError(f"{name} must be 2-D with contiguous rows, got shape "
+                          f"{tuple(tensor.shape)} strides {tuple(tensor.stride())}")
+    return tensor.stride(0) if tensor.shape[0] > 1 else max(tensor.stride(0), tensor.shape[1])
+
+
+def _ptr(tensor):
+    return 0 if tensor is None else tensor.data_ptr()
+
+
+def embed(table, pos_table, ids, positions, out):
+    """out[t] = table[ids[t]] + pos_table[positions[t]] as float (pos_table may be None)."""
+    _check(table, "table", ndim=2)
+    _check(ids, "ids", torch.int32, 1)
+    _check(out, "out", torch.float32, 2)
+    tokens = ids.numel()
+    width = table.shape[1]
+    if not (table.is_contiguous() and out.is_contiguous() and ids.is_contiguous()):
+        raise KernelError("embed: tensors must be contiguous")
+    if out.shape[0] < tokens or out.shape[1] != width:
+        raise KernelError(f"embed: out {tuple(out.shape)} does not fit {tokens} rows of {width}")
+    max_positions = 0
+    if pos_table is not None:
+        _check(pos_table, "pos_table", table.dtype, 2)
+        _check(positions, "positions", torch.int32, 1)
+        if pos_table.shape[1] != width or not pos_table.is_contiguous():
+            raise KernelError("embed: position table must be contiguous and as wide as the table")
+        if positions.numel() != tokens or not positions.is_contiguous():
+            raise KernelError("embed: one position per token is needed")
+        max_positions = pos_table.shape[0]
+    _call("ps_embed", table.data_ptr(), _ptr(pos_table), ids.data_ptr(),
+          _ptr(positions if pos_table is not None else None), out.data_ptr(), tokens, width,
+          table.shape[0], max_positions, dtype_code(table.dtype), _stream())
+    return out
+
+
+def norm(x, gamma, beta, eps, out, rows=None, rms=False):
+    """out[r] = norm(x[rows[r]]) * gamma + beta; statistics in float."""
+    _check(x, "x", torch.float32, 2)
+    _check(gamma, "gamma", torch.float32, 1)
+    _check(out, "out", ndim=2)
+    width = x.shape[1]
+    if not (x.is_contiguous() and out.is_contiguous() and gamma.is_contiguous()):
+        raise KernelError("norm: tensors must be contiguous")
+    if gamma.numel() != width or out.shape[1] != width:
+        raise KernelError("norm: widths of x, gamma and out differ")
+    if beta is not None:
+        _check(beta, "beta", torch.float32, 1)
+        if beta.numel() != width or not beta.is_contiguous():
+            raise KernelError("norm: beta does not match the width")
+    if rows is not None:
+        _check(rows, "rows", torch.int32, 1)
+        n_rows = rows.numel()
+    else:
+        n_rows = x.shape[0]
+    if out.shape[0] < n_rows:
+        raise KernelError("norm: out has too few rows")
+    _call("ps_norm", x.data_ptr(), _ptr(rows), gamma.data_ptr(), _ptr(beta), out.data_ptr(),
+          n_rows, width, float(eps), 1 if rms else 0, dtype_code(out.dtype), _stream())
+    return out
+
+
+def gemm_nt(a, w, bias, out, epilogue="none"):
+    """out[m, n] = epilogue(sum_k a[m, k] w[n, k] + bias[n]).
+
+    ``epilogue='residual'`` adds the product into the float tensor ``out``."""
+    _check(a, "a", ndim=2)
+    _check(w, "w", a.dtype, 2)
+    _check(out, "out", ndim=2)
+    lda = _rows(a, "a")
+    ldc = _rows(out, "out")
+    m, k = a.shape
+    n = w.shape[0]
+    if w.shape[1] != k or not w.is_contiguous():
+        raise KernelError(f"gemm_nt: w {tuple(w.shape)} must be contiguous [n, {k}]")
+    if out.shape[0] != m or out.shape[1] != n:
+        raise KernelError(f"gemm_nt: out {tuple(out.shape)} must be [{m}, {n}]")
+    if bias is not None:
+        _check(bias, "bias", torch.float32, 1)
+        if bias.numel() != n or not bias.is_contiguous():
+            raise KernelError("gemm_nt: bias does not match n")
+    if epilogue not in EPILOGUES:
+        raise KernelError(f"gemm_nt: unknown epilogue {epilogue!r}")
+    _call("ps_gemm_nt", a.data_ptr(), w.data_ptr(), _ptr(bias), out.data_ptr(), m, n, k, lda, ldc,
+          dtype_code(a.dtype), dtype_code(out.dtype), EPILOGUES[epilogue], _stream())
+    return out
+
+
+def _check_pools(k_pool, v_pool, dtype):
+    _check(k_pool, "k_pool", dtype, 4)
+    _check(v_pool, "v_pool", dtype, 4)
+    if k_pool.shape != v_pool.shape or not (k_pool.is_contiguous() and v_pool.is_contiguous()):
+        raise KernelError("key and value pools must be contiguous and of one shape")
+    return k_pool.shape  # pages, kv_heads, page_size, head_dim
+
+
+def _check_step_index(tok_item, tok_pos, tables, tokens):
+    _check(tok_item, "tok_item", torch.int32, 1)
+    _check(tok_pos, "tok_pos", torch.int32, 1)
+    _check(tables, "tables", torch.int32, 2)
+    if tok_item.numel() < tokens or tok_pos.numel() < tokens:
+        raise KernelError("one item index and one position per token are needed")
+    if not (tok_item.is_contiguous() and tok_pos.is_contiguous() and tables.is_contiguous()):
+        raise KernelError("step index tensors must be contiguous")
+
+
+def kv_write(k, v, k_pool, v_pool, tok_item, tok_pos, tables):
+    """Store rows of k and v ([tokens, kv_heads*head_dim]) at their positions' pages."""
+    _check(k, "k", ndim=2)
+    _check(v, "v", k.dtype, 2)
+    pages, kv_heads, page_size, head_dim = _check_pools(k_pool, v_pool, k.dtype)
+    stride = _rows(k, "k")
+    if _rows(v, "v") != stride or v.shape != k.shape:
+        raise KernelError("kv_write: k and v must share shape and row stride")
+    if k.shape[1] != kv_heads * head_dim:
+        raise KernelError(f"kv_write: rows of {k.shape[1]} do not match {kv_heads} x {head_dim}")
+    tokens = k.shape[0]
+    _check_step_index(tok_item, tok_pos, tables, tokens)
+    _call("ps_kv_write", k.data_ptr(), v.data_ptr(), stride, k_pool.data_ptr(), v_pool.data_ptr(),
+          tok_item.data_ptr(), tok_pos.data_ptr(), tables.data_ptr(), tables.shape[1], tokens,
+          kv_heads, head_dim, page_size, pages, dtype_code(k.dtype), _stream())
+
+
+def attention_rowwise(q, k_pool, v_pool, out, tok_item, tok_pos, tables, heads, scale, window=0):
+    """out[t, h] = softmax(q[t, h] . K * scale) V over the cached keys of t's request."""
+    _check(q, "q", ndim=2)
+    _check(out, "out", q.dtype, 2)
+    pages, kv_heads, page_size, head_dim = _check_pools(k_pool, v_pool, q.dtype)
+    q_stride = _rows(q, "q")
+    out_stride = _rows(out, "out")
+    tokens = q.shape[0]
+    if q.shape[1] != heads * head_dim or out.shape[1] != heads * head_dim or out.shape[0] != tokens:
+        raise KernelError("attention: q/out rows must hold heads x head_dim values")
+    _check_step_index(tok_item, tok_pos, tables, tokens)
+    _call("ps_attention_rowwise", q.data_ptr(), q_stride, k_pool.data_ptr(), v_pool.data_ptr(),
+          out.data_ptr(), out_stride, tok_item.data_ptr(), tok_pos.data_ptr(), tables.data_ptr(),
+          tables.shape[1], tokens, heads, kv_heads, head_dim, page_size, pages, float(scale),
+          int(window), dtype_code(q.dtype), _stream())
+    return out
+
+
+def sample(logits, inv_temperature, uniform, out):
+    """out[r] = argmax(logits[r]) where inv_temperature[r] == 0, else the inverse-CDF draw of
+    softmax(logits[r] * inv_temperature[r]) at uniform[r]."""
+    _check(logits, "logits", torch.float32, 2)
+    _check(out, "out", torch.int32, 1)
+    ld = _rows(logits, "logits")
+    rows, vocab = logits.shape
+    if out.numel() < rows:
+        raise KernelError("sample: out has too few entries")
+    if inv_temperature is not None:
+        _check(inv_temperature, "inv_temperature", torch.float32, 1)
+        _check(uniform, "uniform", torch.float32, 1)
+        if inv_temperature.numel() < rows or uniform.numel() < rows:
+            raise KernelError("sample: one temperature and one uniform number per row are needed")
+    _call("ps_sample", logits.data_ptr(), ld, _ptr(inv_temperature), _ptr(uniform),
+          out.data_ptr(), rows, vocab, _stream())
+    return out
+
+
+def device_info():
+    units = ctypes.c_int(0)
+    lds = ctypes.c_int(0)
+    arch = ctypes.create_string_buffer(64)
+    fn = load_library().ps_device_info
+    fn.restype = c_int
+    status = fn(ctypes.byref(units), ctypes.byref(lds), arch, 64)
+    if status != 0:
+        raise KernelError(load_library().ps_last_error().decode())
+    return {"compute_units": units.value, "lds_bytes": lds.value, "arch": arch.value.decode()}

@@ -1,0 +1,76 @@
+"""Multi-head attention over the paged cache."""
+
+from ..ops import kernels
+from ..weights.loader import MATRIX, VECTOR, ParamSpec
+from .base import Mixer, PagedKVSpec
+from .registry import register_mixer
+
+
+@register_mixer("attention")
+class Attention(Mixer):
+    """Packed QKV projection, cache write, attention over the request's cached keys,
+    output projection added to the residual stream.
+
+    One product gives ``[q | k | v]`` (src/model/paged_decoder.py:47-53); head ``j`` owns
+    columns ``j*head_dim`` onward of each part (``:63-69``).  Keys and values of the
+    step's tokens are stored before attention runs, so a token attends to itself and a
+    prompt portion, a whole prompt and a decoded token are one case: every query at
+    position p reads keys ``0..p`` (the last ``window`` of them) from the pages.
+    ``scale`` multiplies the scores (``head_dim**-0.5`` in src/model/paged_attention.py:27).
+    """
+
+    def __init__(self, width: int, dtype, heads: int, kv_heads: int, head_dim: int, scale: float,
+                 window: int = 0, bias: bool = True):
+        if heads % kv_heads != 0:
+            raise ValueError(f"heads ({heads}) must be a multiple of kv_heads ({kv_heads})")
+        if head_dim % 16 != 0 or head_dim > 256:
+            raise ValueError(f"head_dim {head_dim} must be a multiple of 16 up to 256")
+        self.width = width
+        self.dtype = dtype
+        self.heads = heads
+        self.kv_heads = kv_heads
+        self.head_dim = head_dim
+        self.scale = float(scale)
+        self.window = int(window)
+        self.bias = bias
+        self.q_cols = heads * head_dim
+        self.kv_cols = kv_heads * head_dim
+        self.position = None
+
+    def parameters(self):
+        total = self.q_cols + 2 * self.kv_cols
+        params = {
+            "qkv.weight": ParamSpec((total, self.width), MATRIX),
+            "out.weight": ParamSpec((self.width, self.q_cols), MATRIX),
+        }
+        if self.bias:
+            params["qkv.bias"] = ParamSpec((total,), VECTOR)
+            params["out.bias"] = ParamSpec((self.width,), VECTOR)
+        return params
+
+    def bind(self, tensors):
+        self.qkv_weight = tensors["qkv.weight"]
+        self.out_weight = tensors["out.weight"]
+        self.qkv_bias = tensors.get("qkv.bias")
+        self.out_bias = tensors.get("out.bias")
+
+    def cache_spec(self):
+        return PagedKVSpec(self.kv_heads, self.head_dim, self.window)
+
+    def forward(self, x, residual, ctx, cache):
+        tokens = ctx.tokens
+        total = self.q_cols + 2 * self.kv_cols
+        qkv = ctx.workspace.rows("qkv", total, self.dtype)[:tokens]
+        kernels.gemm_nt(x, self.qkv_weight, self.qkv_bias, qkv)
+        q = qkv[:, :self.q_cols]
+        k = qkv[:, self.q_cols:self.q_cols + self.kv_cols]
+        v = qkv[:, self.q_cols + self.kv_cols:]
+        if self.position is not None:
+            self.position.apply_to_qk(q, k, ctx)
+        tables = ctx.tables[cache.group]
+        if cache.writes:
+            kernels.kv_write(k, v, cache.k_pool, cache.v_pool, ctx.tok_item, ctx.positions, tables)
+        context = ctx.workspace.rows("attn", self.q_cols, self.dtype)[:tokens]
+        kernels.attention_rowwise(q, cache.k_pool, cache.v_pool, context, ctx.tok_item,
+                                  ctx.positions, tables, self.heads, self.scale, self.window)
+        kernels.gemm_nt(context, self.out_weight, self.out_bias, residual, epilogue="residual")

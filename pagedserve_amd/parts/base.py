@@ -1,0 +1,153 @@
+"""Interfaces of the parts that a layer is put together from.
+
+A part is built from sizes and constants only, declares the parameters it needs
+(``parameters``), receives them once (``bind``) and is then called with the step's
+tensors.  It never sees the model's configuration.
+
+* ``Norm.forward(h, out, rows=None)``: ``h`` is the float residual stream ``[T, d]``;
+  writes the normed rows in the engine dtype.
+* ``Mixer.forward(x, residual, ctx, cache)``: ``x`` is ``[T, d]`` in the engine dtype;
+  the mixer ADDS its output to the float ``residual`` in place.  ``cache`` is the
+  ``CacheView`` of this call of the layer: pools of a paged key/value entry, or the
+  state tensor ``[max_slots, ...]`` of a mixer that declared a ``StateSpec``.
+* ``FeedForward.forward(x, residual, ctx)``: same contract without a cache.
+* ``PositionEncoding``: ``embedding_table()`` is added to the token embedding when it
+  is not ``None``; ``apply_to_qk(q, k, ctx)`` may transform queries and keys in place
+  before they are cached (the default does nothing).
+
+Folding the residual sum into the part lets the last matrix product of a part add
+in float in its own epilogue instead of a separate pass over the stream.
+"""
+
+from dataclasses import dataclass
+from typing import Dict, List, Optional
+
+import torch
+
+from ..weights.loader import ParamSpec
+
+
+@dataclass(frozen=True)
+class PagedKVSpec:
+    """A mixer that caches keys and values of every (or the last ``window``) positions."""
+
+    kv_heads: int
+    head_dim: int
+    window: int = 0
+
+
+@dataclass(frozen=True)
+class SlotStateSpec:
+    """A mixer that keeps a fixed-size state per request."""
+
+    shape: tuple
+    dtype: torch.dtype = torch.float32
+
+
+@dataclass
+class CacheView:
+    """What one call of a layer may touch in the cache."""
+
+    entry: int
+    writes: bool
+    group: Optional[int] = None                # index of the cache group (paged entries)
+    k_pool: Optional[torch.Tensor] = None      # [pages, kv_heads, page, head_dim]
+    v_pool: Optional[torch.Tensor] = None
+    state: Optional[torch.Tensor] = None       # [max_slots, ...]
+
+
+class Part:
+    def parameters(self) -> Dict[str, ParamSpec]:
+        return {}
+
+    def bind(self, tensors: Dict[str, torch.Tensor]):
+        for name in self.parameters():
+            setattr(self, name.replace(".", "_"), tensors[name])
+
+
+class Norm(Part):
+    def forward(self, h, out, rows=None):
+        raise NotImplementedError
+
+
+class PositionEncoding(Part):
+    def embedding_table(self):
+        return None
+
+    def apply_to_qk(self, q, k, ctx):
+        return None
+
+
+class Mixer(Part):
+    def cache_spec(self):
+        """``PagedKVSpec``, ``SlotStateSpec`` or ``None``."""
+        return None
+
+    def set_position(self, position: PositionEncoding):
+        self.position = position
+
+    def forward(self, x, residual, ctx, cache: CacheView):
+        raise NotImplementedError
+
+
+class FeedForward(Part):
+    def forward(self, x, residual, ctx):
+        raise NotImplementedError
+
+
+class Workspace:
+    """Activation buffers that live as long as the engine.
+
+    ``rows(name, columns, dtype)`` returns a ``[max_rows, columns]`` tensor that is
+    allocated on first use and never moves afterwards, so kernels captured in a HIP
+    graph keep valid addresses.  Buffers are shared by all layers (they run one after
+    the other)."""
+
+    def __init__(self, max_rows: int, device):
+        self.max_rows = max_rows
+        self.device = torch.device(device)
+        self._buffers: Dict[tuple, torch.Tensor] = {}
+
+    def rows(self, name: str, columns: int, dtype: torch.dtype, max_rows: Optional[int] = None):
+        key = (name, columns, dtype, max_rows or self.max_rows)
+        buffer = self._buffers.get(key)
+        if buffer is None:
+            buffer = torch.empty((max_rows or self.max_rows, columns), dtype=dtype, device=self.device)
+            self._buffers[key] = buffer
+        return buffer
+
+    def bytes(self) -> int:
+        return sum(buffer.numel() * buffer.element_size() for buffer in self._buffers.values())
+
+
+@dataclass
+class StepItem:
+    """One request's share of a step (host side)."""
+
+    request_id: object
+    slot: int
+    start: int      # position of its first token in the request
+    count: int      # tokens in this step
+    offset: int     # index of its first token in the step's flat token list
+
+
+@dataclass
+class StepContext:
+    """Everything a part may read about the running step."""
+
+    tokens: int
+    dtype: torch.dtype
+    device: torch.device
+    items: List[StepItem]
+    token_ids: torch.Tensor     # int32 [T]
+    positions: torch.Tensor     # int32 [T]   position of each token in its request
+    tok_item: torch.Tensor      # int32 [T]   index into ``items``
+    cu_tokens: torch.Tensor     # int32 [items + 1]
+    kv_lens: torch.Tensor       # int32 [items]  cached length after this step
+    slots: torch.Tensor         # int32 [items]
+    tables: List[torch.Tensor]  # per cache group: int32 [items, pages per request]
+    page_size: int
+    workspace: Workspace
+    decode_only: bool = False   # every item brings exactly one token
+    max_kv_len: int = 0
+    extra: Optional[dict] = None

@@ -1,0 +1,44 @@
+"""Feed-forward parts."""
+
+from ..ops import kernels
+from ..weights.loader import MATRIX, VECTOR, ParamSpec
+from .base import FeedForward
+from .registry import register_feed_forward
+
+ACTIVATIONS = ("gelu_tanh", "gelu_erf")
+
+
+@register_feed_forward("dense")
+class DenseFeedForward(FeedForward):
+    """``residual += act(x W_up + b_up) W_down + b_down``
+    (src/model/paged_decoder.py:178-179,224-228; activations ``:273-280``)."""
+
+    def __init__(self, width: int, dtype, inner: int, activation: str, bias: bool = True):
+        if activation not in ACTIVATIONS:
+            raise ValueError(f"unknown activation {activation!r}; known: {', '.join(ACTIVATIONS)}")
+        self.width = width
+        self.dtype = dtype
+        self.inner = inner
+        self.activation = activation
+        self.bias = bias
+
+    def parameters(self):
+        params = {
+            "up.weight": ParamSpec((self.inner, self.width), MATRIX),
+            "down.weight": ParamSpec((self.width, self.inner), MATRIX),
+        }
+        if self.bias:
+            params["up.bias"] = ParamSpec((self.inner,), VECTOR)
+            params["down.bias"] = ParamSpec((self.width,), VECTOR)
+        return params
+
+    def bind(self, tensors):
+        self.up_weight = tensors["up.weight"]
+        self.down_weight = tensors["down.weight"]
+        self.up_bias = tensors.get("up.bias")
+        self.down_bias = tensors.get("down.bias")
+
+    def forward(self, x, residual, ctx):
+        hidden = ctx.workspace.rows("ffn", self.inner, self.dtype)[:ctx.tokens]
+        kernels.gemm_nt(x, self.up_weight, self.up_bias, hidden, epilogue=self.activation)
+        kernels.gemm_nt(hidden, self.down_weight, self.down_bias, residual, epilogue="residual")

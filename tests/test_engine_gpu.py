@@ -1,0 +1,110 @@
+"""The engine against the plain implementation under every way of cutting the work."""
+
+import json
+import os
+import subprocess
+import sys
+
+import numpy as np
+import pytest
+import torch
+
+import helpers
+
+pytestmark = pytest.mark.gpu
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+# prompts + decoded tokens of BASELINE's tiny workloads, as given token sequences
+LENGTHS = {"A": [5 + 16, 17 + 16, 31 + 16, 90], "B": [1 + 24, 9 + 24, 40 + 24, 64 + 24, 100 + 24, 200]}
+
+
+def _requests(which, config):
+    return {f"r{i}": helpers.random_tokens(n, config["vocab_size"], 100 + i)
+            for i, n in enumerate(LENGTHS[which])}
+
+
+def _engine(folder, dtype, page_size, pages, max_step_tokens=512):
+    from pagedserve_amd.engine import Engine
+    from pagedserve_amd.model import load_model
+
+    model, _ = load_model(folder, dtype=dtype, device="cuda")
+    return Engine(model, num_pages=pages, page_size=page_size, max_requests=8,
+                  max_step_tokens=max_step_tokens)
+
+
+@pytest.fixture(scope="module")
+def folders(tmp_path_factory):
+    base = tmp_path_factory.mktemp("models")
+    return {which: helpers.tiny_folder(base, which) for which in ("A", "B")}
+
+
+@pytest.fixture(scope="module")
+def references(folders):
+    out = {}
+    for which, (folder, config, _) in folders.items():
+        requests = _requests(which, config)
+        for bf16 in (False, True):
+            out[(which, bf16)] = {rid: helpers.plain_logits(folder, tokens, bfloat16=bf16)
+                                  for rid, tokens in requests.items()}
+    return out
+
+
+CUTS = {
+    "whole": helpers.trace_whole,
+    "tail_decoded": helpers.trace_tail_decoded,
+    "portions": helpers.trace_portions,
+    "mixed": helpers.trace_mixed,
+}
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("which", ["A", "B"])
+@pytest.mark.parametrize("cut", list(CUTS))
+def test_cuts_match_plain(folders, references, which, dtype, cut):
+    folder, config, page_size = folders[which]
+    requests = _requests(which, config)
+    steps = CUTS[cut](requests)
+    budget = helpers.live_token_budget(steps)
+    # exactly the pages that the live requests need at their peak: pages are used again
+    engine = _engine(folder, dtype, page_size, pages=-(-budget // page_size))
+    rows = helpers.replay_in_process(engine, steps)
+    engine.cache.check_invariants()
+    assert not engine.cache.requests
+    assert len(rows) == sum(len(tokens) for tokens in requests.values())
+    error, scale, where = helpers.max_error(rows, references[(which, dtype == "bfloat16")])
+    assert error <= helpers.TOLERANCE[dtype] * scale, (error, scale, where)
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_trace_run_program(folders, references, tmp_path, dtype):
+    """bin/trace_run as a user calls it: JSON lines in, <step>.f32 files and 'done' lines out."""
+    folder, config, page_size = folders["B"]
+    requests = _requests("B", config)
+    steps = helpers.trace_mixed(requests, seed=3)
+    budget = helpers.live_token_budget(steps)
+    out_dir = tmp_path / "out"
+    process = subprocess.run(
+        [sys.executable, os.path.join(ROOT, "bin", "trace_run"), "--model", folder, "--dtype", dtype,
+         "--out", str(out_dir), "--max-tokens", str(budget)],
+        input="\n".join(json.dumps(step) for step in steps) + "\n", capture_output=True, text=True,
+        timeout=600)
+    assert process.returncode == 0, process.stderr[-2000:]
+    done = [line for line in process.stdout.splitlines() if line.startswith("done ")]
+    assert done == [f"done {step['step']}" for step in steps]
+    reference = references[("B", dtype == "bfloat16")]
+    held = {}
+    worst, scale = 0.0, 0.0
+    for step in steps:
+        wanted = sum(len(entry["want"]) for entry in step["entries"])
+        values = np.fromfile(out_dir / f"{step['step']}.f32", dtype="<f4").reshape(wanted, config["vocab_size"])
+        row = 0
+        for entry in step["entries"]:
+            start = held.get(entry["id"], 0)
+            for place in entry["want"]:
+                expected = reference[entry["id"]][start + place]
+                worst = max(worst, float((torch.from_numpy(values[row]).double() - expected).abs().max()))
+                scale = max(scale, float(expected.abs().max()))
+                row += 1
+            held[entry["id"]] = start + len(entry["tokens"])
+    assert worst <= helpers.TOLERANCE[dtype] * scale, (worst, scale)

@@ -1,0 +1,361 @@
+"""Each HIP kernel alone against a plain float64 torch formula, at sizes that differ
+from the engine's tiny models (ragged widths, odd row counts, head sizes 16..128)."""
+
+import math
+
+import pytest
+import torch
+from torch.nn import functional as F
+
+pytestmark = pytest.mark.gpu
+
+DTYPES = [torch.float32, torch.bfloat16]
+
+
+def _tol(dtype):
+    return (2e-5, 2e-5) if dtype == torch.float32 else (2e-2, 2e-2)
+
+
+def _rand(shape, dtype, seed, scale=1.0):
+    g = torch.Generator().manual_seed(seed)
+    return (torch.randn(shape, generator=g) * scale).to(dtype).cuda()
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("tokens,width,vocab,positions", [(1, 64, 50, 9), (37, 100, 257, 64), (300, 768, 1000, 128)])
+def test_embed(dtype, tokens, width, vocab, positions):
+    from pagedserve_amd.ops import kernels
+
+    table = _rand((vocab, width), dtype, 0)
+    pos_table = _rand((positions, width), dtype, 1)
+    g = torch.Generator().manual_seed(2)
+    ids = torch.randint(0, vocab, (tokens,), generator=g).int().cuda()
+    pos = torch.randint(0, positions, (tokens,), generator=g).int().cuda()
+    out = torch.full((tokens, width), float("nan"), device="cuda")
+    kernels.embed(table, pos_table, ids, pos, out)
+    expected = F.embedding(ids.long(), table.float()) + F.embedding(pos.long(), pos_table.float())
+    torch.testing.assert_close(out, expected, atol=0, rtol=0)
+    kernels.embed(table, None, ids, pos, out)
+    torch.testing.assert_close(out, F.embedding(ids.long(), table.float()), atol=0, rtol=0)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("rows,width", [(1, 768), (8, 768), (32, 768), (5, 96), (3, 1600), (7, 50)])
+def test_layernorm_matches_library(dtype, rows, width):
+    # shapes (1, 8, 32) x 768 are those of testing/test_triton_residual_layernorm.py:7-35
+    from pagedserve_amd.ops import kernels
+
+    x = _rand((rows, width), torch.float32, 515)
+    gamma = _rand((width,), torch.float32, 516)
+    beta = _rand((width,), torch.float32, 517)
+    out = torch.empty((rows, width), dtype=dtype, device="cuda")
+    kernels.norm(x, gamma, beta, 1e-5, out)
+    expected = F.layer_norm(x.double(), (width,), gamma.double(), beta.double(), 1e-5)
+    atol, rtol = _tol(dtype)
+    torch.testing.assert_close(out.double(), expected, atol=atol, rtol=rtol)
+
+
+def test_layernorm_eps_and_gather():
+    """A row of tiny variance tells eps 1e-5 from 1e-6; `rows` gathers and reorders."""
+    from pagedserve_amd.ops import kernels
+
+    width = 64
+    x = torch.zeros(4, width, device="cuda")
+    x[1] = _rand((width,), torch.float32, 3) * 1e-3 + 5.0
+    x[3] = _rand((width,), torch.float32, 4)
+    gamma = torch.ones(width, device="cuda")
+    beta = torch.zeros(width, device="cuda")
+    rows = torch.tensor([3, 1], dtype=torch.int32, device="cuda")
+    for eps in (1e-5, 1e-6):
+        out = torch.empty(2, width, device="cuda")
+        kernels.norm(x, gamma, beta, eps, out, rows=rows)
+        expected = F.layer_norm(x[[3, 1]].double(), (width,), None, None, eps)
+        torch.testing.assert_close(out.double(), expected, atol=1e-5, rtol=1e-5)
+    a = torch.empty(2, width, device="cuda")
+    b = torch.empty(2, width, device="cuda")
+    kernels.norm(x, gamma, beta, 1e-5, a, rows=rows)
+    kernels.norm(x, gamma, beta, 1e-6, b, rows=rows)
+    assert (a[1] - b[1]).abs().max() > 1e-2          # the tiny-variance row feels eps
+    # a constant row maps to beta
+    const = torch.full((1, width), 3.0, device="cuda")
+    out = torch.empty(1, width, device="cuda")
+    kernels.norm(const, gamma, beta + 0.25, 1e-5, out)
+    torch.testing.assert_close(out, torch.full_like(out, 0.25), atol=1e-6, rtol=0)
+
+
+def test_rmsnorm():
+    from pagedserve_amd.ops import kernels
+
+    x = _rand((6, 80), torch.float32, 5)
+    gamma = _rand((80,), torch.float32, 6)
+    out = torch.empty(6, 80, device="cuda")
+    kernels.norm(x, gamma, None, 1e-6, out, rms=True)
+    xd = x.double()
+    expected = xd / torch.sqrt((xd * xd).mean(-1, keepdim=True) + 1e-6) * gamma.double()
+    torch.testing.assert_close(out.double(), expected, atol=2e-5, rtol=2e-5)
+
+
+GEMM_SHAPES = [(1, 50, 64), (5, 1000, 96), (64, 2304, 768), (130, 70, 320), (33, 257, 100),
+               (256, 768, 3072), (2, 50257, 64)]
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("m,n,k", GEMM_SHAPES)
+@pytest.mark.parametrize("epilogue", ["none", "gelu_tanh", "gelu_erf", "residual"])
+def test_gemm_nt(dtype, m, n, k, epilogue):
+    from pagedserve_amd.ops import kernels
+
+    if epilogue != "none" and n > 5000:
+        pytest.skip("one epilogue is enough at the vocabulary size")
+    a = _rand((m, k), dtype, 10, 1.0)
+    w = _rand((n, k), dtype, 11, 1.0 / math.sqrt(k))
+    bias = _rand((n,), torch.float32, 12)
+    product = a.double() @ w.double().t() + bias.double()
+    if epilogue == "residual":
+        out = _rand((m, n), torch.float32, 13)
+        expected = out.double() + product
+    else:
+        out_dtype = dtype
+        out = torch.full((m, n), float("nan"), dtype=out_dtype, device="cuda")
+        if epilogue == "gelu_tanh":
+            expected = F.gelu(product, approximate="tanh")
+        elif epilogue == "gelu_erf":
+            expected = F.gelu(product)
+        else:
+            expected = product
+    kernels.gemm_nt(a, w, bias, out, epilogue=epilogue)
+    atol, rtol = _tol(dtype)
+    torch.testing.assert_close(out.double(), expected, atol=atol * 2, rtol=rtol)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_gemm_float_logits_and_strided_views(dtype):
+    """bfloat16 operands with float output (the head), inputs and outputs that are column
+    slices of wider buffers, and no bias."""
+    from pagedserve_amd.ops import kernels
+
+    wide = _rand((9, 300), dtype, 20)
+    a = wide[:, 100:196]
+    w = _rand((77, 96), dtype, 21, 0.1)
+    out_wide = torch.zeros((9, 200), dtype=torch.float32, device="cuda")
+    out = out_wide[:, 50:127]
+    kernels.gemm_nt(a, w, None, out)
+    expected = a.double() @ w.double().t()
+    atol, rtol = (2e-5, 2e-5) if dtype == torch.float32 else (2e-3, 2e-3)
+    torch.testing.assert_close(out.double(), expected, atol=atol, rtol=rtol)
+    assert float(out_wide[:, :50].abs().max()) == 0 and float(out_wide[:, 127:].abs().max()) == 0
+
+
+def test_gemm_identity_and_one_hot():
+    from pagedserve_amd.ops import kernels
+
+    w = _rand((40, 40), torch.float32, 30)
+    eye = torch.eye(40, device="cuda")
+    out = torch.empty(40, 40, device="cuda")
+    kernels.gemm_nt(eye, w, None, out)           # row m of out = column m of w^T... = w[:, m]
+    torch.testing.assert_close(out, w.t().contiguous(), atol=0, rtol=0)
+    kernels.gemm_nt(w, eye, None, out)
+    torch.testing.assert_close(out, w, atol=0, rtol=0)
+
+
+def _paged_fixture(dtype, batch_lens, kv_heads, head_dim, page_size, seed, extra_pages=5):
+    """Fragmented pools and tables for requests of the given cached lengths."""
+    g = torch.Generator().manual_seed(seed)
+    pages_per = [-(-length // page_size) for length in batch_lens]
+    width = max(pages_per) + 2
+    total = sum(pages_per) + extra_pages
+    order = torch.randperm(total, generator=g).tolist()
+    tables = torch.full((len(batch_lens), width), -1, dtype=torch.int32)
+    cursor = 0
+    for index, count in enumerate(pages_per):
+        tables[index, :count] = torch.tensor(order[cursor:cursor + count], dtype=torch.int32)
+        cursor += count
+    k_pool = (torch.randn((total, kv_heads, page_size, head_dim), generator=g)).to(dtype).cuda()
+    v_pool = (torch.randn((total, kv_heads, page_size, head_dim), generator=g)).to(dtype).cuda()
+    return k_pool, v_pool, tables.cuda()
+
+
+def _gather(pool, table, length, page_size):
+    pages = table[: -(-length // page_size)].long()
+    return pool[pages].permute(1, 0, 2, 3).reshape(pool.shape[1], -1, pool.shape[3])[:, :length]
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("heads,kv_heads,head_dim,page_size", [(1, 1, 32, 16), (4, 4, 16, 8), (6, 2, 48, 16), (3, 3, 128, 4), (12, 12, 64, 16)])
+def test_attention_rowwise_decode_contexts(dtype, heads, kv_heads, head_dim, page_size):
+    """Single-token queries over fragmented tables; contexts around page edges as in
+    testing/test_triton_correctness_matrix.py:9 (1, 15, 16, 17, 31, 32, 33, 128, 512)."""
+    from pagedserve_amd.ops import kernels
+
+    contexts = [1, 15, 16, 17, 31, 32, 33, 128, 512]
+    k_pool, v_pool, tables = _paged_fixture(dtype, contexts, kv_heads, head_dim, page_size, 17)
+    q = _rand((len(contexts), heads * head_dim), dtype, 18)
+    out = torch.empty_like(q)
+    tok_item = torch.arange(len(contexts), dtype=torch.int32, device="cuda")
+    tok_pos = torch.tensor([c - 1 for c in contexts], dtype=torch.int32, device="cuda")
+    scale = head_dim ** -0.5
+    kernels.attention_rowwise(q, k_pool, v_pool, out, tok_item, tok_pos, tables, heads, scale)
+    group = heads // kv_heads
+    for index, context in enumerate(contexts):
+        keys = _gather(k_pool, tables[index], context, page_size).double()
+        values = _gather(v_pool, tables[index], context, page_size).double()
+        keys = keys.repeat_interleave(group, 0)
+        values = values.repeat_interleave(group, 0)
+        query = q[index].double().reshape(heads, 1, head_dim)
+        expected = F.scaled_dot_product_attention(query, keys, values).reshape(-1)
+        atol, rtol = (3e-5, 3e-5) if dtype == torch.float32 else (2e-2, 2e-2)
+        torch.testing.assert_close(out[index].double(), expected, atol=atol, rtol=rtol)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("window", [0, 5, 16, 40])
+def test_attention_rowwise_portion_and_window(dtype, window):
+    """A portion of 23 queries that continues 30 cached keys; with and without a window;
+    page tails hold NaN to prove they are never read into the result."""
+    from pagedserve_amd.ops import kernels
+    import plain_gpt2
+
+    heads, head_dim, page_size, past, new = 2, 32, 8, 30, 23
+    total = past + new
+    k_pool, v_pool, tables = _paged_fixture(dtype, [total], heads, head_dim, page_size, 23)
+    pages = tables[0, : -(-total // page_size)].long()
+    last = pages[-1]
+    k_pool[last, :, total % page_size:] = float("nan")
+    v_pool[last, :, total % page_size:] = float("nan")
+    keys = _gather(k_pool, tables[0], total, page_size).double()
+    values = _gather(v_pool, tables[0], total, page_size).double()
+    g = torch.Generator().manual_seed(5)
+    q_all = torch.randn((heads, total, head_dim), generator=g).to(dtype).cuda()
+    expected = plain_gpt2.causal_attention(q_all.double().cpu(), keys.cpu(), values.cpu(),
+                                           head_dim ** -0.5, window=window)[:, past:]
+    q = q_all[:, past:].permute(1, 0, 2).reshape(new, heads * head_dim).contiguous()
+    out = torch.empty_like(q)
+    tok_item = torch.zeros(new, dtype=torch.int32, device="cuda")
+    tok_pos = torch.arange(past, total, dtype=torch.int32, device="cuda")
+    kernels.attention_rowwise(q, k_pool, v_pool, out, tok_item, tok_pos, tables, heads,
+                              head_dim ** -0.5, window=window)
+    got = out.double().cpu().reshape(new, heads, head_dim).permute(1, 0, 2)
+    atol, rtol = (3e-5, 3e-5) if dtype == torch.float32 else (2e-2, 2e-2)
+    torch.testing.assert_close(got, expected, atol=atol, rtol=rtol)
+
+
+def test_attention_far_key_stands_out():
+    """One key among 700 is made to dominate: the output must be its value.  A kernel that
+    skips a page, mixes two requests' tables or misplaces an offset fails this."""
+    from pagedserve_amd.ops import kernels
+
+    heads, head_dim, page_size, context = 2, 64, 16, 700
+    for dtype in DTYPES:
+        k_pool, v_pool, tables = _paged_fixture(dtype, [context, context], heads, head_dim, page_size, 31)
+        k_pool *= 0.1
+        q = _rand((2, heads * head_dim), dtype, 32, 0.1)
+        targets = [(0, 0, 3), (0, 1, 367), (1, 0, 688), (1, 1, 699)]
+        for item, head, key in targets:
+            page = int(tables[item, key // page_size])
+            direction = q[item, head * head_dim:(head + 1) * head_dim].float()
+            direction = direction / direction.norm()
+            q[item, head * head_dim:(head + 1) * head_dim] = (direction * 8.0).to(dtype)
+            k_pool[page, head, key % page_size] = (direction * 40.0).to(dtype)
+        out = torch.empty_like(q)
+        tok_item = torch.arange(2, dtype=torch.int32, device="cuda")
+        tok_pos = torch.full((2,), context - 1, dtype=torch.int32, device="cuda")
+        kernels.attention_rowwise(q, k_pool, v_pool, out, tok_item, tok_pos, tables, heads, head_dim ** -0.5)
+        for item, head, key in targets:
+            page = int(tables[item, key // page_size])
+            expected = v_pool[page, head, key % page_size].float()
+            got = out[item, head * head_dim:(head + 1) * head_dim].float()
+            torch.testing.assert_close(got, expected, atol=2e-2, rtol=2e-2)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_kv_write_places_tokens(dtype):
+    """Token t of a request lands at (table[t // page], t % page)
+    (testing/test_project.py:66-88) and nothing else in the pool changes."""
+    from pagedserve_amd.ops import kernels
+
+    kv_heads, head_dim, page_size = 3, 16, 4
+    lens = [5, 9]
+    k_pool, v_pool, tables = _paged_fixture(dtype, lens, kv_heads, head_dim, page_size, 41)
+    before_k, before_v = k_pool.clone(), v_pool.clone()
+    starts = [2, 0]      # request 0 already holds 2 tokens
+    tok_item, tok_pos = [], []
+    for item, (start, length) in enumerate(zip(starts, lens)):
+        for position in range(start, length):
+            tok_item.append(item)
+            tok_pos.append(position)
+    tokens = len(tok_item)
+    wide = _rand((tokens, 5 * kv_heads * head_dim), dtype, 42)
+    k = wide[:, kv_heads * head_dim:2 * kv_heads * head_dim]
+    v = wide[:, 3 * kv_heads * head_dim:4 * kv_heads * head_dim]
+    kernels.kv_write(k, v, k_pool, v_pool, torch.tensor(tok_item, dtype=torch.int32, device="cuda"),
+                     torch.tensor(tok_pos, dtype=torch.int32, device="cuda"), tables)
+    touched = torch.zeros(k_pool.shape[:3], dtype=torch.bool)
+    for t, (item, position) in enumerate(zip(tok_item, tok_pos)):
+        page = int(tables[item, position // page_size])
+        torch.testing.assert_close(k_pool[page, :, position % page_size], k[t].reshape(kv_heads, head_dim), atol=0, rtol=0)
+        torch.testing.assert_close(v_pool[page, :, position % page_size], v[t].reshape(kv_heads, head_dim), atol=0, rtol=0)
+        touched[page, :, position % page_size] = True
+    untouched = ~touched.cuda()
+    assert torch.equal(k_pool[untouched].view(torch.int16 if dtype == torch.bfloat16 else torch.int32),
+                       before_k[untouched].view(torch.int16 if dtype == torch.bfloat16 else torch.int32))
+    assert torch.equal(v_pool[untouched].view(torch.int16 if dtype == torch.bfloat16 else torch.int32),
+                       before_v[untouched].view(torch.int16 if dtype == torch.bfloat16 else torch.int32))
+
+
+def test_sample_argmax_and_ties():
+    from pagedserve_amd.ops import kernels
+
+    for vocab in (7, 257, 1000, 50257):
+        logits = _rand((5, vocab), torch.float32, vocab)
+        logits[2, vocab // 2] = 50.0
+        logits[3, 1] = 60.0
+        logits[3, vocab - 1] = 60.0      # tie: the lowest id wins
+        out = torch.empty(5, dtype=torch.int32, device="cuda")
+        kernels.sample(logits, None, None, out)
+        assert out.tolist() == torch.argmax(logits, dim=-1).tolist()
+        assert out[3].item() == 1
+
+
+def test_sample_temperature_inverse_cdf():
+    from pagedserve_amd.ops import kernels
+
+    vocab = 1000
+    logits = _rand((64, vocab), torch.float32, 77, 2.0)
+    g = torch.Generator().manual_seed(78)
+    uniform = torch.rand(64, generator=g).cuda()
+    temperature = 0.8
+    inv_t = torch.full((64,), 1.0 / temperature, device="cuda")
+    inv_t[0] = 0.0   # greedy row inside a sampling batch
+    out = torch.empty(64, dtype=torch.int32, device="cuda")
+    kernels.sample(logits, inv_t, uniform, out)
+    probs = torch.softmax(logits.double() / temperature, dim=-1)
+    cdf = probs.cumsum(-1)
+    assert out[0].item() == int(torch.argmax(logits[0]))
+    for row in range(1, 64):
+        token = out[row].item()
+        upper = float(cdf[row, token])
+        lower = float(cdf[row, token - 1]) if token > 0 else 0.0
+        assert lower - 1e-5 <= float(uniform[row]) <= upper + 1e-5, (row, token)
+    # frequencies follow the probabilities on a small vocabulary
+    small = torch.tensor([[0.0, 1.0, 2.0, -1.0, 0.5]], device="cuda").repeat(4000, 1)
+    u = torch.rand(4000, generator=g).cuda()
+    toks = torch.empty(4000, dtype=torch.int32, device="cuda")
+    kernels.sample(small, torch.ones(4000, device="cuda"), u, toks)
+    freq = torch.bincount(toks.long().cpu(), minlength=5).double() / 4000
+    assert (freq - torch.softmax(small[0].double().cpu(), -1)).abs().max() < 0.03
+
+
+def test_kernels_refuse_bad_sizes():
+    from pagedserve_amd.ops import kernels
+
+    q = torch.zeros((1, 40), device="cuda")
+    pool = torch.zeros((2, 1, 4, 40), device="cuda")
+    idx = torch.zeros(1, dtype=torch.int32, device="cuda")
+    tables = torch.zeros((1, 2), dtype=torch.int32, device="cuda")
+    with pytest.raises(kernels.KernelError, match="multiple of 16"):
+        kernels.attention_rowwise(q, pool, pool.clone(), q.clone(), idx, idx, tables, 1, 1.0)
+    with pytest.raises(kernels.KernelError, match="GPU"):
+        kernels.norm(torch.zeros(2, 4), torch.ones(4), None, 1e-5, torch.zeros(2, 4))
+    with pytest.raises(kernels.KernelError):
+        kernels.gemm_nt(torch.zeros(2, 8, device="cuda"), torch.zeros(3, 9, device="cuda"), None,
+                        torch.zeros(2, 3, device="cuda"))
