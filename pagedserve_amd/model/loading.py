@@ -39,6 +39,35 @@ def load_model(folder, dtype="float32", device="cuda"):
     return model, config
 
 
+def random_model(config, seed=0, dtype="bfloat16", device="cuda"):
+    """A bound model with random weights of ``config`` (typed, or a raw config.json dict),
+    made in memory: the same draws, layouts and casts as writing a folder and loading it."""
+    from ..weights.loader import target_dtype
+
+    if isinstance(config, dict):
+        architecture = resolve_architecture(config)
+        config = architecture.config_class.from_dict(config)
+    else:
+        architecture = resolve_architecture({"architectures": [config.architecture]})
+    spec = architecture.build_spec(config)
+    engine_dtype = resolve_dtype(dtype)
+    model = DecoderModel(spec, engine_dtype, device)
+    drawn = architecture.random_tensors(config, seed)
+    sources = architecture.weight_sources(config, spec)
+    tensors = {}
+    for target, param in model.parameters().items():
+        source = sources[target]
+        tensor = drawn[source.name]
+        if source.transpose:
+            tensor = tensor.transpose(0, 1)
+        if tuple(tensor.shape) != tuple(param.shape):
+            raise ValueError(f"random tensor {source.name} has shape {tuple(tensor.shape)}, "
+                             f"parameter {target} needs {tuple(param.shape)}")
+        tensors[target] = tensor.to(target_dtype(param.role, engine_dtype)).contiguous().to(device)
+    model.bind(tensors)
+    return model, config
+
+
 def write_random_model(folder, config, seed=0, store_dtype=torch.float32, prefix="transformer."):
     """Write ``config.json`` and ``model.safetensors`` of a random model of ``config``.
 

@@ -1,0 +1,196 @@
+"""Generation through the entry points, long decoding, the first tokens of a sequence,
+sampling, and the command line."""
+
+import os
+import subprocess
+import sys
+
+import pytest
+import torch
+
+import helpers
+import plain_gpt2
+
+pytestmark = pytest.mark.gpu
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+@pytest.fixture(scope="module")
+def folders(tmp_path_factory):
+    base = tmp_path_factory.mktemp("gen_models")
+    return {which: helpers.tiny_folder(base, which) for which in ("A", "B")}
+
+
+# the tiny workloads: A: prompts 5, 17, 31 -> 16 tokens; B: 1, 9, 40, 64, 100 -> 24 tokens,
+# portions of 32, mixed batches
+WORKLOADS = {"A": ([5, 17, 31], 16, dict(scheduling_strategy="orca")),
+             "B": ([1, 9, 40, 64, 100], 24, dict(scheduling_strategy="sarathi", prefill_chunk_size=32,
+                                                max_prefill_requests=2))}
+
+
+@pytest.mark.parametrize("which", ["A", "B"])
+def test_greedy_generation_matches_plain(folders, which):
+    from pagedserve_amd.engine.llm import LLM
+    from pagedserve_amd.sampling import SamplingParams
+
+    folder, config, page_size = folders[which]
+    lengths, new_tokens, options = WORKLOADS[which]
+    prompts = [helpers.random_tokens(n, config["vocab_size"], 300 + i) for i, n in enumerate(lengths)]
+    raw, weights = plain_gpt2.read_model_folder(folder)
+    expected = [plain_gpt2.greedy_generate(raw, weights, prompt, new_tokens) for prompt in prompts]
+    llm = LLM(folder, dtype="float32", block_size=page_size, num_kv_pages=40, max_batch_size=4,
+              eos_token_id=None, **options)
+    outputs = llm.generate(prompts, SamplingParams(max_new_tokens=new_tokens))
+    assert [o.token_ids for o in outputs] == expected
+    assert all(o.finish_reason == "length" for o in outputs)
+    llm.engine.cache.check_invariants()
+    assert not llm.engine.cache.requests
+    # bfloat16 runs the same workload; its tokens follow the rounded model closely
+    llm16 = LLM(folder, dtype="bfloat16", block_size=page_size, num_kv_pages=40, max_batch_size=4,
+                eos_token_id=None, **options)
+    outputs16 = llm16.generate(prompts, SamplingParams(max_new_tokens=new_tokens))
+    first = [o.token_ids[0] for o in outputs16]
+    assert sum(a == e[0] for a, e in zip(first, expected)) >= len(prompts) - 1
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_long_decoding(folders, dtype):
+    """Two prompt tokens, then 250 tokens decoded one by one up to the last position."""
+    from pagedserve_amd.engine import Engine, StepEntry
+    from pagedserve_amd.model import load_model
+
+    folder, config, page_size = folders["B"]
+    tokens = helpers.random_tokens(config["n_positions"], config["vocab_size"], 400)
+    reference = helpers.plain_logits(folder, tokens, bfloat16=dtype == "bfloat16")
+    model, _ = load_model(folder, dtype=dtype)
+    engine = Engine(model, num_pages=config["n_positions"] // page_size, page_size=page_size,
+                    max_requests=2, max_step_tokens=64)
+    rows = {}
+    out = engine.step([StepEntry("r", tokens[:2], [0, 1])])
+    rows[0], rows[1] = out.logits[0].double().cpu(), out.logits[1].double().cpu()
+    for position in range(2, len(tokens)):
+        out = engine.step([StepEntry("r", [tokens[position]], [0])])
+        rows[position] = out.logits[0].double().cpu()
+    error = max(float((rows[p] - reference[p]).abs().max()) for p in rows)
+    scale = float(reference.abs().max())
+    assert error <= helpers.TOLERANCE[dtype] * scale, (error, scale)
+    from pagedserve_amd.engine import StepError
+    with pytest.raises(StepError, match="position"):
+        engine.step([StepEntry("r", [1], [0])])          # the position table is exhausted
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_first_tokens_of_a_sequence(folders, dtype):
+    """Positions 0, 1, 2 in every arrangement: alone, one by one, and beside another request."""
+    from pagedserve_amd.engine import Engine, StepEntry
+    from pagedserve_amd.model import load_model
+
+    folder, config, page_size = folders["A"]
+    tokens = helpers.random_tokens(3, config["vocab_size"], 410)
+    other = helpers.random_tokens(11, config["vocab_size"], 411)
+    reference = helpers.plain_logits(folder, tokens, bfloat16=dtype == "bfloat16")
+    model, _ = load_model(folder, dtype=dtype)
+    engine = Engine(model, num_pages=8, page_size=page_size, max_requests=4, max_step_tokens=32)
+    tolerance = helpers.TOLERANCE[dtype] * float(reference.abs().max())
+    whole = engine.step([StepEntry("a", tokens, [0, 1, 2])]).logits.double().cpu()
+    assert float((whole - reference).abs().max()) <= tolerance
+    for position in range(3):
+        entries = [StepEntry("b", [tokens[position]], [0])]
+        if position == 1:
+            entries.insert(0, StepEntry("c", other, [10]))
+        got = engine.step(entries).logits[-1].double().cpu()
+        assert float((got - reference[position]).abs().max()) <= tolerance
+    single = engine.step([StepEntry("d", tokens[:1], [0])]).logits[0].double().cpu()
+    assert float((single - reference[0]).abs().max()) <= tolerance
+
+
+def test_step_refuses_what_it_cannot_run(folders):
+    from pagedserve_amd.cache import CacheFull
+    from pagedserve_amd.engine import Engine, StepEntry, StepError
+    from pagedserve_amd.model import load_model
+
+    folder, config, page_size = folders["A"]
+    model, _ = load_model(folder, dtype="float32")
+    engine = Engine(model, num_pages=4, page_size=page_size, max_requests=2, max_step_tokens=16)
+    with pytest.raises(StepError, match="at least one"):
+        engine.step([])
+    with pytest.raises(StepError, match="twice"):
+        engine.step([StepEntry("a", [1], []), StepEntry("a", [2], [])])
+    with pytest.raises(StepError, match="vocabulary"):
+        engine.step([StepEntry("a", [config["vocab_size"]], [])])
+    with pytest.raises(StepError, match="place"):
+        engine.step([StepEntry("a", [1, 2], [2])])
+    with pytest.raises(StepError, match="max_step_tokens"):
+        engine.step([StepEntry("a", [1] * 17, [])])
+    with pytest.raises(StepError, match="live requests"):
+        engine.step([StepEntry("a", [1], []), StepEntry("b", [1], []), StepEntry("c", [1], [])])
+    engine.step([StepEntry("a", [1] * 16, [])])
+    engine.step([StepEntry("a", [1] * 16, [])])
+    with pytest.raises(CacheFull):
+        engine.step([StepEntry("b", [1], [0])])            # all four pages are held by "a"
+    assert not engine.is_live("b")                          # a refused newcomer leaves no trace
+    engine.cache.check_invariants()
+    engine.finish("a")
+    assert engine.step([StepEntry("b", [1], [0])]).logits.shape == (1, config["vocab_size"])
+
+
+def test_temperature_sampling_is_reproducible_and_batch_independent(folders):
+    from pagedserve_amd.engine.llm import LLM
+    from pagedserve_amd.sampling import SamplingParams, uniform_for
+
+    folder, config, page_size = folders["A"]
+    prompts = [helpers.random_tokens(n, config["vocab_size"], 500 + n) for n in (4, 9, 13)]
+    params = SamplingParams(temperature=0.8, seed=7, max_new_tokens=12)
+    kwargs = dict(dtype="float32", block_size=page_size, num_kv_pages=32, max_batch_size=4, eos_token_id=None)
+    together = [o.token_ids for o in LLM(folder, **kwargs).generate(prompts, params)]
+    again = [o.token_ids for o in LLM(folder, **kwargs).generate(prompts, params)]
+    assert together == again
+    # request ids are part of the key: the same prompts alone, as request 0, 1, 2 of their own engines
+    alone = LLM(folder, scheduling_strategy="sarathi", prefill_chunk_size=3, **kwargs)
+    assert [o.token_ids for o in alone.generate(prompts, params)] == together
+    other_seed = [o.token_ids for o in LLM(folder, **kwargs).generate(
+        prompts, SamplingParams(temperature=0.8, seed=8, max_new_tokens=12))]
+    assert other_seed != together
+    # each drawn token is the inverse-CDF point of the plain model's distribution at the same uniform number
+    raw, weights = plain_gpt2.read_model_folder(folder)
+    checked = 0
+    for request, (prompt, tokens) in enumerate(zip(prompts, together)):
+        sequence = list(prompt)
+        for index, token in enumerate(tokens):
+            logits = plain_gpt2.forward_logits(raw, weights, sequence)[-1]
+            cdf = torch.softmax(logits / 0.8, dim=-1).cumsum(-1)
+            u = uniform_for(7, request, index)
+            upper = float(cdf[token])
+            lower = float(cdf[token - 1]) if token > 0 else 0.0
+            assert lower - 1e-4 <= u <= upper + 1e-4, (request, index, token, u, lower, upper)
+            sequence.append(token)
+            checked += 1
+    assert checked == 36
+
+
+def test_command_line(folders):
+    """main.py as a user runs it: the built-in random model with the byte tokenizer, and a folder."""
+    run = subprocess.run([sys.executable, os.path.join(ROOT, "main.py"), "--dtype", "bfloat16",
+                          "--strategy", "sarathi", "--prefill-chunk-size", "4", "--max-batch-size", "4",
+                          "--kv-cache-memory-mb", "8"], capture_output=True, text=True, timeout=600)
+    assert run.returncode == 0, run.stderr[-2000:]
+    lines = [line for line in run.stdout.splitlines() if line.startswith("request ")]
+    assert len(lines) == 2 and lines[0].startswith("request 0:")
+    folder, config, page_size = folders["A"]
+    prompt = helpers.random_tokens(6, config["vocab_size"], 600)
+    run = subprocess.run([sys.executable, os.path.join(ROOT, "main.py"), "--model", folder,
+                          "--prompt-ids", ",".join(map(str, prompt)), "--max-new-tokens", "5",
+                          "--block-size", str(page_size), "--num-kv-pages", "16", "--ignore-eos"],
+                         capture_output=True, text=True, timeout=600)
+    assert run.returncode == 0, run.stderr[-2000:]
+    raw, weights = plain_gpt2.read_model_folder(folder)
+    expected = plain_gpt2.greedy_generate(raw, weights, prompt, 5)
+    assert f"tokens={expected}" in run.stdout
+
+
+def test_smoke_entry():
+    sys.path.insert(0, ROOT)
+    import __graft_entry__
+
+    __graft_entry__.smoke()

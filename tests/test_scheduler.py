@@ -1,0 +1,290 @@
+"""The scheduler's decisions, on the CPU, above a stand-in for the step function that does
+the cache bookkeeping of the real engine and returns made-up logits."""
+
+import random
+from types import SimpleNamespace
+
+import pytest
+import torch
+
+from pagedserve_amd.cache import CacheGroupSpec, CacheManager
+from pagedserve_amd.engine.engine import StepOutput
+from pagedserve_amd.engine.scheduler import (ORCA_STRATEGY, SARATHI_STRATEGY,
+                                             ContinuousBatchScheduler)
+from pagedserve_amd.sampling import SamplingParams, uniform_for
+
+VOCAB = 50
+
+
+class FakeEngine:
+    """Cache bookkeeping as in Engine.step; logits put all mass on a token that depends on
+    the request's whole history, so outputs tell whether every token arrived in order."""
+
+    def __init__(self, pages=64, page_size=4, max_requests=8, max_step_tokens=64, max_positions=128,
+                 window=0):
+        self.spec = SimpleNamespace(vocab_size=VOCAB, max_positions=max_positions)
+        groups = [CacheGroupSpec((0,), 1, 16, 0)]
+        if window:
+            groups.append(CacheGroupSpec((1,), 1, 16, window))
+        self.cache = CacheManager(groups, pages, page_size, max_requests, torch.float32, "cpu",
+                                  max_positions=max_positions, allocate_pools=False)
+        self.max_requests = max_requests
+        self.max_step_tokens = max_step_tokens
+        self.history = {}
+        self.steps = []
+        self.fail_next = False
+
+    def step(self, entries):
+        if self.fail_next:
+            self.fail_next = False
+            raise RuntimeError("injected failure")
+        assert sum(len(e.tokens) for e in entries) <= self.max_step_tokens
+        assert len({e.request_id for e in entries}) == len(entries)
+        rows = []
+        for entry in entries:
+            if entry.request_id not in self.cache.requests:
+                self.cache.admit(entry.request_id)
+                self.history[entry.request_id] = []
+            start = self.cache.length(entry.request_id)
+            self.cache.grow(entry.request_id, start + len(entry.tokens))
+        for entry in entries:
+            start = self.cache.length(entry.request_id)
+            self.history[entry.request_id].extend(entry.tokens)
+            self.cache.commit(entry.request_id, start + len(entry.tokens))
+            for place in entry.want:
+                assert place == len(entry.tokens) - 1
+                seen = self.history[entry.request_id]
+                row = torch.zeros(VOCAB)
+                row[(sum(seen) * 7 + len(seen)) % (VOCAB - 1)] = 5.0   # never VOCAB-1 (the end token)
+                rows.append(row)
+        self.steps.append([(e.request_id, list(e.tokens), list(e.want)) for e in entries])
+        self.cache.check_invariants()
+        logits = torch.stack(rows) if rows else torch.zeros((0, VOCAB))
+        return StepOutput(logits=logits, rows=[])
+
+    def finish(self, request_id):
+        self.cache.release(request_id)
+        del self.history[request_id]
+
+
+class ArgmaxSampler:
+    def sample(self, logits, params, keys, indices, seeds):
+        return logits.argmax(-1).tolist()
+
+
+def expected_tokens(prompt, count):
+    seen, out = list(prompt), []
+    for _ in range(count):
+        token = (sum(seen) * 7 + len(seen)) % (VOCAB - 1)
+        out.append(token)
+        seen.append(token)
+    return out
+
+
+def make(strategy=ORCA_STRATEGY, engine=None, **kwargs):
+    engine = engine or FakeEngine()
+    kwargs.setdefault("max_batch_size", engine.max_requests)
+    return ContinuousBatchScheduler(engine, ArgmaxSampler(), tokenizer=None,
+                                    scheduling_strategy=strategy, **kwargs), engine
+
+
+def test_orca_runs_whole_prompts_together():
+    # testing/test_project.py:940-988: two prompts of different length in one step,
+    # finished after two tokens, nothing reserved, nothing left in the manager
+    scheduler, engine = make(max_batch_size=4)
+    a = scheduler.add_token_request([1, 2, 3], max_new_tokens=2)
+    b = scheduler.add_token_request([4, 5, 6, 7, 8], max_new_tokens=2)
+    first = scheduler.step()
+    assert set(first) == {a, b}
+    assert engine.steps[0] == [(a, [1, 2, 3], [2]), (b, [4, 5, 6, 7, 8], [4])]
+    second = scheduler.step()
+    assert set(second) == {a, b} and not scheduler.has_work()
+    assert engine.steps[1] == [(a, [first[a]], [0]), (b, [first[b]], [0])]
+    assert scheduler.reserved_blocks == [0] and not engine.cache.requests
+    assert scheduler.finished[a].generated_token_ids == expected_tokens([1, 2, 3], 2)
+    assert scheduler.finished[b].finish_reason == "length"
+    assert scheduler.step() == {}
+
+
+def test_sarathi_chunks_and_piggybacks():
+    # testing/test_project.py:991-1051: chunk 2 -> {}, {}, {A}; B's first portion rides with A's decode
+    scheduler, engine = make(SARATHI_STRATEGY, prefill_chunk_size=2, max_batch_size=4)
+    a = scheduler.add_token_request([1, 2, 3, 4, 5], max_new_tokens=3)
+    assert scheduler.step() == {} and scheduler.waiting[0].prefill_cursor == 2
+    assert scheduler.step() == {} and scheduler.waiting[0].prefill_cursor == 4
+    assert engine.cache.length(a) == 4
+    emitted = scheduler.step()
+    assert set(emitted) == {a} and not scheduler.waiting and a in scheduler.active
+    assert [step[0][2] for step in engine.steps] == [[], [], [0]]
+    b = scheduler.add_token_request([9, 8, 7], max_new_tokens=1)
+    emitted = scheduler.step()
+    assert set(emitted) == {a}
+    assert engine.steps[-1] == [(a, [scheduler.active[a].generated_token_ids[0]], [0]), (b, [9, 8], [])]
+    assert engine.cache.length(a) == 6 and engine.cache.length(b) == 2
+    emitted = scheduler.step()
+    assert set(emitted) == {a, b}
+    assert not scheduler.has_work()
+    assert scheduler.finished[a].generated_token_ids == expected_tokens([1, 2, 3, 4, 5], 3)
+    assert scheduler.finished[b].generated_token_ids == expected_tokens([9, 8, 7], 1)
+
+
+def test_token_budget_cuts_prompts_in_both_strategies():
+    for strategy in (ORCA_STRATEGY, SARATHI_STRATEGY):
+        scheduler, engine = make(strategy, max_num_batched_tokens=6, prefill_chunk_size=4,
+                                 max_prefill_requests=8)
+        a = scheduler.add_token_request(list(range(1, 11)), max_new_tokens=2)
+        b = scheduler.add_token_request([3, 3, 3], max_new_tokens=2)
+        scheduler.run_until_complete()
+        assert all(sum(len(tokens) for _, tokens, _ in step) <= 6 for step in engine.steps)
+        assert scheduler.finished[a].generated_token_ids == expected_tokens(list(range(1, 11)), 2)
+        assert scheduler.finished[b].generated_token_ids == expected_tokens([3, 3, 3], 2)
+        portions = [len(tokens) for step in engine.steps for rid, tokens, _ in step if rid == a and len(tokens) > 1]
+        assert sum(portions) == 10 and max(portions) <= (6 if strategy == ORCA_STRATEGY else 4)
+
+
+def test_results_do_not_depend_on_strategy_chunk_or_batch_limit():
+    prompts = [[(i * 5 + j) % VOCAB for j in range(3 + 4 * i)] for i in range(6)]
+    outputs = []
+    for strategy, kwargs in ((ORCA_STRATEGY, {}), (ORCA_STRATEGY, {"max_batch_size": 2}),
+                             (SARATHI_STRATEGY, {"prefill_chunk_size": 2}),
+                             (SARATHI_STRATEGY, {"prefill_chunk_size": 5, "max_prefill_requests": 3}),
+                             (ORCA_STRATEGY, {"max_num_batched_tokens": 7})):
+        scheduler, _ = make(strategy, **kwargs)
+        ids = [scheduler.add_token_request(p, max_new_tokens=4 + i) for i, p in enumerate(prompts)]
+        scheduler.run_until_complete()
+        outputs.append([scheduler.finished[i].generated_token_ids for i in ids])
+        assert all(len(tokens) == 4 + i for i, tokens in enumerate(outputs[-1]))
+    assert all(out == outputs[0] for out in outputs)
+    assert outputs[0] == [expected_tokens(p, 4 + i) for i, p in enumerate(prompts)]
+
+
+def test_when_pages_run_out_requests_wait_in_order():
+    # 6 pages of 4 tokens.  Each request reserves ceil((6 + 6) / 4) = 3 pages: two fit.
+    engine = FakeEngine(pages=6, page_size=4)
+    scheduler, _ = make(engine=engine, max_batch_size=8)
+    ids = [scheduler.add_token_request([i + 1] * 6, max_new_tokens=6) for i in range(4)]
+    scheduler.step()
+    assert scheduler.reserved_blocks == [6]
+    assert [rid for rid, _, _ in engine.steps[0]] == ids[:2]       # the third waits, and so does the fourth
+    assert [r.request_id for r in scheduler.waiting] == ids[2:]
+    small = scheduler.add_token_request([7], max_new_tokens=1)     # would fit, but may not overtake
+    order = []
+    while scheduler.has_work():
+        before = set(scheduler.finished)
+        scheduler.step()
+        order.extend(sorted(set(scheduler.finished) - before))
+        assert scheduler.reserved_blocks[0] <= 6
+        engine.cache.check_invariants()
+    assert order.index(small) > order.index(ids[2])
+    assert scheduler.reserved_blocks == [0] and engine.cache.pools[0].num_free == 6
+    for i, rid in enumerate(ids):
+        assert scheduler.finished[rid].generated_token_ids == expected_tokens([i + 1] * 6, 6)
+    # sarathi: the head of the queue waits likewise while decodes go on
+    engine = FakeEngine(pages=6, page_size=4)
+    scheduler, _ = make(SARATHI_STRATEGY, engine=engine, prefill_chunk_size=8)
+    ids = [scheduler.add_token_request([i + 1] * 6, max_new_tokens=6) for i in range(3)]
+    scheduler.run_until_complete()
+    assert all(len(scheduler.finished[rid].generated_token_ids) == 6 for rid in ids)
+
+
+def test_request_that_can_never_fit_is_refused_at_once():
+    engine = FakeEngine(pages=3, page_size=4)
+    scheduler, _ = make(engine=engine)
+    with pytest.raises(ValueError, match="never be scheduled"):
+        scheduler.add_token_request([1] * 10, max_new_tokens=5)
+    assert not scheduler.waiting
+    scheduler.add_token_request([1] * 6, max_new_tokens=6)          # exactly 3 pages
+    scheduler.run_until_complete()
+
+
+def test_request_validation():
+    scheduler, _ = make()
+    for bad in ([], [1, VOCAB], [-1], [1.5], [True]):
+        with pytest.raises(ValueError):
+            scheduler.add_token_request(bad, max_new_tokens=1)
+    with pytest.raises(ValueError):
+        scheduler.add_token_request([1], max_new_tokens=0)
+    with pytest.raises(ValueError, match="context limit"):
+        scheduler.add_token_request([1] * 100, max_new_tokens=29)   # 129 > 128
+    scheduler.add_token_request([1] * 100, max_new_tokens=28)
+    with pytest.raises(ValueError, match="tokenizer"):
+        scheduler.add_request("hello")
+    with pytest.raises(ValueError, match="strategy"):
+        make("fifo")
+    with pytest.raises(ValueError):
+        make(max_batch_size=0)
+    with pytest.raises(ValueError):
+        make(max_batch_size=100)
+    with pytest.raises(ValueError):
+        make(max_num_batched_tokens=10 ** 6)
+
+
+def test_end_token_stops_unless_ignored():
+    class EosSampler:
+        def sample(self, logits, params, keys, indices, seeds):
+            return [VOCAB - 1 if index == 1 else 3 for index in indices]
+
+    engine = FakeEngine()
+    scheduler = ContinuousBatchScheduler(engine, EosSampler(), eos_token_id=VOCAB - 1, max_batch_size=8)
+    a = scheduler.add_token_request([1, 2], max_new_tokens=5)
+    b = scheduler.add_token_request([1, 2], max_new_tokens=5, sampling=SamplingParams(ignore_eos=True, max_new_tokens=5))
+    scheduler.run_until_complete()
+    assert scheduler.finished[a].generated_token_ids == [3, VOCAB - 1]
+    assert scheduler.finished[a].finish_reason == "stop"
+    assert len(scheduler.finished[b].generated_token_ids) == 5 and scheduler.finished[b].finish_reason == "length"
+    assert not engine.cache.requests
+
+
+def test_failed_step_unreserves_new_requests():
+    scheduler, engine = make()
+    a = scheduler.add_token_request([1, 2, 3], max_new_tokens=2)
+    engine.fail_next = True
+    with pytest.raises(RuntimeError, match="injected"):
+        scheduler.step()
+    # src/scheduler/orca_scheduler.py:243-247
+    assert scheduler.reserved_blocks == [0] and scheduler.waiting[0].reserved_blocks == []
+    scheduler.run_until_complete()
+    assert scheduler.finished[a].generated_token_ids == expected_tokens([1, 2, 3], 2)
+
+
+def test_window_group_reserves_less():
+    engine = FakeEngine(pages=[40, 6], page_size=4, window=8, max_step_tokens=8)
+    scheduler, _ = make(SARATHI_STRATEGY, engine=engine, prefill_chunk_size=8)
+    rid = scheduler.add_token_request([2] * 60, max_new_tokens=20)
+    assert scheduler._required_blocks(scheduler.waiting[0]) == [20, 5]
+    scheduler.run_until_complete()
+    assert len(scheduler.finished[rid].generated_token_ids) == 20
+    assert engine.cache.pools[1].peak_allocated <= 5
+
+
+@pytest.mark.parametrize("seed", range(5))
+def test_random_arrivals_finish_with_exact_outputs(seed):
+    rng = random.Random(seed)
+    strategy = rng.choice([ORCA_STRATEGY, SARATHI_STRATEGY])
+    engine = FakeEngine(pages=rng.choice([12, 20, 64]), page_size=4, max_requests=6, max_step_tokens=32)
+    scheduler, _ = make(strategy, engine=engine, max_batch_size=rng.choice([2, 4, 6]),
+                        prefill_chunk_size=rng.choice([1, 3, 8]), max_num_batched_tokens=rng.choice([8, 32]))
+    expected = {}
+    pending = 25
+    while pending or scheduler.has_work():
+        if pending and rng.random() < 0.5:
+            prompt = [rng.randrange(VOCAB) for _ in range(rng.randint(1, 20))]
+            count = rng.randint(1, 12)
+            expected[scheduler.add_token_request(prompt, max_new_tokens=count)] = expected_tokens(prompt, count)
+            pending -= 1
+        if scheduler.has_work():
+            scheduler.step()
+    assert {rid: r.generated_token_ids for rid, r in scheduler.finished.items()} == expected
+    assert scheduler.reserved_blocks == [0] and not engine.cache.requests
+
+
+def test_uniform_numbers_are_a_function_of_seed_request_and_index():
+    a = uniform_for(7, 3, 0)
+    assert a == uniform_for(7, 3, 0) and 0.0 <= a < 1.0
+    assert len({uniform_for(7, 3, i) for i in range(100)}) == 100
+    assert uniform_for(7, 4, 0) != a and uniform_for(8, 3, 0) != a
+    values = [uniform_for(1, r, i) for r in range(50) for i in range(200)]
+    assert abs(sum(values) / len(values) - 0.5) < 0.01
+    assert float(torch.tensor(values, dtype=torch.float32).max()) < 1.0
+    with pytest.raises(ValueError):
+        SamplingParams(temperature=-1)
