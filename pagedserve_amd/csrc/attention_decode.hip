@@ -1,0 +1,295 @@
+// Split-KV paged attention for single queries: the decode kernel.
+//
+// One 256-thread block per (query token, head, split).  A token's visible keys are cut into
+// `splits` contiguous ranges so that a small batch still fills the chip (the reference's
+// Triton kernel runs one program per (request, head), src/kernels/triton_paged_attention.py:
+// 84-86, which leaves most CUs idle at batch 1).  Inside a block, LPK lanes share one key:
+// each lane loads 8 consecutive head dimensions of it (16 bytes of bfloat16), so a wave's
+// load of 64/LPK keys is one contiguous run inside a page; the partial dot products are
+// summed over the LPK lanes with shuffles.  Every lane group keeps its own online-softmax
+// state (running max m, sum l, 8 accumulators; float, as in src/kernels/
+// triton_paged_attention.py:219-223) over the keys it visits and the states are merged once
+// at the end: across lane groups by shuffles, across the four waves through LDS.  With one
+// split the block writes the output; otherwise it writes (acc, m, l) and
+// attention_reduce_kernel merges the splits.
+#include <math.h>
+
+#include "common.h"
+#include "pagedserve_hip.h"
+
+#define AD_UNROLL 4
+#define AD_WAVES 4
+
+template <typename T>
+__device__ inline void load8(const T* p, float* out);
+
+template <>
+__device__ inline void load8<float>(const float* p, float* out) {
+  const float4 a = *reinterpret_cast<const float4*>(p);
+  const float4 b = *reinterpret_cast<const float4*>(p + 4);
+  out[0] = a.x; out[1] = a.y; out[2] = a.z; out[3] = a.w;
+  out[4] = b.x; out[5] = b.y; out[6] = b.z; out[7] = b.w;
+}
+
+template <>
+__device__ inline void load8<bf16_t>(const bf16_t* p, float* out) {
+  const uint4 raw = *reinterpret_cast<const uint4*>(p);
+  const uint32_t w[4] = {raw.x, raw.y, raw.z, raw.w};
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    out[2 * i] = __uint_as_float(w[i] << 16);
+    out[2 * i + 1] = __uint_as_float(w[i] & 0xffff0000u);
+  }
+}
+
+// Merge the online-softmax state (m, l, acc) with another one.
+__device__ inline void merge_state(float& m, float& l, float* acc, float m_o, float l_o,
+                                   const float* acc_o, int n) {
+  const float m_n = fmaxf(m, m_o);
+  const float c1 = (m == -INFINITY) ? 0.f : expf(m - m_n);
+  const float c2 = (m_o == -INFINITY) ? 0.f : expf(m_o - m_n);
+  l = l * c1 + l_o * c2;
+  for (int i = 0; i < n; ++i) acc[i] = acc[i] * c1 + acc_o[i] * c2;
+  m = m_n;
+}
+
+template <typename T, int LPK>
+__global__ __launch_bounds__(64 * AD_WAVES) void attention_decode_kernel(
+    const T* __restrict__ q, int64_t q_stride, const T* __restrict__ k_pool,
+    const T* __restrict__ v_pool, T* __restrict__ out, int64_t out_stride,
+    float* __restrict__ partial, const int* __restrict__ tok_list,
+    const int* __restrict__ tok_item, const int* __restrict__ tok_pos,
+    const int* __restrict__ tables, int table_width, int heads, int kv_heads, int head_dim,
+    int page_size, int page_shift, int num_pages, float scale, int window, int splits) {
+  constexpr int GROUPS = 64 / LPK;               // keys per wave load
+  constexpr int KEYS_PER_WAVE = GROUPS * AD_UNROLL;
+  __shared__ float s_acc[AD_WAVES][256];
+  __shared__ float s_ml[AD_WAVES][2];
+
+  const int n = blockIdx.x;
+  const int head = blockIdx.y;
+  const int split = blockIdx.z;
+  const int t = tok_list ? tok_list[n] : n;
+  const int kv_head = head / (heads / kv_heads);
+  const int lane = threadIdx.x & 63;
+  const int wave = threadIdx.x >> 6;
+  const int group = lane / LPK;
+  const int dim0 = (lane % LPK) * 8;
+  const bool has_dims = dim0 < head_dim;
+
+  const int pos = tok_pos[t];
+  const int* table = tables + (int64_t)tok_item[t] * table_width;
+  const int first_key = (window > 0 && pos - window + 1 > 0) ? pos - window + 1 : 0;
+  const int end_key = pos + 1;
+  int chunk = (end_key - first_key + splits - 1) / splits;
+  chunk = (chunk + KEYS_PER_WAVE - 1) / KEYS_PER_WAVE * KEYS_PER_WAVE;
+  const int range_begin = first_key + split * chunk;
+  const int range_end = range_begin + chunk < end_key ? range_begin + chunk : end_key;
+
+  float qf[8];
+#pragma unroll
+  for (int i = 0; i < 8; ++i)
+    qf[i] = has_dims ? to_float<T>(q[(int64_t)t * q_stride + (int64_t)head * head_dim + dim0 + i])
+                     : 0.f;
+
+  float m = -INFINITY, l = 0.f;
+  float acc[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+
+  for (int base = range_begin + wave * KEYS_PER_WAVE; base < range_end;
+       base += AD_WAVES * KEYS_PER_WAVE) {
+    float kf[AD_UNROLL][8], vf[AD_UNROLL][8];
+    bool valid[AD_UNROLL];
+#pragma unroll
+    for (int u = 0; u < AD_UNROLL; ++u) {
+      const int key = base + u * GROUPS + group;
+      valid[u] = false;
+      if (key < range_end) {
+        const int logical = page_shift >= 0 ? (key >> page_shift) : key / page_size;
+        const int page = logical < table_width ? table[logical] : -1;
+        if (page >= 0 && page < num_pages) {
+          valid[u] = true;
+          if (has_dims) {
+            const int64_t offset =
+                (((int64_t)page * kv_heads + kv_head) * page_size + (key - logical * page_size)) *
+                    head_dim + dim0;
+            load8<T>(k_pool + offset, kf[u]);
+            load8<T>(v_pool + offset, vf[u]);
+          }
+        }
+      }
+      if (!valid[u] || !has_dims) {
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+          kf[u][i] = 0.f;
+          vf[u][i] = 0.f;
+        }
+      }
+    }
+    float s[AD_UNROLL];
+    float m_new = m;
+#pragma unroll
+    for (int u = 0; u < AD_UNROLL; ++u) {
+      float dot = 0.f;
+#pragma unroll
+      for (int i = 0; i < 8; ++i) dot = fmaf(qf[i], kf[u][i], dot);
+#pragma unroll
+      for (int offset = LPK / 2; offset > 0; offset >>= 1) dot += __shfl_xor(dot, offset, 64);
+      s[u] = valid[u] ? dot * scale : -INFINITY;
+      m_new = fmaxf(m_new, s[u]);
+    }
+    if (m_new != -INFINITY) {
+      const float correction = (m == -INFINITY) ? 0.f : expf(m - m_new);
+      l *= correction;
+#pragma unroll
+      for (int i = 0; i < 8; ++i) acc[i] *= correction;
+#pragma unroll
+      for (int u = 0; u < AD_UNROLL; ++u) {
+        const float p = valid[u] ? expf(s[u] - m_new) : 0.f;
+        l += p;
+#pragma unroll
+        for (int i = 0; i < 8; ++i) acc[i] = fmaf(p, vf[u][i], acc[i]);
+      }
+      m = m_new;
+    }
+  }
+
+  // merge the lane groups of this wave
+#pragma unroll
+  for (int offset = LPK; offset < 64; offset <<= 1) {
+    const float m_o = __shfl_xor(m, offset, 64);
+    const float l_o = __shfl_xor(l, offset, 64);
+    float acc_o[8];
+#pragma unroll
+    for (int i = 0; i < 8; ++i) acc_o[i] = __shfl_xor(acc[i], offset, 64);
+    merge_state(m, l, acc, m_o, l_o, acc_o, 8);
+  }
+  if (group == 0 && has_dims) {
+#pragma unroll
+    for (int i = 0; i < 8; ++i) s_acc[wave][dim0 + i] = acc[i];
+  }
+  if (lane == 0) {
+    s_ml[wave][0] = m;
+    s_ml[wave][1] = l;
+  }
+  __syncthreads();
+
+  // merge the waves: one thread per head dimension
+  const int d = threadIdx.x;
+  float block_m = -INFINITY;
+#pragma unroll
+  for (int w = 0; w < AD_WAVES; ++w) block_m = fmaxf(block_m, s_ml[w][0]);
+  float block_l = 0.f, value = 0.f;
+#pragma unroll
+  for (int w = 0; w < AD_WAVES; ++w) {
+    const float c = (s_ml[w][0] == -INFINITY) ? 0.f : expf(s_ml[w][0] - block_m);
+    block_l += s_ml[w][1] * c;
+    if (d < head_dim) value += s_acc[w][d] * c;
+  }
+  if (splits == 1) {
+    if (d < head_dim)
+      out[(int64_t)t * out_stride + (int64_t)head * head_dim + d] = from_float<T>(value / block_l);
+  } else {
+    float* dst = partial + (((int64_t)n * heads + head) * splits + split) * (head_dim + 2);
+    if (d < head_dim) dst[d] = value;
+    if (d == 0) {
+      dst[head_dim] = block_m;
+      dst[head_dim + 1] = block_l;
+    }
+  }
+}
+
+// out = sum_s acc_s e^{m_s - M} / sum_s l_s e^{m_s - M}
+template <typename T>
+__global__ __launch_bounds__(64) void attention_reduce_kernel(
+    const float* __restrict__ partial, T* __restrict__ out, int64_t out_stride,
+    const int* __restrict__ tok_list, int heads, int head_dim, int splits) {
+  const int n = blockIdx.x;
+  const int head = blockIdx.y;
+  const int t = tok_list ? tok_list[n] : n;
+  const float* src = partial + ((int64_t)n * heads + head) * splits * (head_dim + 2);
+  float total_m = -INFINITY;
+  for (int s = 0; s < splits; ++s) total_m = fmaxf(total_m, src[s * (head_dim + 2) + head_dim]);
+  float total_l = 0.f;
+  for (int s = 0; s < splits; ++s) {
+    const float m_s = src[s * (head_dim + 2) + head_dim];
+    if (m_s != -INFINITY) total_l += src[s * (head_dim + 2) + head_dim + 1] * expf(m_s - total_m);
+  }
+  for (int d = threadIdx.x; d < head_dim; d += 64) {
+    float value = 0.f;
+    for (int s = 0; s < splits; ++s) {
+      const float m_s = src[s * (head_dim + 2) + head_dim];
+      if (m_s != -INFINITY) value += src[s * (head_dim + 2) + d] * expf(m_s - total_m);
+    }
+    out[(int64_t)t * out_stride + (int64_t)head * head_dim + d] = from_float<T>(value / total_l);
+  }
+}
+
+template <typename T>
+static int launch_decode(const void* q, int64_t q_stride, const void* k_pool, const void* v_pool,
+                         void* out, int64_t out_stride, float* partial, const int* tok_list,
+                         const int* tok_item, const int* tok_pos, const int* tables,
+                         int table_width, int count, int heads, int kv_heads, int head_dim,
+                         int page_size, int num_pages, float scale, int window, int splits,
+                         hipStream_t s) {
+  int page_shift = -1;
+  if ((page_size & (page_size - 1)) == 0) {
+    page_shift = 0;
+    while ((1 << page_shift) < page_size) ++page_shift;
+  }
+  dim3 grid(count, heads, splits);
+  dim3 block(64 * AD_WAVES);
+#define PS_LAUNCH_AD(LPK)                                                                        \
+  hipLaunchKernelGGL((attention_decode_kernel<T, LPK>), grid, block, 0, s, (const T*)q, q_stride, \
+                     (const T*)k_pool, (const T*)v_pool, (T*)out, out_stride, partial, tok_list, \
+                     tok_item, tok_pos, tables, table_width, heads, kv_heads, head_dim,          \
+                     page_size, page_shift, num_pages, scale, window, splits)
+  const int lanes = head_dim / 8;
+  if (lanes <= 2) PS_LAUNCH_AD(2);
+  else if (lanes <= 4) PS_LAUNCH_AD(4);
+  else if (lanes <= 8) PS_LAUNCH_AD(8);
+  else if (lanes <= 16) PS_LAUNCH_AD(16);
+  else PS_LAUNCH_AD(32);
+#undef PS_LAUNCH_AD
+  PS_CHECK_LAUNCH("ps_attention_decode");
+  if (splits > 1) {
+    hipLaunchKernelGGL(attention_reduce_kernel<T>, dim3(count, heads), dim3(64), 0, s, partial,
+                       (T*)out, out_stride, tok_list, heads, head_dim, splits);
+    PS_CHECK_LAUNCH("ps_attention_decode(reduce)");
+  }
+  return 0;
+}
+
+extern "C" int ps_attention_decode(const void* q, int64_t q_stride, const void* k_pool,
+                                   const void* v_pool, void* out, int64_t out_stride,
+                                   float* partial, int64_t partial_floats, const int* tok_list,
+                                   const int* tok_item, const int* tok_pos, const int* tables,
+                                   int table_width, int count, int heads, int kv_heads,
+                                   int head_dim, int page_size, int num_pages, float scale,
+                                   int window, int splits, int dtype, void* stream) {
+  PS_REQUIRE(count >= 0 && heads > 0 && kv_heads > 0 && page_size > 0 && num_pages > 0 &&
+                 table_width > 0,
+             "ps_attention_decode: bad sizes");
+  PS_REQUIRE(heads % kv_heads == 0,
+             "ps_attention_decode: heads (%d) must be a multiple of kv_heads (%d)", heads, kv_heads);
+  PS_REQUIRE(head_dim > 0 && head_dim % 16 == 0 && head_dim <= 256,
+             "ps_attention_decode: head_dim %d must be a multiple of 16 up to 256", head_dim);
+  PS_REQUIRE(window >= 0, "ps_attention_decode: negative window");
+  PS_REQUIRE(splits >= 1 && splits <= 65535 && heads <= 65535,
+             "ps_attention_decode: splits %d / heads %d out of range", splits, heads);
+  PS_REQUIRE(dtype == PS_F32 || dtype == PS_BF16, "ps_attention_decode: unknown dtype %d", dtype);
+  if (splits > 1) {
+    const int64_t need = (int64_t)count * heads * splits * (head_dim + 2);
+    PS_REQUIRE(partial != nullptr && partial_floats >= need,
+               "ps_attention_decode: %lld floats of scratch needed for %d splits, %lld given",
+               (long long)need, splits, (long long)partial_floats);
+  }
+  if (count == 0) return 0;
+  hipStream_t s = (hipStream_t)stream;
+  if (dtype == PS_F32)
+    return launch_decode<float>(q, q_stride, k_pool, v_pool, out, out_stride, partial, tok_list,
+                                tok_item, tok_pos, tables, table_width, count, heads, kv_heads,
+                                head_dim, page_size, num_pages, scale, window, splits, s);
+  return launch_decode<bf16_t>(q, q_stride, k_pool, v_pool, out, out_stride, partial, tok_list,
+                               tok_item, tok_pos, tables, table_width, count, heads, kv_heads,
+                               head_dim, page_size, num_pages, scale, window, splits, s);
+}

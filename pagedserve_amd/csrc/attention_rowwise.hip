@@ -19,14 +19,14 @@ template <typename T>
 __global__ __launch_bounds__(64) void attention_rowwise_kernel(
     const T* __restrict__ q, int64_t q_stride, const T* __restrict__ k_pool,
     const T* __restrict__ v_pool, T* __restrict__ out, int64_t out_stride,
-    const int* __restrict__ tok_item, const int* __restrict__ tok_pos,
-    const int* __restrict__ tables, int table_width, int heads, int kv_heads, int head_dim,
-    int page_size, int num_pages, float scale, int window) {
+    const int* __restrict__ tok_list, const int* __restrict__ tok_item,
+    const int* __restrict__ tok_pos, const int* __restrict__ tables, int table_width, int heads,
+    int kv_heads, int head_dim, int page_size, int num_pages, float scale, int window) {
   __shared__ float q_row[256];
   __shared__ float prob[64];
   __shared__ int64_t key_base[64];
 
-  const int t = blockIdx.x;
+  const int t = tok_list ? tok_list[blockIdx.x] : blockIdx.x;
   const int head = blockIdx.y;
   const int kv_head = head / (heads / kv_heads);
   const int lane = threadIdx.x;
@@ -96,8 +96,9 @@ __global__ __launch_bounds__(64) void attention_rowwise_kernel(
 
 extern "C" int ps_attention_rowwise(const void* q, int64_t q_stride, const void* k_pool,
                                     const void* v_pool, void* out, int64_t out_stride,
-                                    const int* tok_item, const int* tok_pos, const int* tables,
-                                    int table_width, int tokens, int heads, int kv_heads,
+                                    const int* tok_list, const int* tok_item, const int* tok_pos,
+                                    const int* tables, int table_width, int tokens, int heads,
+                                    int kv_heads,
                                     int head_dim, int page_size, int num_pages, float scale,
                                     int window, int dtype, void* stream) {
   PS_REQUIRE(tokens >= 0 && heads > 0 && kv_heads > 0 && page_size > 0 && num_pages > 0 &&
@@ -117,12 +118,12 @@ extern "C" int ps_attention_rowwise(const void* q, int64_t q_stride, const void*
   if (dtype == PS_F32)
     hipLaunchKernelGGL(attention_rowwise_kernel<float>, grid, dim3(64), 0, s, (const float*)q,
                        q_stride, (const float*)k_pool, (const float*)v_pool, (float*)out,
-                       out_stride, tok_item, tok_pos, tables, table_width, heads, kv_heads,
+                       out_stride, tok_list, tok_item, tok_pos, tables, table_width, heads, kv_heads,
                        head_dim, page_size, num_pages, scale, window);
   else
     hipLaunchKernelGGL(attention_rowwise_kernel<bf16_t>, grid, dim3(64), 0, s, (const bf16_t*)q,
                        q_stride, (const bf16_t*)k_pool, (const bf16_t*)v_pool, (bf16_t*)out,
-                       out_stride, tok_item, tok_pos, tables, table_width, heads, kv_heads,
+                       out_stride, tok_list, tok_item, tok_pos, tables, table_width, heads, kv_heads,
                        head_dim, page_size, num_pages, scale, window);
   PS_CHECK_LAUNCH("ps_attention_rowwise");
   return 0;

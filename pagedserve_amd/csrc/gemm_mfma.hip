@@ -1,0 +1,335 @@
+// Matrix products on the matrix cores (MFMA) of gfx950:  C[m, n] = epi(sum_k A[m, k] W[n, k] + b[n]).
+//
+// Two kernels.
+//
+// gemm_nt_tiled_kernel — many rows (prompt portions).  128 x 128 outputs per 256-thread block,
+//   four waves in a 2 x 2 arrangement, each wave 2 x 2 tiles of 32 x 32.  A and W tiles of 64
+//   bytes of k per row go global -> registers -> LDS (two buffers, one barrier per k tile);
+//   every lane reads 16 bytes of k for its row from LDS.  For bfloat16 that is the operand of
+//   one v_mfma_f32_32x32x16_bf16; for float the four values feed four v_mfma_f32_32x32x2_f32
+//   (both operands use the same assignment of k to lanes and instructions, which is all a dot
+//   product needs).  The float instantiation multiplies true 32-bit inputs.
+//
+// gemm_nt_skinny_kernel — up to 64 rows (decode), bfloat16.  The product is bound by reading W
+//   once, so weights go straight from global memory into MFMA operands: a wave owns 16 weight
+//   rows, every lane loads 32 contiguous bytes of one row per 64 k, and v_mfma_f32_16x16x32_bf16
+//   takes the weights as its row operand and up to four blocks of 16 activation rows as column
+//   operands.  K may be split over blocks; partial sums are then added into the float output
+//   with hardware float atomics (only the residual epilogue allows it).
+//
+// Accumulation is float in all cases.  Shapes that the kernels cannot take (k not a multiple
+// of 8 elements, unaligned rows) are refused by ps_gemm_nt_mfma_supported and run on the
+// plain kernel instead.
+#include "common.h"
+#include "pagedserve_hip.h"
+
+typedef __attribute__((__vector_size__(8 * sizeof(__bf16)))) __bf16 bf16x8;
+typedef __attribute__((__vector_size__(16 * sizeof(float)))) float f32x16;
+typedef __attribute__((__vector_size__(4 * sizeof(float)))) float f32x4;
+
+#define TG_BM 128
+#define TG_BN 128
+#define TG_ROW_BYTES 64   // k bytes per row and stage
+#define TG_LDS_STRIDE 80  // padded row stride in bytes (keeps 16-byte alignment)
+
+template <typename T>
+struct Mma;
+
+template <>
+struct Mma<bf16_t> {
+  static constexpr int K_PER_CHUNK = 8;  // elements in 16 bytes
+  __device__ static inline void step(const uint4& a, const uint4& b, f32x16& acc) {
+    acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(*reinterpret_cast<const bf16x8*>(&a),
+                                                  *reinterpret_cast<const bf16x8*>(&b), acc, 0, 0, 0);
+  }
+};
+
+template <>
+struct Mma<float> {
+  static constexpr int K_PER_CHUNK = 4;
+  __device__ static inline void step(const uint4& a, const uint4& b, f32x16& acc) {
+    acc = __builtin_amdgcn_mfma_f32_32x32x2f32(__uint_as_float(a.x), __uint_as_float(b.x), acc, 0, 0, 0);
+    acc = __builtin_amdgcn_mfma_f32_32x32x2f32(__uint_as_float(a.y), __uint_as_float(b.y), acc, 0, 0, 0);
+    acc = __builtin_amdgcn_mfma_f32_32x32x2f32(__uint_as_float(a.z), __uint_as_float(b.z), acc, 0, 0, 0);
+    acc = __builtin_amdgcn_mfma_f32_32x32x2f32(__uint_as_float(a.w), __uint_as_float(b.w), acc, 0, 0, 0);
+  }
+};
+
+template <typename T, typename TOut, int EPI>
+__global__ __launch_bounds__(256) void gemm_nt_tiled_kernel(
+    const T* __restrict__ a, const T* __restrict__ w, const float* __restrict__ bias,
+    TOut* __restrict__ c, int m, int n, int k, int lda, int ldc, int tiles_n) {
+  constexpr int KC = Mma<T>::K_PER_CHUNK;            // elements per 16-byte chunk
+  constexpr int BK = TG_ROW_BYTES / (int)sizeof(T);  // elements of k per stage
+  __shared__ __attribute__((aligned(16))) unsigned char lds[2][(TG_BM + TG_BN) * TG_LDS_STRIDE];
+
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = tid >> 6;
+  const int wave_m = wave >> 1;
+  const int wave_n = wave & 1;
+  const int tile_m = blockIdx.x / tiles_n;
+  const int tile_n = blockIdx.x - tile_m * tiles_n;
+  const int m0 = tile_m * TG_BM;
+  const int n0 = tile_n * TG_BN;
+
+  // global -> register staging: 512 chunks of 16 bytes per operand, two per thread
+  uint4 stage_a[2], stage_w[2];
+  auto load_global = [&](int k0) {
+#pragma unroll
+    for (int i = 0; i < 2; ++i) {
+      const int chunk = tid + i * 256;
+      const int row = chunk >> 2;
+      const int kk = k0 + (chunk & 3) * KC;
+      const uint4 zero = {0u, 0u, 0u, 0u};
+      stage_a[i] = (m0 + row < m && kk < k)
+                       ? *reinterpret_cast<const uint4*>(a + (int64_t)(m0 + row) * lda + kk)
+                       : zero;
+      stage_w[i] = (n0 + row < n && kk < k)
+                       ? *reinterpret_cast<const uint4*>(w + (int64_t)(n0 + row) * k + kk)
+                       : zero;
+    }
+  };
+  auto store_lds = [&](int buffer) {
+#pragma unroll
+    for (int i = 0; i < 2; ++i) {
+      const int chunk = tid + i * 256;
+      const int row = chunk >> 2;
+      const int offset = row * TG_LDS_STRIDE + (chunk & 3) * 16;
+      *reinterpret_cast<uint4*>(&lds[buffer][offset]) = stage_a[i];
+      *reinterpret_cast<uint4*>(&lds[buffer][TG_BM * TG_LDS_STRIDE + offset]) = stage_w[i];
+    }
+  };
+
+  f32x16 acc[2][2];
+#pragma unroll
+  for (int i = 0; i < 2; ++i)
+#pragma unroll
+    for (int j = 0; j < 2; ++j)
+#pragma unroll
+      for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.f;
+
+  const int k_tiles = (k + BK - 1) / BK;
+  load_global(0);
+  store_lds(0);
+  __syncthreads();
+  for (int kt = 0; kt < k_tiles; ++kt) {
+    const int buffer = kt & 1;
+    if (kt + 1 < k_tiles) load_global((kt + 1) * BK);
+    // 64 bytes of k per row = two 32-byte halves; lanes 0..31 take the first 16 bytes of a
+    // half, lanes 32..63 the second
+#pragma unroll
+    for (int half = 0; half < 2; ++half) {
+      uint4 fa[2], fw[2];
+      const int kbyte = half * 32 + (lane >> 5) * 16;
+#pragma unroll
+      for (int i = 0; i < 2; ++i) {
+        const int row = wave_m * 64 + i * 32 + (lane & 31);
+        fa[i] = *reinterpret_cast<const uint4*>(&lds[buffer][row * TG_LDS_STRIDE + kbyte]);
+      }
+#pragma unroll
+      for (int j = 0; j < 2; ++j) {
+        const int row = wave_n * 64 + j * 32 + (lane & 31);
+        fw[j] = *reinterpret_cast<const uint4*>(
+            &lds[buffer][TG_BM * TG_LDS_STRIDE + row * TG_LDS_STRIDE + kbyte]);
+      }
+#pragma unroll
+      for (int i = 0; i < 2; ++i)
+#pragma unroll
+        for (int j = 0; j < 2; ++j) Mma<T>::step(fa[i], fw[j], acc[i][j]);
+    }
+    if (kt + 1 < k_tiles) store_lds(buffer ^ 1);
+    __syncthreads();
+  }
+
+  // element e of a 32 x 32 accumulator: row (e / 4) * 8 + (lane / 32) * 4 + e % 4, column lane % 32
+#pragma unroll
+  for (int j = 0; j < 2; ++j) {
+    const int col = n0 + wave_n * 64 + j * 32 + (lane & 31);
+    if (col >= n) continue;
+    const float b = bias ? bias[col] : 0.f;
+#pragma unroll
+    for (int i = 0; i < 2; ++i) {
+#pragma unroll
+      for (int e = 0; e < 16; ++e) {
+        const int row = m0 + wave_m * 64 + i * 32 + (e >> 2) * 8 + (lane >> 5) * 4 + (e & 3);
+        if (row >= m) continue;
+        float v = apply_activation<EPI>(acc[i][j][e] + b);
+        TOut* dst = c + (int64_t)row * ldc + col;
+        if (EPI == PS_EPI_RESIDUAL) v += to_float<TOut>(*dst);
+        *dst = from_float<TOut>(v);
+      }
+    }
+  }
+}
+
+// ------------------------------------------------------------------------------- skinny
+#define SK_WAVES 4
+#define SK_ROWS (16 * SK_WAVES)
+
+template <typename TOut, int EPI, int MB>
+__global__ __launch_bounds__(64 * SK_WAVES) void gemm_nt_skinny_kernel(
+    const bf16_t* __restrict__ a, const bf16_t* __restrict__ w, const float* __restrict__ bias,
+    TOut* __restrict__ c, int m, int n, int k, int lda, int ldc, int k_chunk, int k_splits) {
+  const int lane = threadIdx.x & 63;
+  const int wave = threadIdx.x >> 6;
+  const int n0 = blockIdx.x * SK_ROWS + wave * 16;
+  if (n0 >= n) return;
+  const int split = blockIdx.y;
+  const int k_begin = split * k_chunk;
+  const int k_end = k_begin + k_chunk < k ? k_begin + k_chunk : k;
+  const int sub = lane & 15;
+  const int group = lane >> 4;
+  const int w_row = n0 + sub < n ? n0 + sub : n - 1;
+  const bf16_t* w_ptr = w + (int64_t)w_row * k + group * 16;
+  const bf16_t* a_ptr[MB];
+#pragma unroll
+  for (int b = 0; b < MB; ++b) {
+    const int row = b * 16 + sub < m ? b * 16 + sub : m - 1;
+    a_ptr[b] = a + (int64_t)row * lda + group * 16;
+  }
+  f32x4 acc[MB];
+#pragma unroll
+  for (int b = 0; b < MB; ++b) acc[b] = f32x4{0.f, 0.f, 0.f, 0.f};
+
+  const uint4 zero = {0u, 0u, 0u, 0u};
+  for (int k0 = k_begin; k0 < k_end; k0 += 64) {
+    const int kk = k0 + group * 16;
+    const bool first = kk < k_end;
+    const bool second = kk + 8 < k_end;
+    const uint4 w0 = first ? *reinterpret_cast<const uint4*>(w_ptr + k0) : zero;
+    const uint4 w1 = second ? *reinterpret_cast<const uint4*>(w_ptr + k0 + 8) : zero;
+#pragma unroll
+    for (int b = 0; b < MB; ++b) {
+      const uint4 x0 = first ? *reinterpret_cast<const uint4*>(a_ptr[b] + k0) : zero;
+      const uint4 x1 = second ? *reinterpret_cast<const uint4*>(a_ptr[b] + k0 + 8) : zero;
+      acc[b] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(*reinterpret_cast<const bf16x8*>(&w0),
+                                                       *reinterpret_cast<const bf16x8*>(&x0),
+                                                       acc[b], 0, 0, 0);
+      acc[b] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(*reinterpret_cast<const bf16x8*>(&w1),
+                                                       *reinterpret_cast<const bf16x8*>(&x1),
+                                                       acc[b], 0, 0, 0);
+    }
+  }
+
+  // element i of a 16 x 16 accumulator: weight row (lane / 16) * 4 + i, activation row lane % 16
+#pragma unroll
+  for (int b = 0; b < MB; ++b) {
+    const int row = b * 16 + sub;
+    if (row >= m) continue;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int col = n0 + group * 4 + i;
+      if (col >= n) continue;
+      float v = acc[b][i];
+      if (bias != nullptr && split == 0) v += bias[col];
+      TOut* dst = c + (int64_t)row * ldc + col;
+      if (EPI == PS_EPI_RESIDUAL) {
+        if (k_splits > 1) {
+          unsafeAtomicAdd(reinterpret_cast<float*>(dst), v);
+        } else {
+          *dst = from_float<TOut>(v + to_float<TOut>(*dst));
+        }
+      } else {
+        *dst = from_float<TOut>(apply_activation<EPI>(v));
+      }
+    }
+  }
+}
+
+// --------------------------------------------------------------------------------- host
+static bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
+
+bool ps_gemm_nt_mfma_supported(const void* a, const void* w, int k, int lda, int dtype) {
+  const int per_chunk = dtype == PS_BF16 ? 8 : 4;
+  return k % per_chunk == 0 && lda % per_chunk == 0 && aligned16(a) && aligned16(w);
+}
+
+template <typename T, typename TOut>
+static int launch_tiled(const void* a, const void* w, const float* bias, void* c, int m, int n,
+                        int k, int lda, int ldc, int epilogue, hipStream_t s) {
+  const int tiles_m = (m + TG_BM - 1) / TG_BM;
+  const int tiles_n = (n + TG_BN - 1) / TG_BN;
+  dim3 grid(tiles_m * tiles_n);
+#define PS_LAUNCH_TG(EPI)                                                                    \
+  hipLaunchKernelGGL((gemm_nt_tiled_kernel<T, TOut, EPI>), grid, dim3(256), 0, s, (const T*)a, \
+                     (const T*)w, bias, (TOut*)c, m, n, k, lda, ldc, tiles_n)
+  switch (epilogue) {
+    case PS_EPI_NONE: PS_LAUNCH_TG(PS_EPI_NONE); break;
+    case PS_EPI_GELU_TANH: PS_LAUNCH_TG(PS_EPI_GELU_TANH); break;
+    case PS_EPI_GELU_ERF: PS_LAUNCH_TG(PS_EPI_GELU_ERF); break;
+    case PS_EPI_RESIDUAL: PS_LAUNCH_TG(PS_EPI_RESIDUAL); break;
+    default: ps_set_error("ps_gemm_nt: unknown epilogue %d", epilogue); return 1;
+  }
+#undef PS_LAUNCH_TG
+  PS_CHECK_LAUNCH("ps_gemm_nt(tiled)");
+  return 0;
+}
+
+template <typename TOut, int EPI>
+static void launch_skinny_mb(const void* a, const void* w, const float* bias, void* c, int m,
+                             int n, int k, int lda, int ldc, int k_chunk, int k_splits,
+                             hipStream_t s) {
+  dim3 grid((n + SK_ROWS - 1) / SK_ROWS, k_splits);
+  dim3 block(64 * SK_WAVES);
+#define PS_LAUNCH_SK(MB)                                                                       \
+  hipLaunchKernelGGL((gemm_nt_skinny_kernel<TOut, EPI, MB>), grid, block, 0, s,                \
+                     (const bf16_t*)a, (const bf16_t*)w, bias, (TOut*)c, m, n, k, lda, ldc,    \
+                     k_chunk, k_splits)
+  const int blocks = (m + 15) / 16;
+  if (blocks <= 1) PS_LAUNCH_SK(1);
+  else if (blocks == 2) PS_LAUNCH_SK(2);
+  else if (blocks == 3) PS_LAUNCH_SK(3);
+  else PS_LAUNCH_SK(4);
+#undef PS_LAUNCH_SK
+}
+
+template <typename TOut>
+static int launch_skinny(const void* a, const void* w, const float* bias, void* c, int m, int n,
+                         int k, int lda, int ldc, int epilogue, hipStream_t s) {
+  // Split k only where partial sums can be added in place, and only to fill the chip.
+  int k_splits = 1;
+  if (epilogue == PS_EPI_RESIDUAL) {
+    const int waves = (n + 15) / 16;
+    const int wanted = (1024 + waves - 1) / waves;
+    const int possible = k / 128 > 0 ? k / 128 : 1;
+    k_splits = wanted < possible ? wanted : possible;
+    if (k_splits < 1) k_splits = 1;
+  }
+  int k_chunk = (k + k_splits - 1) / k_splits;
+  k_chunk = (k_chunk + 63) / 64 * 64;
+  k_splits = (k + k_chunk - 1) / k_chunk;
+  switch (epilogue) {
+    case PS_EPI_NONE:
+      launch_skinny_mb<TOut, PS_EPI_NONE>(a, w, bias, c, m, n, k, lda, ldc, k_chunk, k_splits, s);
+      break;
+    case PS_EPI_GELU_TANH:
+      launch_skinny_mb<TOut, PS_EPI_GELU_TANH>(a, w, bias, c, m, n, k, lda, ldc, k_chunk, k_splits, s);
+      break;
+    case PS_EPI_GELU_ERF:
+      launch_skinny_mb<TOut, PS_EPI_GELU_ERF>(a, w, bias, c, m, n, k, lda, ldc, k_chunk, k_splits, s);
+      break;
+    case PS_EPI_RESIDUAL:
+      launch_skinny_mb<TOut, PS_EPI_RESIDUAL>(a, w, bias, c, m, n, k, lda, ldc, k_chunk, k_splits, s);
+      break;
+    default: ps_set_error("ps_gemm_nt: unknown epilogue %d", epilogue); return 1;
+  }
+  PS_CHECK_LAUNCH("ps_gemm_nt(skinny)");
+  return 0;
+}
+
+int ps_gemm_nt_mfma(const void* a, const void* w, const float* bias, void* c, int m, int n, int k,
+                    int lda, int ldc, int dtype, int c_dtype, int epilogue, hipStream_t s) {
+  if (dtype == PS_BF16 && m <= 64) {
+    if (c_dtype == PS_F32) return launch_skinny<float>(a, w, bias, c, m, n, k, lda, ldc, epilogue, s);
+    return launch_skinny<bf16_t>(a, w, bias, c, m, n, k, lda, ldc, epilogue, s);
+  }
+  if (dtype == PS_F32 && c_dtype == PS_F32)
+    return launch_tiled<float, float>(a, w, bias, c, m, n, k, lda, ldc, epilogue, s);
+  if (dtype == PS_BF16 && c_dtype == PS_F32)
+    return launch_tiled<bf16_t, float>(a, w, bias, c, m, n, k, lda, ldc, epilogue, s);
+  if (dtype == PS_BF16 && c_dtype == PS_BF16)
+    return launch_tiled<bf16_t, bf16_t>(a, w, bias, c, m, n, k, lda, ldc, epilogue, s);
+  ps_set_error("ps_gemm_nt: unsupported dtype pair (in %d, out %d)", dtype, c_dtype);
+  return 1;
+}

@@ -42,14 +42,25 @@ int ps_kv_write(const void* k, const void* v, int64_t stride, void* k_pool, void
                 int tokens, int kv_heads, int head_dim, int page_size, int num_pages, int dtype,
                 void* stream);
 
-// Attention of every token of the step over its request's cached keys 0..position
-// (or the last `window` of them), one wave per (token, head).  Any head_dim that is a
-// multiple of 16 up to 256; heads must be a multiple of kv_heads.
+// Attention of `tokens` tokens of the step (those listed in tok_list, or all when it is
+// null) over their requests' cached keys 0..position (or the last `window` of them), one
+// wave per (token, head).  Any head_dim that is a multiple of 16 up to 256; heads must be a
+// multiple of kv_heads.
 int ps_attention_rowwise(const void* q, int64_t q_stride, const void* k_pool, const void* v_pool,
-                         void* out, int64_t out_stride, const int* tok_item, const int* tok_pos,
-                         const int* tables, int table_width, int tokens, int heads, int kv_heads,
-                         int head_dim, int page_size, int num_pages, float scale, int window,
-                         int dtype, void* stream);
+                         void* out, int64_t out_stride, const int* tok_list, const int* tok_item,
+                         const int* tok_pos, const int* tables, int table_width, int tokens,
+                         int heads, int kv_heads, int head_dim, int page_size, int num_pages,
+                         float scale, int window, int dtype, void* stream);
+
+// The same result for single queries, with each token's keys cut into `splits` ranges that
+// run as separate blocks; `partial` is scratch of count * heads * splits * (head_dim + 2)
+// floats (unused when splits == 1).
+int ps_attention_decode(const void* q, int64_t q_stride, const void* k_pool, const void* v_pool,
+                        void* out, int64_t out_stride, float* partial, int64_t partial_floats,
+                        const int* tok_list, const int* tok_item, const int* tok_pos,
+                        const int* tables, int table_width, int count, int heads, int kv_heads,
+                        int head_dim, int page_size, int num_pages, float scale, int window,
+                        int splits, int dtype, void* stream);
 
 // tokens[r] = argmax (inv_temperature[r] == 0) or a draw from softmax(logits * inv_temperature[r])
 // by inverse CDF at uniform[r] in [0, 1).

@@ -61,7 +61,7 @@ class Engine:
         self.views = model.cache_views(self.cache)
         self.workspace = Workspace(max_step_tokens, self.device)
         self.table_width = -(-self.spec.max_positions // page_size)
-        capacity = (4 * max_step_tokens + 3 * max_requests + 1
+        capacity = (5 * max_step_tokens + 3 * max_requests + 1
                     + len(groups) * max_requests * self.table_width + 16)
         self._meta_device = torch.empty(capacity, dtype=torch.int32, device=self.device)
         self._meta_host = [torch.empty(capacity, dtype=torch.int32, pin_memory=True) for _ in range(2)]
@@ -152,13 +152,15 @@ class Engine:
         tokens = sum(len(entry.tokens) for entry in entries)
         items = len(entries)
         wanted = sum(len(entry.want) for entry in entries)
+        singles = sum(1 for entry in entries if len(entry.tokens) == 1)
         groups = len(self.cache.groups)
         width = self.table_width
         offsets = {}
         cursor = 0
         for name, size in (("token_ids", tokens), ("positions", tokens), ("tok_item", tokens),
                            ("cu_tokens", items + 1), ("kv_lens", items), ("slots", items),
-                           ("rows", wanted)):
+                           ("rows", wanted), ("single_tokens", singles),
+                           ("portion_tokens", tokens - singles)):
             offsets[name] = (cursor, size)
             cursor += size
         for group in range(groups):
@@ -176,6 +178,7 @@ class Engine:
 
         token_ids, positions, tok_item = section("token_ids"), section("positions"), section("tok_item")
         cu, kv_lens, slots, rows = section("cu_tokens"), section("kv_lens"), section("slots"), section("rows")
+        single_tokens, portion_tokens = section("single_tokens"), section("portion_tokens")
         tables = [section(f"tables{group}").reshape(items, width) for group in range(groups)]
         for table in tables:
             table.fill(-1)
@@ -184,6 +187,8 @@ class Engine:
         flat = 0
         row_cursor = 0
         max_kv = 0
+        single_cursor = 0
+        portion_cursor = 0
         for index, entry in enumerate(entries):
             record = self.cache.requests[entry.request_id]
             count = len(entry.tokens)
@@ -202,6 +207,13 @@ class Engine:
                 rows[row_cursor] = flat + int(place)
                 row_keys.append((entry.request_id, start + int(place)))
                 row_cursor += 1
+            if count == 1:
+                single_tokens[single_cursor] = flat
+                single_cursor += 1
+            else:
+                portion_tokens[portion_cursor:portion_cursor + count] = np.arange(
+                    flat, flat + count, dtype=np.int32)
+                portion_cursor += count
             step_items.append(StepItem(entry.request_id, record.slot, start, count, flat))
             flat += count
         cu[items] = flat
@@ -221,7 +233,9 @@ class Engine:
             cu_tokens=view("cu_tokens"), kv_lens=view("kv_lens"), slots=view("slots"),
             tables=[view(f"tables{group}").view(items, width) for group in range(groups)],
             page_size=self.page_size, workspace=self.workspace,
-            decode_only=all(len(entry.tokens) == 1 for entry in entries), max_kv_len=max_kv)
+            decode_only=singles == items, max_kv_len=max_kv,
+            single_tokens=view("single_tokens"), portion_tokens=view("portion_tokens"),
+            max_positions=self.spec.max_positions)
         return ctx, view("rows"), row_keys
 
     def _run(self, entries) -> StepOutput:

@@ -29,8 +29,11 @@ _SIGNATURES = {
     "ps_kv_write": [c_void_p, c_void_p, c_int64, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
                     c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_void_p],
     "ps_attention_rowwise": [c_void_p, c_int64, c_void_p, c_void_p, c_void_p, c_int64, c_void_p,
-                             c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_int,
-                             c_float, c_int, c_int, c_void_p],
+                             c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int,
+                             c_int, c_float, c_int, c_int, c_void_p],
+    "ps_attention_decode": [c_void_p, c_int64, c_void_p, c_void_p, c_void_p, c_int64, c_void_p,
+                            c_int64, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int,
+                            c_int, c_int, c_int, c_int, c_float, c_int, c_int, c_int, c_void_p],
     "ps_sample": [c_void_p, c_int64, c_void_p, c_void_p, c_void_p, c_int, c_int, c_void_p],
 }
 
@@ -207,8 +210,7 @@ def kv_write(k, v, k_pool, v_pool, tok_item, tok_pos, tables):
           kv_heads, head_dim, page_size, pages, dtype_code(k.dtype), _stream())
 
 
-def attention_rowwise(q, k_pool, v_pool, out, tok_item, tok_pos, tables, heads, scale, window=0):
-    """out[t, h] = softmax(q[t, h] . K * scale) V over the cached keys of t's request."""
+def _attention_args(q, k_pool, v_pool, out, tok_item, tok_pos, tables, heads, tok_list):
     _check(q, "q", ndim=2)
     _check(out, "out", q.dtype, 2)
     pages, kv_heads, page_size, head_dim = _check_pools(k_pool, v_pool, q.dtype)
@@ -218,10 +220,52 @@ def attention_rowwise(q, k_pool, v_pool, out, tok_item, tok_pos, tables, heads, 
     if q.shape[1] != heads * head_dim or out.shape[1] != heads * head_dim or out.shape[0] != tokens:
         raise KernelError("attention: q/out rows must hold heads x head_dim values")
     _check_step_index(tok_item, tok_pos, tables, tokens)
+    count = tokens
+    if tok_list is not None:
+        _check(tok_list, "tok_list", torch.int32, 1)
+        if not tok_list.is_contiguous():
+            raise KernelError("attention: tok_list must be contiguous")
+        count = tok_list.numel()
+    return pages, kv_heads, page_size, head_dim, q_stride, out_stride, count
+
+
+def attention_rowwise(q, k_pool, v_pool, out, tok_item, tok_pos, tables, heads, scale, window=0,
+                      tok_list=None):
+    """out[t, h] = softmax(q[t, h] . K * scale) V over the cached keys of t's request, for the
+    tokens in ``tok_list`` (all when it is None)."""
+    pages, kv_heads, page_size, head_dim, q_stride, out_stride, count = _attention_args(
+        q, k_pool, v_pool, out, tok_item, tok_pos, tables, heads, tok_list)
     _call("ps_attention_rowwise", q.data_ptr(), q_stride, k_pool.data_ptr(), v_pool.data_ptr(),
-          out.data_ptr(), out_stride, tok_item.data_ptr(), tok_pos.data_ptr(), tables.data_ptr(),
-          tables.shape[1], tokens, heads, kv_heads, head_dim, page_size, pages, float(scale),
-          int(window), dtype_code(q.dtype), _stream())
+          out.data_ptr(), out_stride, _ptr(tok_list), tok_item.data_ptr(), tok_pos.data_ptr(),
+          tables.data_ptr(), tables.shape[1], count, heads, kv_heads, head_dim, page_size, pages,
+          float(scale), int(window), dtype_code(q.dtype), _stream())
+    return out
+
+
+def decode_keys_per_block(head_dim: int) -> int:
+    """Keys that one block of the split-KV kernel visits per iteration."""
+    lanes = head_dim // 8
+    lanes_per_key = 2 if lanes <= 2 else 4 if lanes <= 4 else 8 if lanes <= 8 else 16 if lanes <= 16 else 32
+    return (64 // lanes_per_key) * 4 * 4
+
+
+def attention_decode(q, k_pool, v_pool, out, tok_item, tok_pos, tables, heads, scale, splits,
+                     partial=None, window=0, tok_list=None):
+    """The same result as ``attention_rowwise`` by the split-KV kernel; ``partial`` is float
+    scratch of ``count * heads * splits * (head_dim + 2)`` values when ``splits > 1``."""
+    pages, kv_heads, page_size, head_dim, q_stride, out_stride, count = _attention_args(
+        q, k_pool, v_pool, out, tok_item, tok_pos, tables, heads, tok_list)
+    floats = 0
+    if splits > 1:
+        _check(partial, "partial", torch.float32)
+        if not partial.is_contiguous():
+            raise KernelError("attention_decode: scratch must be contiguous")
+        floats = partial.numel()
+    _call("ps_attention_decode", q.data_ptr(), q_stride, k_pool.data_ptr(), v_pool.data_ptr(),
+          out.data_ptr(), out_stride, _ptr(partial if splits > 1 else None), floats,
+          _ptr(tok_list), tok_item.data_ptr(), tok_pos.data_ptr(), tables.data_ptr(),
+          tables.shape[1], count, heads, kv_heads, head_dim, page_size, pages, float(scale),
+          int(window), int(splits), dtype_code(q.dtype), _stream())
     return out
 
 

@@ -1,5 +1,7 @@
 """Multi-head attention over the paged cache."""
 
+import torch
+
 from ..ops import kernels
 from ..weights.loader import MATRIX, VECTOR, ParamSpec
 from .base import Mixer, PagedKVSpec
@@ -71,6 +73,30 @@ class Attention(Mixer):
         if cache.writes:
             kernels.kv_write(k, v, cache.k_pool, cache.v_pool, ctx.tok_item, ctx.positions, tables)
         context = ctx.workspace.rows("attn", self.q_cols, self.dtype)[:tokens]
-        kernels.attention_rowwise(q, cache.k_pool, cache.v_pool, context, ctx.tok_item,
-                                  ctx.positions, tables, self.heads, self.scale, self.window)
+        singles = ctx.single_tokens.numel() if ctx.single_tokens is not None else 0
+        if singles:
+            # one-token items: keys of a request are cut into ranges so that few requests
+            # still fill the chip
+            splits = self._splits(singles, ctx.max_kv_len)
+            partial = None
+            if splits > 1:
+                # _splits keeps singles * heads * splits below 1024 + singles * heads
+                worst = (1024 + ctx.workspace.max_rows * self.heads) * (self.head_dim + 2)
+                partial = ctx.workspace.flat("attn_partial", worst, torch.float32)
+            kernels.attention_decode(q, cache.k_pool, cache.v_pool, context, ctx.tok_item,
+                                     ctx.positions, tables, self.heads, self.scale, splits,
+                                     partial=partial, window=self.window,
+                                     tok_list=None if singles == tokens else ctx.single_tokens)
+        if singles < tokens:
+            kernels.attention_rowwise(q, cache.k_pool, cache.v_pool, context, ctx.tok_item,
+                                      ctx.positions, tables, self.heads, self.scale, self.window,
+                                      tok_list=None if singles == 0 else ctx.portion_tokens)
         kernels.gemm_nt(context, self.out_weight, self.out_bias, residual, epilogue="residual")
+
+    def _splits(self, count: int, max_kv_len: int) -> int:
+        """Ranges per request: enough blocks for about four per compute unit, never more
+        than the keys of the longest request can feed."""
+        visible = max_kv_len if self.window <= 0 else min(max_kv_len, self.window)
+        most = max(1, -(-visible // kernels.decode_keys_per_block(self.head_dim)))
+        wanted = max(1, -(-1024 // (count * self.heads)))
+        return min(most, wanted, 64)

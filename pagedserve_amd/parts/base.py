@@ -116,6 +116,16 @@ class Workspace:
             self._buffers[key] = buffer
         return buffer
 
+    def flat(self, name: str, numel: int, dtype: torch.dtype):
+        """A 1-D scratch buffer of at least ``numel`` elements; callers ask for their worst
+        case so that it is allocated once."""
+        key = (name, dtype)
+        buffer = self._buffers.get(key)
+        if buffer is None or buffer.numel() < numel:
+            buffer = torch.empty(numel, dtype=dtype, device=self.device)
+            self._buffers[key] = buffer
+        return buffer
+
     def bytes(self) -> int:
         return sum(buffer.numel() * buffer.element_size() for buffer in self._buffers.values())
 
@@ -149,5 +159,8 @@ class StepContext:
     page_size: int
     workspace: Workspace
     decode_only: bool = False   # every item brings exactly one token
-    max_kv_len: int = 0
+    max_kv_len: int = 0         # longest cached length after this step (host value)
+    single_tokens: Optional[torch.Tensor] = None   # int32: step indices of one-token items
+    portion_tokens: Optional[torch.Tensor] = None  # int32: step indices of all other tokens
+    max_positions: int = 0
     extra: Optional[dict] = None

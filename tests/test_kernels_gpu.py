@@ -96,8 +96,11 @@ def test_rmsnorm():
     torch.testing.assert_close(out.double(), expected, atol=2e-5, rtol=2e-5)
 
 
+# rows 1..64 take the skinny kernel in bfloat16, more rows the tiled one; k = 100 and 66 are
+# not multiples of 8 and fall to the plain kernel
 GEMM_SHAPES = [(1, 50, 64), (5, 1000, 96), (64, 2304, 768), (130, 70, 320), (33, 257, 100),
-               (256, 768, 3072), (2, 50257, 64)]
+               (256, 768, 3072), (2, 50257, 64), (17, 768, 768), (48, 100, 3072), (65, 192, 96),
+               (300, 1000, 320), (129, 257, 66), (8, 768, 3072), (512, 2304, 768)]
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
@@ -240,6 +243,44 @@ def test_attention_rowwise_portion_and_window(dtype, window):
     torch.testing.assert_close(got, expected, atol=atol, rtol=rtol)
 
 
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("heads,kv_heads,head_dim,page_size", [(1, 1, 32, 16), (4, 4, 16, 8), (6, 2, 48, 16), (3, 3, 128, 4), (12, 12, 64, 16), (2, 1, 256, 16), (5, 5, 80, 12)])
+@pytest.mark.parametrize("splits", [1, 2, 5, 16])
+def test_attention_decode_split_kv(dtype, heads, kv_heads, head_dim, page_size, splits):
+    """The split-KV kernel over fragmented tables at the contexts of
+    testing/test_triton_correctness_matrix.py:9, for any number of splits (also more than the
+    keys can feed), listed tokens in any order, and a window."""
+    from pagedserve_amd.ops import kernels
+
+    contexts = [1, 15, 16, 17, 31, 32, 33, 128, 512, 1024]
+    k_pool, v_pool, tables = _paged_fixture(dtype, contexts, kv_heads, head_dim, page_size, 19)
+    count = len(contexts)
+    q = _rand((count, heads * head_dim), dtype, 20)
+    tok_item = torch.arange(count, dtype=torch.int32, device="cuda")
+    tok_pos = torch.tensor([c - 1 for c in contexts], dtype=torch.int32, device="cuda")
+    scale = head_dim ** -0.5
+    partial = torch.full((count * heads * splits * (head_dim + 2),), float("nan"), device="cuda")
+    atol, rtol = (3e-5, 3e-5) if dtype == torch.float32 else (2e-2, 2e-2)
+    for window in (0, 20):
+        expected = torch.empty_like(q)
+        kernels.attention_rowwise(q, k_pool, v_pool, expected, tok_item, tok_pos, tables, heads, scale, window=window)
+        out = torch.full_like(q, float("nan"))
+        kernels.attention_decode(q, k_pool, v_pool, out, tok_item, tok_pos, tables, heads, scale, splits,
+                                 partial=partial, window=window)
+        torch.testing.assert_close(out.double(), expected.double(), atol=atol, rtol=rtol)
+    # a list of tokens: only those rows are written
+    chosen = torch.tensor([7, 2, 9], dtype=torch.int32, device="cuda")
+    out = torch.full_like(q, 7.0)
+    kernels.attention_decode(q, k_pool, v_pool, out, tok_item, tok_pos, tables, heads, scale, splits,
+                             partial=partial, tok_list=chosen)
+    kernels.attention_rowwise(q, k_pool, v_pool, expected, tok_item, tok_pos, tables, heads, scale)
+    for row in range(count):
+        if row in (7, 2, 9):
+            torch.testing.assert_close(out[row].double(), expected[row].double(), atol=atol, rtol=rtol)
+        else:
+            assert float((out[row].float() - 7.0).abs().max()) == 0.0
+
+
 def test_attention_far_key_stands_out():
     """One key among 700 is made to dominate: the output must be its value.  A kernel that
     skips a page, mixes two requests' tables or misplaces an offset fails this."""
@@ -257,15 +298,21 @@ def test_attention_far_key_stands_out():
             direction = direction / direction.norm()
             q[item, head * head_dim:(head + 1) * head_dim] = (direction * 8.0).to(dtype)
             k_pool[page, head, key % page_size] = (direction * 40.0).to(dtype)
-        out = torch.empty_like(q)
         tok_item = torch.arange(2, dtype=torch.int32, device="cuda")
         tok_pos = torch.full((2,), context - 1, dtype=torch.int32, device="cuda")
-        kernels.attention_rowwise(q, k_pool, v_pool, out, tok_item, tok_pos, tables, heads, head_dim ** -0.5)
-        for item, head, key in targets:
-            page = int(tables[item, key // page_size])
-            expected = v_pool[page, head, key % page_size].float()
-            got = out[item, head * head_dim:(head + 1) * head_dim].float()
-            torch.testing.assert_close(got, expected, atol=2e-2, rtol=2e-2)
+        partial = torch.empty(2 * heads * 7 * (head_dim + 2), device="cuda")
+        for kernel in ("rowwise", "decode1", "decode7"):
+            out = torch.empty_like(q)
+            if kernel == "rowwise":
+                kernels.attention_rowwise(q, k_pool, v_pool, out, tok_item, tok_pos, tables, heads, head_dim ** -0.5)
+            else:
+                kernels.attention_decode(q, k_pool, v_pool, out, tok_item, tok_pos, tables, heads,
+                                         head_dim ** -0.5, int(kernel[6:]), partial=partial)
+            for item, head, key in targets:
+                page = int(tables[item, key // page_size])
+                expected = v_pool[page, head, key % page_size].float()
+                got = out[item, head * head_dim:(head + 1) * head_dim].float()
+                torch.testing.assert_close(got, expected, atol=2e-2, rtol=2e-2)
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
