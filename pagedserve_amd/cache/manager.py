@@ -23,6 +23,7 @@ state tensors live on the device given at construction.
 from dataclasses import dataclass, field
 from typing import Dict, Hashable, List, Optional, Sequence, Tuple
 
+import numpy as np
 import torch
 
 
@@ -151,6 +152,13 @@ class CacheManager:
                 (max_slots,) + tuple(spec.shape), dtype=spec.dtype, device=self.device)
         self.free_slots: List[int] = list(range(max_slots - 1, -1, -1))
         self.requests: Dict[Hashable, RequestCache] = {}
+        # Block tables as arrays [slot, logical page] (-1: no page), kept in step with the
+        # lists, so that a step gathers its rows with one indexing operation.
+        self.table_arrays: Optional[List[np.ndarray]] = None
+        if max_positions is not None:
+            width = -(-max_positions // page_size)
+            self.table_arrays = [np.full((max_slots, width), RELEASED, dtype=np.int32)
+                                 for _ in self.groups]
 
     # ------------------------------------------------------------------ sizes
     def bytes_per_page(self, group_index: int) -> int:
@@ -226,6 +234,8 @@ class CacheManager:
             raise
         for group_index, page in taken:
             record.tables[group_index].append(page)
+            if self.table_arrays is not None:
+                self.table_arrays[group_index][record.slot, len(record.tables[group_index]) - 1] = page
 
     def commit(self, request_id: Hashable, new_length: int):
         """The step that wrote positions ``< new_length`` succeeded."""
@@ -248,6 +258,8 @@ class CacheManager:
                 if table[page] != RELEASED:
                     self.pools[group_index].free(table[page])
                     table[page] = RELEASED
+                    if self.table_arrays is not None:
+                        self.table_arrays[group_index][record.slot, page] = RELEASED
                 page += 1
 
     def release(self, request_id: Hashable):
@@ -259,9 +271,10 @@ class CacheManager:
             live = [page for page in table if page != RELEASED]
             if len(live) != len(set(live)):
                 raise RuntimeError("request holds a page twice")
-            # newest page first, so that the request's first page is reused first
             for page in live:
                 self.pools[group_index].free(page)
+            if self.table_arrays is not None:
+                self.table_arrays[group_index][record.slot, :] = RELEASED
         self.free_slots.append(record.slot)
 
     def table(self, request_id: Hashable, group_index: int) -> List[int]:

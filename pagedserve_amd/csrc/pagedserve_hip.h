@@ -67,6 +67,13 @@ int ps_attention_decode(const void* q, int64_t q_stride, const void* k_pool, con
 int ps_sample(const float* logits, int64_t ld, const float* inv_temperature, const float* uniform,
               int* tokens, int rows, int vocab, void* stream);
 
+// Record the launches issued on `stream` between begin and end into an executable graph.
+int ps_graph_begin(void* stream);
+int ps_graph_end(void* stream, void** exec_out, int* node_count);
+int ps_graph_abort(void* stream);
+int ps_graph_launch(void* exec, void* stream);
+int ps_graph_destroy(void* exec);
+
 #ifdef __cplusplus
 }
 #endif

@@ -68,7 +68,13 @@ class Engine:
         self._meta_events = [None, None]
         self._meta_turn = 0
         self._logits = None
+        # The engine's work runs on a stream of its own (default priority): a capture cannot
+        # record from the default stream.
+        self.stream = torch.cuda.Stream(device=self.device)
         self.use_graphs = use_graphs
+        self._graphs = {}        # key -> StepGraph
+        self._graph_seen = set()  # keys that ran once without a graph (buffers exist now)
+        self._graph_failures = {}
         self.steps = 0
 
     # ------------------------------------------------------------------ admin
@@ -81,6 +87,13 @@ class Engine:
     def finish(self, request_id):
         """The request is over: its pages and its slot go back."""
         self.cache.release(request_id)
+
+    def graph_summary(self) -> dict:
+        """Counters in the manner of src/model/paged_decoder.py:498-507."""
+        return {"enabled": self.use_graphs, "captured_graphs": len(self._graphs),
+                "graph_replays": sum(graph.replays for graph in self._graphs.values()),
+                "graph_nodes": {str(key): graph.nodes for key, graph in self._graphs.items()},
+                "capture_failures": list(self._graph_failures.values())}
 
     def _logit_buffer(self, rows: int) -> torch.Tensor:
         if self._logits is None or self._logits.shape[0] < rows:
@@ -95,6 +108,8 @@ class Engine:
             raise StepError("a step needs at least one entry")
         seen = set()
         total = 0
+        new = 0
+        vocab = self.spec.vocab_size
         for entry in entries:
             if entry.request_id in seen:
                 # src/model/iteration.py:61-63
@@ -103,15 +118,15 @@ class Engine:
             count = len(entry.tokens)
             if count == 0:
                 raise StepError(f"request {entry.request_id!r} brings no tokens")
-            for token in entry.tokens:
-                if not 0 <= int(token) < self.spec.vocab_size:
-                    raise StepError(f"token {token} of request {entry.request_id!r} is outside "
-                                    f"the vocabulary of {self.spec.vocab_size}")
-            for index in entry.want:
-                if not 0 <= int(index) < count:
-                    raise StepError(f"request {entry.request_id!r} wants logits at place {index} "
-                                    f"of {count} tokens")
-            have = self.cache.length(entry.request_id) if self.is_live(entry.request_id) else 0
+            if min(entry.tokens) < 0 or max(entry.tokens) >= vocab:
+                raise StepError(f"a token of request {entry.request_id!r} is outside "
+                                f"the vocabulary of {vocab}")
+            if entry.want and (min(entry.want) < 0 or max(entry.want) >= count):
+                raise StepError(f"request {entry.request_id!r} wants logits at place "
+                                f"{max(entry.want)} of {count} tokens")
+            record = self.cache.requests.get(entry.request_id)
+            have = record.length if record is not None else 0
+            new += record is None
             if have + count > self.spec.max_positions:
                 # src/model/paged_decoder.py:521-522
                 raise StepError(f"request {entry.request_id!r} would reach position "
@@ -119,7 +134,6 @@ class Engine:
             total += count
         if total > self.max_step_tokens:
             raise StepError(f"step of {total} tokens exceeds max_step_tokens={self.max_step_tokens}")
-        new = sum(1 for entry in entries if not self.is_live(entry.request_id))
         if len(self.cache.requests) + new > self.max_requests:
             raise StepError(f"more than {self.max_requests} live requests")
 
@@ -127,33 +141,44 @@ class Engine:
         entries = list(entries)
         self._validate(entries)
         admitted = []
+        cache = self.cache
         try:
             for entry in entries:
-                if not self.is_live(entry.request_id):
-                    self.cache.admit(entry.request_id)
+                record = cache.requests.get(entry.request_id)
+                if record is None:
+                    cache.admit(entry.request_id)
                     admitted.append(entry.request_id)
-                self.cache.grow(entry.request_id,
-                                self.cache.length(entry.request_id) + len(entry.tokens))
-            output = self._run(entries)
+                    record = cache.requests[entry.request_id]
+                cache.grow(entry.request_id, record.length + len(entry.tokens))
+            caller = torch.cuda.current_stream(self.device)
+            # the caller may still be reading the last step's logits
+            self.stream.wait_stream(caller)
+            with torch.cuda.stream(self.stream):
+                output = self._run(entries)
+            caller.wait_stream(self.stream)
         except Exception:
             # requests that this step admitted leave no trace
             # (src/scheduler/orca_scheduler.py:243-247)
             for request_id in admitted:
-                self.cache.release(request_id)
+                cache.release(request_id)
             raise
         for entry in entries:
-            self.cache.commit(entry.request_id,
-                              self.cache.length(entry.request_id) + len(entry.tokens))
+            cache.commit(entry.request_id, cache.requests[entry.request_id].length + len(entry.tokens))
         self.steps += 1
         return output
 
     def _pack(self, entries):
-        """Fill the packed index buffer on the host; returns views of the device copy."""
-        tokens = sum(len(entry.tokens) for entry in entries)
+        """Fill the packed index buffer on the host, copy it, and return the step context.
+
+        The layout depends only on (tokens, items, wanted rows, one-token items)."""
+        cache = self.cache
+        counts = [len(entry.tokens) for entry in entries]
+        tokens = sum(counts)
         items = len(entries)
-        wanted = sum(len(entry.want) for entry in entries)
-        singles = sum(1 for entry in entries if len(entry.tokens) == 1)
-        groups = len(self.cache.groups)
+        wants = [len(entry.want) for entry in entries]
+        wanted = sum(wants)
+        singles = counts.count(1)
+        groups = len(cache.groups)
         width = self.table_width
         offsets = {}
         cursor = 0
@@ -176,47 +201,60 @@ class Engine:
             begin, size = offsets[name]
             return host[begin:begin + size]
 
-        token_ids, positions, tok_item = section("token_ids"), section("positions"), section("tok_item")
-        cu, kv_lens, slots, rows = section("cu_tokens"), section("kv_lens"), section("slots"), section("rows")
-        single_tokens, portion_tokens = section("single_tokens"), section("portion_tokens")
-        tables = [section(f"tables{group}").reshape(items, width) for group in range(groups)]
-        for table in tables:
-            table.fill(-1)
+        records = [cache.requests[entry.request_id] for entry in entries]
+        starts = [record.length for record in records]
+        slot_list = [record.slot for record in records]
+        section("slots")[:] = slot_list
         step_items = []
         row_keys = []
-        flat = 0
-        row_cursor = 0
-        max_kv = 0
-        single_cursor = 0
-        portion_cursor = 0
-        for index, entry in enumerate(entries):
-            record = self.cache.requests[entry.request_id]
-            count = len(entry.tokens)
-            start = record.length
-            token_ids[flat:flat + count] = np.asarray(entry.tokens, dtype=np.int32)
-            positions[flat:flat + count] = np.arange(start, start + count, dtype=np.int32)
-            tok_item[flat:flat + count] = index
-            cu[index] = flat
-            kv_lens[index] = start + count
-            max_kv = max(max_kv, start + count)
-            slots[index] = record.slot
-            for group, table in enumerate(tables):
-                pages = record.tables[group]
-                table[index, :len(pages)] = pages
-            for place in entry.want:
-                rows[row_cursor] = flat + int(place)
-                row_keys.append((entry.request_id, start + int(place)))
-                row_cursor += 1
-            if count == 1:
-                single_tokens[single_cursor] = flat
-                single_cursor += 1
-            else:
-                portion_tokens[portion_cursor:portion_cursor + count] = np.arange(
-                    flat, flat + count, dtype=np.int32)
-                portion_cursor += count
-            step_items.append(StepItem(entry.request_id, record.slot, start, count, flat))
-            flat += count
-        cu[items] = flat
+        if tokens == items:
+            # every item brings one token: no per-item loops over numpy slices
+            section("token_ids")[:] = [entry.tokens[0] for entry in entries]
+            section("positions")[:] = starts
+            index = np.arange(items + 1, dtype=np.int32)
+            section("tok_item")[:] = index[:items]
+            section("cu_tokens")[:] = index
+            section("kv_lens")[:] = [start + 1 for start in starts]
+            section("single_tokens")[:] = index[:items]
+            rows = section("rows")
+            row_cursor = 0
+            for flat, (entry, record, start) in enumerate(zip(entries, records, starts)):
+                if entry.want:
+                    rows[row_cursor] = flat
+                    row_keys.append((entry.request_id, start))
+                    row_cursor += 1
+                step_items.append(StepItem(entry.request_id, record.slot, start, 1, flat))
+            max_kv = max(starts) + 1
+        else:
+            token_ids, positions = section("token_ids"), section("positions")
+            tok_item, cu, kv_lens = section("tok_item"), section("cu_tokens"), section("kv_lens")
+            rows = section("rows")
+            single_tokens, portion_tokens = section("single_tokens"), section("portion_tokens")
+            flat = row_cursor = single_cursor = portion_cursor = max_kv = 0
+            for index, (entry, record, start, count) in enumerate(zip(entries, records, starts, counts)):
+                token_ids[flat:flat + count] = entry.tokens
+                positions[flat:flat + count] = np.arange(start, start + count, dtype=np.int32)
+                tok_item[flat:flat + count] = index
+                cu[index] = flat
+                kv_lens[index] = start + count
+                max_kv = max(max_kv, start + count)
+                if count == 1:
+                    single_tokens[single_cursor] = flat
+                    single_cursor += 1
+                else:
+                    portion_tokens[portion_cursor:portion_cursor + count] = np.arange(
+                        flat, flat + count, dtype=np.int32)
+                    portion_cursor += count
+                for place in entry.want:
+                    rows[row_cursor] = flat + int(place)
+                    row_keys.append((entry.request_id, start + int(place)))
+                    row_cursor += 1
+                step_items.append(StepItem(entry.request_id, record.slot, start, count, flat))
+                flat += count
+            cu[items] = flat
+        slot_index = np.asarray(slot_list, dtype=np.int64)
+        for group in range(groups):
+            section(f"tables{group}").reshape(items, width)[:] = cache.table_arrays[group][slot_index]
         device = self._meta_device
         device[:cursor].copy_(self._meta_host[turn][:cursor], non_blocking=True)
         event = torch.cuda.Event()
@@ -241,5 +279,36 @@ class Engine:
     def _run(self, entries) -> StepOutput:
         ctx, rows, row_keys = self._pack(entries)
         logits = self._logit_buffer(len(row_keys))
-        out = self.model.forward(ctx, self.views, rows, logits)
-        return StepOutput(logits=out, rows=row_keys)
+        graph_key = None
+        if self.use_graphs and ctx.decode_only and len(row_keys) == ctx.tokens:
+            # A step of single tokens that all want their logits.  Every launch argument is
+            # then a function of the number of items (and of buffer addresses).
+            graph_key = (ctx.tokens, logits.data_ptr())
+        if graph_key is None or graph_key in self._graph_failures:
+            out = self.model.forward(ctx, self.views, rows, logits)
+            return StepOutput(logits=out, rows=row_keys)
+        # launch shapes inside a graph must not depend on this step's lengths
+        ctx.max_kv_len = self.spec.max_positions
+        graph = self._graphs.get(graph_key)
+        if graph is None:
+            if graph_key not in self._graph_seen:
+                # first time: run directly, so that every buffer exists before a capture
+                self._graph_seen.add(graph_key)
+                out = self.model.forward(ctx, self.views, rows, logits)
+                return StepOutput(logits=out, rows=row_keys)
+            from ..ops.kernels import KernelError, StepGraph
+
+            graph = StepGraph()
+            StepGraph.begin()
+            try:
+                self.model.forward(ctx, self.views, rows, logits)
+                graph.end()
+            except Exception as error:       # the capture is abandoned, the step runs directly
+                StepGraph.abort()
+                self._graph_failures[graph_key] = f"{type(error).__name__}: {error}"
+                ctx.max_kv_len = max(item.start + 1 for item in ctx.items)
+                out = self.model.forward(ctx, self.views, rows, logits)
+                return StepOutput(logits=out, rows=row_keys)
+            self._graphs[graph_key] = graph
+        graph.launch()
+        return StepOutput(logits=logits[:len(row_keys)], rows=row_keys)

@@ -288,6 +288,56 @@ def sample(logits, inv_temperature, uniform, out):
     return out
 
 
+class StepGraph:
+    """An executable HIP graph of the launches issued between ``begin`` and ``end`` on the
+    current (non-default) stream."""
+
+    def __init__(self):
+        self.handle = None
+        self.nodes = 0
+        self.replays = 0
+
+    @staticmethod
+    def begin():
+        lib = load_library()
+        lib.ps_graph_begin.argtypes = [c_void_p]
+        lib.ps_graph_begin.restype = c_int
+        if lib.ps_graph_begin(_stream()) != 0:
+            raise KernelError(lib.ps_last_error().decode())
+
+    def end(self):
+        lib = load_library()
+        lib.ps_graph_end.argtypes = [c_void_p, ctypes.POINTER(c_void_p), ctypes.POINTER(c_int)]
+        lib.ps_graph_end.restype = c_int
+        handle = c_void_p()
+        nodes = c_int(0)
+        if lib.ps_graph_end(_stream(), ctypes.byref(handle), ctypes.byref(nodes)) != 0:
+            raise KernelError(lib.ps_last_error().decode())
+        self.handle = handle
+        self.nodes = nodes.value
+
+    @staticmethod
+    def abort():
+        lib = load_library()
+        lib.ps_graph_abort.argtypes = [c_void_p]
+        lib.ps_graph_abort(_stream())
+
+    def launch(self):
+        lib = load_library()
+        lib.ps_graph_launch.argtypes = [c_void_p, c_void_p]
+        lib.ps_graph_launch.restype = c_int
+        if lib.ps_graph_launch(self.handle, _stream()) != 0:
+            raise KernelError(lib.ps_last_error().decode())
+        self.replays += 1
+
+    def destroy(self):
+        if self.handle is not None:
+            lib = load_library()
+            lib.ps_graph_destroy.argtypes = [c_void_p]
+            lib.ps_graph_destroy(self.handle)
+            self.handle = None
+
+
 def device_info():
     units = ctypes.c_int(0)
     lds = ctypes.c_int(0)

@@ -108,3 +108,62 @@ def test_trace_run_program(folders, references, tmp_path, dtype):
                 row += 1
             held[entry["id"]] = start + len(entry["tokens"])
     assert worst <= helpers.TOLERANCE[dtype] * scale, (worst, scale)
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_graph_replay_matches_direct_launches(folders, references, dtype):
+    """Decode steps replayed from a captured HIP graph give the logits of direct launches, on
+    every replay, with other work of the engine (a prompt portion, a batch of another size, a
+    finished request whose pages go to a new one) between the replays."""
+    from pagedserve_amd.engine import StepEntry
+
+    folder, config, page_size = folders["B"]
+    requests = _requests("B", config)
+    outputs = {}
+    for use_graphs in (False, True):
+        names = ["r2", "r3", "r4"]
+        from pagedserve_amd.engine import Engine
+        from pagedserve_amd.model import load_model
+
+        model, _ = load_model(folder, dtype=dtype)
+        engine = Engine(model, num_pages=30, page_size=page_size, max_requests=4,
+                        max_step_tokens=128, use_graphs=use_graphs)
+        rows = {}
+
+        def run(entries):
+            out = engine.step(entries)
+            values = out.logits.double().cpu()
+            for index, key in enumerate(out.rows):
+                rows[key] = values[index]
+
+        cursor = {}
+        for name in names:
+            run([StepEntry(name, requests[name][:20], list(range(20)))])
+            cursor[name] = 20
+        for turn in range(30):
+            live = [name for name in names if cursor[name] < len(requests[name])]
+            batch = live if turn % 5 else live[:1]
+            run([StepEntry(name, [requests[name][cursor[name]]], [0]) for name in batch])
+            for name in batch:
+                cursor[name] += 1
+            if turn == 7:       # a prompt portion of another request between two replays
+                run([StepEntry("r1", requests["r1"][:9], list(range(9)))])
+                engine.finish("r1")
+            if turn == 15:      # r2 ends; its pages go to a newcomer that joins the decode batch
+                engine.finish("r2")
+                names[0] = "r0"
+                run([StepEntry("r0", requests["r0"][:3], [0, 1, 2])])
+                cursor["r0"] = 3
+        outputs[use_graphs] = rows
+        if use_graphs:
+            summary = engine.graph_summary()
+            assert summary["captured_graphs"] >= 2 and summary["graph_replays"] >= 15, summary
+            assert not summary["capture_failures"], summary
+            assert all(nodes > 10 for nodes in summary["graph_nodes"].values())
+    reference = references[("B", dtype == "bfloat16")]
+    for rows in outputs.values():
+        error, scale, where = helpers.max_error(rows, reference)
+        assert error <= helpers.TOLERANCE[dtype] * scale, (error, scale, where)
+    assert outputs[True].keys() == outputs[False].keys()
+    worst = max(float((outputs[True][key] - outputs[False][key]).abs().max()) for key in outputs[True])
+    assert worst <= helpers.TOLERANCE[dtype] * 0.2 * float(reference["r4"].abs().max())
