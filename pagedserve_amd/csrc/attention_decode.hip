@@ -198,28 +198,26 @@ __global__ __launch_bounds__(64 * AD_WAVES) void attention_decode_kernel(
   }
 }
 
-// out = sum_s acc_s e^{m_s - M} / sum_s l_s e^{m_s - M}
+// out = sum_s acc_s e^{m_s - M} / sum_s l_s e^{m_s - M}.  One wave per (token, head); lane s
+// first fetches (m_s, l_s) of split s (splits <= 64), so the weights cost one trip to memory.
 template <typename T>
 __global__ __launch_bounds__(64) void attention_reduce_kernel(
     const float* __restrict__ partial, T* __restrict__ out, int64_t out_stride,
     const int* __restrict__ tok_list, int heads, int head_dim, int splits) {
   const int n = blockIdx.x;
   const int head = blockIdx.y;
+  const int lane = threadIdx.x;
   const int t = tok_list ? tok_list[n] : n;
-  const float* src = partial + ((int64_t)n * heads + head) * splits * (head_dim + 2);
-  float total_m = -INFINITY;
-  for (int s = 0; s < splits; ++s) total_m = fmaxf(total_m, src[s * (head_dim + 2) + head_dim]);
-  float total_l = 0.f;
-  for (int s = 0; s < splits; ++s) {
-    const float m_s = src[s * (head_dim + 2) + head_dim];
-    if (m_s != -INFINITY) total_l += src[s * (head_dim + 2) + head_dim + 1] * expf(m_s - total_m);
-  }
-  for (int d = threadIdx.x; d < head_dim; d += 64) {
+  const int stride = head_dim + 2;
+  const float* src = partial + ((int64_t)n * heads + head) * splits * stride;
+  const float m_s = lane < splits ? src[lane * stride + head_dim] : -INFINITY;
+  const float l_s = lane < splits ? src[lane * stride + head_dim + 1] : 0.f;
+  const float total_m = wave_max(m_s);
+  const float weight = (m_s == -INFINITY) ? 0.f : expf(m_s - total_m);
+  const float total_l = wave_sum(l_s * weight);
+  for (int d = lane; d < head_dim; d += 64) {
     float value = 0.f;
-    for (int s = 0; s < splits; ++s) {
-      const float m_s = src[s * (head_dim + 2) + head_dim];
-      if (m_s != -INFINITY) value += src[s * (head_dim + 2) + d] * expf(m_s - total_m);
-    }
+    for (int s = 0; s < splits; ++s) value = fmaf(src[s * stride + d], __shfl(weight, s, 64), value);
     out[(int64_t)t * out_stride + (int64_t)head * head_dim + d] = from_float<T>(value / total_l);
   }
 }
@@ -274,7 +272,7 @@ extern "C" int ps_attention_decode(const void* q, int64_t q_stride, const void* 
   PS_REQUIRE(head_dim > 0 && head_dim % 16 == 0 && head_dim <= 256,
              "ps_attention_decode: head_dim %d must be a multiple of 16 up to 256", head_dim);
   PS_REQUIRE(window >= 0, "ps_attention_decode: negative window");
-  PS_REQUIRE(splits >= 1 && splits <= 65535 && heads <= 65535,
+  PS_REQUIRE(splits >= 1 && splits <= 64 && heads <= 65535,
              "ps_attention_decode: splits %d / heads %d out of range", splits, heads);
   PS_REQUIRE(dtype == PS_F32 || dtype == PS_BF16, "ps_attention_decode: unknown dtype %d", dtype);
   if (splits > 1) {

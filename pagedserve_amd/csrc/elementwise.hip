@@ -75,12 +75,54 @@ extern "C" int ps_embed(const void* table, const void* pos_table, const int* ids
 
 // ---------------------------------------------------------------- norms
 // mean, centred values, biased variance of the centred values, rsqrt(var + eps), scale and
-// shift (reference: src/kernels/triton_residual_layernorm.py:25-39).  One block per row; the
-// row is read three times (it stays in cache), so any width works.
+// shift (reference: src/kernels/triton_residual_layernorm.py:25-39).
+//
+// norm_wave_kernel: one wave per row, the row held in registers (width <= 64 * VPT): one
+// trip to memory, reductions by shuffles, no barrier.  norm_block_kernel: one block per row,
+// the row read three times (it stays in cache), any width.
+template <typename T, bool RMS, int VPT>
+__global__ __launch_bounds__(256) void norm_wave_kernel(
+    const float* __restrict__ x, const int* __restrict__ rows, const float* __restrict__ gamma,
+    const float* __restrict__ beta, T* __restrict__ out, int n_rows, int width, float eps) {
+  const int lane = threadIdx.x & 63;
+  const int r = blockIdx.x * 4 + (threadIdx.x >> 6);
+  if (r >= n_rows) return;
+  const float* src = x + (int64_t)(rows ? rows[r] : r) * width;
+  float v[VPT];
+  float sum = 0.f;
+#pragma unroll
+  for (int i = 0; i < VPT; ++i) {
+    const int col = lane + i * 64;
+    v[i] = col < width ? src[col] : 0.f;
+    sum += v[i];
+  }
+  float mean = 0.f;
+  if (!RMS) mean = wave_sum(sum) / (float)width;
+  float sq = 0.f;
+#pragma unroll
+  for (int i = 0; i < VPT; ++i) {
+    const int col = lane + i * 64;
+    const float c = col < width ? v[i] - mean : 0.f;
+    v[i] = c;
+    sq += c * c;
+  }
+  const float inv_std = 1.0f / sqrtf(wave_sum(sq) / (float)width + eps);
+  T* dst = out + (int64_t)r * width;
+#pragma unroll
+  for (int i = 0; i < VPT; ++i) {
+    const int col = lane + i * 64;
+    if (col < width) {
+      float y = v[i] * inv_std * gamma[col];
+      if (!RMS && beta != nullptr) y += beta[col];
+      dst[col] = from_float<T>(y);
+    }
+  }
+}
+
 template <typename T, bool RMS>
-__global__ void norm_kernel(const float* __restrict__ x, const int* __restrict__ rows,
-                            const float* __restrict__ gamma, const float* __restrict__ beta,
-                            T* __restrict__ out, int width, float eps) {
+__global__ void norm_block_kernel(const float* __restrict__ x, const int* __restrict__ rows,
+                                  const float* __restrict__ gamma, const float* __restrict__ beta,
+                                  T* __restrict__ out, int width, float eps) {
   __shared__ float scratch[16];
   const int r = blockIdx.x;
   const float* src = x + (int64_t)(rows ? rows[r] : r) * width;
@@ -105,6 +147,26 @@ __global__ void norm_kernel(const float* __restrict__ x, const int* __restrict__
   }
 }
 
+template <typename T, bool RMS>
+static void launch_norm(const float* x, const int* rows, const float* gamma, const float* beta,
+                        void* out, int n_rows, int width, float eps, hipStream_t s) {
+  const int per_lane = (width + 63) / 64;
+  const dim3 grid((n_rows + 3) / 4);
+#define PS_LAUNCH_NW(VPT)                                                                       \
+  hipLaunchKernelGGL((norm_wave_kernel<T, RMS, VPT>), grid, dim3(256), 0, s, x, rows, gamma, beta, \
+                     (T*)out, n_rows, width, eps)
+  if (per_lane <= 2) PS_LAUNCH_NW(2);
+  else if (per_lane <= 4) PS_LAUNCH_NW(4);
+  else if (per_lane <= 8) PS_LAUNCH_NW(8);
+  else if (per_lane <= 12) PS_LAUNCH_NW(12);
+  else if (per_lane <= 16) PS_LAUNCH_NW(16);
+  else if (per_lane <= 32) PS_LAUNCH_NW(32);
+  else
+    hipLaunchKernelGGL((norm_block_kernel<T, RMS>), dim3(n_rows), dim3(256), 0, s, x, rows, gamma,
+                       beta, (T*)out, width, eps);
+#undef PS_LAUNCH_NW
+}
+
 extern "C" int ps_norm(const float* x, const int* rows, const float* gamma, const float* beta,
                        void* out, int n_rows, int width, float eps, int rms, int out_dtype,
                        void* stream) {
@@ -112,17 +174,14 @@ extern "C" int ps_norm(const float* x, const int* rows, const float* gamma, cons
   PS_REQUIRE(out_dtype == PS_F32 || out_dtype == PS_BF16, "ps_norm: unknown dtype %d", out_dtype);
   PS_REQUIRE(eps > 0.f, "ps_norm: eps must be positive");
   if (n_rows == 0) return 0;
-  const int threads = width >= 1024 ? 256 : (width >= 256 ? 128 : 64);
   hipStream_t s = (hipStream_t)stream;
-#define PS_LAUNCH_NORM(T, RMS)                                                              \
-  hipLaunchKernelGGL((norm_kernel<T, RMS>), dim3(n_rows), dim3(threads), 0, s, x, rows, gamma, \
-                     beta, (T*)out, width, eps)
   if (out_dtype == PS_F32) {
-    if (rms) PS_LAUNCH_NORM(float, true); else PS_LAUNCH_NORM(float, false);
+    if (rms) launch_norm<float, true>(x, rows, gamma, beta, out, n_rows, width, eps, s);
+    else launch_norm<float, false>(x, rows, gamma, beta, out, n_rows, width, eps, s);
   } else {
-    if (rms) PS_LAUNCH_NORM(bf16_t, true); else PS_LAUNCH_NORM(bf16_t, false);
+    if (rms) launch_norm<bf16_t, true>(x, rows, gamma, beta, out, n_rows, width, eps, s);
+    else launch_norm<bf16_t, false>(x, rows, gamma, beta, out, n_rows, width, eps, s);
   }
-#undef PS_LAUNCH_NORM
   PS_CHECK_LAUNCH("ps_norm");
   return 0;
 }

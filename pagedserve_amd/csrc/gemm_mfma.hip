@@ -11,11 +11,14 @@
 //   product needs).  The float instantiation multiplies true 32-bit inputs.
 //
 // gemm_nt_skinny_kernel — up to 64 rows (decode), bfloat16.  The product is bound by reading W
-//   once, so weights go straight from global memory into MFMA operands: a wave owns 16 weight
-//   rows, every lane loads 32 contiguous bytes of one row per 64 k, and v_mfma_f32_16x16x32_bf16
-//   takes the weights as its row operand and up to four blocks of 16 activation rows as column
-//   operands.  K may be split over blocks; partial sums are then added into the float output
-//   with hardware float atomics (only the residual epilogue allows it).
+//   once, and at these sizes by the latency of that one trip to memory, so weights go straight
+//   from global memory into MFMA operands and every wave issues all its loads before it
+//   multiplies.  A block owns 16 weight rows; its four waves take a quarter of k each (every
+//   lane loads 32 contiguous bytes of one row per 64 k) and feed v_mfma_f32_16x16x32_bf16 with
+//   the weights as row operand and up to four blocks of 16 activation rows as column operands;
+//   the four partial tiles are summed through LDS.  K may also be split over blocks; those
+//   partial sums are added into the float output with hardware float atomics (only the
+//   residual epilogue allows it).
 //
 // Accumulation is float in all cases.  Shapes that the kernels cannot take (k not a multiple
 // of 8 elements, unaligned rows) are refused by ps_gemm_nt_mfma_supported and run on the
@@ -165,16 +168,16 @@ __global__ __launch_bounds__(256) void gemm_nt_tiled_kernel(
 
 // ------------------------------------------------------------------------------- skinny
 #define SK_WAVES 4
-#define SK_ROWS (16 * SK_WAVES)
+#define SK_UNROLL 4   // 64-k steps whose loads are issued together
 
 template <typename TOut, int EPI, int MB>
 __global__ __launch_bounds__(64 * SK_WAVES) void gemm_nt_skinny_kernel(
     const bf16_t* __restrict__ a, const bf16_t* __restrict__ w, const float* __restrict__ bias,
     TOut* __restrict__ c, int m, int n, int k, int lda, int ldc, int k_chunk, int k_splits) {
+  __shared__ float partial[SK_WAVES][MB][4][64];
   const int lane = threadIdx.x & 63;
   const int wave = threadIdx.x >> 6;
-  const int n0 = blockIdx.x * SK_ROWS + wave * 16;
-  if (n0 >= n) return;
+  const int n0 = blockIdx.x * 16;
   const int split = blockIdx.y;
   const int k_begin = split * k_chunk;
   const int k_end = k_begin + k_chunk < k ? k_begin + k_chunk : k;
@@ -193,46 +196,61 @@ __global__ __launch_bounds__(64 * SK_WAVES) void gemm_nt_skinny_kernel(
   for (int b = 0; b < MB; ++b) acc[b] = f32x4{0.f, 0.f, 0.f, 0.f};
 
   const uint4 zero = {0u, 0u, 0u, 0u};
-  for (int k0 = k_begin; k0 < k_end; k0 += 64) {
-    const int kk = k0 + group * 16;
-    const bool first = kk < k_end;
-    const bool second = kk + 8 < k_end;
-    const uint4 w0 = first ? *reinterpret_cast<const uint4*>(w_ptr + k0) : zero;
-    const uint4 w1 = second ? *reinterpret_cast<const uint4*>(w_ptr + k0 + 8) : zero;
+  // wave `wave` takes the 64-k steps wave, wave + 4, ... of the block's range
+  for (int k0 = k_begin + wave * 64; k0 < k_end; k0 += SK_WAVES * SK_UNROLL * 64) {
+    uint4 wf[SK_UNROLL][2], xf[SK_UNROLL][MB][2];
 #pragma unroll
-    for (int b = 0; b < MB; ++b) {
-      const uint4 x0 = first ? *reinterpret_cast<const uint4*>(a_ptr[b] + k0) : zero;
-      const uint4 x1 = second ? *reinterpret_cast<const uint4*>(a_ptr[b] + k0 + 8) : zero;
-      acc[b] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(*reinterpret_cast<const bf16x8*>(&w0),
-                                                       *reinterpret_cast<const bf16x8*>(&x0),
-                                                       acc[b], 0, 0, 0);
-      acc[b] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(*reinterpret_cast<const bf16x8*>(&w1),
-                                                       *reinterpret_cast<const bf16x8*>(&x1),
-                                                       acc[b], 0, 0, 0);
+    for (int u = 0; u < SK_UNROLL; ++u) {
+      const int ku = k0 + u * SK_WAVES * 64;
+      const int kk = ku + group * 16;
+      const bool first = kk < k_end;
+      const bool second = kk + 8 < k_end;
+      wf[u][0] = first ? *reinterpret_cast<const uint4*>(w_ptr + ku) : zero;
+      wf[u][1] = second ? *reinterpret_cast<const uint4*>(w_ptr + ku + 8) : zero;
+#pragma unroll
+      for (int b = 0; b < MB; ++b) {
+        xf[u][b][0] = first ? *reinterpret_cast<const uint4*>(a_ptr[b] + ku) : zero;
+        xf[u][b][1] = second ? *reinterpret_cast<const uint4*>(a_ptr[b] + ku + 8) : zero;
+      }
     }
+#pragma unroll
+    for (int u = 0; u < SK_UNROLL; ++u)
+#pragma unroll
+      for (int b = 0; b < MB; ++b)
+#pragma unroll
+        for (int h = 0; h < 2; ++h)
+          acc[b] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(
+              *reinterpret_cast<const bf16x8*>(&wf[u][h]),
+              *reinterpret_cast<const bf16x8*>(&xf[u][b][h]), acc[b], 0, 0, 0);
   }
 
-  // element i of a 16 x 16 accumulator: weight row (lane / 16) * 4 + i, activation row lane % 16
+#pragma unroll
+  for (int b = 0; b < MB; ++b)
+#pragma unroll
+    for (int i = 0; i < 4; ++i) partial[wave][b][i][lane] = acc[b][i];
+  __syncthreads();
+
+  // element i of a 16 x 16 accumulator: weight row (lane / 16) * 4 + i, activation row lane % 16.
+  // Thread (wave, lane) finishes element i = wave of every block b.
+  const int i = wave;
+  const int col = n0 + group * 4 + i;
+  if (col >= n) return;
 #pragma unroll
   for (int b = 0; b < MB; ++b) {
     const int row = b * 16 + sub;
     if (row >= m) continue;
-#pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      const int col = n0 + group * 4 + i;
-      if (col >= n) continue;
-      float v = acc[b][i];
-      if (bias != nullptr && split == 0) v += bias[col];
-      TOut* dst = c + (int64_t)row * ldc + col;
-      if (EPI == PS_EPI_RESIDUAL) {
-        if (k_splits > 1) {
-          unsafeAtomicAdd(reinterpret_cast<float*>(dst), v);
-        } else {
-          *dst = from_float<TOut>(v + to_float<TOut>(*dst));
-        }
+    float v = partial[0][b][i][lane] + partial[1][b][i][lane] + partial[2][b][i][lane] +
+              partial[3][b][i][lane];
+    if (bias != nullptr && split == 0) v += bias[col];
+    TOut* dst = c + (int64_t)row * ldc + col;
+    if (EPI == PS_EPI_RESIDUAL) {
+      if (k_splits > 1) {
+        unsafeAtomicAdd(reinterpret_cast<float*>(dst), v);
       } else {
-        *dst = from_float<TOut>(apply_activation<EPI>(v));
+        *dst = from_float<TOut>(v + to_float<TOut>(*dst));
       }
+    } else {
+      *dst = from_float<TOut>(apply_activation<EPI>(v));
     }
   }
 }
@@ -270,7 +288,7 @@ template <typename TOut, int EPI>
 static void launch_skinny_mb(const void* a, const void* w, const float* bias, void* c, int m,
                              int n, int k, int lda, int ldc, int k_chunk, int k_splits,
                              hipStream_t s) {
-  dim3 grid((n + SK_ROWS - 1) / SK_ROWS, k_splits);
+  dim3 grid((n + 15) / 16, k_splits);
   dim3 block(64 * SK_WAVES);
 #define PS_LAUNCH_SK(MB)                                                                       \
   hipLaunchKernelGGL((gemm_nt_skinny_kernel<TOut, EPI, MB>), grid, block, 0, s,                \
@@ -287,17 +305,12 @@ static void launch_skinny_mb(const void* a, const void* w, const float* bias, vo
 template <typename TOut>
 static int launch_skinny(const void* a, const void* w, const float* bias, void* c, int m, int n,
                          int k, int lda, int ldc, int epilogue, hipStream_t s) {
-  // Split k only where partial sums can be added in place, and only to fill the chip.
+  // A block covers 1024 k with one round of loads.  Longer k is split over blocks where the
+  // partial sums can be added in place (residual epilogue), else the block loops.
   int k_splits = 1;
-  if (epilogue == PS_EPI_RESIDUAL) {
-    const int waves = (n + 15) / 16;
-    const int wanted = (1024 + waves - 1) / waves;
-    const int possible = k / 128 > 0 ? k / 128 : 1;
-    k_splits = wanted < possible ? wanted : possible;
-    if (k_splits < 1) k_splits = 1;
-  }
+  if (epilogue == PS_EPI_RESIDUAL && k > 1024) k_splits = (k + 1023) / 1024;
   int k_chunk = (k + k_splits - 1) / k_splits;
-  k_chunk = (k_chunk + 63) / 64 * 64;
+  k_chunk = (k_chunk + 255) / 256 * 256;
   k_splits = (k + k_chunk - 1) / k_chunk;
   switch (epilogue) {
     case PS_EPI_NONE:

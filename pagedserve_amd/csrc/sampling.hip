@@ -2,106 +2,132 @@
 // the reference's path, src/scheduler/orca_scheduler.py:250) or a draw from
 // softmax(logits / temperature) by inverse CDF.  The uniform number of a row is made by the
 // host from (seed, request, step), so a draw does not depend on what else is in the batch.
-// One 256-thread block per row; thread i owns the contiguous id range [i*c, (i+1)*c), which
-// fixes the order of every sum.
+//
+// One 1024-thread block per row.  The maximum is found with coalesced strided reads.  For a
+// draw, wave w owns the contiguous id range [w * seg, (w + 1) * seg): it sums
+// exp((l - max) / T) over its range 64 ids at a time, thread 0 picks the range that holds
+// uniform * total, and that wave walks its range again with a prefix sum over each 64 ids to
+// find the first id whose cumulative mass exceeds the goal.
 #include <math.h>
 
 #include "common.h"
 #include "pagedserve_hip.h"
 
-#define SM_THREADS 256
+#define SM_THREADS 1024
+#define SM_WAVES (SM_THREADS / 64)
 
 __global__ __launch_bounds__(SM_THREADS) void sample_kernel(
     const float* __restrict__ logits, int64_t ld, const float* __restrict__ inv_temperature,
     const float* __restrict__ uniform, int* __restrict__ tokens, int vocab) {
-  __shared__ float s_val[SM_THREADS];
-  __shared__ int s_idx[SM_THREADS];
-  __shared__ float s_sum[SM_THREADS];
+  __shared__ float s_val[SM_WAVES];
+  __shared__ int s_idx[SM_WAVES];
+  __shared__ float s_sum[SM_WAVES];
   __shared__ int s_choice;
   __shared__ float s_before;
   __shared__ float s_goal;
 
   const int r = blockIdx.x;
   const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = tid >> 6;
   const float* row = logits + (int64_t)r * ld;
-  const int chunk = (vocab + SM_THREADS - 1) / SM_THREADS;
-  const int begin = tid * chunk;
-  const int end = begin + chunk < vocab ? begin + chunk : vocab;
 
   // maximum and its first index
   float best = -INFINITY;
   int best_idx = vocab;
-  for (int i = begin; i < end; ++i) {
+  for (int i = tid; i < vocab; i += SM_THREADS) {
     const float v = row[i];
     if (v > best) {
       best = v;
       best_idx = i;
     }
   }
-  s_val[tid] = best;
-  s_idx[tid] = best_idx;
-  __syncthreads();
-  for (int stride = SM_THREADS / 2; stride > 0; stride >>= 1) {
-    if (tid < stride) {
-      const float other = s_val[tid + stride];
-      const int other_idx = s_idx[tid + stride];
-      if (other > s_val[tid] || (other == s_val[tid] && other_idx < s_idx[tid])) {
-        s_val[tid] = other;
-        s_idx[tid] = other_idx;
-      }
+#pragma unroll
+  for (int offset = 32; offset > 0; offset >>= 1) {
+    const float other = __shfl_xor(best, offset, 64);
+    const int other_idx = __shfl_xor(best_idx, offset, 64);
+    if (other > best || (other == best && other_idx < best_idx)) {
+      best = other;
+      best_idx = other_idx;
     }
-    __syncthreads();
   }
-  const float row_max = s_val[0];
-  const int row_argmax = s_idx[0] < vocab ? s_idx[0] : 0;
+  if (lane == 0) {
+    s_val[wave] = best;
+    s_idx[wave] = best_idx;
+  }
+  __syncthreads();
+  float row_max = s_val[0];
+  int row_argmax = s_idx[0];
+#pragma unroll
+  for (int w = 1; w < SM_WAVES; ++w) {
+    if (s_val[w] > row_max || (s_val[w] == row_max && s_idx[w] < row_argmax)) {
+      row_max = s_val[w];
+      row_argmax = s_idx[w];
+    }
+  }
+  if (row_argmax >= vocab) row_argmax = 0;
   const float inv_t = inv_temperature ? inv_temperature[r] : 0.f;
   if (inv_t <= 0.f) {
     if (tid == 0) tokens[r] = row_argmax;
     return;
   }
 
-  // unnormalised probabilities exp((l - max) / T), summed per thread range
+  // unnormalised probabilities exp((l - max) / T), summed per wave range
+  const int seg = ((vocab + SM_WAVES - 1) / SM_WAVES + 63) / 64 * 64;
+  const int begin = wave * seg;
+  const int end = begin + seg < vocab ? begin + seg : vocab;
   float partial = 0.f;
-  for (int i = begin; i < end; ++i) partial += expf((row[i] - row_max) * inv_t);
-  s_sum[tid] = partial;
+  for (int i = begin + lane; i < end; i += 64) partial += expf((row[i] - row_max) * inv_t);
+  partial = wave_sum(partial);
+  if (lane == 0) s_sum[wave] = partial;
   __syncthreads();
   if (tid == 0) {
     float total = 0.f;
-    for (int i = 0; i < SM_THREADS; ++i) total += s_sum[i];
+    for (int w = 0; w < SM_WAVES; ++w) total += s_sum[w];
     const float goal = uniform[r] * total;
     float before = 0.f;
     int choice = -1;
-    for (int i = 0; i < SM_THREADS; ++i) {
-      if (s_sum[i] > 0.f && before + s_sum[i] > goal) {
-        choice = i;
+    for (int w = 0; w < SM_WAVES; ++w) {
+      if (s_sum[w] > 0.f && before + s_sum[w] > goal) {
+        choice = w;
         break;
       }
-      before += s_sum[i];
+      before += s_sum[w];
     }
     if (choice < 0) {
       // rounding left the goal at or beyond the total: the last non-empty range takes it
-      choice = SM_THREADS - 1;
+      choice = SM_WAVES - 1;
       while (choice > 0 && s_sum[choice] <= 0.f) --choice;
       before = 0.f;
-      for (int i = 0; i < choice; ++i) before += s_sum[i];
+      for (int w = 0; w < choice; ++w) before += s_sum[w];
     }
     s_choice = choice;
     s_before = before;
     s_goal = goal;
   }
   __syncthreads();
-  if (tid == s_choice) {
-    float running = s_before;
-    int token = end - 1 >= begin ? end - 1 : row_argmax;
-    for (int i = begin; i < end; ++i) {
-      running += expf((row[i] - row_max) * inv_t);
-      if (running > s_goal) {
-        token = i;
-        break;
-      }
+  if (wave != s_choice) return;
+  float running = s_before;
+  const float goal = s_goal;
+  int token = -1;
+  int last_positive = -1;
+  for (int base = begin; base < end && token < 0; base += 64) {
+    const int i = base + lane;
+    const float e = i < end ? expf((row[i] - row_max) * inv_t) : 0.f;
+    float prefix = e;  // inclusive prefix sum over the wave
+#pragma unroll
+    for (int offset = 1; offset < 64; offset <<= 1) {
+      const float other = __shfl_up(prefix, offset, 64);
+      if (lane >= offset) prefix += other;
     }
-    tokens[r] = token;
+    const unsigned long long hits = __ballot(i < end && e > 0.f && running + prefix > goal);
+    const unsigned long long positive = __ballot(i < end && e > 0.f);
+    if (positive) last_positive = base + 63 - __clzll(positive);
+    if (hits) token = base + __ffsll((long long)hits) - 1;
+    running += __shfl(prefix, 63, 64);
   }
+  if (token < 0) token = last_positive >= 0 ? last_positive : row_argmax;
+  if (lane == 0) tokens[r] = token;
 }
 
 extern "C" int ps_sample(const float* logits, int64_t ld, const float* inv_temperature,

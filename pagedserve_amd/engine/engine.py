@@ -61,7 +61,7 @@ class Engine:
         self.views = model.cache_views(self.cache)
         self.workspace = Workspace(max_step_tokens, self.device)
         self.table_width = -(-self.spec.max_positions // page_size)
-        capacity = (5 * max_step_tokens + 3 * max_requests + 1
+        capacity = (6 * max_step_tokens + 5 * max_requests + 1
                     + len(groups) * max_requests * self.table_width + 16)
         self._meta_device = torch.empty(capacity, dtype=torch.int32, device=self.device)
         self._meta_host = [torch.empty(capacity, dtype=torch.int32, pin_memory=True) for _ in range(2)]
@@ -178,6 +178,8 @@ class Engine:
         wants = [len(entry.want) for entry in entries]
         wanted = sum(wants)
         singles = counts.count(1)
+        # items with several tokens are cut into tiles of 64 queries for the tiled kernel
+        tiles = sum(-(-count // 64) for count in counts if count > 1)
         groups = len(cache.groups)
         width = self.table_width
         offsets = {}
@@ -185,7 +187,8 @@ class Engine:
         for name, size in (("token_ids", tokens), ("positions", tokens), ("tok_item", tokens),
                            ("cu_tokens", items + 1), ("kv_lens", items), ("slots", items),
                            ("rows", wanted), ("single_tokens", singles),
-                           ("portion_tokens", tokens - singles)):
+                           ("portion_tokens", tokens - singles), ("tile_item", tiles),
+                           ("tile_q0", tiles)):
             offsets[name] = (cursor, size)
             cursor += size
         for group in range(groups):
@@ -230,7 +233,8 @@ class Engine:
             tok_item, cu, kv_lens = section("tok_item"), section("cu_tokens"), section("kv_lens")
             rows = section("rows")
             single_tokens, portion_tokens = section("single_tokens"), section("portion_tokens")
-            flat = row_cursor = single_cursor = portion_cursor = max_kv = 0
+            tile_item, tile_q0 = section("tile_item"), section("tile_q0")
+            flat = row_cursor = single_cursor = portion_cursor = max_kv = tile_cursor = 0
             for index, (entry, record, start, count) in enumerate(zip(entries, records, starts, counts)):
                 token_ids[flat:flat + count] = entry.tokens
                 positions[flat:flat + count] = np.arange(start, start + count, dtype=np.int32)
@@ -245,6 +249,10 @@ class Engine:
                     portion_tokens[portion_cursor:portion_cursor + count] = np.arange(
                         flat, flat + count, dtype=np.int32)
                     portion_cursor += count
+                    for q0 in range(0, count, 64):
+                        tile_item[tile_cursor] = index
+                        tile_q0[tile_cursor] = q0
+                        tile_cursor += 1
                 for place in entry.want:
                     rows[row_cursor] = flat + int(place)
                     row_keys.append((entry.request_id, start + int(place)))
@@ -273,7 +281,8 @@ class Engine:
             page_size=self.page_size, workspace=self.workspace,
             decode_only=singles == items, max_kv_len=max_kv,
             single_tokens=view("single_tokens"), portion_tokens=view("portion_tokens"),
-            max_positions=self.spec.max_positions)
+            max_positions=self.spec.max_positions,
+            tile_item=view("tile_item"), tile_q0=view("tile_q0"))
         return ctx, view("rows"), row_keys
 
     def _run(self, entries) -> StepOutput:

@@ -34,6 +34,9 @@ _SIGNATURES = {
     "ps_attention_decode": [c_void_p, c_int64, c_void_p, c_void_p, c_void_p, c_int64, c_void_p,
                             c_int64, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int,
                             c_int, c_int, c_int, c_int, c_float, c_int, c_int, c_int, c_void_p],
+    "ps_attention_prefill": [c_void_p, c_int64, c_void_p, c_void_p, c_void_p, c_int64, c_void_p,
+                             c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int,
+                             c_int, c_int, c_int, c_float, c_int, c_int, c_void_p],
     "ps_sample": [c_void_p, c_int64, c_void_p, c_void_p, c_void_p, c_int, c_int, c_void_p],
 }
 
@@ -266,6 +269,43 @@ def attention_decode(q, k_pool, v_pool, out, tok_item, tok_pos, tables, heads, s
           _ptr(tok_list), tok_item.data_ptr(), tok_pos.data_ptr(), tables.data_ptr(),
           tables.shape[1], count, heads, kv_heads, head_dim, page_size, pages, float(scale),
           int(window), int(splits), dtype_code(q.dtype), _stream())
+    return out
+
+
+PREFILL_TILE = 64
+
+
+def prefill_supported(dtype, head_dim) -> bool:
+    """Whether the tiled matrix-core kernel takes this storage type and head size."""
+    return dtype == torch.bfloat16 and head_dim % 16 == 0 and head_dim <= 128
+
+
+def attention_prefill(q, k_pool, v_pool, out, tile_item, tile_q0, cu_tokens, kv_lens, tables,
+                      heads, scale, window=0):
+    """Attention of items with several tokens, 64 queries per block, on the matrix cores."""
+    _check(q, "q", torch.bfloat16, 2)
+    _check(out, "out", torch.bfloat16, 2)
+    pages, kv_heads, page_size, head_dim = _check_pools(k_pool, v_pool, q.dtype)
+    q_stride = _rows(q, "q")
+    out_stride = _rows(out, "out")
+    if q.shape[1] != heads * head_dim or out.shape != q.shape:
+        raise KernelError("attention_prefill: q/out rows must hold heads x head_dim values")
+    for name, tensor in (("tile_item", tile_item), ("tile_q0", tile_q0), ("cu_tokens", cu_tokens),
+                         ("kv_lens", kv_lens)):
+        _check(tensor, name, torch.int32, 1)
+        if not tensor.is_contiguous():
+            raise KernelError(f"attention_prefill: {name} must be contiguous")
+    _check(tables, "tables", torch.int32, 2)
+    tiles = tile_item.numel()
+    items = kv_lens.numel()
+    if tile_q0.numel() != tiles or cu_tokens.numel() != items + 1 or tables.shape[0] != items \
+            or not tables.is_contiguous():
+        raise KernelError("attention_prefill: inconsistent tile or item arrays")
+    _call("ps_attention_prefill", q.data_ptr(), q_stride, k_pool.data_ptr(), v_pool.data_ptr(),
+          out.data_ptr(), out_stride, tile_item.data_ptr(), tile_q0.data_ptr(), tiles,
+          cu_tokens.data_ptr(), kv_lens.data_ptr(), tables.data_ptr(), tables.shape[1], heads,
+          kv_heads, head_dim, page_size, pages, float(scale), int(window), dtype_code(q.dtype),
+          _stream())
     return out
 
 

@@ -87,7 +87,11 @@ class Attention(Mixer):
                                      ctx.positions, tables, self.heads, self.scale, splits,
                                      partial=partial, window=self.window,
                                      tok_list=None if singles == tokens else ctx.single_tokens)
-        if singles < tokens:
+        if singles < tokens and kernels.prefill_supported(self.dtype, self.head_dim):
+            kernels.attention_prefill(q, cache.k_pool, cache.v_pool, context, ctx.tile_item,
+                                      ctx.tile_q0, ctx.cu_tokens, ctx.kv_lens, tables,
+                                      self.heads, self.scale, self.window)
+        elif singles < tokens:
             kernels.attention_rowwise(q, cache.k_pool, cache.v_pool, context, ctx.tok_item,
                                       ctx.positions, tables, self.heads, self.scale, self.window,
                                       tok_list=None if singles == 0 else ctx.portion_tokens)

@@ -163,4 +163,6 @@ class StepContext:
     single_tokens: Optional[torch.Tensor] = None   # int32: step indices of one-token items
     portion_tokens: Optional[torch.Tensor] = None  # int32: step indices of all other tokens
     max_positions: int = 0
+    tile_item: Optional[torch.Tensor] = None       # int32: item of each 64-query tile
+    tile_q0: Optional[torch.Tensor] = None         # int32: first query of the tile in its item
     extra: Optional[dict] = None

@@ -407,3 +407,73 @@ def test_kernels_refuse_bad_sizes():
     with pytest.raises(kernels.KernelError):
         kernels.gemm_nt(torch.zeros(2, 8, device="cuda"), torch.zeros(3, 9, device="cuda"), None,
                         torch.zeros(2, 3, device="cuda"))
+
+
+@pytest.mark.parametrize("heads,kv_heads,head_dim,page_size", [(1, 1, 32, 16), (4, 4, 16, 8), (6, 2, 48, 16), (2, 2, 128, 4), (12, 12, 64, 16), (3, 1, 80, 12)])
+@pytest.mark.parametrize("window", [0, 37])
+def test_attention_prefill_tiles(heads, kv_heads, head_dim, page_size, window):
+    """The tiled kernel against the row-wise one: fresh prompts and later portions of many
+    lengths in one launch (1 < count, portions that start inside a page, more than one tile,
+    a tile's last rows empty), fragmented tables, NaN behind every request's last key."""
+    from pagedserve_amd.ops import kernels
+
+    dtype = torch.bfloat16
+    # (cached before the portion, tokens of the portion)
+    items = [(0, 2), (0, 64), (0, 65), (0, 200), (30, 23), (17, 130), (100, 16), (63, 3), (250, 70)]
+    totals = [past + new for past, new in items]
+    k_pool, v_pool, tables = _paged_fixture(dtype, totals, kv_heads, head_dim, page_size, 51)
+    for index, total in enumerate(totals):
+        if total % page_size:
+            last = int(tables[index, total // page_size])
+            k_pool[last, :, total % page_size:] = float("nan")
+            v_pool[last, :, total % page_size:] = float("nan")
+    tokens = sum(new for _, new in items)
+    q = _rand((tokens, heads * head_dim), dtype, 52)
+    tok_item, tok_pos, tile_item, tile_q0, cu = [], [], [], [], [0]
+    for index, (past, new) in enumerate(items):
+        tok_item += [index] * new
+        tok_pos += list(range(past, past + new))
+        cu.append(cu[-1] + new)
+        for q0 in range(0, new, 64):
+            tile_item.append(index)
+            tile_q0.append(q0)
+
+    def dev(values):
+        return torch.tensor(values, dtype=torch.int32, device="cuda")
+
+    scale = head_dim ** -0.5
+    expected = torch.empty_like(q)
+    kernels.attention_rowwise(q, k_pool, v_pool, expected, dev(tok_item), dev(tok_pos), tables, heads, scale, window=window)
+    out = torch.full_like(q, float("nan"))
+    kernels.attention_prefill(q, k_pool, v_pool, out, dev(tile_item), dev(tile_q0), dev(cu), dev(totals),
+                              tables, heads, scale, window=window)
+    assert torch.isfinite(out.float()).all()
+    torch.testing.assert_close(out.double(), expected.double(), atol=2e-2, rtol=2e-2)
+
+
+def test_attention_prefill_far_key_and_causality():
+    """One early key is made to dominate for late queries only if they may see it; the query
+    just before it must not feel it (a mask off by one would)."""
+    from pagedserve_amd.ops import kernels
+
+    heads, head_dim, page_size, total = 1, 64, 16, 300
+    k_pool, v_pool, tables = _paged_fixture(torch.bfloat16, [total], heads, head_dim, page_size, 61)
+    k_pool *= 0.05
+    q = _rand((total, head_dim), torch.bfloat16, 62, 0.05)
+    direction = torch.ones(head_dim, device="cuda") / 8.0
+    target = 137
+    page = int(tables[0, target // page_size])
+    k_pool[page, 0, target % page_size] = (direction * 40).to(torch.bfloat16)
+    for row in (136, 137, 138, 299):
+        q[row] = (direction * 8).to(torch.bfloat16)
+    out = torch.empty_like(q)
+
+    def dev(values):
+        return torch.tensor(values, dtype=torch.int32, device="cuda")
+
+    kernels.attention_prefill(q, k_pool, v_pool, out, dev([0, 0, 0, 0, 0]), dev([0, 64, 128, 192, 256]),
+                              dev([0, total]), dev([total]), tables, heads, head_dim ** -0.5)
+    value = v_pool[page, 0, target % page_size].float()
+    for row in (137, 138, 299):
+        torch.testing.assert_close(out[row].float(), value, atol=2e-2, rtol=2e-2)
+    assert float((out[136].float() - value).abs().max()) > 0.3
