@@ -18,7 +18,6 @@
 #include "pagedserve_hip.h"
 
 #define AD_UNROLL 4
-#define AD_WAVES 4
 
 template <typename T>
 __device__ inline void load8(const T* p, float* out);
@@ -53,7 +52,7 @@ __device__ inline void merge_state(float& m, float& l, float* acc, float m_o, fl
   m = m_n;
 }
 
-template <typename T, int LPK>
+template <typename T, int LPK, int AD_WAVES>
 __global__ __launch_bounds__(64 * AD_WAVES) void attention_decode_kernel(
     const T* __restrict__ q, int64_t q_stride, const T* __restrict__ k_pool,
     const T* __restrict__ v_pool, T* __restrict__ out, int64_t out_stride,
@@ -99,24 +98,30 @@ __global__ __launch_bounds__(64 * AD_WAVES) void attention_decode_kernel(
        base += AD_WAVES * KEYS_PER_WAVE) {
     float kf[AD_UNROLL][8], vf[AD_UNROLL][8];
     bool valid[AD_UNROLL];
+    // Every load is unconditional from a clamped address and masked afterwards, so that the
+    // table entries, then all keys and values of the iteration, travel together.
+    int page[AD_UNROLL], within[AD_UNROLL];
 #pragma unroll
     for (int u = 0; u < AD_UNROLL; ++u) {
       const int key = base + u * GROUPS + group;
-      valid[u] = false;
-      if (key < range_end) {
-        const int logical = page_shift >= 0 ? (key >> page_shift) : key / page_size;
-        const int page = logical < table_width ? table[logical] : -1;
-        if (page >= 0 && page < num_pages) {
-          valid[u] = true;
-          if (has_dims) {
-            const int64_t offset =
-                (((int64_t)page * kv_heads + kv_head) * page_size + (key - logical * page_size)) *
-                    head_dim + dim0;
-            load8<T>(k_pool + offset, kf[u]);
-            load8<T>(v_pool + offset, vf[u]);
-          }
-        }
-      }
+      const int safe_key = key < range_end ? key : range_end - 1;
+      const int logical = page_shift >= 0 ? (safe_key >> page_shift) : safe_key / page_size;
+      within[u] = safe_key - logical * page_size;
+      page[u] = table[logical < table_width ? logical : table_width - 1];
+      valid[u] = key < range_end && logical < table_width;
+    }
+#pragma unroll
+    for (int u = 0; u < AD_UNROLL; ++u) {
+      valid[u] = valid[u] && page[u] >= 0 && page[u] < num_pages;
+      const int safe_page = valid[u] ? page[u] : 0;
+      const int64_t offset =
+          (((int64_t)safe_page * kv_heads + kv_head) * page_size + within[u]) * head_dim +
+          (has_dims ? dim0 : 0);
+      load8<T>(k_pool + offset, kf[u]);
+      load8<T>(v_pool + offset, vf[u]);
+    }
+#pragma unroll
+    for (int u = 0; u < AD_UNROLL; ++u) {
       if (!valid[u] || !has_dims) {
 #pragma unroll
         for (int i = 0; i < 8; ++i) {
@@ -175,6 +180,7 @@ __global__ __launch_bounds__(64 * AD_WAVES) void attention_decode_kernel(
 
   // merge the waves: one thread per head dimension
   const int d = threadIdx.x;
+  if (d >= 256) return;
   float block_m = -INFINITY;
 #pragma unroll
   for (int w = 0; w < AD_WAVES; ++w) block_m = fmaxf(block_m, s_ml[w][0]);
@@ -228,19 +234,27 @@ static int launch_decode(const void* q, int64_t q_stride, const void* k_pool, co
                          const int* tok_item, const int* tok_pos, const int* tables,
                          int table_width, int count, int heads, int kv_heads, int head_dim,
                          int page_size, int num_pages, float scale, int window, int splits,
-                         hipStream_t s) {
+                         int waves, hipStream_t s) {
   int page_shift = -1;
   if ((page_size & (page_size - 1)) == 0) {
     page_shift = 0;
     while ((1 << page_shift) < page_size) ++page_shift;
   }
   dim3 grid(count, heads, splits);
-  dim3 block(64 * AD_WAVES);
-#define PS_LAUNCH_AD(LPK)                                                                        \
-  hipLaunchKernelGGL((attention_decode_kernel<T, LPK>), grid, block, 0, s, (const T*)q, q_stride, \
-                     (const T*)k_pool, (const T*)v_pool, (T*)out, out_stride, partial, tok_list, \
-                     tok_item, tok_pos, tables, table_width, heads, kv_heads, head_dim,          \
-                     page_size, page_shift, num_pages, scale, window, splits)
+#define PS_LAUNCH_ADW(LPK, WAVES)                                                                \
+  hipLaunchKernelGGL((attention_decode_kernel<T, LPK, WAVES>), grid, dim3(64 * WAVES), 0, s,     \
+                     (const T*)q, q_stride, (const T*)k_pool, (const T*)v_pool, (T*)out,         \
+                     out_stride, partial, tok_list, tok_item, tok_pos, tables, table_width,      \
+                     heads, kv_heads, head_dim, page_size, page_shift, num_pages, scale, window, \
+                     splits)
+#define PS_LAUNCH_AD(LPK)            \
+  do {                               \
+    if (waves == 16) {               \
+      PS_LAUNCH_ADW(LPK, 16);        \
+    } else {                         \
+      PS_LAUNCH_ADW(LPK, 4);         \
+    }                                \
+  } while (0)
   const int lanes = head_dim / 8;
   if (lanes <= 2) PS_LAUNCH_AD(2);
   else if (lanes <= 4) PS_LAUNCH_AD(4);
@@ -248,6 +262,7 @@ static int launch_decode(const void* q, int64_t q_stride, const void* k_pool, co
   else if (lanes <= 16) PS_LAUNCH_AD(16);
   else PS_LAUNCH_AD(32);
 #undef PS_LAUNCH_AD
+#undef PS_LAUNCH_ADW
   PS_CHECK_LAUNCH("ps_attention_decode");
   if (splits > 1) {
     hipLaunchKernelGGL(attention_reduce_kernel<T>, dim3(count, heads), dim3(64), 0, s, partial,
@@ -263,7 +278,7 @@ extern "C" int ps_attention_decode(const void* q, int64_t q_stride, const void* 
                                    const int* tok_item, const int* tok_pos, const int* tables,
                                    int table_width, int count, int heads, int kv_heads,
                                    int head_dim, int page_size, int num_pages, float scale,
-                                   int window, int splits, int dtype, void* stream) {
+                                   int window, int splits, int waves, int dtype, void* stream) {
   PS_REQUIRE(count >= 0 && heads > 0 && kv_heads > 0 && page_size > 0 && num_pages > 0 &&
                  table_width > 0,
              "ps_attention_decode: bad sizes");
@@ -275,6 +290,8 @@ extern "C" int ps_attention_decode(const void* q, int64_t q_stride, const void* 
   PS_REQUIRE(splits >= 1 && splits <= 64 && heads <= 65535,
              "ps_attention_decode: splits %d / heads %d out of range", splits, heads);
   PS_REQUIRE(dtype == PS_F32 || dtype == PS_BF16, "ps_attention_decode: unknown dtype %d", dtype);
+  PS_REQUIRE(waves == 4 || waves == 16, "ps_attention_decode: blocks have 4 or 16 waves, not %d",
+             waves);
   if (splits > 1) {
     const int64_t need = (int64_t)count * heads * splits * (head_dim + 2);
     PS_REQUIRE(partial != nullptr && partial_floats >= need,
@@ -286,8 +303,8 @@ extern "C" int ps_attention_decode(const void* q, int64_t q_stride, const void* 
   if (dtype == PS_F32)
     return launch_decode<float>(q, q_stride, k_pool, v_pool, out, out_stride, partial, tok_list,
                                 tok_item, tok_pos, tables, table_width, count, heads, kv_heads,
-                                head_dim, page_size, num_pages, scale, window, splits, s);
+                                head_dim, page_size, num_pages, scale, window, splits, waves, s);
   return launch_decode<bf16_t>(q, q_stride, k_pool, v_pool, out, out_stride, partial, tok_list,
                                tok_item, tok_pos, tables, table_width, count, heads, kv_heads,
-                               head_dim, page_size, num_pages, scale, window, splits, s);
+                               head_dim, page_size, num_pages, scale, window, splits, waves, s);
 }

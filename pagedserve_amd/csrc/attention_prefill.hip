@@ -108,17 +108,19 @@ __global__ __launch_bounds__(256) void attention_prefill_kernel(
       const int key_local = c / (NDB * 2);
       const int dc = c - key_local * (NDB * 2);
       const int key = k0 + key_local;
-      uint4 kv = {0u, 0u, 0u, 0u}, vv = {0u, 0u, 0u, 0u};
-      if (key < key_end) {
-        const int logical = page_shift >= 0 ? (key >> page_shift) : key / page_size;
-        const int page = logical < table_width ? table[logical] : -1;
-        if (page >= 0 && page < num_pages) {
-          const int64_t offset =
-              (((int64_t)page * kv_heads + kv_head) * page_size + (key - logical * page_size)) * HD +
-              dc * 8;
-          kv = *reinterpret_cast<const uint4*>(k_pool + offset);
-          vv = *reinterpret_cast<const uint4*>(v_pool + offset);
-        }
+      // unconditional loads from clamped addresses, zeroed afterwards
+      const int safe_key = key < key_end ? key : key_end - 1;
+      const int logical = page_shift >= 0 ? (safe_key >> page_shift) : safe_key / page_size;
+      const int page = table[logical < table_width ? logical : table_width - 1];
+      const bool ok = key < key_end && logical < table_width && page >= 0 && page < num_pages;
+      const int64_t offset =
+          (((int64_t)(ok ? page : 0) * kv_heads + kv_head) * page_size +
+           (safe_key - logical * page_size)) * HD + dc * 8;
+      uint4 kv = *reinterpret_cast<const uint4*>(k_pool + offset);
+      uint4 vv = *reinterpret_cast<const uint4*>(v_pool + offset);
+      if (!ok) {
+        kv = uint4{0u, 0u, 0u, 0u};
+        vv = uint4{0u, 0u, 0u, 0u};
       }
       *reinterpret_cast<uint4*>(&k_lds[key_local * K_STRIDE + dc * 16]) = kv;
       const uint32_t words[4] = {vv.x, vv.y, vv.z, vv.w};

@@ -88,12 +88,21 @@ __global__ __launch_bounds__(256) void norm_wave_kernel(
   const int r = blockIdx.x * 4 + (threadIdx.x >> 6);
   if (r >= n_rows) return;
   const float* src = x + (int64_t)(rows ? rows[r] : r) * width;
-  float v[VPT];
-  float sum = 0.f;
+  // Loads are unconditional (index clamped, value selected afterwards): a load under a
+  // branch would wait for the one before it, and the row would cost VPT trips to memory.
+  float v[VPT], g[VPT], b[VPT];
 #pragma unroll
   for (int i = 0; i < VPT; ++i) {
     const int col = lane + i * 64;
-    v[i] = col < width ? src[col] : 0.f;
+    const int safe = col < width ? col : width - 1;
+    v[i] = src[safe];
+    g[i] = gamma[safe];
+    b[i] = (!RMS && beta != nullptr) ? beta[safe] : 0.f;
+  }
+  float sum = 0.f;
+#pragma unroll
+  for (int i = 0; i < VPT; ++i) {
+    if (lane + i * 64 >= width) v[i] = 0.f;
     sum += v[i];
   }
   float mean = 0.f;
@@ -111,11 +120,7 @@ __global__ __launch_bounds__(256) void norm_wave_kernel(
 #pragma unroll
   for (int i = 0; i < VPT; ++i) {
     const int col = lane + i * 64;
-    if (col < width) {
-      float y = v[i] * inv_std * gamma[col];
-      if (!RMS && beta != nullptr) y += beta[col];
-      dst[col] = from_float<T>(y);
-    }
+    if (col < width) dst[col] = from_float<T>(v[i] * inv_std * g[i] + b[i]);
   }
 }
 

@@ -20,10 +20,20 @@
 //   partial sums are added into the float output with hardware float atomics (only the
 //   residual epilogue allows it).
 //
+// gemm_nt_skinny_norm_kernel — the skinny kernel for up to 16 rows with the norm of its input
+//   fused in front: while the block's weight loads are in flight, each wave normalises four of
+//   the float input rows in registers (statistics by shuffles, as the norm kernel) and leaves
+//   them in LDS as bfloat16; the product then reads its column operand from LDS.  One launch
+//   and one trip to memory instead of two launches.
+//
+// Both kernels can also store the key and value columns of a [q | k | v] output into cache
+// pages from their epilogue (KvScatter).
+//
 // Accumulation is float in all cases.  Shapes that the kernels cannot take (k not a multiple
 // of 8 elements, unaligned rows) are refused by ps_gemm_nt_mfma_supported and run on the
 // plain kernel instead.
 #include "common.h"
+#include "linear.h"
 #include "pagedserve_hip.h"
 
 typedef __attribute__((__vector_size__(8 * sizeof(__bf16)))) __bf16 bf16x8;
@@ -61,7 +71,7 @@ struct Mma<float> {
 template <typename T, typename TOut, int EPI>
 __global__ __launch_bounds__(256) void gemm_nt_tiled_kernel(
     const T* __restrict__ a, const T* __restrict__ w, const float* __restrict__ bias,
-    TOut* __restrict__ c, int m, int n, int k, int lda, int ldc, int tiles_n) {
+    TOut* __restrict__ c, int m, int n, int k, int lda, int ldc, int tiles_n, KvScatter scatter) {
   constexpr int KC = Mma<T>::K_PER_CHUNK;            // elements per 16-byte chunk
   constexpr int BK = TG_ROW_BYTES / (int)sizeof(T);  // elements of k per stage
   __shared__ __attribute__((aligned(16))) unsigned char lds[2][(TG_BM + TG_BN) * TG_LDS_STRIDE];
@@ -85,12 +95,16 @@ __global__ __launch_bounds__(256) void gemm_nt_tiled_kernel(
       const int row = chunk >> 2;
       const int kk = k0 + (chunk & 3) * KC;
       const uint4 zero = {0u, 0u, 0u, 0u};
-      stage_a[i] = (m0 + row < m && kk < k)
-                       ? *reinterpret_cast<const uint4*>(a + (int64_t)(m0 + row) * lda + kk)
-                       : zero;
-      stage_w[i] = (n0 + row < n && kk < k)
-                       ? *reinterpret_cast<const uint4*>(w + (int64_t)(n0 + row) * k + kk)
-                       : zero;
+      // unconditional loads from clamped addresses, zeroed afterwards
+      const bool k_ok = kk < k;
+      const bool a_ok = m0 + row < m && k_ok;
+      const bool w_ok = n0 + row < n && k_ok;
+      stage_a[i] = *reinterpret_cast<const uint4*>(a + (int64_t)(a_ok ? m0 + row : 0) * lda +
+                                                   (a_ok ? kk : 0));
+      stage_w[i] = *reinterpret_cast<const uint4*>(w + (int64_t)(w_ok ? n0 + row : 0) * k +
+                                                   (w_ok ? kk : 0));
+      if (!a_ok) stage_a[i] = zero;
+      if (!w_ok) stage_w[i] = zero;
     }
   };
   auto store_lds = [&](int buffer) {
@@ -161,6 +175,7 @@ __global__ __launch_bounds__(256) void gemm_nt_tiled_kernel(
         TOut* dst = c + (int64_t)row * ldc + col;
         if (EPI == PS_EPI_RESIDUAL) v += to_float<TOut>(*dst);
         *dst = from_float<TOut>(v);
+        if (EPI == PS_EPI_NONE) kv_scatter_store<TOut>(scatter, row, col, v);
       }
     }
   }
@@ -170,10 +185,44 @@ __global__ __launch_bounds__(256) void gemm_nt_tiled_kernel(
 #define SK_WAVES 4
 #define SK_UNROLL 4   // 64-k steps whose loads are issued together
 
+// Sum the four waves' partial tiles and finish element (row sub, column n0 + group*4 + wave).
+template <typename TOut, int EPI, int MB>
+__device__ inline void skinny_epilogue(float (*partial)[MB][4][64], const float* bias, TOut* c,
+                                       int m, int n, int ldc, int n0, int split, int k_splits,
+                                       const KvScatter& scatter) {
+  const int lane = threadIdx.x & 63;
+  const int i = threadIdx.x >> 6;
+  const int sub = lane & 15;
+  const int group = lane >> 4;
+  const int col = n0 + group * 4 + i;
+  if (col >= n) return;
+#pragma unroll
+  for (int b = 0; b < MB; ++b) {
+    const int row = b * 16 + sub;
+    if (row >= m) continue;
+    float v = partial[0][b][i][lane] + partial[1][b][i][lane] + partial[2][b][i][lane] +
+              partial[3][b][i][lane];
+    if (bias != nullptr && split == 0) v += bias[col];
+    TOut* dst = c + (int64_t)row * ldc + col;
+    if (EPI == PS_EPI_RESIDUAL) {
+      if (k_splits > 1) {
+        unsafeAtomicAdd(reinterpret_cast<float*>(dst), v);
+      } else {
+        *dst = from_float<TOut>(v + to_float<TOut>(*dst));
+      }
+    } else {
+      v = apply_activation<EPI>(v);
+      *dst = from_float<TOut>(v);
+      if (EPI == PS_EPI_NONE) kv_scatter_store<TOut>(scatter, row, col, v);
+    }
+  }
+}
+
 template <typename TOut, int EPI, int MB>
 __global__ __launch_bounds__(64 * SK_WAVES) void gemm_nt_skinny_kernel(
     const bf16_t* __restrict__ a, const bf16_t* __restrict__ w, const float* __restrict__ bias,
-    TOut* __restrict__ c, int m, int n, int k, int lda, int ldc, int k_chunk, int k_splits) {
+    TOut* __restrict__ c, int m, int n, int k, int lda, int ldc, int k_chunk, int k_splits,
+    KvScatter scatter) {
   __shared__ float partial[SK_WAVES][MB][4][64];
   const int lane = threadIdx.x & 63;
   const int wave = threadIdx.x >> 6;
@@ -205,12 +254,26 @@ __global__ __launch_bounds__(64 * SK_WAVES) void gemm_nt_skinny_kernel(
       const int kk = ku + group * 16;
       const bool first = kk < k_end;
       const bool second = kk + 8 < k_end;
-      wf[u][0] = first ? *reinterpret_cast<const uint4*>(w_ptr + ku) : zero;
-      wf[u][1] = second ? *reinterpret_cast<const uint4*>(w_ptr + ku + 8) : zero;
+      // unconditional loads from a clamped offset, zeroed afterwards: loads under a branch
+      // would not be issued together
+      const int o0 = first ? ku : k_begin - group * 16;
+      const int o1 = second ? ku + 8 : k_begin - group * 16;
+      wf[u][0] = *reinterpret_cast<const uint4*>(w_ptr + o0);
+      wf[u][1] = *reinterpret_cast<const uint4*>(w_ptr + o1);
 #pragma unroll
       for (int b = 0; b < MB; ++b) {
-        xf[u][b][0] = first ? *reinterpret_cast<const uint4*>(a_ptr[b] + ku) : zero;
-        xf[u][b][1] = second ? *reinterpret_cast<const uint4*>(a_ptr[b] + ku + 8) : zero;
+        xf[u][b][0] = *reinterpret_cast<const uint4*>(a_ptr[b] + o0);
+        xf[u][b][1] = *reinterpret_cast<const uint4*>(a_ptr[b] + o1);
+      }
+      if (!first) {
+        wf[u][0] = zero;
+#pragma unroll
+        for (int b = 0; b < MB; ++b) xf[u][b][0] = zero;
+      }
+      if (!second) {
+        wf[u][1] = zero;
+#pragma unroll
+        for (int b = 0; b < MB; ++b) xf[u][b][1] = zero;
       }
     }
 #pragma unroll
@@ -229,30 +292,121 @@ __global__ __launch_bounds__(64 * SK_WAVES) void gemm_nt_skinny_kernel(
 #pragma unroll
     for (int i = 0; i < 4; ++i) partial[wave][b][i][lane] = acc[b][i];
   __syncthreads();
+  // element i of a 16 x 16 accumulator: weight row (lane / 16) * 4 + i, activation row lane % 16
+  skinny_epilogue<TOut, EPI, MB>(partial, bias, c, m, n, ldc, n0, split, k_splits, scatter);
+}
 
-  // element i of a 16 x 16 accumulator: weight row (lane / 16) * 4 + i, activation row lane % 16.
-  // Thread (wave, lane) finishes element i = wave of every block b.
-  const int i = wave;
-  const int col = n0 + group * 4 + i;
-  if (col >= n) return;
+// ---------------------------------------------------------------- skinny with fused norm
+#define SN_MAX_K 1024              // one round of loads covers it: 4 waves x 4 steps x 64
+#define SN_VPT (SN_MAX_K / 64)     // values of a row per lane
+#define SN_STRIDE (SN_MAX_K + 8)   // LDS row stride in elements (16-byte aligned, skewed)
+
+template <typename TOut, int EPI>
+__global__ __launch_bounds__(64 * SK_WAVES) void gemm_nt_skinny_norm_kernel(
+    NormPrologue norm, const bf16_t* __restrict__ w, const float* __restrict__ bias,
+    TOut* __restrict__ c, int m, int n, int k, int ldc, KvScatter scatter) {
+  __shared__ float partial[SK_WAVES][1][4][64];
+  __shared__ __attribute__((aligned(16))) bf16_t xs[16 * SN_STRIDE];
+  const int lane = threadIdx.x & 63;
+  const int wave = threadIdx.x >> 6;
+  const int n0 = blockIdx.x * 16;
+  const int sub = lane & 15;
+  const int group = lane >> 4;
+  const int w_row = n0 + sub < n ? n0 + sub : n - 1;
+  const bf16_t* w_ptr = w + (int64_t)w_row * k + group * 16;
+  const uint4 zero = {0u, 0u, 0u, 0u};
+
+  // 1. this wave's weights: all loads leave now and arrive while the rows are normalised
+  uint4 wf[SK_UNROLL][2];
+  bool first[SK_UNROLL], second[SK_UNROLL];
 #pragma unroll
-  for (int b = 0; b < MB; ++b) {
-    const int row = b * 16 + sub;
-    if (row >= m) continue;
-    float v = partial[0][b][i][lane] + partial[1][b][i][lane] + partial[2][b][i][lane] +
-              partial[3][b][i][lane];
-    if (bias != nullptr && split == 0) v += bias[col];
-    TOut* dst = c + (int64_t)row * ldc + col;
-    if (EPI == PS_EPI_RESIDUAL) {
-      if (k_splits > 1) {
-        unsafeAtomicAdd(reinterpret_cast<float*>(dst), v);
-      } else {
-        *dst = from_float<TOut>(v + to_float<TOut>(*dst));
+  for (int u = 0; u < SK_UNROLL; ++u) {
+    const int ku = wave * 64 + u * SK_WAVES * 64;
+    const int kk = ku + group * 16;
+    first[u] = kk < k;
+    second[u] = kk + 8 < k;
+    wf[u][0] = *reinterpret_cast<const uint4*>(w_ptr + (first[u] ? ku : -group * 16));
+    wf[u][1] = *reinterpret_cast<const uint4*>(w_ptr + (second[u] ? ku + 8 : -group * 16));
+  }
+
+  // 2. rows wave, wave + 4, wave + 8, wave + 12: statistics and normalisation in registers
+  //    (mean, centred values, biased variance, rsqrt(var + eps), scale, shift; reference:
+  //    src/kernels/triton_residual_layernorm.py:25-39), result to LDS as bfloat16
+  {
+    float g[SN_VPT], bt[SN_VPT];
+#pragma unroll
+    for (int i = 0; i < SN_VPT; ++i) {
+      const int col = lane + i * 64;
+      const int safe = col < k ? col : k - 1;
+      g[i] = norm.gamma[safe];
+      bt[i] = (!norm.rms && norm.beta != nullptr) ? norm.beta[safe] : 0.f;
+    }
+#pragma unroll
+    for (int pass = 0; pass < 2; ++pass) {   // two rows at a time keep the registers in hand
+      float v[2][SN_VPT];
+      int token[2];
+#pragma unroll
+      for (int j = 0; j < 2; ++j) {
+        token[j] = wave + (pass * 2 + j) * SK_WAVES;
+        const int t = token[j] < m ? token[j] : m - 1;
+        const float* src = norm.h + (int64_t)(norm.rows ? norm.rows[t] : t) * norm.ldh;
+#pragma unroll
+        for (int i = 0; i < SN_VPT; ++i) {
+          const int col = lane + i * 64;
+          v[j][i] = src[col < k ? col : k - 1];
+        }
       }
-    } else {
-      *dst = from_float<TOut>(apply_activation<EPI>(v));
+#pragma unroll
+      for (int j = 0; j < 2; ++j) {
+        float sum = 0.f;
+#pragma unroll
+        for (int i = 0; i < SN_VPT; ++i) {
+          if (lane + i * 64 >= k) v[j][i] = 0.f;
+          sum += v[j][i];
+        }
+        const float mean = norm.rms ? 0.f : wave_sum(sum) / (float)k;
+        float sq = 0.f;
+#pragma unroll
+        for (int i = 0; i < SN_VPT; ++i) {
+          const float centred = lane + i * 64 < k ? v[j][i] - mean : 0.f;
+          v[j][i] = centred;
+          sq += centred * centred;
+        }
+        const float inv_std = 1.0f / sqrtf(wave_sum(sq) / (float)k + norm.eps);
+        if (token[j] < 16) {
+#pragma unroll
+          for (int i = 0; i < SN_VPT; ++i) {
+            const int col = lane + i * 64;
+            if (col < k)
+              xs[token[j] * SN_STRIDE + col] =
+                  token[j] < m ? float_to_bf16(v[j][i] * inv_std * g[i] + bt[i]) : bf16_t{0};
+          }
+        }
+      }
     }
   }
+  __syncthreads();
+
+  // 3. the product: column operand from LDS
+  f32x4 acc = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+  for (int u = 0; u < SK_UNROLL; ++u) {
+    const int ku = wave * 64 + u * SK_WAVES * 64;
+    const int kk = ku + group * 16;
+    uint4 x0 = zero, x1 = zero;
+    if (first[u]) x0 = *reinterpret_cast<const uint4*>(&xs[sub * SN_STRIDE + kk]);
+    if (second[u]) x1 = *reinterpret_cast<const uint4*>(&xs[sub * SN_STRIDE + kk + 8]);
+    const uint4 w0 = first[u] ? wf[u][0] : zero;
+    const uint4 w1 = second[u] ? wf[u][1] : zero;
+    acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(*reinterpret_cast<const bf16x8*>(&w0),
+                                                  *reinterpret_cast<const bf16x8*>(&x0), acc, 0, 0, 0);
+    acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(*reinterpret_cast<const bf16x8*>(&w1),
+                                                  *reinterpret_cast<const bf16x8*>(&x1), acc, 0, 0, 0);
+  }
+#pragma unroll
+  for (int i = 0; i < 4; ++i) partial[wave][0][i][lane] = acc[i];
+  __syncthreads();
+  skinny_epilogue<TOut, EPI, 1>(partial, bias, c, m, n, ldc, n0, 0, 1, scatter);
 }
 
 // --------------------------------------------------------------------------------- host
@@ -263,37 +417,43 @@ bool ps_gemm_nt_mfma_supported(const void* a, const void* w, int k, int lda, int
   return k % per_chunk == 0 && lda % per_chunk == 0 && aligned16(a) && aligned16(w);
 }
 
+// Whether norm + product run as one launch.
+bool ps_norm_gemm_fusable(const void* w, int m, int k, int dtype) {
+  return dtype == PS_BF16 && m <= 16 && k <= SN_MAX_K && k % 8 == 0 && aligned16(w);
+}
+
 template <typename T, typename TOut>
 static int launch_tiled(const void* a, const void* w, const float* bias, void* c, int m, int n,
-                        int k, int lda, int ldc, int epilogue, hipStream_t s) {
+                        int k, int lda, int ldc, int epilogue, const KvScatter& scatter,
+                        hipStream_t s) {
   const int tiles_m = (m + TG_BM - 1) / TG_BM;
   const int tiles_n = (n + TG_BN - 1) / TG_BN;
   dim3 grid(tiles_m * tiles_n);
 #define PS_LAUNCH_TG(EPI)                                                                    \
   hipLaunchKernelGGL((gemm_nt_tiled_kernel<T, TOut, EPI>), grid, dim3(256), 0, s, (const T*)a, \
-                     (const T*)w, bias, (TOut*)c, m, n, k, lda, ldc, tiles_n)
+                     (const T*)w, bias, (TOut*)c, m, n, k, lda, ldc, tiles_n, scatter)
   switch (epilogue) {
     case PS_EPI_NONE: PS_LAUNCH_TG(PS_EPI_NONE); break;
     case PS_EPI_GELU_TANH: PS_LAUNCH_TG(PS_EPI_GELU_TANH); break;
     case PS_EPI_GELU_ERF: PS_LAUNCH_TG(PS_EPI_GELU_ERF); break;
     case PS_EPI_RESIDUAL: PS_LAUNCH_TG(PS_EPI_RESIDUAL); break;
-    default: ps_set_error("ps_gemm_nt: unknown epilogue %d", epilogue); return 1;
+    default: ps_set_error("ps_linear: unknown epilogue %d", epilogue); return 1;
   }
 #undef PS_LAUNCH_TG
-  PS_CHECK_LAUNCH("ps_gemm_nt(tiled)");
+  PS_CHECK_LAUNCH("ps_linear(tiled)");
   return 0;
 }
 
 template <typename TOut, int EPI>
 static void launch_skinny_mb(const void* a, const void* w, const float* bias, void* c, int m,
                              int n, int k, int lda, int ldc, int k_chunk, int k_splits,
-                             hipStream_t s) {
+                             const KvScatter& scatter, hipStream_t s) {
   dim3 grid((n + 15) / 16, k_splits);
   dim3 block(64 * SK_WAVES);
 #define PS_LAUNCH_SK(MB)                                                                       \
   hipLaunchKernelGGL((gemm_nt_skinny_kernel<TOut, EPI, MB>), grid, block, 0, s,                \
                      (const bf16_t*)a, (const bf16_t*)w, bias, (TOut*)c, m, n, k, lda, ldc,    \
-                     k_chunk, k_splits)
+                     k_chunk, k_splits, scatter)
   const int blocks = (m + 15) / 16;
   if (blocks <= 1) PS_LAUNCH_SK(1);
   else if (blocks == 2) PS_LAUNCH_SK(2);
@@ -304,7 +464,8 @@ static void launch_skinny_mb(const void* a, const void* w, const float* bias, vo
 
 template <typename TOut>
 static int launch_skinny(const void* a, const void* w, const float* bias, void* c, int m, int n,
-                         int k, int lda, int ldc, int epilogue, hipStream_t s) {
+                         int k, int lda, int ldc, int epilogue, const KvScatter& scatter,
+                         hipStream_t s) {
   // A block covers 1024 k with one round of loads.  Longer k is split over blocks where the
   // partial sums can be added in place (residual epilogue), else the block loops.
   int k_splits = 1;
@@ -312,37 +473,67 @@ static int launch_skinny(const void* a, const void* w, const float* bias, void* 
   int k_chunk = (k + k_splits - 1) / k_splits;
   k_chunk = (k_chunk + 255) / 256 * 256;
   k_splits = (k + k_chunk - 1) / k_chunk;
+#define PS_SKINNY_CASE(EPI)                                                                      \
+  case EPI:                                                                                      \
+    launch_skinny_mb<TOut, EPI>(a, w, bias, c, m, n, k, lda, ldc, k_chunk, k_splits, scatter, s); \
+    break
   switch (epilogue) {
-    case PS_EPI_NONE:
-      launch_skinny_mb<TOut, PS_EPI_NONE>(a, w, bias, c, m, n, k, lda, ldc, k_chunk, k_splits, s);
-      break;
-    case PS_EPI_GELU_TANH:
-      launch_skinny_mb<TOut, PS_EPI_GELU_TANH>(a, w, bias, c, m, n, k, lda, ldc, k_chunk, k_splits, s);
-      break;
-    case PS_EPI_GELU_ERF:
-      launch_skinny_mb<TOut, PS_EPI_GELU_ERF>(a, w, bias, c, m, n, k, lda, ldc, k_chunk, k_splits, s);
-      break;
-    case PS_EPI_RESIDUAL:
-      launch_skinny_mb<TOut, PS_EPI_RESIDUAL>(a, w, bias, c, m, n, k, lda, ldc, k_chunk, k_splits, s);
-      break;
-    default: ps_set_error("ps_gemm_nt: unknown epilogue %d", epilogue); return 1;
+    PS_SKINNY_CASE(PS_EPI_NONE);
+    PS_SKINNY_CASE(PS_EPI_GELU_TANH);
+    PS_SKINNY_CASE(PS_EPI_GELU_ERF);
+    PS_SKINNY_CASE(PS_EPI_RESIDUAL);
+    default: ps_set_error("ps_linear: unknown epilogue %d", epilogue); return 1;
   }
-  PS_CHECK_LAUNCH("ps_gemm_nt(skinny)");
+#undef PS_SKINNY_CASE
+  PS_CHECK_LAUNCH("ps_linear(skinny)");
   return 0;
 }
 
+template <typename TOut>
+static int launch_skinny_norm(const NormPrologue& norm, const void* w, const float* bias, void* c,
+                              int m, int n, int k, int ldc, int epilogue, const KvScatter& scatter,
+                              hipStream_t s) {
+  dim3 grid((n + 15) / 16);
+  dim3 block(64 * SK_WAVES);
+#define PS_NORM_CASE(EPI)                                                                     \
+  case EPI:                                                                                   \
+    hipLaunchKernelGGL((gemm_nt_skinny_norm_kernel<TOut, EPI>), grid, block, 0, s, norm,       \
+                       (const bf16_t*)w, bias, (TOut*)c, m, n, k, ldc, scatter);              \
+    break
+  switch (epilogue) {
+    PS_NORM_CASE(PS_EPI_NONE);
+    PS_NORM_CASE(PS_EPI_GELU_TANH);
+    PS_NORM_CASE(PS_EPI_GELU_ERF);
+    PS_NORM_CASE(PS_EPI_RESIDUAL);
+    default: ps_set_error("ps_linear: unknown epilogue %d", epilogue); return 1;
+  }
+#undef PS_NORM_CASE
+  PS_CHECK_LAUNCH("ps_linear(skinny, fused norm)");
+  return 0;
+}
+
+int ps_norm_gemm_fused(const NormPrologue& norm, const void* w, const float* bias, void* c, int m,
+                       int n, int k, int ldc, int c_dtype, int epilogue, const KvScatter& scatter,
+                       hipStream_t s) {
+  if (c_dtype == PS_F32)
+    return launch_skinny_norm<float>(norm, w, bias, c, m, n, k, ldc, epilogue, scatter, s);
+  return launch_skinny_norm<bf16_t>(norm, w, bias, c, m, n, k, ldc, epilogue, scatter, s);
+}
+
 int ps_gemm_nt_mfma(const void* a, const void* w, const float* bias, void* c, int m, int n, int k,
-                    int lda, int ldc, int dtype, int c_dtype, int epilogue, hipStream_t s) {
+                    int lda, int ldc, int dtype, int c_dtype, int epilogue,
+                    const KvScatter& scatter, hipStream_t s) {
   if (dtype == PS_BF16 && m <= 64) {
-    if (c_dtype == PS_F32) return launch_skinny<float>(a, w, bias, c, m, n, k, lda, ldc, epilogue, s);
-    return launch_skinny<bf16_t>(a, w, bias, c, m, n, k, lda, ldc, epilogue, s);
+    if (c_dtype == PS_F32)
+      return launch_skinny<float>(a, w, bias, c, m, n, k, lda, ldc, epilogue, scatter, s);
+    return launch_skinny<bf16_t>(a, w, bias, c, m, n, k, lda, ldc, epilogue, scatter, s);
   }
   if (dtype == PS_F32 && c_dtype == PS_F32)
-    return launch_tiled<float, float>(a, w, bias, c, m, n, k, lda, ldc, epilogue, s);
+    return launch_tiled<float, float>(a, w, bias, c, m, n, k, lda, ldc, epilogue, scatter, s);
   if (dtype == PS_BF16 && c_dtype == PS_F32)
-    return launch_tiled<bf16_t, float>(a, w, bias, c, m, n, k, lda, ldc, epilogue, s);
+    return launch_tiled<bf16_t, float>(a, w, bias, c, m, n, k, lda, ldc, epilogue, scatter, s);
   if (dtype == PS_BF16 && c_dtype == PS_BF16)
-    return launch_tiled<bf16_t, bf16_t>(a, w, bias, c, m, n, k, lda, ldc, epilogue, s);
-  ps_set_error("ps_gemm_nt: unsupported dtype pair (in %d, out %d)", dtype, c_dtype);
+    return launch_tiled<bf16_t, bf16_t>(a, w, bias, c, m, n, k, lda, ldc, epilogue, scatter, s);
+  ps_set_error("ps_linear: unsupported dtype pair (in %d, out %d)", dtype, c_dtype);
   return 1;
 }

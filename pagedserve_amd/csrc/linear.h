@@ -1,0 +1,47 @@
+// What the matrix-product kernels may fuse around the product: a norm in front of it and the
+// scatter of key/value columns into cache pages behind it.
+#pragma once
+
+#include "common.h"
+
+struct KvScatter {
+  void* k_pool;          // null: no scatter
+  void* v_pool;
+  const int* tok_item;
+  const int* tok_pos;
+  const int* tables;
+  int table_width, q_cols, kv_cols, head_dim, kv_heads, page_size, page_shift, num_pages;
+};
+
+struct NormPrologue {
+  const float* h;        // null: no norm
+  const int* rows;
+  const float* gamma;
+  const float* beta;
+  float eps;
+  int rms;
+  int ldh;
+};
+
+// Column `col` of output row `row` also goes into the cache when it is a key or value column:
+// token at position p of item r lands at (page = table[r][p / page], offset = p % page)
+// (reference: src/model/kv_manager.py:303-308,403-404).
+template <typename T>
+__device__ inline void kv_scatter_store(const KvScatter& s, int row, int col, float v) {
+  if (s.k_pool == nullptr || col < s.q_cols) return;
+  int within = col - s.q_cols;
+  T* pool = reinterpret_cast<T*>(s.k_pool);
+  if (within >= s.kv_cols) {
+    within -= s.kv_cols;
+    pool = reinterpret_cast<T*>(s.v_pool);
+  }
+  const int head = within / s.head_dim;
+  const int dim = within - head * s.head_dim;
+  const int pos = s.tok_pos[row];
+  const int logical = s.page_shift >= 0 ? (pos >> s.page_shift) : pos / s.page_size;
+  if (logical >= s.table_width) return;
+  const int page = s.tables[(int64_t)s.tok_item[row] * s.table_width + logical];
+  if (page < 0 || page >= s.num_pages) return;
+  pool[(((int64_t)page * s.kv_heads + head) * s.page_size + (pos - logical * s.page_size)) *
+           s.head_dim + dim] = from_float<T>(v);
+}

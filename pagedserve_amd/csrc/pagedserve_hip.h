@@ -34,6 +34,38 @@ int ps_norm(const float* x, const int* rows, const float* gamma, const float* be
 int ps_gemm_nt(const void* a, const void* w, const float* bias, void* c, int m, int n, int k,
                int lda, int ldc, int dtype, int c_dtype, int epilogue, void* stream);
 
+// A linear layer with what may be fused around it.
+//   * norm_h != null: the input rows are norm(norm_h[norm_rows ? norm_rows[r] : r]) * gamma
+//     (+ beta) instead of `a`; `norm_out` ([m, k] of `dtype`) is scratch for when the norm
+//     cannot be fused into the product (it is fused for bfloat16, m <= 16, k <= 1024);
+//   * k_pool != null: the output is [q | k | v] columns (q_cols, then kv_cols twice); besides
+//     being written to c, the k and v columns of row t are stored in the cache at the page
+//     slot of position tok_pos[t] of item tok_item[t] (what ps_kv_write does).
+typedef struct PsLinearArgs {
+  const void* a;
+  const void* w;
+  const float* bias;
+  void* c;
+  int m, n, k, lda, ldc;
+  int dtype, c_dtype, epilogue;
+  const float* norm_h;
+  const int* norm_rows;
+  const float* gamma;
+  const float* beta;
+  void* norm_out;
+  float eps;
+  int rms;
+  int ldh;
+  void* k_pool;
+  void* v_pool;
+  const int* tok_item;
+  const int* tok_pos;
+  const int* tables;
+  int table_width, q_cols, kv_cols, head_dim, kv_heads, page_size, num_pages;
+} PsLinearArgs;
+
+int ps_linear(const PsLinearArgs* args, void* stream);
+
 // Store keys and values of the step's tokens into their pages.
 //   k, v: [tokens, kv_heads * head_dim] with row stride `stride`;
 //   pools: [pages, kv_heads, page_size, head_dim].
@@ -53,14 +85,14 @@ int ps_attention_rowwise(const void* q, int64_t q_stride, const void* k_pool, co
                          float scale, int window, int dtype, void* stream);
 
 // The same result for single queries, with each token's keys cut into `splits` ranges that
-// run as separate blocks; `partial` is scratch of count * heads * splits * (head_dim + 2)
-// floats (unused when splits == 1).
+// run as separate blocks of `waves` (4 or 16) waves; `partial` is scratch of
+// count * heads * splits * (head_dim + 2) floats (unused when splits == 1).
 int ps_attention_decode(const void* q, int64_t q_stride, const void* k_pool, const void* v_pool,
                         void* out, int64_t out_stride, float* partial, int64_t partial_floats,
                         const int* tok_list, const int* tok_item, const int* tok_pos,
                         const int* tables, int table_width, int count, int heads, int kv_heads,
                         int head_dim, int page_size, int num_pages, float scale, int window,
-                        int splits, int dtype, void* stream);
+                        int splits, int waves, int dtype, void* stream);
 
 // Tiled attention on the matrix cores for items that bring several tokens (bfloat16, head_dim a
 // multiple of 16 up to 128).  Tile i covers queries tile_q0[i] .. tile_q0[i] + 63 of item

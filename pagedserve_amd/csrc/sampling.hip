@@ -35,11 +35,20 @@ __global__ __launch_bounds__(SM_THREADS) void sample_kernel(
   // maximum and its first index
   float best = -INFINITY;
   int best_idx = vocab;
-  for (int i = tid; i < vocab; i += SM_THREADS) {
-    const float v = row[i];
-    if (v > best) {
-      best = v;
-      best_idx = i;
+  for (int i0 = tid; i0 < vocab; i0 += 4 * SM_THREADS) {
+    float v[4];
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {   // four loads in flight, index clamped, masked below
+      const int i = i0 + u * SM_THREADS;
+      v[u] = row[i < vocab ? i : vocab - 1];
+    }
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+      const int i = i0 + u * SM_THREADS;
+      if (i < vocab && v[u] > best) {
+        best = v[u];
+        best_idx = i;
+      }
     }
   }
 #pragma unroll

@@ -131,9 +131,11 @@ class DecoderModel:
         if wanted == 0:
             return logits_out[:0]
         final = ctx.workspace.rows("final", self.spec.width, self.dtype)[:wanted]
-        self.final_norm.forward(h, final, rows=logit_rows)
+        pending = self.final_norm.pending(h, final, rows=logit_rows)
+        if pending is None:
+            pending = self.final_norm.forward(h, final, rows=logit_rows)
         # logits = f @ table^T without bias, always float
         # (src/model/paged_decoder.py:295-301,605)
         out = logits_out[:wanted]
-        kernels.gemm_nt(final, self.head_weight, None, out)
+        kernels.linear(pending, self.head_weight, None, out)
         return out

@@ -33,7 +33,8 @@ _SIGNATURES = {
                              c_int, c_float, c_int, c_int, c_void_p],
     "ps_attention_decode": [c_void_p, c_int64, c_void_p, c_void_p, c_void_p, c_int64, c_void_p,
                             c_int64, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int,
-                            c_int, c_int, c_int, c_int, c_float, c_int, c_int, c_int, c_void_p],
+                            c_int, c_int, c_int, c_int, c_float, c_int, c_int, c_int, c_int,
+                            c_void_p],
     "ps_attention_prefill": [c_void_p, c_int64, c_void_p, c_void_p, c_void_p, c_int64, c_void_p,
                              c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int,
                              c_int, c_int, c_int, c_float, c_int, c_int, c_void_p],
@@ -178,6 +179,126 @@ def gemm_nt(a, w, bias, out, epilogue="none"):
     return out
 
 
+class _LinearArgs(ctypes.Structure):
+    _fields_ = [
+        ("a", c_void_p), ("w", c_void_p), ("bias", c_void_p), ("c", c_void_p),
+        ("m", c_int), ("n", c_int), ("k", c_int), ("lda", c_int), ("ldc", c_int),
+        ("dtype", c_int), ("c_dtype", c_int), ("epilogue", c_int),
+        ("norm_h", c_void_p), ("norm_rows", c_void_p), ("gamma", c_void_p), ("beta", c_void_p),
+        ("norm_out", c_void_p), ("eps", c_float), ("rms", c_int), ("ldh", c_int),
+        ("k_pool", c_void_p), ("v_pool", c_void_p), ("tok_item", c_void_p), ("tok_pos", c_void_p),
+        ("tables", c_void_p),
+        ("table_width", c_int), ("q_cols", c_int), ("kv_cols", c_int), ("head_dim", c_int),
+        ("kv_heads", c_int), ("page_size", c_int), ("num_pages", c_int),
+    ]
+
+
+class PendingNorm:
+    """A norm that has not run yet: the float rows, the parameters, and scratch for the
+    normed rows.  ``linear`` fuses it into the product when the kernel can; ``materialize``
+    runs it on its own."""
+
+    def __init__(self, h, gamma, beta, eps, rms, scratch, rows=None):
+        self.h = h
+        self.gamma = gamma
+        self.beta = beta
+        self.eps = float(eps)
+        self.rms = bool(rms)
+        self.scratch = scratch
+        self.rows = rows
+
+    @property
+    def count(self):
+        return self.rows.numel() if self.rows is not None else self.h.shape[0]
+
+    def materialize(self):
+        count = self.count
+        return norm(self.h, self.gamma, self.beta, self.eps, self.scratch[:count], rows=self.rows,
+                    rms=self.rms)[:count]
+
+
+def linear(x, w, bias, out, epilogue="none", scatter=None):
+    """out = epilogue(x w^T + bias) where ``x`` is a tensor or a ``PendingNorm``.
+
+    ``scatter = (k_pool, v_pool, tok_item, tok_pos, tables, q_cols, kv_cols)`` also stores the
+    key and value columns of a ``[q | k | v]`` output into their cache pages."""
+    _check(w, "w", ndim=2)
+    _check(out, "out", ndim=2)
+    n, k = w.shape
+    if not w.is_contiguous():
+        raise KernelError("linear: w must be contiguous")
+    args = _LinearArgs()
+    if isinstance(x, PendingNorm):
+        _check(x.h, "norm input", torch.float32, 2)
+        _check(x.gamma, "gamma", torch.float32, 1)
+        if x.h.shape[1] != k or x.gamma.numel() != k or not x.h.is_contiguous():
+            raise KernelError("linear: norm input rows must be contiguous and k wide")
+        if x.beta is not None:
+            _check(x.beta, "beta", torch.float32, 1)
+        m = x.count
+        _check(x.scratch, "norm scratch", w.dtype, 2)
+        if x.scratch.shape[0] < m or x.scratch.shape[1] != k or not x.scratch.is_contiguous():
+            raise KernelError("linear: norm scratch must be contiguous [>= m, k]")
+        if x.rows is not None:
+            _check(x.rows, "rows", torch.int32, 1)
+        args.norm_h = x.h.data_ptr()
+        args.norm_rows = _ptr(x.rows)
+        args.gamma = x.gamma.data_ptr()
+        args.beta = _ptr(x.beta)
+        args.norm_out = x.scratch.data_ptr()
+        args.eps = x.eps
+        args.rms = 1 if x.rms else 0
+        args.ldh = k
+        args.lda = k
+    else:
+        _check(x, "x", w.dtype, 2)
+        if x.shape[1] != k:
+            raise KernelError(f"linear: x {tuple(x.shape)} does not match w {tuple(w.shape)}")
+        m = x.shape[0]
+        args.a = x.data_ptr()
+        args.lda = _rows(x, "x")
+    if out.shape[0] != m or out.shape[1] != n:
+        raise KernelError(f"linear: out {tuple(out.shape)} must be [{m}, {n}]")
+    if bias is not None:
+        _check(bias, "bias", torch.float32, 1)
+        if bias.numel() != n or not bias.is_contiguous():
+            raise KernelError("linear: bias does not match n")
+    if epilogue not in EPILOGUES:
+        raise KernelError(f"linear: unknown epilogue {epilogue!r}")
+    args.w = w.data_ptr()
+    args.bias = _ptr(bias)
+    args.c = out.data_ptr()
+    args.m, args.n, args.k = m, n, k
+    args.ldc = _rows(out, "out")
+    args.dtype = dtype_code(w.dtype)
+    args.c_dtype = dtype_code(out.dtype)
+    args.epilogue = EPILOGUES[epilogue]
+    if scatter is not None:
+        k_pool, v_pool, tok_item, tok_pos, tables, q_cols, kv_cols = scatter
+        pages, kv_heads, page_size, head_dim = _check_pools(k_pool, v_pool, w.dtype)
+        _check_step_index(tok_item, tok_pos, tables, m)
+        args.k_pool = k_pool.data_ptr()
+        args.v_pool = v_pool.data_ptr()
+        args.tok_item = tok_item.data_ptr()
+        args.tok_pos = tok_pos.data_ptr()
+        args.tables = tables.data_ptr()
+        args.table_width = tables.shape[1]
+        args.q_cols, args.kv_cols = int(q_cols), int(kv_cols)
+        args.head_dim, args.kv_heads = head_dim, kv_heads
+        args.page_size, args.num_pages = page_size, pages
+    lib = load_library()
+    fn = _BOUND.get("ps_linear")
+    if fn is None:
+        fn = lib.ps_linear
+        fn.argtypes = [ctypes.POINTER(_LinearArgs), c_void_p]
+        fn.restype = c_int
+        _BOUND["ps_linear"] = fn
+    status = fn(ctypes.byref(args), _stream())
+    if status != 0:
+        raise KernelError(f"ps_linear failed ({status}): {lib.ps_last_error().decode('utf-8', 'replace')}")
+    return out
+
+
 def _check_pools(k_pool, v_pool, dtype):
     _check(k_pool, "k_pool", dtype, 4)
     _check(v_pool, "v_pool", dtype, 4)
@@ -245,15 +366,15 @@ def attention_rowwise(q, k_pool, v_pool, out, tok_item, tok_pos, tables, heads, 
     return out
 
 
-def decode_keys_per_block(head_dim: int) -> int:
+def decode_keys_per_block(head_dim: int, waves: int = 4) -> int:
     """Keys that one block of the split-KV kernel visits per iteration."""
     lanes = head_dim // 8
     lanes_per_key = 2 if lanes <= 2 else 4 if lanes <= 4 else 8 if lanes <= 8 else 16 if lanes <= 16 else 32
-    return (64 // lanes_per_key) * 4 * 4
+    return (64 // lanes_per_key) * 4 * waves
 
 
 def attention_decode(q, k_pool, v_pool, out, tok_item, tok_pos, tables, heads, scale, splits,
-                     partial=None, window=0, tok_list=None):
+                     partial=None, window=0, tok_list=None, waves=4):
     """The same result as ``attention_rowwise`` by the split-KV kernel; ``partial`` is float
     scratch of ``count * heads * splits * (head_dim + 2)`` values when ``splits > 1``."""
     pages, kv_heads, page_size, head_dim, q_stride, out_stride, count = _attention_args(
@@ -268,7 +389,7 @@ def attention_decode(q, k_pool, v_pool, out, tok_item, tok_pos, tables, heads, s
           out.data_ptr(), out_stride, _ptr(partial if splits > 1 else None), floats,
           _ptr(tok_list), tok_item.data_ptr(), tok_pos.data_ptr(), tables.data_ptr(),
           tables.shape[1], count, heads, kv_heads, head_dim, page_size, pages, float(scale),
-          int(window), int(splits), dtype_code(q.dtype), _stream())
+          int(window), int(splits), int(waves), dtype_code(q.dtype), _stream())
     return out
 
 

@@ -21,6 +21,8 @@ class Attention(Mixer):
     ``scale`` multiplies the scores (``head_dim**-0.5`` in src/model/paged_attention.py:27).
     """
 
+    accepts_pending_norm = True
+
     def __init__(self, width: int, dtype, heads: int, kv_heads: int, head_dim: int, scale: float,
                  window: int = 0, bias: bool = True):
         if heads % kv_heads != 0:
@@ -63,21 +65,29 @@ class Attention(Mixer):
         tokens = ctx.tokens
         total = self.q_cols + 2 * self.kv_cols
         qkv = ctx.workspace.rows("qkv", total, self.dtype)[:tokens]
-        kernels.gemm_nt(x, self.qkv_weight, self.qkv_bias, qkv)
+        tables = ctx.tables[cache.group]
         q = qkv[:, :self.q_cols]
         k = qkv[:, self.q_cols:self.q_cols + self.kv_cols]
         v = qkv[:, self.q_cols + self.kv_cols:]
-        if self.position is not None:
-            self.position.apply_to_qk(q, k, ctx)
-        tables = ctx.tables[cache.group]
-        if cache.writes:
-            kernels.kv_write(k, v, cache.k_pool, cache.v_pool, ctx.tok_item, ctx.positions, tables)
+        rotates = self.position is not None and self.position.transforms_qk
+        if cache.writes and not rotates:
+            # keys and values go to their pages from the product's own epilogue
+            kernels.linear(x, self.qkv_weight, self.qkv_bias, qkv,
+                           scatter=(cache.k_pool, cache.v_pool, ctx.tok_item, ctx.positions, tables,
+                                    self.q_cols, self.kv_cols))
+        else:
+            kernels.linear(x, self.qkv_weight, self.qkv_bias, qkv)
+            if rotates:
+                self.position.apply_to_qk(q, k, ctx)
+            if cache.writes:
+                kernels.kv_write(k, v, cache.k_pool, cache.v_pool, ctx.tok_item, ctx.positions,
+                                 tables)
         context = ctx.workspace.rows("attn", self.q_cols, self.dtype)[:tokens]
         singles = ctx.single_tokens.numel() if ctx.single_tokens is not None else 0
         if singles:
             # one-token items: keys of a request are cut into ranges so that few requests
             # still fill the chip
-            splits = self._splits(singles, ctx.max_kv_len)
+            splits, waves = self._splits(singles, ctx.max_kv_len)
             partial = None
             if splits > 1:
                 # _splits keeps singles * heads * splits below 1024 + singles * heads
@@ -85,7 +95,7 @@ class Attention(Mixer):
                 partial = ctx.workspace.flat("attn_partial", worst, torch.float32)
             kernels.attention_decode(q, cache.k_pool, cache.v_pool, context, ctx.tok_item,
                                      ctx.positions, tables, self.heads, self.scale, splits,
-                                     partial=partial, window=self.window,
+                                     partial=partial, window=self.window, waves=waves,
                                      tok_list=None if singles == tokens else ctx.single_tokens)
         if singles < tokens and kernels.prefill_supported(self.dtype, self.head_dim):
             kernels.attention_prefill(q, cache.k_pool, cache.v_pool, context, ctx.tile_item,
@@ -95,12 +105,17 @@ class Attention(Mixer):
             kernels.attention_rowwise(q, cache.k_pool, cache.v_pool, context, ctx.tok_item,
                                       ctx.positions, tables, self.heads, self.scale, self.window,
                                       tok_list=None if singles == 0 else ctx.portion_tokens)
-        kernels.gemm_nt(context, self.out_weight, self.out_bias, residual, epilogue="residual")
+        kernels.linear(context, self.out_weight, self.out_bias, residual, epilogue="residual")
 
-    def _splits(self, count: int, max_kv_len: int) -> int:
-        """Ranges per request: enough blocks for about four per compute unit, never more
-        than the keys of the longest request can feed."""
+    def _splits(self, count: int, max_kv_len: int):
+        """(ranges per request, waves per block).  With enough (token, head) pairs and long
+        contexts one block of 16 waves takes a whole request's keys and no second launch is
+        needed to merge ranges; few pairs are cut into ranges so that the chip is filled,
+        never into more than the keys of the longest request can feed."""
         visible = max_kv_len if self.window <= 0 else min(max_kv_len, self.window)
-        most = max(1, -(-visible // kernels.decode_keys_per_block(self.head_dim)))
-        wanted = max(1, -(-1024 // (count * self.heads)))
-        return min(most, wanted, 64)
+        pairs = count * self.heads
+        if pairs >= 64 and visible > kernels.decode_keys_per_block(self.head_dim, 4):
+            return 1, 16
+        most = max(1, -(-visible // kernels.decode_keys_per_block(self.head_dim, 4)))
+        wanted = max(1, -(-1024 // pairs))
+        return min(most, wanted, 64), 4

@@ -6,6 +6,10 @@ tensors.  It never sees the model's configuration.
 
 * ``Norm.forward(h, out, rows=None)``: ``h`` is the float residual stream ``[T, d]``;
   writes the normed rows in the engine dtype.
+* ``Norm.pending(h, scratch, rows=None)``: the same norm as an object that has not run
+  yet (``ops.kernels.PendingNorm``); a part that sets ``accepts_pending_norm = True`` gets
+  this instead of normed rows and may hand it to ``kernels.linear``, which runs norm and
+  product as one launch where it can.  Other parts get the tensor.
 * ``Mixer.forward(x, residual, ctx, cache)``: ``x`` is ``[T, d]`` in the engine dtype;
   the mixer ADDS its output to the float ``residual`` in place.  ``cache`` is the
   ``CacheView`` of this call of the layer: pools of a paged key/value entry, or the
@@ -69,8 +73,14 @@ class Norm(Part):
     def forward(self, h, out, rows=None):
         raise NotImplementedError
 
+    def pending(self, h, scratch, rows=None):
+        """This norm of ``h`` as a ``PendingNorm``, or ``None`` if it can only run on its own."""
+        return None
+
 
 class PositionEncoding(Part):
+    transforms_qk = False   # True when apply_to_qk changes queries or keys
+
     def embedding_table(self):
         return None
 
@@ -79,6 +89,8 @@ class PositionEncoding(Part):
 
 
 class Mixer(Part):
+    accepts_pending_norm = False
+
     def cache_spec(self):
         """``PagedKVSpec``, ``SlotStateSpec`` or ``None``."""
         return None
@@ -91,6 +103,8 @@ class Mixer(Part):
 
 
 class FeedForward(Part):
+    accepts_pending_norm = False
+
     def forward(self, x, residual, ctx):
         raise NotImplementedError
 

@@ -20,10 +20,16 @@ class PreNormBlock:
         return {"norm1": self.norm1, "mixer": self.mixer, "norm2": self.norm2,
                 "feed_forward": self.feed_forward}
 
+    def _normed(self, norm, part, h, ctx):
+        """Input of ``part``: the norm as a pending object if the part takes one, else rows."""
+        scratch = ctx.workspace.rows("normed", self.width, self.dtype)[:ctx.tokens]
+        if getattr(part, "accepts_pending_norm", False):
+            pending = norm.pending(h, scratch)
+            if pending is not None:
+                return pending
+        return norm.forward(h, scratch)
+
     def forward(self, h, ctx, cache):
-        normed = ctx.workspace.rows("normed", self.width, self.dtype)[:ctx.tokens]
-        self.norm1.forward(h, normed)
-        self.mixer.forward(normed, h, ctx, cache)
-        self.norm2.forward(h, normed)
-        self.feed_forward.forward(normed, h, ctx)
+        self.mixer.forward(self._normed(self.norm1, self.mixer, h, ctx), h, ctx, cache)
+        self.feed_forward.forward(self._normed(self.norm2, self.feed_forward, h, ctx), h, ctx)
         return h

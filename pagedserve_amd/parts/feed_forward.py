@@ -13,6 +13,8 @@ class DenseFeedForward(FeedForward):
     """``residual += act(x W_up + b_up) W_down + b_down``
     (src/model/paged_decoder.py:178-179,224-228; activations ``:273-280``)."""
 
+    accepts_pending_norm = True
+
     def __init__(self, width: int, dtype, inner: int, activation: str, bias: bool = True):
         if activation not in ACTIVATIONS:
             raise ValueError(f"unknown activation {activation!r}; known: {', '.join(ACTIVATIONS)}")
@@ -40,5 +42,5 @@ class DenseFeedForward(FeedForward):
 
     def forward(self, x, residual, ctx):
         hidden = ctx.workspace.rows("ffn", self.inner, self.dtype)[:ctx.tokens]
-        kernels.gemm_nt(x, self.up_weight, self.up_bias, hidden, epilogue=self.activation)
-        kernels.gemm_nt(hidden, self.down_weight, self.down_bias, residual, epilogue="residual")
+        kernels.linear(x, self.up_weight, self.up_bias, hidden, epilogue=self.activation)
+        kernels.linear(hidden, self.down_weight, self.down_bias, residual, epilogue="residual")

@@ -22,6 +22,9 @@ class LayerNorm(Norm):
     def forward(self, h, out, rows=None):
         return kernels.norm(h, self.gamma, self.beta, self.eps, out, rows=rows, rms=False)
 
+    def pending(self, h, scratch, rows=None):
+        return kernels.PendingNorm(h, self.gamma, self.beta, self.eps, False, scratch, rows)
+
 
 @register_norm("rmsnorm")
 class RMSNorm(Norm):
@@ -37,3 +40,6 @@ class RMSNorm(Norm):
 
     def forward(self, h, out, rows=None):
         return kernels.norm(h, self.gamma, None, self.eps, out, rows=rows, rms=True)
+
+    def pending(self, h, scratch, rows=None):
+        return kernels.PendingNorm(h, self.gamma, None, self.eps, True, scratch, rows)

@@ -477,3 +477,95 @@ def test_attention_prefill_far_key_and_causality():
     for row in (137, 138, 299):
         torch.testing.assert_close(out[row].float(), value, atol=2e-2, rtol=2e-2)
     assert float((out[136].float() - value).abs().max()) > 0.3
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("m,n,k", [(1, 48, 64), (8, 2304, 768), (16, 100, 1024), (13, 257, 96), (17, 192, 768), (5, 64, 1600), (200, 320, 96)])
+@pytest.mark.parametrize("epilogue", ["none", "gelu_tanh", "residual"])
+@pytest.mark.parametrize("rms", [False, True])
+def test_linear_with_pending_norm(dtype, m, n, k, epilogue, rms):
+    """Norm + product as one call: fused for bfloat16 with up to 16 rows and k <= 1024, two
+    launches otherwise; with and without a row gather."""
+    from pagedserve_amd.ops import kernels
+
+    h = _rand((m + 3, k), torch.float32, 70, 2.0) + 0.5
+    gamma = 1.0 + _rand((k,), torch.float32, 71, 0.2)
+    beta = None if rms else _rand((k,), torch.float32, 72, 0.2)
+    w = _rand((n, k), dtype, 73, 1.0 / math.sqrt(k))
+    bias = _rand((n,), torch.float32, 74)
+    for rows in (None, torch.randperm(m + 3)[:m].int().cuda()):
+        source = h[:m] if rows is None else h
+        count = m
+        scratch = torch.empty((count, k), dtype=dtype, device="cuda")
+        pending = kernels.PendingNorm(source, gamma, beta, 1e-6, rms, scratch, rows)
+        picked = (source if rows is None else source[rows.long()]).double()
+        if rms:
+            normed = picked / torch.sqrt((picked * picked).mean(-1, keepdim=True) + 1e-6) * gamma.double()
+        else:
+            normed = F.layer_norm(picked, (k,), gamma.double(), beta.double(), 1e-6)
+        if dtype == torch.bfloat16:
+            normed = normed.to(torch.bfloat16).double()
+        product = normed @ w.double().t() + bias.double()
+        if epilogue == "residual":
+            out = _rand((count, n), torch.float32, 75)
+            expected = out.double() + product
+        else:
+            out = torch.full((count, n), float("nan"), dtype=dtype, device="cuda")
+            expected = F.gelu(product, approximate="tanh") if epilogue == "gelu_tanh" else product
+        kernels.linear(pending, w, bias, out, epilogue=epilogue)
+        atol, rtol = (4e-5, 2e-5) if dtype == torch.float32 else (4e-2, 2e-2)
+        torch.testing.assert_close(out.double(), expected, atol=atol, rtol=rtol)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("m", [1, 9, 40, 150])
+@pytest.mark.parametrize("k", [64, 100])
+def test_linear_scatters_keys_and_values(dtype, m, k):
+    """A [q | k | v] product that also stores k and v in their pages equals product + kv_write
+    (k = 100 takes the plain kernel, which scatters in a second launch)."""
+    from pagedserve_amd.ops import kernels
+
+    heads, kv_heads, head_dim, page_size = 4, 2, 16, 8
+    q_cols, kv_cols = heads * head_dim, kv_heads * head_dim
+    n = q_cols + 2 * kv_cols
+    lens = [m // 2 + 3, m - m // 2 + 11] if m > 1 else [5]
+    k_pool, v_pool, tables = _paged_fixture(dtype, lens, kv_heads, head_dim, page_size, 81)
+    tok_item, tok_pos = [], []
+    counts = [m // 2, m - m // 2] if m > 1 else [1]
+    for item, (count, length) in enumerate(zip(counts, lens)):
+        tok_item += [item] * count
+        tok_pos += list(range(length - count, length))
+    tok_item = torch.tensor(tok_item, dtype=torch.int32, device="cuda")
+    tok_pos = torch.tensor(tok_pos, dtype=torch.int32, device="cuda")
+    x = _rand((m, k), dtype, 82)
+    w = _rand((n, k), dtype, 83, 1.0 / math.sqrt(k))
+    bias = _rand((n,), torch.float32, 84)
+    plain = torch.empty((m, n), dtype=dtype, device="cuda")
+    kernels.linear(x, w, bias, plain)
+    k_ref, v_ref = k_pool.clone(), v_pool.clone()
+    kernels.kv_write(plain[:, q_cols:q_cols + kv_cols], plain[:, q_cols + kv_cols:], k_ref, v_ref, tok_item, tok_pos, tables)
+    out = torch.empty_like(plain)
+    kernels.linear(x, w, bias, out, scatter=(k_pool, v_pool, tok_item, tok_pos, tables, q_cols, kv_cols))
+    torch.testing.assert_close(out, plain, atol=0, rtol=0)
+    assert torch.equal(k_pool.view(torch.int16 if dtype == torch.bfloat16 else torch.int32),
+                       k_ref.view(torch.int16 if dtype == torch.bfloat16 else torch.int32))
+    assert torch.equal(v_pool.view(torch.int16 if dtype == torch.bfloat16 else torch.int32),
+                       v_ref.view(torch.int16 if dtype == torch.bfloat16 else torch.int32))
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_attention_decode_sixteen_waves(dtype):
+    from pagedserve_amd.ops import kernels
+
+    heads, head_dim, page_size = 12, 64, 16
+    contexts = [1, 17, 300, 513, 1024, 700, 64, 999]
+    k_pool, v_pool, tables = _paged_fixture(dtype, contexts, heads, head_dim, page_size, 91)
+    q = _rand((len(contexts), heads * head_dim), dtype, 92)
+    tok_item = torch.arange(len(contexts), dtype=torch.int32, device="cuda")
+    tok_pos = torch.tensor([c - 1 for c in contexts], dtype=torch.int32, device="cuda")
+    expected = torch.empty_like(q)
+    kernels.attention_rowwise(q, k_pool, v_pool, expected, tok_item, tok_pos, tables, heads, 0.125)
+    out = torch.full_like(q, float("nan"))
+    kernels.attention_decode(q, k_pool, v_pool, out, tok_item, tok_pos, tables, heads, 0.125, 1, waves=16)
+    atol, rtol = (3e-5, 3e-5) if dtype == torch.float32 else (2e-2, 2e-2)
+    torch.testing.assert_close(out.double(), expected.double(), atol=atol, rtol=rtol)
