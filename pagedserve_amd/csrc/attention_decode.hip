@@ -17,29 +17,38 @@
 #include "common.h"
 #include "pagedserve_hip.h"
 
-#define AD_UNROLL 4
 
+// Eight consecutive elements as they lie in memory; widened to float when they are used, so
+// that many of them can be in flight without filling the register file.
 template <typename T>
-__device__ inline void load8(const T* p, float* out);
+struct Raw8;
 
 template <>
-__device__ inline void load8<float>(const float* p, float* out) {
-  const float4 a = *reinterpret_cast<const float4*>(p);
-  const float4 b = *reinterpret_cast<const float4*>(p + 4);
-  out[0] = a.x; out[1] = a.y; out[2] = a.z; out[3] = a.w;
-  out[4] = b.x; out[5] = b.y; out[6] = b.z; out[7] = b.w;
-}
-
-template <>
-__device__ inline void load8<bf16_t>(const bf16_t* p, float* out) {
-  const uint4 raw = *reinterpret_cast<const uint4*>(p);
-  const uint32_t w[4] = {raw.x, raw.y, raw.z, raw.w};
-#pragma unroll
-  for (int i = 0; i < 4; ++i) {
-    out[2 * i] = __uint_as_float(w[i] << 16);
-    out[2 * i + 1] = __uint_as_float(w[i] & 0xffff0000u);
+struct Raw8<float> {
+  float4 a, b;
+  __device__ inline void load(const float* p) {
+    a = *reinterpret_cast<const float4*>(p);
+    b = *reinterpret_cast<const float4*>(p + 4);
   }
-}
+  __device__ inline void widen(float* out) const {
+    out[0] = a.x; out[1] = a.y; out[2] = a.z; out[3] = a.w;
+    out[4] = b.x; out[5] = b.y; out[6] = b.z; out[7] = b.w;
+  }
+};
+
+template <>
+struct Raw8<bf16_t> {
+  uint4 raw;
+  __device__ inline void load(const bf16_t* p) { raw = *reinterpret_cast<const uint4*>(p); }
+  __device__ inline void widen(float* out) const {
+    const uint32_t w[4] = {raw.x, raw.y, raw.z, raw.w};
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      out[2 * i] = __uint_as_float(w[i] << 16);
+      out[2 * i + 1] = __uint_as_float(w[i] & 0xffff0000u);
+    }
+  }
+};
 
 // Merge the online-softmax state (m, l, acc) with another one.
 __device__ inline void merge_state(float& m, float& l, float* acc, float m_o, float l_o,
@@ -52,7 +61,7 @@ __device__ inline void merge_state(float& m, float& l, float* acc, float m_o, fl
   m = m_n;
 }
 
-template <typename T, int LPK, int AD_WAVES>
+template <typename T, int LPK, int AD_WAVES, int AD_UNROLL>
 __global__ __launch_bounds__(64 * AD_WAVES) void attention_decode_kernel(
     const T* __restrict__ q, int64_t q_stride, const T* __restrict__ k_pool,
     const T* __restrict__ v_pool, T* __restrict__ out, int64_t out_stride,
@@ -96,7 +105,7 @@ __global__ __launch_bounds__(64 * AD_WAVES) void attention_decode_kernel(
 
   for (int base = range_begin + wave * KEYS_PER_WAVE; base < range_end;
        base += AD_WAVES * KEYS_PER_WAVE) {
-    float kf[AD_UNROLL][8], vf[AD_UNROLL][8];
+    Raw8<T> kr[AD_UNROLL], vr[AD_UNROLL];
     bool valid[AD_UNROLL];
     // Every load is unconditional from a clamped address and masked afterwards, so that the
     // table entries, then all keys and values of the iteration, travel together.
@@ -117,26 +126,19 @@ __global__ __launch_bounds__(64 * AD_WAVES) void attention_decode_kernel(
       const int64_t offset =
           (((int64_t)safe_page * kv_heads + kv_head) * page_size + within[u]) * head_dim +
           (has_dims ? dim0 : 0);
-      load8<T>(k_pool + offset, kf[u]);
-      load8<T>(v_pool + offset, vf[u]);
-    }
-#pragma unroll
-    for (int u = 0; u < AD_UNROLL; ++u) {
-      if (!valid[u] || !has_dims) {
-#pragma unroll
-        for (int i = 0; i < 8; ++i) {
-          kf[u][i] = 0.f;
-          vf[u][i] = 0.f;
-        }
-      }
+      kr[u].load(k_pool + offset);
+      vr[u].load(v_pool + offset);
     }
     float s[AD_UNROLL];
     float m_new = m;
 #pragma unroll
     for (int u = 0; u < AD_UNROLL; ++u) {
+      float kf[8];
+      kr[u].widen(kf);
       float dot = 0.f;
 #pragma unroll
-      for (int i = 0; i < 8; ++i) dot = fmaf(qf[i], kf[u][i], dot);
+      for (int i = 0; i < 8; ++i) dot = fmaf(qf[i], kf[i], dot);
+      if (!has_dims) dot = 0.f;
 #pragma unroll
       for (int offset = LPK / 2; offset > 0; offset >>= 1) dot += __shfl_xor(dot, offset, 64);
       s[u] = valid[u] ? dot * scale : -INFINITY;
@@ -151,11 +153,18 @@ __global__ __launch_bounds__(64 * AD_WAVES) void attention_decode_kernel(
       for (int u = 0; u < AD_UNROLL; ++u) {
         const float p = valid[u] ? expf(s[u] - m_new) : 0.f;
         l += p;
+        float vf[8];
+        vr[u].widen(vf);
+        // a masked key was loaded from a clamped address and may hold anything, also NaN
 #pragma unroll
-        for (int i = 0; i < 8; ++i) acc[i] = fmaf(p, vf[u][i], acc[i]);
+        for (int i = 0; i < 8; ++i) acc[i] = valid[u] ? fmaf(p, vf[i], acc[i]) : acc[i];
       }
       m = m_new;
     }
+  }
+  if (!has_dims) {
+#pragma unroll
+    for (int i = 0; i < 8; ++i) acc[i] = 0.f;
   }
 
   // merge the lane groups of this wave
@@ -242,7 +251,8 @@ static int launch_decode(const void* q, int64_t q_stride, const void* k_pool, co
   }
   dim3 grid(count, heads, splits);
 #define PS_LAUNCH_ADW(LPK, WAVES)                                                                \
-  hipLaunchKernelGGL((attention_decode_kernel<T, LPK, WAVES>), grid, dim3(64 * WAVES), 0, s,     \
+  hipLaunchKernelGGL((attention_decode_kernel<T, LPK, WAVES, (WAVES == 16 ? 8 : 4)>), grid,      \
+                     dim3(64 * WAVES), 0, s,                                                     \
                      (const T*)q, q_stride, (const T*)k_pool, (const T*)v_pool, (T*)out,         \
                      out_stride, partial, tok_list, tok_item, tok_pos, tables, table_width,      \
                      heads, kv_heads, head_dim, page_size, page_shift, num_pages, scale, window, \

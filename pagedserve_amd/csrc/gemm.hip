@@ -14,7 +14,7 @@ int ps_norm_gemm_fused(const NormPrologue& norm, const void* w, const float* bia
                        int n, int k, int ldc, int c_dtype, int epilogue, const KvScatter& scatter,
                        hipStream_t s);
 bool ps_gemm_nt_mfma_supported(const void* a, const void* w, int k, int lda, int dtype);
-bool ps_norm_gemm_fusable(const void* w, int m, int k, int dtype);
+bool ps_norm_gemm_fusable(const void* w, const NormPrologue& norm, int m, int n, int k, int dtype);
 
 extern "C" int ps_linear(const PsLinearArgs* p, void* stream) {
   PS_REQUIRE(p != nullptr, "ps_linear: no arguments");
@@ -71,8 +71,8 @@ extern "C" int ps_linear(const PsLinearArgs* p, void* stream) {
   const void* a = p->a;
   int lda = p->lda;
   if (has_norm) {
-    if (ps_norm_gemm_fusable(p->w, m, k, p->dtype)) {
-      NormPrologue norm = {p->norm_h, p->norm_rows, p->gamma, p->beta, p->eps, p->rms, p->ldh};
+    NormPrologue norm = {p->norm_h, p->norm_rows, p->gamma, p->beta, p->eps, p->rms, p->ldh};
+    if (ps_norm_gemm_fusable(p->w, norm, m, n, k, p->dtype)) {
       return ps_norm_gemm_fused(norm, p->w, p->bias, p->c, m, n, k, p->ldc, p->c_dtype,
                                 p->epilogue, scatter, s);
     }

@@ -298,7 +298,6 @@ __global__ __launch_bounds__(64 * SK_WAVES) void gemm_nt_skinny_kernel(
 
 // ---------------------------------------------------------------- skinny with fused norm
 #define SN_MAX_K 1024              // one round of loads covers it: 4 waves x 4 steps x 64
-#define SN_VPT (SN_MAX_K / 64)     // values of a row per lane
 #define SN_STRIDE (SN_MAX_K + 8)   // LDS row stride in elements (16-byte aligned, skewed)
 
 template <typename TOut, int EPI>
@@ -331,57 +330,79 @@ __global__ __launch_bounds__(64 * SK_WAVES) void gemm_nt_skinny_norm_kernel(
 
   // 2. rows wave, wave + 4, wave + 8, wave + 12: statistics and normalisation in registers
   //    (mean, centred values, biased variance, rsqrt(var + eps), scale, shift; reference:
-  //    src/kernels/triton_residual_layernorm.py:25-39), result to LDS as bfloat16
+  //    src/kernels/triton_residual_layernorm.py:25-39), result to LDS as bfloat16.  A lane
+  //    owns columns 4 * lane + 256 * i (one 16-byte load each); all loads of the four rows and
+  //    of the scale and shift leave together.
   {
-    float g[SN_VPT], bt[SN_VPT];
+    constexpr int V4 = SN_MAX_K / 256;
+    const float4 zero4 = {0.f, 0.f, 0.f, 0.f};
+    float4 g[V4], bt[V4], v[4][V4];
+    bool in_row[V4];
+    const float* src[4];
 #pragma unroll
-    for (int i = 0; i < SN_VPT; ++i) {
-      const int col = lane + i * 64;
-      const int safe = col < k ? col : k - 1;
-      g[i] = norm.gamma[safe];
-      bt[i] = (!norm.rms && norm.beta != nullptr) ? norm.beta[safe] : 0.f;
+    for (int j = 0; j < 4; ++j) {
+      const int token = wave + j * SK_WAVES;
+      const int t = token < m ? token : m - 1;
+      src[j] = norm.h + (int64_t)(norm.rows ? norm.rows[t] : t) * norm.ldh;
     }
 #pragma unroll
-    for (int pass = 0; pass < 2; ++pass) {   // two rows at a time keep the registers in hand
-      float v[2][SN_VPT];
-      int token[2];
+    for (int i = 0; i < V4; ++i) {
+      const int col = 4 * lane + 256 * i;
+      in_row[i] = col < k;
+      const int safe = in_row[i] ? col : 0;
+      g[i] = *reinterpret_cast<const float4*>(norm.gamma + safe);
+      bt[i] = (!norm.rms && norm.beta != nullptr)
+                  ? *reinterpret_cast<const float4*>(norm.beta + safe)
+                  : zero4;
 #pragma unroll
-      for (int j = 0; j < 2; ++j) {
-        token[j] = wave + (pass * 2 + j) * SK_WAVES;
-        const int t = token[j] < m ? token[j] : m - 1;
-        const float* src = norm.h + (int64_t)(norm.rows ? norm.rows[t] : t) * norm.ldh;
+      for (int j = 0; j < 4; ++j) v[j][i] = *reinterpret_cast<const float4*>(src[j] + safe);
+    }
+    float sum[4], sq[4], mean[4], inv_std[4];
 #pragma unroll
-        for (int i = 0; i < SN_VPT; ++i) {
-          const int col = lane + i * 64;
-          v[j][i] = src[col < k ? col : k - 1];
-        }
+    for (int j = 0; j < 4; ++j) {
+      sum[j] = 0.f;
+#pragma unroll
+      for (int i = 0; i < V4; ++i) {
+        if (!in_row[i]) v[j][i] = zero4;
+        sum[j] += (v[j][i].x + v[j][i].y) + (v[j][i].z + v[j][i].w);
       }
+    }
 #pragma unroll
-      for (int j = 0; j < 2; ++j) {
-        float sum = 0.f;
+    for (int j = 0; j < 4; ++j) mean[j] = norm.rms ? 0.f : wave_sum(sum[j]) / (float)k;
 #pragma unroll
-        for (int i = 0; i < SN_VPT; ++i) {
-          if (lane + i * 64 >= k) v[j][i] = 0.f;
-          sum += v[j][i];
+    for (int j = 0; j < 4; ++j) {
+      sq[j] = 0.f;
+#pragma unroll
+      for (int i = 0; i < V4; ++i) {
+        if (in_row[i]) {
+          v[j][i].x -= mean[j];
+          v[j][i].y -= mean[j];
+          v[j][i].z -= mean[j];
+          v[j][i].w -= mean[j];
         }
-        const float mean = norm.rms ? 0.f : wave_sum(sum) / (float)k;
-        float sq = 0.f;
+        sq[j] += (v[j][i].x * v[j][i].x + v[j][i].y * v[j][i].y) +
+                 (v[j][i].z * v[j][i].z + v[j][i].w * v[j][i].w);
+      }
+    }
 #pragma unroll
-        for (int i = 0; i < SN_VPT; ++i) {
-          const float centred = lane + i * 64 < k ? v[j][i] - mean : 0.f;
-          v[j][i] = centred;
-          sq += centred * centred;
-        }
-        const float inv_std = 1.0f / sqrtf(wave_sum(sq) / (float)k + norm.eps);
-        if (token[j] < 16) {
+    for (int j = 0; j < 4; ++j) inv_std[j] = 1.0f / sqrtf(wave_sum(sq[j]) / (float)k + norm.eps);
 #pragma unroll
-          for (int i = 0; i < SN_VPT; ++i) {
-            const int col = lane + i * 64;
-            if (col < k)
-              xs[token[j] * SN_STRIDE + col] =
-                  token[j] < m ? float_to_bf16(v[j][i] * inv_std * g[i] + bt[i]) : bf16_t{0};
-          }
+    for (int j = 0; j < 4; ++j) {
+      const int token = wave + j * SK_WAVES;
+      const bool live = token < m;
+#pragma unroll
+      for (int i = 0; i < V4; ++i) {
+        if (!in_row[i]) continue;
+        uint2 packed = {0u, 0u};
+        if (live) {
+          const float y0 = v[j][i].x * inv_std[j] * g[i].x + bt[i].x;
+          const float y1 = v[j][i].y * inv_std[j] * g[i].y + bt[i].y;
+          const float y2 = v[j][i].z * inv_std[j] * g[i].z + bt[i].z;
+          const float y3 = v[j][i].w * inv_std[j] * g[i].w + bt[i].w;
+          packed.x = (uint32_t)float_to_bf16(y0).bits | ((uint32_t)float_to_bf16(y1).bits << 16);
+          packed.y = (uint32_t)float_to_bf16(y2).bits | ((uint32_t)float_to_bf16(y3).bits << 16);
         }
+        *reinterpret_cast<uint2*>(&xs[token * SN_STRIDE + 4 * lane + 256 * i]) = packed;
       }
     }
   }
@@ -418,8 +439,11 @@ bool ps_gemm_nt_mfma_supported(const void* a, const void* w, int k, int lda, int
 }
 
 // Whether norm + product run as one launch.
-bool ps_norm_gemm_fusable(const void* w, int m, int k, int dtype) {
-  return dtype == PS_BF16 && m <= 16 && k <= SN_MAX_K && k % 8 == 0 && aligned16(w);
+// Every block normalises the rows again, so the fusion only pays while there are few blocks.
+bool ps_norm_gemm_fusable(const void* w, const NormPrologue& norm, int m, int n, int k, int dtype) {
+  return dtype == PS_BF16 && m <= 16 && n <= 8192 && k <= SN_MAX_K && k % 8 == 0 &&
+         norm.ldh % 4 == 0 && aligned16(w) && aligned16(norm.h) && aligned16(norm.gamma) &&
+         (norm.beta == nullptr || aligned16(norm.beta));
 }
 
 template <typename T, typename TOut>

@@ -370,7 +370,7 @@ def decode_keys_per_block(head_dim: int, waves: int = 4) -> int:
     """Keys that one block of the split-KV kernel visits per iteration."""
     lanes = head_dim // 8
     lanes_per_key = 2 if lanes <= 2 else 4 if lanes <= 4 else 8 if lanes <= 8 else 16 if lanes <= 16 else 32
-    return (64 // lanes_per_key) * 4 * waves
+    return (64 // lanes_per_key) * (8 if waves == 16 else 4) * waves
 
 
 def attention_decode(q, k_pool, v_pool, out, tok_item, tok_pos, tables, heads, scale, splits,

@@ -163,20 +163,29 @@ def test_gemm_identity_and_one_hot():
 
 
 def _paged_fixture(dtype, batch_lens, kv_heads, head_dim, page_size, seed, extra_pages=5):
-    """Fragmented pools and tables for requests of the given cached lengths."""
+    """Fragmented pools and tables for requests of the given cached lengths.  Whatever no
+    request owns holds NaN: page 0 and the other spare pages, and the slots behind each
+    request's last key, so a kernel that lets a masked or clamped load reach its result fails."""
     g = torch.Generator().manual_seed(seed)
     pages_per = [-(-length // page_size) for length in batch_lens]
     width = max(pages_per) + 2
     total = sum(pages_per) + extra_pages
-    order = torch.randperm(total, generator=g).tolist()
+    order = (torch.randperm(total - 1, generator=g) + 1).tolist()     # page 0 stays unowned
     tables = torch.full((len(batch_lens), width), -1, dtype=torch.int32)
+    owned = torch.zeros(total, page_size, dtype=torch.bool)
     cursor = 0
-    for index, count in enumerate(pages_per):
-        tables[index, :count] = torch.tensor(order[cursor:cursor + count], dtype=torch.int32)
+    for index, (count, length) in enumerate(zip(pages_per, batch_lens)):
+        pages = order[cursor:cursor + count]
+        tables[index, :count] = torch.tensor(pages, dtype=torch.int32)
+        for logical, page in enumerate(pages):
+            owned[page, :max(0, min(page_size, length - logical * page_size))] = True
         cursor += count
-    k_pool = (torch.randn((total, kv_heads, page_size, head_dim), generator=g)).to(dtype).cuda()
-    v_pool = (torch.randn((total, kv_heads, page_size, head_dim), generator=g)).to(dtype).cuda()
-    return k_pool, v_pool, tables.cuda()
+    k_pool = torch.randn((total, kv_heads, page_size, head_dim), generator=g)
+    v_pool = torch.randn((total, kv_heads, page_size, head_dim), generator=g)
+    hole = ~owned[:, None, :, None].expand_as(k_pool)
+    k_pool[hole] = float("nan")
+    v_pool[hole] = float("nan")
+    return k_pool.to(dtype).cuda(), v_pool.to(dtype).cuda(), tables.cuda()
 
 
 def _gather(pool, table, length, page_size):
