@@ -31,9 +31,7 @@ typedef __attribute__((__vector_size__(4 * sizeof(float)))) float f32x4;
 #define AP_QUERIES 64   // queries per block
 #define AP_V_STRIDE (AP_KEYS * 2 + 16)
 
-__device__ inline uint32_t pack_bf16(float lo, float hi) {
-  return (uint32_t)float_to_bf16(lo).bits | ((uint32_t)float_to_bf16(hi).bits << 16);
-}
+__device__ inline uint32_t pack_bf16(float lo, float hi) { return pack2_bf16(lo, hi); }
 
 template <int NDB>  // head_dim / 16
 __global__ __launch_bounds__(256) void attention_prefill_kernel(

@@ -31,8 +31,14 @@ __host__ __device__ inline float bf16_to_float(bf16_t v) {
   return c.f;
 }
 
-// Round to nearest, ties to even; NaN stays NaN.
+// Round to nearest, ties to even; NaN stays NaN.  On the device this is the hardware
+// conversion of gfx950 (v_cvt_pk_bf16_f32).
 __host__ __device__ inline bf16_t float_to_bf16(float f) {
+#if defined(__HIP_DEVICE_COMPILE__)
+  bf16_t native;
+  native.bits = __builtin_bit_cast(uint16_t, (__bf16)f);
+  return native;
+#endif
   union {
     uint32_t u;
     float f;
@@ -46,6 +52,14 @@ __host__ __device__ inline bf16_t float_to_bf16(float f) {
   uint32_t rounding = 0x7fffu + ((c.u >> 16) & 1u);
   out.bits = (uint16_t)((c.u + rounding) >> 16);
   return out;
+}
+
+// Two floats to two bfloat16 in one 32-bit word (lo in the low half).
+__device__ inline uint32_t pack2_bf16(float lo, float hi) {
+  typedef __attribute__((__vector_size__(2 * sizeof(float)))) float f32x2_t;
+  typedef __attribute__((__vector_size__(2 * sizeof(__bf16)))) __bf16 bf16x2_t;
+  const f32x2_t pair = {lo, hi};
+  return __builtin_bit_cast(uint32_t, __builtin_convertvector(pair, bf16x2_t));
 }
 
 template <typename T>

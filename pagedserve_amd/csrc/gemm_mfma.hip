@@ -357,10 +357,15 @@ __global__ __launch_bounds__(64 * SK_WAVES) void gemm_nt_skinny_norm_kernel(
 #pragma unroll
       for (int j = 0; j < 4; ++j) v[j][i] = *reinterpret_cast<const float4*>(src[j] + safe);
     }
+    // rows beyond m (the same for the whole wave) are not worked on
+    bool live_row[4];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) live_row[j] = wave + j * SK_WAVES < m;
     float sum[4], sq[4], mean[4], inv_std[4];
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
       sum[j] = 0.f;
+      if (!live_row[j]) continue;
 #pragma unroll
       for (int i = 0; i < V4; ++i) {
         if (!in_row[i]) v[j][i] = zero4;
@@ -368,10 +373,12 @@ __global__ __launch_bounds__(64 * SK_WAVES) void gemm_nt_skinny_norm_kernel(
       }
     }
 #pragma unroll
-    for (int j = 0; j < 4; ++j) mean[j] = norm.rms ? 0.f : wave_sum(sum[j]) / (float)k;
+    for (int j = 0; j < 4; ++j)
+      mean[j] = (norm.rms || !live_row[j]) ? 0.f : wave_sum(sum[j]) / (float)k;
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
       sq[j] = 0.f;
+      if (!live_row[j]) continue;
 #pragma unroll
       for (int i = 0; i < V4; ++i) {
         if (in_row[i]) {
@@ -385,7 +392,8 @@ __global__ __launch_bounds__(64 * SK_WAVES) void gemm_nt_skinny_norm_kernel(
       }
     }
 #pragma unroll
-    for (int j = 0; j < 4; ++j) inv_std[j] = 1.0f / sqrtf(wave_sum(sq[j]) / (float)k + norm.eps);
+    for (int j = 0; j < 4; ++j)
+      inv_std[j] = live_row[j] ? 1.0f / sqrtf(wave_sum(sq[j]) / (float)k + norm.eps) : 0.f;
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
       const int token = wave + j * SK_WAVES;
@@ -399,8 +407,8 @@ __global__ __launch_bounds__(64 * SK_WAVES) void gemm_nt_skinny_norm_kernel(
           const float y1 = v[j][i].y * inv_std[j] * g[i].y + bt[i].y;
           const float y2 = v[j][i].z * inv_std[j] * g[i].z + bt[i].z;
           const float y3 = v[j][i].w * inv_std[j] * g[i].w + bt[i].w;
-          packed.x = (uint32_t)float_to_bf16(y0).bits | ((uint32_t)float_to_bf16(y1).bits << 16);
-          packed.y = (uint32_t)float_to_bf16(y2).bits | ((uint32_t)float_to_bf16(y3).bits << 16);
+          packed.x = pack2_bf16(y0, y1);
+          packed.y = pack2_bf16(y2, y3);
         }
         *reinterpret_cast<uint2*>(&xs[token * SN_STRIDE + 4 * lane + 256 * i]) = packed;
       }
