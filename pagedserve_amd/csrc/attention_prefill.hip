@@ -100,35 +100,58 @@ __global__ __launch_bounds__(256) void attention_prefill_kernel(
 #pragma unroll
   for (int db = 0; db < NDB; ++db) acc[db] = f32x4{0.f, 0.f, 0.f, 0.f};
 
-  for (int k0 = key_begin / AP_KEYS * AP_KEYS; k0 < key_end; k0 += AP_KEYS) {
-    __syncthreads();   // the previous tile has been consumed
-    for (int c = tid; c < AP_KEYS * NDB * 2; c += 256) {
+  // Each thread moves CHUNKS 16-byte pieces of a K tile and of a V tile; the next tile's
+  // pieces are loaded into registers while the current tile is being multiplied.
+  constexpr int CHUNKS = (AP_KEYS * NDB * 2 + 255) / 256;
+  uint4 k_next[CHUNKS], v_next[CHUNKS];
+  auto fetch_tile = [&](int k0) {
+#pragma unroll
+    for (int i = 0; i < CHUNKS; ++i) {
+      const int c = tid + i * 256;
       const int key_local = c / (NDB * 2);
       const int dc = c - key_local * (NDB * 2);
       const int key = k0 + key_local;
       // unconditional loads from clamped addresses, zeroed afterwards
-      const int safe_key = key < key_end ? key : key_end - 1;
+      const int safe_key = (key < key_end && key_local < AP_KEYS) ? key : key_end - 1;
       const int logical = page_shift >= 0 ? (safe_key >> page_shift) : safe_key / page_size;
       const int page = table[logical < table_width ? logical : table_width - 1];
-      const bool ok = key < key_end && logical < table_width && page >= 0 && page < num_pages;
+      const bool ok = key < key_end && key_local < AP_KEYS && logical < table_width && page >= 0 &&
+                      page < num_pages;
       const int64_t offset =
           (((int64_t)(ok ? page : 0) * kv_heads + kv_head) * page_size +
            (safe_key - logical * page_size)) * HD + dc * 8;
-      uint4 kv = *reinterpret_cast<const uint4*>(k_pool + offset);
-      uint4 vv = *reinterpret_cast<const uint4*>(v_pool + offset);
+      k_next[i] = *reinterpret_cast<const uint4*>(k_pool + offset);
+      v_next[i] = *reinterpret_cast<const uint4*>(v_pool + offset);
       if (!ok) {
-        kv = uint4{0u, 0u, 0u, 0u};
-        vv = uint4{0u, 0u, 0u, 0u};
+        k_next[i] = uint4{0u, 0u, 0u, 0u};
+        v_next[i] = uint4{0u, 0u, 0u, 0u};
       }
-      *reinterpret_cast<uint4*>(&k_lds[key_local * K_STRIDE + dc * 16]) = kv;
-      const uint32_t words[4] = {vv.x, vv.y, vv.z, vv.w};
+    }
+  };
+  auto store_tile = [&]() {
+#pragma unroll
+    for (int i = 0; i < CHUNKS; ++i) {
+      const int c = tid + i * 256;
+      const int key_local = c / (NDB * 2);
+      const int dc = c - key_local * (NDB * 2);
+      if (key_local >= AP_KEYS) continue;
+      *reinterpret_cast<uint4*>(&k_lds[key_local * K_STRIDE + dc * 16]) = k_next[i];
+      const uint32_t words[4] = {v_next[i].x, v_next[i].y, v_next[i].z, v_next[i].w};
 #pragma unroll
       for (int j = 0; j < 8; ++j) {
         const uint16_t value = (uint16_t)(words[j >> 1] >> ((j & 1) * 16));
         *reinterpret_cast<uint16_t*>(&v_lds[(dc * 8 + j) * AP_V_STRIDE + key_local * 2]) = value;
       }
     }
+  };
+
+  const int k_first = key_begin / AP_KEYS * AP_KEYS;
+  fetch_tile(k_first);
+  for (int k0 = k_first; k0 < key_end; k0 += AP_KEYS) {
+    __syncthreads();   // the previous tile has been consumed
+    store_tile();
     __syncthreads();
+    if (k0 + AP_KEYS < key_end) fetch_tile(k0 + AP_KEYS);   // in flight during the products
     // skip tiles that no query of this wave can see
     if (!wave_active || k0 > wave_last) continue;
     if (window > 0 && k0 + AP_KEYS - 1 < wave_first - window + 1) continue;

@@ -68,10 +68,13 @@ struct Mma<float> {
   }
 };
 
+#define TG_DEPTH 4   // k tiles whose global loads are in flight
+
 template <typename T, typename TOut, int EPI>
 __global__ __launch_bounds__(256) void gemm_nt_tiled_kernel(
     const T* __restrict__ a, const T* __restrict__ w, const float* __restrict__ bias,
-    TOut* __restrict__ c, int m, int n, int k, int lda, int ldc, int tiles_n, KvScatter scatter) {
+    TOut* __restrict__ c, int m, int n, int k, int lda, int ldc, int tiles_m, int tiles_n,
+    int k_splits, int k_chunk, KvScatter scatter) {
   constexpr int KC = Mma<T>::K_PER_CHUNK;            // elements per 16-byte chunk
   constexpr int BK = TG_ROW_BYTES / (int)sizeof(T);  // elements of k per stage
   __shared__ __attribute__((aligned(16))) unsigned char lds[2][(TG_BM + TG_BN) * TG_LDS_STRIDE];
@@ -81,38 +84,57 @@ __global__ __launch_bounds__(256) void gemm_nt_tiled_kernel(
   const int wave = tid >> 6;
   const int wave_m = wave >> 1;
   const int wave_n = wave & 1;
-  const int tile_m = blockIdx.x / tiles_n;
-  const int tile_n = blockIdx.x - tile_m * tiles_n;
+  // Consecutive block ids run on different XCDs, each with an L2 of its own.  Blocks are
+  // renumbered so that every XCD works on a contiguous run of tiles (which share rows of A
+  // and, in the next run, rows of W) instead of every XCD fetching every operand tile.
+  const int blocks = gridDim.x;
+  const int per_xcd = blocks / 8;
+  int logical = blockIdx.x;
+  if (blockIdx.x < per_xcd * 8) logical = (blockIdx.x & 7) * per_xcd + (blockIdx.x >> 3);
+  const int tiles = tiles_m * tiles_n;
+  const int split = logical / tiles;
+  const int tile = logical - split * tiles;
+  // walk the tiles column-major in groups of 8 rows, so that a run of blocks reuses W tiles
+  const int tile_n = tile / tiles_m;
+  const int tile_m = tile - tile_n * tiles_m;
   const int m0 = tile_m * TG_BM;
   const int n0 = tile_n * TG_BN;
+  const int k_begin = split * k_chunk;
+  const int k_end = k_begin + k_chunk < k ? k_begin + k_chunk : k;
 
-  // global -> register staging: 512 chunks of 16 bytes per operand, two per thread
-  uint4 stage_a[2], stage_w[2];
-  auto load_global = [&](int k0) {
+  // global -> register staging: 512 chunks of 16 bytes per operand, two per thread; a ring
+  // of TG_DEPTH stages keeps that many k tiles in flight
+  uint4 ring_a[TG_DEPTH][2], ring_w[TG_DEPTH][2];
+  const int load_row = tid >> 2;           // rows load_row and load_row + 64
+  const int load_k = (tid & 3) * KC;
+  const T* a_src[2];
+  const T* w_src[2];
+  bool a_row_ok[2], w_row_ok[2];
+#pragma unroll
+  for (int i = 0; i < 2; ++i) {
+    const int row = load_row + i * 64;
+    a_row_ok[i] = m0 + row < m;
+    w_row_ok[i] = n0 + row < n;
+    a_src[i] = a + (int64_t)(a_row_ok[i] ? m0 + row : 0) * lda + load_k;
+    w_src[i] = w + (int64_t)(w_row_ok[i] ? n0 + row : 0) * k + load_k;
+  }
+  auto load_global = [&](uint4* stage_a, uint4* stage_w, int k0) {
+    // unconditional loads from clamped addresses, zeroed afterwards
+    const bool k_ok = k0 + load_k < k_end;
+    const int kk = k_ok ? k0 : k_begin;
+    const uint4 zero = {0u, 0u, 0u, 0u};
 #pragma unroll
     for (int i = 0; i < 2; ++i) {
-      const int chunk = tid + i * 256;
-      const int row = chunk >> 2;
-      const int kk = k0 + (chunk & 3) * KC;
-      const uint4 zero = {0u, 0u, 0u, 0u};
-      // unconditional loads from clamped addresses, zeroed afterwards
-      const bool k_ok = kk < k;
-      const bool a_ok = m0 + row < m && k_ok;
-      const bool w_ok = n0 + row < n && k_ok;
-      stage_a[i] = *reinterpret_cast<const uint4*>(a + (int64_t)(a_ok ? m0 + row : 0) * lda +
-                                                   (a_ok ? kk : 0));
-      stage_w[i] = *reinterpret_cast<const uint4*>(w + (int64_t)(w_ok ? n0 + row : 0) * k +
-                                                   (w_ok ? kk : 0));
-      if (!a_ok) stage_a[i] = zero;
-      if (!w_ok) stage_w[i] = zero;
+      stage_a[i] = *reinterpret_cast<const uint4*>(a_src[i] + kk);
+      stage_w[i] = *reinterpret_cast<const uint4*>(w_src[i] + kk);
+      if (!(a_row_ok[i] && k_ok)) stage_a[i] = zero;
+      if (!(w_row_ok[i] && k_ok)) stage_w[i] = zero;
     }
   };
-  auto store_lds = [&](int buffer) {
+  auto store_lds = [&](int buffer, const uint4* stage_a, const uint4* stage_w) {
 #pragma unroll
     for (int i = 0; i < 2; ++i) {
-      const int chunk = tid + i * 256;
-      const int row = chunk >> 2;
-      const int offset = row * TG_LDS_STRIDE + (chunk & 3) * 16;
+      const int offset = (load_row + i * 64) * TG_LDS_STRIDE + (tid & 3) * 16;
       *reinterpret_cast<uint4*>(&lds[buffer][offset]) = stage_a[i];
       *reinterpret_cast<uint4*>(&lds[buffer][TG_BM * TG_LDS_STRIDE + offset]) = stage_w[i];
     }
@@ -126,13 +148,7 @@ __global__ __launch_bounds__(256) void gemm_nt_tiled_kernel(
 #pragma unroll
       for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.f;
 
-  const int k_tiles = (k + BK - 1) / BK;
-  load_global(0);
-  store_lds(0);
-  __syncthreads();
-  for (int kt = 0; kt < k_tiles; ++kt) {
-    const int buffer = kt & 1;
-    if (kt + 1 < k_tiles) load_global((kt + 1) * BK);
+  auto compute = [&](int buffer) {
     // 64 bytes of k per row = two 32-byte halves; lanes 0..31 take the first 16 bytes of a
     // half, lanes 32..63 the second
 #pragma unroll
@@ -155,16 +171,35 @@ __global__ __launch_bounds__(256) void gemm_nt_tiled_kernel(
 #pragma unroll
         for (int j = 0; j < 2; ++j) Mma<T>::step(fa[i], fw[j], acc[i][j]);
     }
-    if (kt + 1 < k_tiles) store_lds(buffer ^ 1);
-    __syncthreads();
+  };
+
+  const int k_tiles = (k_end - k_begin + BK - 1) / BK;
+#pragma unroll
+  for (int d = 0; d < TG_DEPTH; ++d) load_global(ring_a[d], ring_w[d], k_begin + d * BK);
+  store_lds(0, ring_a[0], ring_w[0]);
+  __syncthreads();
+  for (int kt0 = 0; kt0 < k_tiles; kt0 += TG_DEPTH) {
+#pragma unroll
+    for (int d = 0; d < TG_DEPTH; ++d) {
+      const int kt = kt0 + d;
+      if (kt < k_tiles) {
+        // stage d held tile kt, which is in LDS already: refill it with tile kt + TG_DEPTH
+        load_global(ring_a[d], ring_w[d], k_begin + (kt + TG_DEPTH) * BK);
+        compute(kt & 1);
+        // tile kt + 1 left TG_DEPTH - 1 iterations ago
+        store_lds((kt + 1) & 1, ring_a[(d + 1) % TG_DEPTH], ring_w[(d + 1) % TG_DEPTH]);
+        __syncthreads();
+      }
+    }
   }
 
   // element e of a 32 x 32 accumulator: row (e / 4) * 8 + (lane / 32) * 4 + e % 4, column lane % 32
+  const bool scatters = EPI == PS_EPI_NONE && scatter.k_pool != nullptr && n0 + TG_BN > scatter.q_cols;
 #pragma unroll
   for (int j = 0; j < 2; ++j) {
     const int col = n0 + wave_n * 64 + j * 32 + (lane & 31);
     if (col >= n) continue;
-    const float b = bias ? bias[col] : 0.f;
+    const float b = (bias && split == 0) ? bias[col] : 0.f;
 #pragma unroll
     for (int i = 0; i < 2; ++i) {
 #pragma unroll
@@ -173,9 +208,15 @@ __global__ __launch_bounds__(256) void gemm_nt_tiled_kernel(
         if (row >= m) continue;
         float v = apply_activation<EPI>(acc[i][j][e] + b);
         TOut* dst = c + (int64_t)row * ldc + col;
-        if (EPI == PS_EPI_RESIDUAL) v += to_float<TOut>(*dst);
+        if (EPI == PS_EPI_RESIDUAL) {
+          if (k_splits > 1) {
+            unsafeAtomicAdd(reinterpret_cast<float*>(dst), v);
+            continue;
+          }
+          v += to_float<TOut>(*dst);
+        }
         *dst = from_float<TOut>(v);
-        if (EPI == PS_EPI_NONE) kv_scatter_store<TOut>(scatter, row, col, v);
+        if (scatters) kv_scatter_store<TOut>(scatter, row, col, v);
       }
     }
   }
@@ -460,10 +501,23 @@ static int launch_tiled(const void* a, const void* w, const float* bias, void* c
                         hipStream_t s) {
   const int tiles_m = (m + TG_BM - 1) / TG_BM;
   const int tiles_n = (n + TG_BN - 1) / TG_BN;
-  dim3 grid(tiles_m * tiles_n);
+  // Few tiles leave compute units idle: where partial sums can be added in place (residual
+  // epilogue) k is split over blocks until about three blocks per unit are in flight.
+  constexpr int bk = TG_ROW_BYTES / (int)sizeof(T);
+  int k_splits = 1;
+  if (epilogue == PS_EPI_RESIDUAL) {
+    const int wanted = (768 + tiles_m * tiles_n - 1) / (tiles_m * tiles_n);
+    const int possible = k / (8 * bk) > 0 ? k / (8 * bk) : 1;
+    k_splits = wanted < possible ? wanted : possible;
+  }
+  int k_chunk = (k + k_splits - 1) / k_splits;
+  k_chunk = (k_chunk + bk - 1) / bk * bk;
+  k_splits = (k + k_chunk - 1) / k_chunk;
+  dim3 grid(tiles_m * tiles_n * k_splits);
 #define PS_LAUNCH_TG(EPI)                                                                    \
   hipLaunchKernelGGL((gemm_nt_tiled_kernel<T, TOut, EPI>), grid, dim3(256), 0, s, (const T*)a, \
-                     (const T*)w, bias, (TOut*)c, m, n, k, lda, ldc, tiles_n, scatter)
+                     (const T*)w, bias, (TOut*)c, m, n, k, lda, ldc, tiles_m, tiles_n,       \
+                     k_splits, k_chunk, scatter)
   switch (epilogue) {
     case PS_EPI_NONE: PS_LAUNCH_TG(PS_EPI_NONE); break;
     case PS_EPI_GELU_TANH: PS_LAUNCH_TG(PS_EPI_GELU_TANH); break;
