@@ -56,8 +56,10 @@ __global__ __launch_bounds__(256) void attention_prefill_kernel(
   const int head = blockIdx.y;
   const int kv_head = head / (heads / kv_heads);
 
-  const int item = tile_item[blockIdx.x];
-  const int q0 = tile_q0[blockIdx.x];
+  // later tiles of a request see more keys: start them first
+  const int tile_index = gridDim.x - 1 - blockIdx.x;
+  const int item = tile_item[tile_index];
+  const int q0 = tile_q0[tile_index];
   const int tok0 = cu_tokens[item];
   const int count = cu_tokens[item + 1] - tok0;
   const int start = kv_lens[item] - count;   // position of the portion's first token
@@ -95,6 +97,9 @@ __global__ __launch_bounds__(256) void attention_prefill_kernel(
                  : uint4{0u, 0u, 0u, 0u};
   }
 
+  // Scores are kept in units of log 2 (scale * log2(e) folded into one factor), so that
+  // every exponential is one v_exp_f32; probabilities are rounded to bfloat16 right after.
+  const float scale_log2 = scale * 1.4426950408889634f;
   float m = -INFINITY, l = 0.f;
   f32x4 acc[NDB];
 #pragma unroll
@@ -104,22 +109,37 @@ __global__ __launch_bounds__(256) void attention_prefill_kernel(
   // pieces are loaded into registers while the current tile is being multiplied.
   constexpr int CHUNKS = (AP_KEYS * NDB * 2 + 255) / 256;
   uint4 k_next[CHUNKS], v_next[CHUNKS];
-  auto fetch_tile = [&](int k0) {
+  int page_next[CHUNKS];
+  // The address of a key needs its page, which is a load of its own: pages are fetched one
+  // tile further ahead than keys, so neither trip to memory is waited for.
+  auto fetch_pages = [&](int k0) {
 #pragma unroll
     for (int i = 0; i < CHUNKS; ++i) {
       const int c = tid + i * 256;
-      const int key_local = c / (NDB * 2);
-      const int dc = c - key_local * (NDB * 2);
+      const int key_local = c % AP_KEYS;
+      const int key = k0 + key_local;
+      const int safe_key = key < key_end ? key : key_end - 1;
+      const int logical = page_shift >= 0 ? (safe_key >> page_shift) : safe_key / page_size;
+      page_next[i] = logical < table_width ? table[logical] : -1;
+    }
+  };
+  auto fetch_tile = [&](int k0) {
+#pragma unroll
+    for (int i = 0; i < CHUNKS; ++i) {
+      // piece c = (8 head dimensions dc, key c % 64): the lanes of a wave hold 64 consecutive
+      // keys of the same dimensions, so the transposed V stores below do not collide in LDS
+      const int c = tid + i * 256;
+      const int dc = c / AP_KEYS;
+      const int key_local = c - dc * AP_KEYS;
       const int key = k0 + key_local;
       // unconditional loads from clamped addresses, zeroed afterwards
-      const int safe_key = (key < key_end && key_local < AP_KEYS) ? key : key_end - 1;
+      const int safe_key = key < key_end ? key : key_end - 1;
       const int logical = page_shift >= 0 ? (safe_key >> page_shift) : safe_key / page_size;
-      const int page = table[logical < table_width ? logical : table_width - 1];
-      const bool ok = key < key_end && key_local < AP_KEYS && logical < table_width && page >= 0 &&
-                      page < num_pages;
+      const int page = page_next[i];
+      const bool ok = key < key_end && dc < NDB * 2 && page >= 0 && page < num_pages;
       const int64_t offset =
           (((int64_t)(ok ? page : 0) * kv_heads + kv_head) * page_size +
-           (safe_key - logical * page_size)) * HD + dc * 8;
+           (safe_key - logical * page_size)) * HD + (dc < NDB * 2 ? dc : 0) * 8;
       k_next[i] = *reinterpret_cast<const uint4*>(k_pool + offset);
       v_next[i] = *reinterpret_cast<const uint4*>(v_pool + offset);
       if (!ok) {
@@ -132,9 +152,9 @@ __global__ __launch_bounds__(256) void attention_prefill_kernel(
 #pragma unroll
     for (int i = 0; i < CHUNKS; ++i) {
       const int c = tid + i * 256;
-      const int key_local = c / (NDB * 2);
-      const int dc = c - key_local * (NDB * 2);
-      if (key_local >= AP_KEYS) continue;
+      const int dc = c / AP_KEYS;
+      const int key_local = c - dc * AP_KEYS;
+      if (dc >= NDB * 2) continue;
       *reinterpret_cast<uint4*>(&k_lds[key_local * K_STRIDE + dc * 16]) = k_next[i];
       const uint32_t words[4] = {v_next[i].x, v_next[i].y, v_next[i].z, v_next[i].w};
 #pragma unroll
@@ -146,12 +166,17 @@ __global__ __launch_bounds__(256) void attention_prefill_kernel(
   };
 
   const int k_first = key_begin / AP_KEYS * AP_KEYS;
+  fetch_pages(k_first);
   fetch_tile(k_first);
+  if (k_first + AP_KEYS < key_end) fetch_pages(k_first + AP_KEYS);
   for (int k0 = k_first; k0 < key_end; k0 += AP_KEYS) {
     __syncthreads();   // the previous tile has been consumed
     store_tile();
     __syncthreads();
-    if (k0 + AP_KEYS < key_end) fetch_tile(k0 + AP_KEYS);   // in flight during the products
+    if (k0 + AP_KEYS < key_end) {
+      fetch_tile(k0 + AP_KEYS);   // in flight during the products
+      if (k0 + 2 * AP_KEYS < key_end) fetch_pages(k0 + 2 * AP_KEYS);
+    }
     // skip tiles that no query of this wave can see
     if (!wave_active || k0 > wave_last) continue;
     if (window > 0 && k0 + AP_KEYS - 1 < wave_first - window + 1) continue;
@@ -174,7 +199,7 @@ __global__ __launch_bounds__(256) void attention_prefill_kernel(
       for (int i = 0; i < 4; ++i) {
         const int key = k0 + kb * 16 + group * 4 + i;
         const bool visible = key <= q_pos && (window <= 0 || q_pos - key < window);
-        s[kb][i] = visible ? sacc[i] * scale : -INFINITY;
+        s[kb][i] = visible ? sacc[i] * scale_log2 : -INFINITY;
         tile_max = fmaxf(tile_max, s[kb][i]);
       }
     }
@@ -185,7 +210,8 @@ __global__ __launch_bounds__(256) void attention_prefill_kernel(
       // nothing visible to this query so far; other lanes of the wave may differ, so the
       // products below still run with zero probabilities
     }
-    const float correction = (m == -INFINITY || m_new == -INFINITY) ? 0.f : expf(m - m_new);
+    const float correction =
+        (m == -INFINITY || m_new == -INFINITY) ? 0.f : __builtin_amdgcn_exp2f(m - m_new);
     float tile_sum = 0.f;
     uint32_t pw[4][2];
 #pragma unroll
@@ -193,7 +219,7 @@ __global__ __launch_bounds__(256) void attention_prefill_kernel(
       float p[4];
 #pragma unroll
       for (int i = 0; i < 4; ++i) {
-        p[i] = (s[kb][i] == -INFINITY) ? 0.f : expf(s[kb][i] - m_new);
+        p[i] = (s[kb][i] == -INFINITY) ? 0.f : __builtin_amdgcn_exp2f(s[kb][i] - m_new);
         tile_sum += p[i];
       }
       pw[kb][0] = pack_bf16(p[0], p[1]);

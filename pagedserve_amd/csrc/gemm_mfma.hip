@@ -195,19 +195,29 @@ __global__ __launch_bounds__(256) void gemm_nt_tiled_kernel(
 
   // element e of a 32 x 32 accumulator: row (e / 4) * 8 + (lane / 32) * 4 + e % 4, column lane % 32
   const bool scatters = EPI == PS_EPI_NONE && scatter.k_pool != nullptr && n0 + TG_BN > scatter.q_cols;
+  int col[2];
+  float b[2];
+  TOut* pool[2] = {nullptr, nullptr};
+  int64_t pool_offset[2] = {0, 0};
 #pragma unroll
   for (int j = 0; j < 2; ++j) {
-    const int col = n0 + wave_n * 64 + j * 32 + (lane & 31);
-    if (col >= n) continue;
-    const float b = (bias && split == 0) ? bias[col] : 0.f;
+    col[j] = n0 + wave_n * 64 + j * 32 + (lane & 31);
+    b[j] = (bias && split == 0 && col[j] < n) ? bias[col[j]] : 0.f;
+    if (scatters && col[j] < n) pool[j] = kv_scatter_col<TOut>(scatter, col[j], &pool_offset[j]);
+  }
 #pragma unroll
-    for (int i = 0; i < 2; ++i) {
+  for (int i = 0; i < 2; ++i) {
 #pragma unroll
-      for (int e = 0; e < 16; ++e) {
-        const int row = m0 + wave_m * 64 + i * 32 + (e >> 2) * 8 + (lane >> 5) * 4 + (e & 3);
-        if (row >= m) continue;
-        float v = apply_activation<EPI>(acc[i][j][e] + b);
-        TOut* dst = c + (int64_t)row * ldc + col;
+    for (int e = 0; e < 16; ++e) {
+      const int row = m0 + wave_m * 64 + i * 32 + (e >> 2) * 8 + (lane >> 5) * 4 + (e & 3);
+      if (row >= m) continue;
+      // the page slot of a row is looked up once for all its columns
+      const int64_t slot = scatters ? kv_scatter_row(scatter, row) : -1;
+#pragma unroll
+      for (int j = 0; j < 2; ++j) {
+        if (col[j] >= n) continue;
+        float v = apply_activation<EPI>(acc[i][j][e] + b[j]);
+        TOut* dst = c + (int64_t)row * ldc + col[j];
         if (EPI == PS_EPI_RESIDUAL) {
           if (k_splits > 1) {
             unsafeAtomicAdd(reinterpret_cast<float*>(dst), v);
@@ -216,7 +226,7 @@ __global__ __launch_bounds__(256) void gemm_nt_tiled_kernel(
           v += to_float<TOut>(*dst);
         }
         *dst = from_float<TOut>(v);
-        if (scatters) kv_scatter_store<TOut>(scatter, row, col, v);
+        if (pool[j] != nullptr && slot >= 0) pool[j][slot + pool_offset[j]] = from_float<TOut>(v);
       }
     }
   }

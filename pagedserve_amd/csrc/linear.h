@@ -23,6 +23,33 @@ struct NormPrologue {
   int ldh;
 };
 
+// The two halves of that address, for kernels that finish many elements of one row or one
+// column: kv_scatter_row gives the element offset of (page, slot) of a token, or -1;
+// kv_scatter_col gives the pool and the offset of (head, dim) inside a page, or null for a
+// query column.
+__device__ inline int64_t kv_scatter_row(const KvScatter& s, int row) {
+  const int pos = s.tok_pos[row];
+  const int logical = s.page_shift >= 0 ? (pos >> s.page_shift) : pos / s.page_size;
+  if (logical >= s.table_width) return -1;
+  const int page = s.tables[(int64_t)s.tok_item[row] * s.table_width + logical];
+  if (page < 0 || page >= s.num_pages) return -1;
+  return ((int64_t)page * s.kv_heads * s.page_size + (pos - logical * s.page_size)) * s.head_dim;
+}
+
+template <typename T>
+__device__ inline T* kv_scatter_col(const KvScatter& s, int col, int64_t* offset) {
+  if (s.k_pool == nullptr || col < s.q_cols) return nullptr;
+  int within = col - s.q_cols;
+  T* pool = reinterpret_cast<T*>(s.k_pool);
+  if (within >= s.kv_cols) {
+    within -= s.kv_cols;
+    pool = reinterpret_cast<T*>(s.v_pool);
+  }
+  const int head = within / s.head_dim;
+  *offset = (int64_t)head * s.page_size * s.head_dim + (within - head * s.head_dim);
+  return pool;
+}
+
 // Column `col` of output row `row` also goes into the cache when it is a key or value column:
 // token at position p of item r lands at (page = table[r][p / page], offset = p % page)
 // (reference: src/model/kv_manager.py:303-308,403-404).
