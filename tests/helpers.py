@@ -220,5 +220,6 @@ def max_error(rows, reference):
     return worst, scale, where
 
 
-# |engine - plain| <= TOLERANCE[dtype] * max|plain logits|
-TOLERANCE = {"float32": 1e-4, "bfloat16": 2e-2}
+# |engine - plain| <= TOLERANCE[dtype] * max|plain logits|.  Measured on MI355X: about 2e-6 in
+# float32 and 2e-3 in bfloat16 at every size from the tiny models to GPT-2 small.
+TOLERANCE = {"float32": 2e-5, "bfloat16": 1e-2}

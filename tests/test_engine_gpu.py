@@ -73,6 +73,7 @@ def test_cuts_match_plain(folders, references, which, dtype, cut):
     assert not engine.cache.requests
     assert len(rows) == sum(len(tokens) for tokens in requests.values())
     error, scale, where = helpers.max_error(rows, references[(which, dtype == "bfloat16")])
+    print(f"cut {cut} {which} {dtype}: error/scale {error / scale:.2e}")
     assert error <= helpers.TOLERANCE[dtype] * scale, (error, scale, where)
 
 
