@@ -37,6 +37,21 @@ class StepEntry:
 class StepOutput:
     logits: torch.Tensor            # float32 [wanted, vocab]; valid until the next step
     rows: List[tuple]               # (request_id, position) of each row
+    tokens: Optional[torch.Tensor] = None   # int32 [wanted]: argmax of each row, if asked for
+
+
+class _ReplayPlan:
+    """What a captured decode step needs on later steps: where each index array lies in the
+    packed buffer (numpy views for both staging buffers), the copy to the device, the graph
+    and its outputs.  Replaying fills a few arrays, copies once and launches once."""
+
+    def __init__(self, graph, used, sections, logits, tokens, items):
+        self.graph = graph
+        self.used = used
+        self.sections = sections       # per staging buffer: dict name -> numpy view
+        self.logits = logits
+        self.tokens = tokens
+        self.items = items
 
 
 class StepError(ValueError):
@@ -65,9 +80,12 @@ class Engine:
                     + len(groups) * max_requests * self.table_width + 16)
         self._meta_device = torch.empty(capacity, dtype=torch.int32, device=self.device)
         self._meta_host = [torch.empty(capacity, dtype=torch.int32, pin_memory=True) for _ in range(2)]
-        self._meta_events = [None, None]
+        self._meta_events = [torch.cuda.Event(), torch.cuda.Event()]
+        self._meta_pending = [False, False]
+        self._meta_owner = [None, None]   # replay plan whose constant arrays a buffer holds
         self._meta_turn = 0
         self._logits = None
+        self._tokens = torch.zeros(max(max_requests, 64), dtype=torch.int32, device=self.device)
         # The engine's work runs on a stream of its own (default priority): a capture cannot
         # record from the default stream.
         self.stream = torch.cuda.Stream(device=self.device)
@@ -91,8 +109,8 @@ class Engine:
     def graph_summary(self) -> dict:
         """Counters in the manner of src/model/paged_decoder.py:498-507."""
         return {"enabled": self.use_graphs, "captured_graphs": len(self._graphs),
-                "graph_replays": sum(graph.replays for graph in self._graphs.values()),
-                "graph_nodes": {str(key): graph.nodes for key, graph in self._graphs.items()},
+                "graph_replays": sum(plan.graph.replays for plan in self._graphs.values()),
+                "graph_nodes": {str(key): plan.graph.nodes for key, plan in self._graphs.items()},
                 "capture_failures": list(self._graph_failures.values())}
 
     def _logit_buffer(self, rows: int) -> torch.Tensor:
@@ -137,7 +155,10 @@ class Engine:
         if len(self.cache.requests) + new > self.max_requests:
             raise StepError(f"more than {self.max_requests} live requests")
 
-    def step(self, entries: Sequence[StepEntry]) -> StepOutput:
+    def step(self, entries: Sequence[StepEntry], greedy: bool = False) -> StepOutput:
+        """Run one batch.  With ``greedy`` the argmax of every wanted row is computed on the
+        GPU as part of the step (inside the graph of a replayed decode step) and returned as
+        ``StepOutput.tokens``."""
         entries = list(entries)
         self._validate(entries)
         admitted = []
@@ -151,11 +172,14 @@ class Engine:
                     record = cache.requests[entry.request_id]
                 cache.grow(entry.request_id, record.length + len(entry.tokens))
             caller = torch.cuda.current_stream(self.device)
-            # the caller may still be reading the last step's logits
-            self.stream.wait_stream(caller)
-            with torch.cuda.stream(self.stream):
-                output = self._run(entries)
-            caller.wait_stream(self.stream)
+            if caller.cuda_stream == self.stream.cuda_stream:
+                output = self._run(entries, greedy)
+            else:
+                # the caller may still be reading the last step's logits
+                self.stream.wait_stream(caller)
+                with torch.cuda.stream(self.stream):
+                    output = self._run(entries, greedy)
+                caller.wait_stream(self.stream)
         except Exception:
             # requests that this step admitted leave no trace
             # (src/scheduler/orca_scheduler.py:243-247)
@@ -196,8 +220,9 @@ class Engine:
             cursor += items * width
         turn = self._meta_turn
         self._meta_turn ^= 1
-        if self._meta_events[turn] is not None:
+        if self._meta_pending[turn]:
             self._meta_events[turn].synchronize()
+        self._meta_owner[turn] = None
         host = self._meta_host[turn].numpy()
 
         def section(name):
@@ -265,9 +290,9 @@ class Engine:
             section(f"tables{group}").reshape(items, width)[:] = cache.table_arrays[group][slot_index]
         device = self._meta_device
         device[:cursor].copy_(self._meta_host[turn][:cursor], non_blocking=True)
-        event = torch.cuda.Event()
-        event.record()
-        self._meta_events[turn] = event
+        self._meta_events[turn].record()
+        self._meta_pending[turn] = True
+        self._last_layout = (offsets, cursor)
 
         def view(name):
             begin, size = offsets[name]
@@ -285,39 +310,99 @@ class Engine:
             tile_item=view("tile_item"), tile_q0=view("tile_q0"))
         return ctx, view("rows"), row_keys
 
-    def _run(self, entries) -> StepOutput:
+    def _forward(self, ctx, rows, logits, wanted, greedy):
+        out = self.model.forward(ctx, self.views, rows, logits)
+        tokens = None
+        if greedy and wanted:
+            from ..ops import kernels
+
+            tokens = kernels.sample(out, None, None, self._tokens[:wanted])
+        return out, tokens
+
+    def _run(self, entries, greedy=False) -> StepOutput:
+        items = len(entries)
+        if self.use_graphs and self._graphs:
+            # a captured step: every entry brings one token and wants its logits
+            plan = self._graphs.get((items, greedy))
+            if (plan is not None and plan.logits.data_ptr() == self._logit_buffer(items).data_ptr()
+                    and all(len(e.tokens) == 1 and len(e.want) == 1 for e in entries)):
+                return self._replay(plan, entries)
         ctx, rows, row_keys = self._pack(entries)
-        logits = self._logit_buffer(len(row_keys))
+        wanted = len(row_keys)
+        logits = self._logit_buffer(wanted)
         graph_key = None
-        if self.use_graphs and ctx.decode_only and len(row_keys) == ctx.tokens:
+        if self.use_graphs and ctx.decode_only and wanted == ctx.tokens:
             # A step of single tokens that all want their logits.  Every launch argument is
             # then a function of the number of items (and of buffer addresses).
-            graph_key = (ctx.tokens, logits.data_ptr())
+            graph_key = (items, greedy)
         if graph_key is None or graph_key in self._graph_failures:
-            out = self.model.forward(ctx, self.views, rows, logits)
-            return StepOutput(logits=out, rows=row_keys)
+            out, tokens = self._forward(ctx, rows, logits, wanted, greedy)
+            return StepOutput(logits=out, rows=row_keys, tokens=tokens)
         # launch shapes inside a graph must not depend on this step's lengths
         ctx.max_kv_len = self.spec.max_positions
-        graph = self._graphs.get(graph_key)
-        if graph is None:
-            if graph_key not in self._graph_seen:
-                # first time: run directly, so that every buffer exists before a capture
-                self._graph_seen.add(graph_key)
-                out = self.model.forward(ctx, self.views, rows, logits)
-                return StepOutput(logits=out, rows=row_keys)
-            from ..ops.kernels import KernelError, StepGraph
+        seen_key = (items, greedy, logits.data_ptr())
+        if seen_key not in self._graph_seen:
+            # first time: run directly, so that every buffer exists before a capture
+            self._graph_seen.add(seen_key)
+            out, tokens = self._forward(ctx, rows, logits, wanted, greedy)
+            return StepOutput(logits=out, rows=row_keys, tokens=tokens)
+        from ..ops.kernels import StepGraph
 
-            graph = StepGraph()
-            StepGraph.begin()
-            try:
-                self.model.forward(ctx, self.views, rows, logits)
-                graph.end()
-            except Exception as error:       # the capture is abandoned, the step runs directly
-                StepGraph.abort()
-                self._graph_failures[graph_key] = f"{type(error).__name__}: {error}"
-                ctx.max_kv_len = max(item.start + 1 for item in ctx.items)
-                out = self.model.forward(ctx, self.views, rows, logits)
-                return StepOutput(logits=out, rows=row_keys)
-            self._graphs[graph_key] = graph
+        graph = StepGraph()
+        StepGraph.begin()
+        try:
+            out, tokens = self._forward(ctx, rows, logits, wanted, greedy)
+            graph.end()
+        except Exception as error:       # the capture is abandoned, the step runs directly
+            StepGraph.abort()
+            self._graph_failures[graph_key] = f"{type(error).__name__}: {error}"
+            ctx.max_kv_len = max(item.start + 1 for item in ctx.items)
+            out, tokens = self._forward(ctx, rows, logits, wanted, greedy)
+            return StepOutput(logits=out, rows=row_keys, tokens=tokens)
+        offsets, used = self._last_layout
+        sections = []
+        for host in self._meta_host:
+            array = host.numpy()
+            views = {name: array[begin:begin + size] for name, (begin, size) in offsets.items()}
+            for group in range(len(self.cache.groups)):
+                views[f"tables{group}"] = views[f"tables{group}"].reshape(items, self.table_width)
+            sections.append(views)
+        old = self._graphs.get(graph_key)
+        if old is not None:
+            old.graph.destroy()
+        self._graphs[graph_key] = _ReplayPlan(graph, used, sections, out, tokens, items)
         graph.launch()
-        return StepOutput(logits=logits[:len(row_keys)], rows=row_keys)
+        return StepOutput(logits=out, rows=row_keys, tokens=tokens)
+
+    def _replay(self, plan, entries) -> StepOutput:
+        """A captured decode step: refresh the per-step indices, copy them, launch the graph."""
+        cache = self.cache
+        turn = self._meta_turn
+        self._meta_turn ^= 1
+        if self._meta_pending[turn]:
+            self._meta_events[turn].synchronize()
+        sections = plan.sections[turn]
+        items = plan.items
+        if self._meta_owner[turn] is not plan:
+            # arrays that are the same on every step of this shape
+            index = np.arange(items + 1, dtype=np.int32)
+            sections["tok_item"][:] = index[:items]
+            sections["cu_tokens"][:] = index
+            sections["single_tokens"][:] = index[:items]
+            sections["rows"][:] = index[:items]
+            self._meta_owner[turn] = plan
+        records = [cache.requests[entry.request_id] for entry in entries]
+        starts = [record.length for record in records]
+        slots = [record.slot for record in records]
+        sections["token_ids"][:] = [entry.tokens[0] for entry in entries]
+        sections["positions"][:] = starts
+        sections["kv_lens"][:] = [start + 1 for start in starts]
+        sections["slots"][:] = slots
+        for group in range(len(cache.groups)):
+            sections[f"tables{group}"][:] = cache.table_arrays[group][slots]
+        self._meta_device[:plan.used].copy_(self._meta_host[turn][:plan.used], non_blocking=True)
+        self._meta_events[turn].record()
+        self._meta_pending[turn] = True
+        plan.graph.launch()
+        rows = [(entry.request_id, start) for entry, start in zip(entries, starts)]
+        return StepOutput(logits=plan.logits, rows=rows, tokens=plan.tokens)

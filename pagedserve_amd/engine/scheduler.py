@@ -235,6 +235,22 @@ class ContinuousBatchScheduler:
 
     # ------------------------------------------------------------------ step
     def step(self) -> Dict[int, int]:
+        """One iteration.  With a real engine the whole iteration (step, token selection and
+        the copy of the tokens) runs on the engine's own stream, which saves the hand-over
+        between streams on every step."""
+        stream = getattr(self.engine, "stream", None)
+        if stream is None:
+            return self._step()
+        import torch
+
+        previous = torch.cuda.current_stream(stream.device)
+        torch.cuda.set_stream(stream)
+        try:
+            return self._step()
+        finally:
+            torch.cuda.set_stream(previous)
+
+    def _step(self) -> Dict[int, int]:
         selected = self.select_requests()
         if not selected:
             if self.waiting or self.active:
@@ -246,20 +262,26 @@ class ContinuousBatchScheduler:
             for g, pages in enumerate(request.reserved_blocks):
                 self.reserved_blocks[g] += pages
         entries = self.build_step_entries(selected)
+        producers = [request for (request, size), entry in zip(selected, entries) if entry.want]
+        # greedy rows are picked on the GPU inside the step (one launch less, and part of the
+        # captured graph of a decode step)
+        greedy = bool(producers) and all(r.sampling.temperature == 0 for r in producers)
         try:
-            output = self.engine.step(entries)
+            output = self.engine.step(entries, greedy=greedy)
         except Exception:
             for request in new_requests:
                 for g, pages in enumerate(request.reserved_blocks):
                     self.reserved_blocks[g] -= pages
                 request.reserved_blocks = []
             raise
-        producers = [request for (request, size), entry in zip(selected, entries) if entry.want]
         if output.logits.shape[0] != len(producers):
             raise RuntimeError("the engine returned a wrong number of logits rows")
-        tokens = self.sampler.sample(
-            output.logits, [r.sampling for r in producers], [r.request_id for r in producers],
-            [len(r.generated_token_ids) for r in producers], [r.seed for r in producers])
+        if getattr(output, "tokens", None) is not None:
+            tokens = output.tokens.tolist()
+        else:
+            tokens = self.sampler.sample(
+                output.logits, [r.sampling for r in producers], [r.request_id for r in producers],
+                [len(r.generated_token_ids) for r in producers], [r.seed for r in producers])
         emitted = {}
         completed_prefill = set()
         next_token = iter(tokens)

@@ -484,11 +484,14 @@ class StepGraph:
         lib.ps_graph_abort(_stream())
 
     def launch(self):
-        lib = load_library()
-        lib.ps_graph_launch.argtypes = [c_void_p, c_void_p]
-        lib.ps_graph_launch.restype = c_int
-        if lib.ps_graph_launch(self.handle, _stream()) != 0:
-            raise KernelError(lib.ps_last_error().decode())
+        fn = _BOUND.get("ps_graph_launch")
+        if fn is None:
+            fn = load_library().ps_graph_launch
+            fn.argtypes = [c_void_p, c_void_p]
+            fn.restype = c_int
+            _BOUND["ps_graph_launch"] = fn
+        if fn(self.handle, torch.cuda.current_stream().cuda_stream) != 0:
+            raise KernelError(load_library().ps_last_error().decode())
         self.replays += 1
 
     def destroy(self):

@@ -15,7 +15,8 @@ pytestmark = pytest.mark.gpu
 
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 
-# prompts + decoded tokens of BASELINE's tiny workloads, as given token sequences
+# prompt + decoded lengths of the two tiny workloads (5, 17, 31 -> 16 tokens; 1, 9, 40, 64, 100 -> 24),
+# as given token sequences, plus one long request each
 LENGTHS = {"A": [5 + 16, 17 + 16, 31 + 16, 90], "B": [1 + 24, 9 + 24, 40 + 24, 64 + 24, 100 + 24, 200]}
 
 

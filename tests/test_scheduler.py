@@ -34,7 +34,7 @@ class FakeEngine:
         self.steps = []
         self.fail_next = False
 
-    def step(self, entries):
+    def step(self, entries, greedy=False):
         if self.fail_next:
             self.fail_next = False
             raise RuntimeError("injected failure")
