@@ -490,6 +490,11 @@ __global__ __launch_bounds__(64 * SK_WAVES) void gemm_nt_skinny_norm_kernel(
 }
 
 // --------------------------------------------------------------------------------- host
+bool ps_gemm_nt_bf16_tiled_supported(const void* a, const void* w, int m, int k, int lda);
+int ps_gemm_nt_bf16_tiled(const void* a, const void* w, const float* bias, void* c, int m, int n,
+                          int k, int lda, int ldc, int c_dtype, int epilogue,
+                          const KvScatter& scatter, hipStream_t s);
+
 static bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
 
 bool ps_gemm_nt_mfma_supported(const void* a, const void* w, int k, int lda, int dtype) {
@@ -624,6 +629,8 @@ int ps_gemm_nt_mfma(const void* a, const void* w, const float* bias, void* c, in
       return launch_skinny<float>(a, w, bias, c, m, n, k, lda, ldc, epilogue, scatter, s);
     return launch_skinny<bf16_t>(a, w, bias, c, m, n, k, lda, ldc, epilogue, scatter, s);
   }
+  if (dtype == PS_BF16 && ps_gemm_nt_bf16_tiled_supported(a, w, m, k, lda))
+    return ps_gemm_nt_bf16_tiled(a, w, bias, c, m, n, k, lda, ldc, c_dtype, epilogue, scatter, s);
   if (dtype == PS_F32 && c_dtype == PS_F32)
     return launch_tiled<float, float>(a, w, bias, c, m, n, k, lda, ldc, epilogue, scatter, s);
   if (dtype == PS_BF16 && c_dtype == PS_F32)

@@ -1,0 +1,322 @@
+// Tiled bfloat16 matrix product for many rows (prompt portions) on gfx950:
+//   C[m, n] = epi(sum_k A[m, k] W[n, k] + b[n]),   k a multiple of 64.
+//
+// Operand tiles go from global memory straight into LDS (global_load_lds_dwordx4: no trip
+// through registers), several k tiles ahead of the one being multiplied.  A stage holds 64
+// values of k (128 bytes) of every row of the block's A and W tiles.  One load instruction of
+// a wave fills 1024 contiguous bytes of LDS, eight rows; which 16-byte piece of its row a
+// lane fetches is chosen so that piece c of row r lands in slot c ^ ((r >> 1) & 7) of the
+// row.  With that, the 16 lanes that read one k piece of 16 consecutive rows for an MFMA
+// operand touch every LDS bank once.
+//
+// Four waves in a 2 x 2 arrangement; a wave owns WM x WN accumulators of 32 x 32
+// (v_mfma_f32_32x32x16_bf16, float accumulation), so a block makes 64 WM x 64 WN outputs.
+// Per k tile there is one wait (own loads of that tile have landed; later tiles stay in
+// flight) and one barrier, after which the stage that was multiplied last is refilled.
+//
+// Rows beyond m or n are fetched from the last valid row instead (they only feed outputs that
+// are never stored).  The epilogue is the one of the other products: bias, GELU, residual
+// add into the float stream, key/value columns into cache pages.
+#include "common.h"
+#include "linear.h"
+#include "pagedserve_hip.h"
+
+typedef __attribute__((__vector_size__(8 * sizeof(__bf16)))) __bf16 bf16x8;
+typedef __attribute__((__vector_size__(16 * sizeof(float)))) float f32x16;
+
+#define TB_BK 64     // values of k per stage
+#define TB_ROW 128   // bytes per row and stage
+
+typedef const __attribute__((address_space(1))) void* global_ptr_t;
+typedef __attribute__((address_space(3))) void* lds_ptr_t;
+
+// gelu_tanh(u) = u * sigmoid(2 z), z = sqrt(2/pi) (u + 0.044715 u^3), with the hardware
+// exponential and reciprocal: its error (about 1e-6 relative) is far below the rounding of a
+// bfloat16 result, which is the only place where it is used.
+__device__ inline float gelu_tanh_fast(float u) {
+  const float z2 = 1.5957691216057308f * (u + 0.044715f * u * u * u);
+  return u * __frcp_rn(1.0f + __expf(-z2));
+}
+
+template <int EPI, typename TOut>
+__device__ inline float finish_value(float v) {
+  if (EPI == PS_EPI_GELU_TANH && sizeof(TOut) == 2) return gelu_tanh_fast(v);
+  return apply_activation<EPI>(v);
+}
+
+// Eight finished values to eight consecutive outputs (16-byte aligned).
+__device__ inline void store8(float* out, const float* v) {
+  *reinterpret_cast<float4*>(out) = make_float4(v[0], v[1], v[2], v[3]);
+  *reinterpret_cast<float4*>(out + 4) = make_float4(v[4], v[5], v[6], v[7]);
+}
+__device__ inline void store8(bf16_t* out, const float* v) {
+  uint4 packed;
+  packed.x = pack2_bf16(v[0], v[1]);
+  packed.y = pack2_bf16(v[2], v[3]);
+  packed.z = pack2_bf16(v[4], v[5]);
+  packed.w = pack2_bf16(v[6], v[7]);
+  *reinterpret_cast<uint4*>(out) = packed;
+}
+
+// Wait until at most `pending` of this wave's loads are in flight, then meet the other waves.
+// The asm statements are compiler barriers for memory as well: LDS reads stay behind them.
+template <int PENDING>
+__device__ inline void wait_loads_and_sync() {
+  asm volatile("s_waitcnt vmcnt(%0)\n\ts_barrier" ::"n"(PENDING) : "memory");
+}
+
+template <int WM, int WN, int STAGES, typename TOut, int EPI>
+__global__ __launch_bounds__(256) void gemm_nt_bf16_tiled_kernel(
+    const bf16_t* __restrict__ a, const bf16_t* __restrict__ w, const float* __restrict__ bias,
+    TOut* __restrict__ c, int m, int n, int k, int lda, int ldc, int tiles_m, int tiles_n,
+    int row_major, KvScatter scatter) {
+  constexpr int BM = 64 * WM, BN = 64 * WN;
+  constexpr int STAGE_BYTES = (BM + BN) * TB_ROW;
+  constexpr int LOADS_A = BM / 32;   // load instructions per wave and stage (8 rows each)
+  constexpr int LOADS_W = BN / 32;
+  constexpr int LOADS = LOADS_A + LOADS_W;
+  static_assert(STAGES >= 2 && STAGES <= 4, "two to four stages");
+  static_assert(LOADS * (STAGES - 2) < 64, "the load counter has six bits");
+  __shared__ __attribute__((aligned(1024))) unsigned char lds[STAGES * STAGE_BYTES];
+
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = tid >> 6;
+  const int wave_m = wave >> 1;
+  const int wave_n = wave & 1;
+  // Consecutive block ids run on different XCDs, each with an L2 of its own: blocks are
+  // renumbered so that every XCD works on a contiguous run of tiles.  A run walked along the
+  // rows of C reads few rows of A and all of W, one walked down the columns few rows of W and
+  // all of A: the host picks the cheaper one.
+  const int blocks = gridDim.x;
+  const int per_xcd = blocks / 8;
+  int logical = blockIdx.x;
+  if (blockIdx.x < per_xcd * 8) logical = (blockIdx.x & 7) * per_xcd + (blockIdx.x >> 3);
+  const int tile_n = row_major ? logical % tiles_n : logical / tiles_m;
+  const int tile_m = row_major ? logical / tiles_n : logical % tiles_m;
+  const int m0 = tile_m * BM;
+  const int n0 = tile_n * BN;
+  const int k_tiles = k / TB_BK;
+
+  // ---- loads: lane l of a load instruction fills slot l % 8 of row l / 8 of its eight rows
+  const bf16_t* src[LOADS];
+  int dst[LOADS];
+#pragma unroll
+  for (int j = 0; j < LOADS; ++j) {
+    const bool is_a = j < LOADS_A;
+    const int group = is_a ? wave * LOADS_A + j : wave * LOADS_W + (j - LOADS_A);
+    const int tile_row = group * 8 + (lane >> 3);
+    const int piece = (lane & 7) ^ ((tile_row >> 1) & 7);
+    if (is_a) {
+      const int row = m0 + tile_row < m ? m0 + tile_row : m - 1;
+      src[j] = a + (int64_t)row * lda + piece * 8;
+      dst[j] = group * 8 * TB_ROW;
+    } else {
+      const int row = n0 + tile_row < n ? n0 + tile_row : n - 1;
+      src[j] = w + (int64_t)row * k + piece * 8;
+      dst[j] = (BM + group * 8) * TB_ROW;
+    }
+  }
+  auto issue = [&](int kt) {
+    unsigned char* stage = lds + (kt % STAGES) * STAGE_BYTES;
+#pragma unroll
+    for (int j = 0; j < LOADS; ++j)
+      __builtin_amdgcn_global_load_lds((global_ptr_t)(src[j] + (int64_t)kt * TB_BK),
+                                       (lds_ptr_t)(stage + dst[j]), 16, 0, 0);
+  };
+
+  f32x16 acc[WM][WN];
+#pragma unroll
+  for (int i = 0; i < WM; ++i)
+#pragma unroll
+    for (int j = 0; j < WN; ++j)
+#pragma unroll
+      for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.f;
+
+  // ---- operands: lane l reads the 16 bytes of k piece 2 s + l / 32 of row l % 32
+  const int key = (lane >> 1) & 7;   // ((row >> 1) & 7) of every row this lane reads
+  const int a_row = (wave_m * WM * 32 + (lane & 31)) * TB_ROW;
+  const int w_row = (BM + wave_n * WN * 32 + (lane & 31)) * TB_ROW;
+  auto compute = [&](int kt) {
+    const unsigned char* stage = lds + (kt % STAGES) * STAGE_BYTES;
+    // the operands of step s + 1 are fetched before the products of step s are issued
+    bf16x8 fa[2][WM], fw[2][WN];
+    auto fetch = [&](int s, bf16x8* da, bf16x8* dw) {
+      const int slot = ((2 * s + (lane >> 5)) ^ key) << 4;
+#pragma unroll
+      for (int i = 0; i < WM; ++i)
+        da[i] = *reinterpret_cast<const bf16x8*>(stage + a_row + i * 32 * TB_ROW + slot);
+#pragma unroll
+      for (int j = 0; j < WN; ++j)
+        dw[j] = *reinterpret_cast<const bf16x8*>(stage + w_row + j * 32 * TB_ROW + slot);
+    };
+    fetch(0, fa[0], fw[0]);
+#pragma unroll
+    for (int s = 0; s < TB_BK / 16; ++s) {
+      if (s + 1 < TB_BK / 16) fetch(s + 1, fa[(s + 1) & 1], fw[(s + 1) & 1]);
+#pragma unroll
+      for (int i = 0; i < WM; ++i)
+#pragma unroll
+        for (int j = 0; j < WN; ++j)
+          acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa[s & 1][i], fw[s & 1][j],
+                                                              acc[i][j], 0, 0, 0);
+    }
+  };
+
+#pragma unroll
+  for (int d = 0; d < STAGES - 1; ++d)
+    if (d < k_tiles) issue(d);
+  for (int kt = 0; kt < k_tiles; ++kt) {
+    // tiles kt + 1 .. kt + STAGES - 2 may stay in flight, as far as they exist
+    const int ahead = k_tiles - 1 - kt < STAGES - 2 ? k_tiles - 1 - kt : STAGES - 2;
+    if (ahead <= 0) wait_loads_and_sync<0>();
+    else if (ahead == 1) wait_loads_and_sync<LOADS>();
+    else wait_loads_and_sync<2 * LOADS>();
+    // the stage of tile kt - 1 is free now: every wave is past its reads
+    if (kt + STAGES - 1 < k_tiles) issue(kt + STAGES - 1);
+    compute(kt);
+  }
+
+  // ---- epilogue.  Element e of a 32 x 32 accumulator is row (e / 4) * 8 + (lane / 32) * 4 +
+  // e % 4, column lane % 32: a lane holds one column.  Each wave turns 32 rows at a time
+  // through a region of LDS of its own, after which a lane holds eight consecutive columns of
+  // one row: bias and activation are applied there and rows leave in pieces of 16 or 32
+  // bytes, eight (or more) lanes to a row.
+  constexpr int EP_STRIDE = WN * 32 + 8;          // floats; 4 rows further is 32 banks further
+  constexpr int EP_CHUNKS = WN * 4;               // pieces of eight columns per row
+  constexpr int EP_ROWS = 64 / EP_CHUNKS;         // rows per pass of the wave
+  static_assert(4 * 32 * EP_STRIDE * 4 <= STAGES * STAGE_BYTES, "the epilogue reuses the stages");
+  wait_loads_and_sync<0>();                       // every wave is past its last operand reads
+  float* region = reinterpret_cast<float*>(lds) + wave * 32 * EP_STRIDE;
+  const int chunk = lane % EP_CHUNKS;
+  const int row_in_pass = lane / EP_CHUNKS;
+  const int col0 = n0 + wave_n * WN * 32 + chunk * 8;
+  const bool full = col0 + 8 <= n;
+  const bool vec_c = ldc % 8 == 0 && (reinterpret_cast<uintptr_t>(c) & 15u) == 0;
+  float b[8];
+#pragma unroll
+  for (int q = 0; q < 8; ++q) b[q] = (bias && col0 + q < n) ? bias[col0 + q] : 0.f;
+  // key and value columns also go into cache pages: eight consecutive columns lie in one head
+  const bool scatters = EPI == PS_EPI_NONE && scatter.k_pool != nullptr && col0 < n &&
+                        col0 + 8 > scatter.q_cols;
+  const bool vec_kv = full && col0 >= scatter.q_cols && scatter.head_dim % 8 == 0 &&
+                      scatter.q_cols % 8 == 0 && scatter.kv_cols % 8 == 0;
+  TOut* pool = nullptr;
+  int64_t pool_offset = 0;
+  if (scatters && vec_kv) pool = kv_scatter_col<TOut>(scatter, col0, &pool_offset);
+
+#pragma unroll
+  for (int i = 0; i < WM; ++i) {
+#pragma unroll
+    for (int j = 0; j < WN; ++j)
+#pragma unroll
+      for (int e = 0; e < 16; ++e)
+        region[((e >> 2) * 8 + (lane >> 5) * 4 + (e & 3)) * EP_STRIDE + j * 32 + (lane & 31)] =
+            acc[i][j][e];
+    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+#pragma unroll 2
+    for (int pass = 0; pass < 32 / EP_ROWS; ++pass) {
+      const int r = pass * EP_ROWS + row_in_pass;
+      const int row = m0 + wave_m * WM * 32 + i * 32 + r;
+      const float4 lo = *reinterpret_cast<const float4*>(region + r * EP_STRIDE + chunk * 8);
+      const float4 hi = *reinterpret_cast<const float4*>(region + r * EP_STRIDE + chunk * 8 + 4);
+      if (row >= m || col0 >= n) continue;
+      float v[8] = {lo.x, lo.y, lo.z, lo.w, hi.x, hi.y, hi.z, hi.w};
+#pragma unroll
+      for (int q = 0; q < 8; ++q) v[q] = finish_value<EPI, TOut>(v[q] + b[q]);
+      TOut* out = c + (int64_t)row * ldc + col0;
+      if (EPI == PS_EPI_RESIDUAL) {
+        float* sum = reinterpret_cast<float*>(out);
+        if (full && vec_c) {
+          float4 o0 = *reinterpret_cast<const float4*>(sum);
+          float4 o1 = *reinterpret_cast<const float4*>(sum + 4);
+          o0.x += v[0]; o0.y += v[1]; o0.z += v[2]; o0.w += v[3];
+          o1.x += v[4]; o1.y += v[5]; o1.z += v[6]; o1.w += v[7];
+          *reinterpret_cast<float4*>(sum) = o0;
+          *reinterpret_cast<float4*>(sum + 4) = o1;
+        } else {
+          for (int q = 0; q < 8; ++q)
+            if (col0 + q < n) sum[q] += v[q];
+        }
+        continue;
+      }
+      if (full && vec_c) {
+        store8(out, v);
+      } else {
+        for (int q = 0; q < 8; ++q)
+          if (col0 + q < n) out[q] = from_float<TOut>(v[q]);
+      }
+      if (scatters) {
+        if (pool != nullptr) {
+          const int64_t slot = kv_scatter_row(scatter, row);
+          if (slot >= 0) store8(pool + slot + pool_offset, v);
+        } else if (!vec_kv) {
+          for (int q = 0; q < 8; ++q)
+            if (col0 + q < n) kv_scatter_store<TOut>(scatter, row, col0 + q, v[q]);
+        }
+      }
+    }
+    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+  }
+}
+
+// --------------------------------------------------------------------------------- host
+bool ps_gemm_nt_bf16_tiled_supported(const void* a, const void* w, int m, int k, int lda) {
+  return m > 64 && k % TB_BK == 0 && lda % 8 == 0 &&
+         (reinterpret_cast<uintptr_t>(a) & 15u) == 0 && (reinterpret_cast<uintptr_t>(w) & 15u) == 0;
+}
+
+template <int WM, int WN, int STAGES, typename TOut>
+static int launch_variant(const void* a, const void* w, const float* bias, void* c, int m, int n,
+                          int k, int lda, int ldc, int epilogue, const KvScatter& scatter,
+                          hipStream_t s) {
+  constexpr int BM = 64 * WM, BN = 64 * WN;
+  const int tiles_m = (m + BM - 1) / BM;
+  const int tiles_n = (n + BN - 1) / BN;
+  // what one XCD's run of tiles fetches into its L2, in rows of k values
+  const int run = (tiles_m * tiles_n + 7) / 8;
+  const int64_t rows_along = (int64_t)((run + tiles_n - 1) / tiles_n) * BM + n;   // along rows of C
+  const int64_t rows_down = (int64_t)((run + tiles_m - 1) / tiles_m) * BN + m;    // down columns
+  const int row_major = rows_along < rows_down ? 1 : 0;
+  dim3 grid(tiles_m * tiles_n);
+#define PS_LAUNCH_TB(EPI)                                                                     \
+  hipLaunchKernelGGL((gemm_nt_bf16_tiled_kernel<WM, WN, STAGES, TOut, EPI>), grid, dim3(256), 0, \
+                     s, (const bf16_t*)a, (const bf16_t*)w, bias, (TOut*)c, m, n, k, lda, ldc, \
+                     tiles_m, tiles_n, row_major, scatter)
+  switch (epilogue) {
+    case PS_EPI_NONE: PS_LAUNCH_TB(PS_EPI_NONE); break;
+    case PS_EPI_GELU_TANH: PS_LAUNCH_TB(PS_EPI_GELU_TANH); break;
+    case PS_EPI_GELU_ERF: PS_LAUNCH_TB(PS_EPI_GELU_ERF); break;
+    case PS_EPI_RESIDUAL: PS_LAUNCH_TB(PS_EPI_RESIDUAL); break;
+    default: ps_set_error("ps_linear: unknown epilogue %d", epilogue); return 1;
+  }
+#undef PS_LAUNCH_TB
+  PS_CHECK_LAUNCH("ps_linear(tiled, bfloat16)");
+  return 0;
+}
+
+// Tile shapes by the number of blocks they give: the chip has 256 compute units, and a product
+// of this size is over in a few microseconds, so filling them counts for more than the reuse
+// inside a large tile.  Long k with few tiles takes deeper prefetch instead.
+template <typename TOut>
+static int launch_tiled_bf16(const void* a, const void* w, const float* bias, void* c, int m,
+                             int n, int k, int lda, int ldc, int epilogue,
+                             const KvScatter& scatter, hipStream_t s) {
+  const int64_t tiles_128 = (int64_t)((m + 127) / 128) * ((n + 127) / 128);
+  const int64_t tiles_128_64 = (int64_t)((m + 127) / 128) * ((n + 63) / 64);
+  if (tiles_128 >= 768)
+    return launch_variant<2, 2, 2, TOut>(a, w, bias, c, m, n, k, lda, ldc, epilogue, scatter, s);
+  if (tiles_128_64 >= 384)
+    return launch_variant<2, 1, 2, TOut>(a, w, bias, c, m, n, k, lda, ldc, epilogue, scatter, s);
+  if (k >= 2048)
+    return launch_variant<1, 1, 4, TOut>(a, w, bias, c, m, n, k, lda, ldc, epilogue, scatter, s);
+  return launch_variant<1, 1, 2, TOut>(a, w, bias, c, m, n, k, lda, ldc, epilogue, scatter, s);
+}
+
+int ps_gemm_nt_bf16_tiled(const void* a, const void* w, const float* bias, void* c, int m, int n,
+                          int k, int lda, int ldc, int c_dtype, int epilogue,
+                          const KvScatter& scatter, hipStream_t s) {
+  if (c_dtype == PS_F32)
+    return launch_tiled_bf16<float>(a, w, bias, c, m, n, k, lda, ldc, epilogue, scatter, s);
+  return launch_tiled_bf16<bf16_t>(a, w, bias, c, m, n, k, lda, ldc, epilogue, scatter, s);
+}

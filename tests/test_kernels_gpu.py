@@ -100,7 +100,10 @@ def test_rmsnorm():
 # not multiples of 8 and fall to the plain kernel
 GEMM_SHAPES = [(1, 50, 64), (5, 1000, 96), (64, 2304, 768), (130, 70, 320), (33, 257, 100),
                (256, 768, 3072), (2, 50257, 64), (17, 768, 768), (48, 100, 3072), (65, 192, 96),
-               (300, 1000, 320), (129, 257, 66), (8, 768, 3072), (512, 2304, 768)]
+               (300, 1000, 320), (129, 257, 66), (8, 768, 3072), (512, 2304, 768),
+               # enough tiles for the larger tile shapes of the bfloat16 tiled kernel, with whole
+               # and with ragged rows of eight columns
+               (1100, 2800, 128), (1027, 2801, 192), (3500, 3530, 64)]
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
@@ -111,6 +114,8 @@ def test_gemm_nt(dtype, m, n, k, epilogue):
 
     if epilogue != "none" and n > 5000:
         pytest.skip("one epilogue is enough at the vocabulary size")
+    if epilogue == "gelu_erf" and m > 1000:
+        pytest.skip("one activation is enough at the large shapes")
     a = _rand((m, k), dtype, 10, 1.0)
     w = _rand((n, k), dtype, 11, 1.0 / math.sqrt(k))
     bias = _rand((n,), torch.float32, 12)
@@ -527,14 +532,17 @@ def test_linear_with_pending_norm(dtype, m, n, k, epilogue, rms):
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
-@pytest.mark.parametrize("m", [1, 9, 40, 150])
-@pytest.mark.parametrize("k", [64, 100])
-def test_linear_scatters_keys_and_values(dtype, m, k):
+@pytest.mark.parametrize("m,k,geometry", [(1, 64, (4, 2, 16, 8)), (9, 64, (4, 2, 16, 8)), (40, 64, (4, 2, 16, 8)),
+                                          (150, 64, (4, 2, 16, 8)), (1, 100, (4, 2, 16, 8)), (9, 100, (4, 2, 16, 8)),
+                                          (40, 100, (4, 2, 16, 8)), (150, 100, (4, 2, 16, 8)),
+                                          (1500, 128, (12, 12, 64, 16)), (700, 64, (5, 1, 48, 12))])
+def test_linear_scatters_keys_and_values(dtype, m, k, geometry):
     """A [q | k | v] product that also stores k and v in their pages equals product + kv_write
-    (k = 100 takes the plain kernel, which scatters in a second launch)."""
+    (k = 100 takes the plain kernel, which scatters in a second launch; the large cases take
+    other tile shapes of the tiled kernel)."""
     from pagedserve_amd.ops import kernels
 
-    heads, kv_heads, head_dim, page_size = 4, 2, 16, 8
+    heads, kv_heads, head_dim, page_size = geometry
     q_cols, kv_cols = heads * head_dim, kv_heads * head_dim
     n = q_cols + 2 * kv_cols
     lens = [m // 2 + 3, m - m // 2 + 11] if m > 1 else [5]
