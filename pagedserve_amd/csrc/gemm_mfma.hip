@@ -624,12 +624,16 @@ int ps_norm_gemm_fused(const NormPrologue& norm, const void* w, const float* bia
 int ps_gemm_nt_mfma(const void* a, const void* w, const float* bias, void* c, int m, int n, int k,
                     int lda, int ldc, int dtype, int c_dtype, int epilogue,
                     const KvScatter& scatter, hipStream_t s) {
-  if (dtype == PS_BF16 && m <= 64) {
+  // Up to 64 rows the skinny kernel has every load of a block in flight at once, which counts
+  // when the weights come from memory and not from a cache; the tiled kernel walks k tile by
+  // tile and wins only where there are tiles enough to fill the chip (the output head).
+  const bool skinny_k = m <= 64 && n < 64 * 256;
+  if (dtype == PS_BF16 && m <= 64 && (skinny_k || !ps_gemm_nt_bf16_tiled_supported(a, w, m, k, lda))) {
     if (c_dtype == PS_F32)
       return launch_skinny<float>(a, w, bias, c, m, n, k, lda, ldc, epilogue, scatter, s);
     return launch_skinny<bf16_t>(a, w, bias, c, m, n, k, lda, ldc, epilogue, scatter, s);
   }
-  if (dtype == PS_BF16 && ps_gemm_nt_bf16_tiled_supported(a, w, m, k, lda))
+  if (dtype == PS_BF16 && !skinny_k && ps_gemm_nt_bf16_tiled_supported(a, w, m, k, lda))
     return ps_gemm_nt_bf16_tiled(a, w, bias, c, m, n, k, lda, ldc, c_dtype, epilogue, scatter, s);
   if (dtype == PS_F32 && c_dtype == PS_F32)
     return launch_tiled<float, float>(a, w, bias, c, m, n, k, lda, ldc, epilogue, scatter, s);

@@ -69,7 +69,7 @@ template <int WM, int WN, int STAGES, typename TOut, int EPI>
 __global__ __launch_bounds__(256) void gemm_nt_bf16_tiled_kernel(
     const bf16_t* __restrict__ a, const bf16_t* __restrict__ w, const float* __restrict__ bias,
     TOut* __restrict__ c, int m, int n, int k, int lda, int ldc, int tiles_m, int tiles_n,
-    int row_major, KvScatter scatter) {
+    int row_major, int k_splits, int k_chunk, KvScatter scatter) {
   constexpr int BM = 64 * WM, BN = 64 * WN;
   constexpr int STAGE_BYTES = (BM + BN) * TB_ROW;
   constexpr int LOADS_A = BM / 32;   // load instructions per wave and stage (8 rows each)
@@ -92,11 +92,15 @@ __global__ __launch_bounds__(256) void gemm_nt_bf16_tiled_kernel(
   const int per_xcd = blocks / 8;
   int logical = blockIdx.x;
   if (blockIdx.x < per_xcd * 8) logical = (blockIdx.x & 7) * per_xcd + (blockIdx.x >> 3);
-  const int tile_n = row_major ? logical % tiles_n : logical / tiles_m;
-  const int tile_m = row_major ? logical / tiles_n : logical % tiles_m;
+  const int tiles = tiles_m * tiles_n;
+  const int split = logical / tiles;
+  const int tile = logical - split * tiles;
+  const int tile_n = row_major ? tile % tiles_n : tile / tiles_m;
+  const int tile_m = row_major ? tile / tiles_n : tile % tiles_m;
   const int m0 = tile_m * BM;
   const int n0 = tile_n * BN;
-  const int k_tiles = k / TB_BK;
+  const int k_begin = split * k_chunk;
+  const int k_tiles = ((k_begin + k_chunk < k ? k_begin + k_chunk : k) - k_begin) / TB_BK;
 
   // ---- loads: lane l of a load instruction fills slot l % 8 of row l / 8 of its eight rows
   const bf16_t* src[LOADS];
@@ -109,11 +113,11 @@ __global__ __launch_bounds__(256) void gemm_nt_bf16_tiled_kernel(
     const int piece = (lane & 7) ^ ((tile_row >> 1) & 7);
     if (is_a) {
       const int row = m0 + tile_row < m ? m0 + tile_row : m - 1;
-      src[j] = a + (int64_t)row * lda + piece * 8;
+      src[j] = a + (int64_t)row * lda + k_begin + piece * 8;
       dst[j] = group * 8 * TB_ROW;
     } else {
       const int row = n0 + tile_row < n ? n0 + tile_row : n - 1;
-      src[j] = w + (int64_t)row * k + piece * 8;
+      src[j] = w + (int64_t)row * k + k_begin + piece * 8;
       dst[j] = (BM + group * 8) * TB_ROW;
     }
   }
@@ -192,10 +196,11 @@ __global__ __launch_bounds__(256) void gemm_nt_bf16_tiled_kernel(
   const int row_in_pass = lane / EP_CHUNKS;
   const int col0 = n0 + wave_n * WN * 32 + chunk * 8;
   const bool full = col0 + 8 <= n;
-  const bool vec_c = ldc % 8 == 0 && (reinterpret_cast<uintptr_t>(c) & 15u) == 0;
+  const bool vec_c = ldc % (16 / (int)sizeof(TOut)) == 0 && (reinterpret_cast<uintptr_t>(c) & 15u) == 0;
+  const bool by_column = !vec_c || k_splits > 1;
   float b[8];
 #pragma unroll
-  for (int q = 0; q < 8; ++q) b[q] = (bias && col0 + q < n) ? bias[col0 + q] : 0.f;
+  for (int q = 0; q < 8; ++q) b[q] = (bias && split == 0 && col0 + q < n) ? bias[col0 + q] : 0.f;
   // key and value columns also go into cache pages: eight consecutive columns lie in one head
   const bool scatters = EPI == PS_EPI_NONE && scatter.k_pool != nullptr && col0 < n &&
                         col0 + 8 > scatter.q_cols;
@@ -214,6 +219,34 @@ __global__ __launch_bounds__(256) void gemm_nt_bf16_tiled_kernel(
         region[((e >> 2) * 8 + (lane >> 5) * 4 + (e & 3)) * EP_STRIDE + j * 32 + (lane & 31)] =
             acc[i][j][e];
     asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+    if (by_column) {
+      // rows that cannot leave in aligned pieces, and partial sums of a split k: a wave's
+      // lanes take consecutive columns of one row
+#pragma unroll 8
+      for (int r = 0; r < 32; ++r) {
+        const int row = m0 + wave_m * WM * 32 + i * 32 + r;
+        if (row >= m) continue;
+#pragma unroll
+        for (int half = 0; half < (WN + 1) / 2; ++half) {
+          const int within = half * 64 + lane;
+          const int col = n0 + wave_n * WN * 32 + within;
+          if (within >= WN * 32 || col >= n) continue;
+          const float bias_here = (bias && split == 0) ? bias[col] : 0.f;
+          const float v = finish_value<EPI, TOut>(region[r * EP_STRIDE + within] + bias_here);
+          TOut* out = c + (int64_t)row * ldc + col;
+          if (EPI == PS_EPI_RESIDUAL) {
+            float* sum = reinterpret_cast<float*>(out);
+            if (k_splits > 1) unsafeAtomicAdd(sum, v);
+            else *sum += v;
+          } else {
+            *out = from_float<TOut>(v);
+            if (EPI == PS_EPI_NONE) kv_scatter_store<TOut>(scatter, row, col, v);
+          }
+        }
+      }
+      asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+      continue;
+    }
 #pragma unroll 2
     for (int pass = 0; pass < 32 / EP_ROWS; ++pass) {
       const int r = pass * EP_ROWS + row_in_pass;
@@ -227,7 +260,7 @@ __global__ __launch_bounds__(256) void gemm_nt_bf16_tiled_kernel(
       TOut* out = c + (int64_t)row * ldc + col0;
       if (EPI == PS_EPI_RESIDUAL) {
         float* sum = reinterpret_cast<float*>(out);
-        if (full && vec_c) {
+        if (full) {
           float4 o0 = *reinterpret_cast<const float4*>(sum);
           float4 o1 = *reinterpret_cast<const float4*>(sum + 4);
           o0.x += v[0]; o0.y += v[1]; o0.z += v[2]; o0.w += v[3];
@@ -240,7 +273,7 @@ __global__ __launch_bounds__(256) void gemm_nt_bf16_tiled_kernel(
         }
         continue;
       }
-      if (full && vec_c) {
+      if (full) {
         store8(out, v);
       } else {
         for (int q = 0; q < 8; ++q)
@@ -262,7 +295,7 @@ __global__ __launch_bounds__(256) void gemm_nt_bf16_tiled_kernel(
 
 // --------------------------------------------------------------------------------- host
 bool ps_gemm_nt_bf16_tiled_supported(const void* a, const void* w, int m, int k, int lda) {
-  return m > 64 && k % TB_BK == 0 && lda % 8 == 0 &&
+  return m > 32 && k % TB_BK == 0 && lda % 8 == 0 &&
          (reinterpret_cast<uintptr_t>(a) & 15u) == 0 && (reinterpret_cast<uintptr_t>(w) & 15u) == 0;
 }
 
@@ -278,11 +311,21 @@ static int launch_variant(const void* a, const void* w, const float* bias, void*
   const int64_t rows_along = (int64_t)((run + tiles_n - 1) / tiles_n) * BM + n;   // along rows of C
   const int64_t rows_down = (int64_t)((run + tiles_m - 1) / tiles_m) * BN + m;    // down columns
   const int row_major = rows_along < rows_down ? 1 : 0;
-  dim3 grid(tiles_m * tiles_n);
+  // Few tiles with a long k leave most of the chip idle: where partial sums can be added in
+  // place (residual epilogue) k is split over blocks.  Float atomics are slow, so this pays
+  // only while the output is small.
+  int k_splits = 1;
+  if (epilogue == PS_EPI_RESIDUAL && tiles_m * tiles_n <= 64 && k >= 1024) {
+    k_splits = 256 / (tiles_m * tiles_n);
+    if (k_splits > k / 256) k_splits = k / 256;
+  }
+  int k_chunk = (k / TB_BK + k_splits - 1) / k_splits * TB_BK;
+  k_splits = (k + k_chunk - 1) / k_chunk;
+  dim3 grid(tiles_m * tiles_n * k_splits);
 #define PS_LAUNCH_TB(EPI)                                                                     \
   hipLaunchKernelGGL((gemm_nt_bf16_tiled_kernel<WM, WN, STAGES, TOut, EPI>), grid, dim3(256), 0, \
                      s, (const bf16_t*)a, (const bf16_t*)w, bias, (TOut*)c, m, n, k, lda, ldc, \
-                     tiles_m, tiles_n, row_major, scatter)
+                     tiles_m, tiles_n, row_major, k_splits, k_chunk, scatter)
   switch (epilogue) {
     case PS_EPI_NONE: PS_LAUNCH_TB(PS_EPI_NONE); break;
     case PS_EPI_GELU_TANH: PS_LAUNCH_TB(PS_EPI_GELU_TANH); break;
@@ -304,9 +347,9 @@ static int launch_tiled_bf16(const void* a, const void* w, const float* bias, vo
                              const KvScatter& scatter, hipStream_t s) {
   const int64_t tiles_128 = (int64_t)((m + 127) / 128) * ((n + 127) / 128);
   const int64_t tiles_128_64 = (int64_t)((m + 127) / 128) * ((n + 63) / 64);
-  if (tiles_128 >= 768)
+  if (m > 64 && tiles_128 >= 768)
     return launch_variant<2, 2, 2, TOut>(a, w, bias, c, m, n, k, lda, ldc, epilogue, scatter, s);
-  if (tiles_128_64 >= 384)
+  if (m > 64 && tiles_128_64 >= 384)
     return launch_variant<2, 1, 2, TOut>(a, w, bias, c, m, n, k, lda, ldc, epilogue, scatter, s);
   if (k >= 2048)
     return launch_variant<1, 1, 4, TOut>(a, w, bias, c, m, n, k, lda, ldc, epilogue, scatter, s);

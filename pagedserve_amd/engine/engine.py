@@ -116,8 +116,11 @@ class Engine:
     def _logit_buffer(self, rows: int) -> torch.Tensor:
         if self._logits is None or self._logits.shape[0] < rows:
             capacity = max(rows, min(self.max_requests, 64))
-            self._logits = torch.empty((capacity, self.spec.vocab_size), dtype=torch.float32,
-                                       device=self.device)
+            # rows start at multiples of 32 bytes, so that kernels store them in aligned pieces
+            vocab = self.spec.vocab_size
+            padded = -(-vocab // 8) * 8
+            self._logits = torch.empty((capacity, padded), dtype=torch.float32,
+                                       device=self.device)[:, :vocab]
         return self._logits
 
     # ------------------------------------------------------------------- step

@@ -108,12 +108,15 @@ class Attention(Mixer):
         kernels.linear(context, self.out_weight, self.out_bias, residual, epilogue="residual")
 
     def _splits(self, count: int, max_kv_len: int):
-        """(ranges per request, waves per block).  With enough (token, head) pairs and long
-        contexts one block of 16 waves takes a whole request's keys and no second launch is
-        needed to merge ranges; few pairs are cut into ranges so that the chip is filled,
-        never into more than the keys of the longest request can feed."""
+        """(ranges per request, waves per block).  Many (token, head) pairs fill the chip with
+        one block of 4 waves each; with fewer pairs and long contexts one block of 16 waves
+        takes a whole request's keys, so that no second launch is needed to merge ranges; few
+        pairs are cut into ranges so that the chip is filled, never into more than the keys
+        of the longest request can feed."""
         visible = max_kv_len if self.window <= 0 else min(max_kv_len, self.window)
         pairs = count * self.heads
+        if pairs >= 384:
+            return 1, 4
         if pairs >= 64 and visible > kernels.decode_keys_per_block(self.head_dim, 4):
             return 1, 16
         most = max(1, -(-visible // kernels.decode_keys_per_block(self.head_dim, 4)))
