@@ -37,12 +37,21 @@ extern "C" int ps_device_info(int* compute_units, int* lds_bytes, char* arch, in
 
 // ---------------------------------------------------------------- embedding
 // h0[t] = wte[id[t]] + wpe[pos[t]]  (reference: src/model/paged_decoder.py:306-314).
+// The id of token t is ids[t], or carried[src[t]] where src[t] >= 0: a token that an earlier
+// step chose on the device and that the host has not seen yet.
 template <typename T>
 __global__ void embed_kernel(const T* __restrict__ table, const T* __restrict__ pos_table,
-                             const int* __restrict__ ids, const int* __restrict__ positions,
-                             float* __restrict__ out, int width) {
+                             const int* __restrict__ ids, const int* __restrict__ src,
+                             const int* __restrict__ carried, const int* __restrict__ positions,
+                             float* __restrict__ out, int width, int vocab) {
   const int t = blockIdx.x;
-  const T* row = table + (int64_t)ids[t] * width;
+  int id = ids[t];
+  if (src != nullptr) {
+    const int from = src[t];
+    if (from >= 0) id = carried[from];
+  }
+  id = id < 0 ? 0 : (id >= vocab ? vocab - 1 : id);   // never a read outside the table
+  const T* row = table + (int64_t)id * width;
   float* dst = out + (int64_t)t * width;
   if (pos_table != nullptr) {
     const T* prow = pos_table + (int64_t)positions[t] * width;
@@ -53,22 +62,24 @@ __global__ void embed_kernel(const T* __restrict__ table, const T* __restrict__ 
   }
 }
 
-extern "C" int ps_embed(const void* table, const void* pos_table, const int* ids,
-                        const int* positions, float* out, int tokens, int width, int vocab,
-                        int max_positions, int dtype, void* stream) {
+extern "C" int ps_embed(const void* table, const void* pos_table, const int* ids, const int* src,
+                        const int* carried, const int* positions, float* out, int tokens,
+                        int width, int vocab, int max_positions, int dtype, void* stream) {
   PS_REQUIRE(tokens >= 0 && width > 0 && vocab > 0, "ps_embed: bad sizes (tokens %d, width %d)",
              tokens, width);
   PS_REQUIRE(dtype == PS_F32 || dtype == PS_BF16, "ps_embed: unknown dtype %d", dtype);
   PS_REQUIRE(pos_table == nullptr || max_positions > 0, "ps_embed: position table without rows");
+  PS_REQUIRE(src == nullptr || carried != nullptr, "ps_embed: carried tokens are missing");
   if (tokens == 0) return 0;
   const int threads = width >= 256 ? 256 : 64;
   hipStream_t s = (hipStream_t)stream;
   if (dtype == PS_F32)
     hipLaunchKernelGGL(embed_kernel<float>, dim3(tokens), dim3(threads), 0, s, (const float*)table,
-                       (const float*)pos_table, ids, positions, out, width);
+                       (const float*)pos_table, ids, src, carried, positions, out, width, vocab);
   else
     hipLaunchKernelGGL(embed_kernel<bf16_t>, dim3(tokens), dim3(threads), 0, s,
-                       (const bf16_t*)table, (const bf16_t*)pos_table, ids, positions, out, width);
+                       (const bf16_t*)table, (const bf16_t*)pos_table, ids, src, carried,
+                       positions, out, width, vocab);
   PS_CHECK_LAUNCH("ps_embed");
   return 0;
 }

@@ -20,10 +20,11 @@ extern "C" {
 const char* ps_last_error(void);
 int ps_device_info(int* compute_units, int* lds_bytes, char* arch, int arch_len);
 
-// out[t, :] = table[ids[t], :] + (pos_table ? pos_table[positions[t], :] : 0), in float.
-int ps_embed(const void* table, const void* pos_table, const int* ids, const int* positions,
-             float* out, int tokens, int width, int vocab, int max_positions, int dtype,
-             void* stream);
+// out[t, :] = table[id(t), :] + (pos_table ? pos_table[positions[t], :] : 0), in float, where
+// id(t) = ids[t], or carried[src[t]] if src is given and src[t] >= 0.
+int ps_embed(const void* table, const void* pos_table, const int* ids, const int* src,
+             const int* carried, const int* positions, float* out, int tokens, int width,
+             int vocab, int max_positions, int dtype, void* stream);
 
 // out[r, :] = norm(x[rows ? rows[r] : r, :]) * gamma (+ beta).  rms != 0: no mean, no beta.
 int ps_norm(const float* x, const int* rows, const float* gamma, const float* beta, void* out,

@@ -31,6 +31,9 @@ class StepEntry:
     request_id: Hashable
     tokens: Sequence[int]
     want: Sequence[int] = field(default_factory=list)
+    # The one token of this entry is not known to the host yet: it is the token that the last
+    # step (a greedy one) chose for its row ``carry``.  ``tokens`` then holds a placeholder.
+    carry: Optional[int] = None
 
 
 @dataclass
@@ -38,6 +41,17 @@ class StepOutput:
     logits: torch.Tensor            # float32 [wanted, vocab]; valid until the next step
     rows: List[tuple]               # (request_id, position) of each row
     tokens: Optional[torch.Tensor] = None   # int32 [wanted]: argmax of each row, if asked for
+    # a copy of ``tokens`` in pinned host memory, complete once ``ready`` has happened; it is
+    # overwritten by the second next greedy step
+    host_tokens: Optional[torch.Tensor] = None
+    ready: Optional[torch.cuda.Event] = None
+
+    def token_list(self) -> List[int]:
+        """The chosen tokens on the host (waits for this step only, not for later ones)."""
+        if self.host_tokens is not None:
+            self.ready.synchronize()
+            return self.host_tokens.tolist()
+        return self.tokens.tolist()
 
 
 class _ReplayPlan:
@@ -76,7 +90,7 @@ class Engine:
         self.views = model.cache_views(self.cache)
         self.workspace = Workspace(max_step_tokens, self.device)
         self.table_width = -(-self.spec.max_positions // page_size)
-        capacity = (6 * max_step_tokens + 5 * max_requests + 1
+        capacity = (7 * max_step_tokens + 5 * max_requests + 1
                     + len(groups) * max_requests * self.table_width + 16)
         self._meta_device = torch.empty(capacity, dtype=torch.int32, device=self.device)
         self._meta_host = [torch.empty(capacity, dtype=torch.int32, pin_memory=True) for _ in range(2)]
@@ -86,6 +100,11 @@ class Engine:
         self._meta_turn = 0
         self._logits = None
         self._tokens = torch.zeros(max(max_requests, 64), dtype=torch.int32, device=self.device)
+        self._tokens_host = [torch.zeros(max(max_requests, 64), dtype=torch.int32, pin_memory=True)
+                             for _ in range(2)]
+        self._tokens_ready = [torch.cuda.Event(), torch.cuda.Event()]
+        self._tokens_turn = 0
+        self._carried_rows = 0    # rows of the last step whose chosen tokens a step may carry on
         # The engine's work runs on a stream of its own (default priority): a capture cannot
         # record from the default stream.
         self.stream = torch.cuda.Stream(device=self.device)
@@ -142,6 +161,9 @@ class Engine:
             if min(entry.tokens) < 0 or max(entry.tokens) >= vocab:
                 raise StepError(f"a token of request {entry.request_id!r} is outside "
                                 f"the vocabulary of {vocab}")
+            if entry.carry is not None and (count != 1 or not 0 <= entry.carry < self._carried_rows):
+                raise StepError(f"request {entry.request_id!r} carries on row {entry.carry} of the "
+                                f"last step, which chose {self._carried_rows} tokens")
             if entry.want and (min(entry.want) < 0 or max(entry.want) >= count):
                 raise StepError(f"request {entry.request_id!r} wants logits at place "
                                 f"{max(entry.want)} of {count} tokens")
@@ -211,7 +233,8 @@ class Engine:
         width = self.table_width
         offsets = {}
         cursor = 0
-        for name, size in (("token_ids", tokens), ("positions", tokens), ("tok_item", tokens),
+        for name, size in (("token_ids", tokens), ("token_src", tokens), ("positions", tokens),
+                           ("tok_item", tokens),
                            ("cu_tokens", items + 1), ("kv_lens", items), ("slots", items),
                            ("rows", wanted), ("single_tokens", singles),
                            ("portion_tokens", tokens - singles), ("tile_item", tiles),
@@ -236,11 +259,14 @@ class Engine:
         starts = [record.length for record in records]
         slot_list = [record.slot for record in records]
         section("slots")[:] = slot_list
+        token_src = section("token_src")
+        token_src[:] = -1
         step_items = []
         row_keys = []
         if tokens == items:
             # every item brings one token: no per-item loops over numpy slices
             section("token_ids")[:] = [entry.tokens[0] for entry in entries]
+            token_src[:] = [-1 if entry.carry is None else entry.carry for entry in entries]
             section("positions")[:] = starts
             index = np.arange(items + 1, dtype=np.int32)
             section("tok_item")[:] = index[:items]
@@ -265,6 +291,8 @@ class Engine:
             flat = row_cursor = single_cursor = portion_cursor = max_kv = tile_cursor = 0
             for index, (entry, record, start, count) in enumerate(zip(entries, records, starts, counts)):
                 token_ids[flat:flat + count] = entry.tokens
+                if entry.carry is not None:
+                    token_src[flat] = entry.carry
                 positions[flat:flat + count] = np.arange(start, start + count, dtype=np.int32)
                 tok_item[flat:flat + count] = index
                 cu[index] = flat
@@ -310,7 +338,8 @@ class Engine:
             decode_only=singles == items, max_kv_len=max_kv,
             single_tokens=view("single_tokens"), portion_tokens=view("portion_tokens"),
             max_positions=self.spec.max_positions,
-            tile_item=view("tile_item"), tile_q0=view("tile_q0"))
+            tile_item=view("tile_item"), tile_q0=view("tile_q0"),
+            token_src=view("token_src"), carried_tokens=self._tokens)
         return ctx, view("rows"), row_keys
 
     def _forward(self, ctx, rows, logits, wanted, greedy):
@@ -323,6 +352,22 @@ class Engine:
         return out, tokens
 
     def _run(self, entries, greedy=False) -> StepOutput:
+        output = self._run_step(entries, greedy)
+        if output.tokens is not None:
+            # the chosen tokens go to the host behind the step, without holding up the next one
+            turn = self._tokens_turn
+            self._tokens_turn ^= 1
+            rows = output.tokens.numel()
+            output.host_tokens = self._tokens_host[turn][:rows]
+            output.host_tokens.copy_(output.tokens, non_blocking=True)
+            output.ready = self._tokens_ready[turn]
+            output.ready.record()
+            self._carried_rows = rows
+        else:
+            self._carried_rows = 0
+        return output
+
+    def _run_step(self, entries, greedy=False) -> StepOutput:
         items = len(entries)
         if self.use_graphs and self._graphs:
             # a captured step: every entry brings one token and wants its logits
@@ -398,6 +443,7 @@ class Engine:
         starts = [record.length for record in records]
         slots = [record.slot for record in records]
         sections["token_ids"][:] = [entry.tokens[0] for entry in entries]
+        sections["token_src"][:] = [-1 if entry.carry is None else entry.carry for entry in entries]
         sections["positions"][:] = starts
         sections["kv_lens"][:] = [start + 1 for start in starts]
         sections["slots"][:] = slots

@@ -22,6 +22,14 @@ requests have reserved (``:119-122,138-142``); otherwise it and everything behin
 (first come, first served).  So a running request never fails for lack of pages, and
 nothing is preempted.  A request whose worst case exceeds the whole pool is refused when
 it is added.
+
+**Running ahead.**  While every running request decodes greedily and nobody waits, the
+iteration after the current one is launched before the current one's tokens have reached
+the host: its entries say "the token that the last step chose for row r" instead of a token
+id, and the host's work for an iteration overlaps the GPU's work for the next.  A request
+that ends by length is known beforehand and left out; one that ends at the end token has one
+token too many computed, which is dropped.  The tokens that a request receives are the same
+either way.
 """
 
 from collections import deque
@@ -55,11 +63,22 @@ class RequestState:
         return self.pending_token_id is None
 
 
+@dataclass
+class _Pending:
+    """An iteration that runs on the GPU and whose tokens the host has not read yet."""
+
+    selected: list            # (request, number of tokens)
+    entries: list
+    producers: list           # requests that receive a token from it, in row order
+    output: object
+    can_carry: bool           # greedy single-token rows: the next iteration may carry them on
+
+
 class ContinuousBatchScheduler:
     def __init__(self, engine, sampler, tokenizer=None, max_batch_size: int = 32,
                  eos_token_id=None, scheduling_strategy: str = ORCA_STRATEGY,
                  prefill_chunk_size: int = 16, max_num_batched_tokens: Optional[int] = None,
-                 max_prefill_requests: Optional[int] = None):
+                 max_prefill_requests: Optional[int] = None, run_ahead: bool = True):
         if max_batch_size <= 0:
             raise ValueError("max_batch_size must be positive")
         if scheduling_strategy not in SUPPORTED_SCHEDULING_STRATEGIES:
@@ -96,6 +115,9 @@ class ContinuousBatchScheduler:
         self.next_request_id = 0
         self.reserved_blocks = [0] * len(engine.cache.groups)
         self.iterations = 0
+        self.run_ahead = run_ahead
+        self.steps_run_ahead = 0
+        self._inflight = None       # a launched iteration whose tokens the host has not read
 
     # ------------------------------------------------------------- admission
     def add_request(self, prompt, max_new_tokens=200, sampling: Optional[SamplingParams] = None):
@@ -251,11 +273,22 @@ class ContinuousBatchScheduler:
             torch.cuda.set_stream(previous)
 
     def _step(self) -> Dict[int, int]:
+        pending = self._inflight
+        self._inflight = None
+        if pending is None:
+            pending = self._launch()
+            if pending is None:
+                return {}
+        self._inflight = self._launch_ahead(pending)
+        return self._resolve(pending)
+
+    def _launch(self) -> Optional["_Pending"]:
+        """Select, reserve, and start one iteration on the GPU."""
         selected = self.select_requests()
         if not selected:
             if self.waiting or self.active:
                 raise RuntimeError("No request can be scheduled with the available KV memory")
-            return {}
+            return None
         new_requests = [request for request, _ in selected if not request.reserved_blocks]
         for request in new_requests:
             request.reserved_blocks = self._required_blocks(request)
@@ -274,10 +307,42 @@ class ContinuousBatchScheduler:
                     self.reserved_blocks[g] -= pages
                 request.reserved_blocks = []
             raise
+        decode_only = all(not request.is_prefilling for request, _ in selected)
+        return _Pending(selected, entries, producers, output, greedy and decode_only)
+
+    def _launch_ahead(self, pending) -> Optional["_Pending"]:
+        """Start the iteration after ``pending`` before ``pending``'s tokens are known, if
+        it is certain which requests it holds: all of ``pending``'s that do not end by
+        length, each carrying on the token that ``pending`` chooses for it."""
+        if (not self.run_ahead or not pending.can_carry or self.waiting
+                or getattr(pending.output, "host_tokens", None) is None
+                or len(self.active) != len(pending.selected)):
+            return None
+        selected, entries = [], []
+        for row, (request, _) in enumerate(pending.selected):
+            if request.finish_reason is not None:
+                continue      # ended at the end token while ``pending`` was already running
+            if len(request.generated_token_ids) + 2 > request.max_new_tokens:
+                continue      # ``pending`` brings its last token
+            selected.append((request, 1))
+            entries.append(StepEntry(request.request_id, [0], [0], carry=row))
+        if not selected:
+            return None
+        try:
+            output = self.engine.step(entries, greedy=True)
+        except ValueError:
+            return None       # the ordinary launch of the next iteration reports it
+        self.steps_run_ahead += 1
+        return _Pending(selected, entries, [request for request, _ in selected], output, True)
+
+    def _resolve(self, pending) -> Dict[int, int]:
+        """Read the tokens of a launched iteration and move its requests on."""
+        selected, entries, producers, output = (pending.selected, pending.entries,
+                                                pending.producers, pending.output)
         if output.logits.shape[0] != len(producers):
             raise RuntimeError("the engine returned a wrong number of logits rows")
         if getattr(output, "tokens", None) is not None:
-            tokens = output.tokens.tolist()
+            tokens = output.token_list() if hasattr(output, "token_list") else output.tokens.tolist()
         else:
             tokens = self.sampler.sample(
                 output.logits, [r.sampling for r in producers], [r.request_id for r in producers],
@@ -286,6 +351,11 @@ class ContinuousBatchScheduler:
         completed_prefill = set()
         next_token = iter(tokens)
         for (request, size), entry in zip(selected, entries):
+            if request.finish_reason is not None:
+                # ended at the end token after this iteration had been launched ahead: the
+                # token computed for it here is dropped
+                next(next_token)
+                continue
             if request.is_prefilling:
                 request.prefill_cursor += size
                 if request.prefill_cursor < len(request.prompt_token_ids):
@@ -317,10 +387,10 @@ class ContinuousBatchScheduler:
         return emitted
 
     def has_work(self) -> bool:
-        return bool(self.waiting or self.active)
+        return bool(self.waiting or self.active or self._inflight is not None)
 
     def run_until_complete(self):
-        while self.waiting or self.active:
+        while self.has_work():
             self.step()
         if self.tokenizer is None:
             return {rid: list(r.generated_token_ids) for rid, r in self.finished.items()}

@@ -124,7 +124,7 @@ class DecoderModel:
         tokens = ctx.tokens
         h = ctx.workspace.rows("residual", self.spec.width, torch.float32)[:tokens]
         kernels.embed(self.embedding_table, self.position.embedding_table(), ctx.token_ids,
-                      ctx.positions, h)
+                      ctx.positions, h, token_src=ctx.token_src, carried=ctx.carried_tokens)
         for call, view in zip(self.spec.schedule, views):
             self.blocks[call.block].forward(h, ctx, view)
         wanted = logit_rows.numel()

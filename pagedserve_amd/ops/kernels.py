@@ -20,8 +20,8 @@ EPILOGUES = {"none": 0, "gelu_tanh": 1, "gelu_erf": 2, "residual": 3}
 _DTYPE_CODE = {torch.float32: F32, torch.bfloat16: BF16}
 
 _SIGNATURES = {
-    "ps_embed": [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int,
-                 c_int, c_void_p],
+    "ps_embed": [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int,
+                 c_int, c_int, c_int, c_int, c_void_p],
     "ps_norm": [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_float, c_int,
                 c_int, c_void_p],
     "ps_gemm_nt": [c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int,
@@ -101,8 +101,10 @@ def _ptr(tensor):
     return 0 if tensor is None else tensor.data_ptr()
 
 
-def embed(table, pos_table, ids, positions, out):
-    """out[t] = table[ids[t]] + pos_table[positions[t]] as float (pos_table may be None)."""
+def embed(table, pos_table, ids, positions, out, token_src=None, carried=None):
+    """out[t] = table[id(t)] + pos_table[positions[t]] as float (pos_table may be None).
+    id(t) is ``ids[t]``, or ``carried[token_src[t]]`` where ``token_src[t] >= 0``: a token
+    that an earlier step chose on the device."""
     _check(table, "table", ndim=2)
     _check(ids, "ids", torch.int32, 1)
     _check(out, "out", torch.float32, 2)
@@ -121,7 +123,13 @@ def embed(table, pos_table, ids, positions, out):
         if positions.numel() != tokens or not positions.is_contiguous():
             raise KernelError("embed: one position per token is needed")
         max_positions = pos_table.shape[0]
-    _call("ps_embed", table.data_ptr(), _ptr(pos_table), ids.data_ptr(),
+    if token_src is not None:
+        _check(token_src, "token_src", torch.int32, 1)
+        _check(carried, "carried", torch.int32, 1)
+        if token_src.numel() != tokens or not token_src.is_contiguous() or not carried.is_contiguous():
+            raise KernelError("embed: one source index per token is needed")
+    _call("ps_embed", table.data_ptr(), _ptr(pos_table), ids.data_ptr(), _ptr(token_src),
+          _ptr(carried if token_src is not None else None),
           _ptr(positions if pos_table is not None else None), out.data_ptr(), tokens, width,
           table.shape[0], max_positions, dtype_code(table.dtype), _stream())
     return out

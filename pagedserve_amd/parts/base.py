@@ -179,4 +179,6 @@ class StepContext:
     max_positions: int = 0
     tile_item: Optional[torch.Tensor] = None       # int32: item of each 64-query tile
     tile_q0: Optional[torch.Tensor] = None         # int32: first query of the tile in its item
+    token_src: Optional[torch.Tensor] = None       # int32 [T]: >= 0: the token is carried_tokens[src]
+    carried_tokens: Optional[torch.Tensor] = None  # int32: tokens that the last step chose
     extra: Optional[dict] = None

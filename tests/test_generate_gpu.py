@@ -54,6 +54,50 @@ def test_greedy_generation_matches_plain(folders, which):
     assert sum(a == e[0] for a, e in zip(first, expected)) >= len(prompts) - 1
 
 
+def test_running_ahead_gives_the_same_tokens_and_stops_at_the_end_token(folders):
+    """Iterations launched before the last one's tokens reached the host change nothing: with
+    an end token that some requests meet on the way and different lengths, every request gets
+    the tokens of the step-by-step run, and the extra token computed for a request that has
+    just ended is dropped."""
+    from pagedserve_amd.engine import ContinuousBatchScheduler, Engine
+    from pagedserve_amd.model import load_model
+    from pagedserve_amd.sampling import Sampler, SamplingParams
+
+    folder, config, page_size = folders["A"]
+    prompts = [helpers.random_tokens(n, config["vocab_size"], 900 + i) for i, n in enumerate([5, 9, 17, 3])]
+    budgets = [40, 23, 31, 12]
+    raw, weights = plain_gpt2.read_model_folder(folder)
+    free_run = [plain_gpt2.greedy_generate(raw, weights, prompt, budget) for prompt, budget in zip(prompts, budgets)]
+    # an end token that the first request produces somewhere in the middle
+    end_token = free_run[0][len(free_run[0]) // 2]
+    expected = []
+    for tokens in free_run:
+        cut = tokens.index(end_token) + 1 if end_token in tokens else len(tokens)
+        expected.append(tokens[:cut])
+    assert any(len(e) < len(f) for e, f in zip(expected, free_run))
+    model, _ = load_model(folder, dtype="float32")
+    results = {}
+    for run_ahead in (False, True):
+        engine = Engine(model, num_pages=64, page_size=page_size, max_requests=4, max_step_tokens=64)
+        scheduler = ContinuousBatchScheduler(engine, Sampler(engine.device, 4), max_batch_size=4,
+                                             eos_token_id=end_token, run_ahead=run_ahead)
+        ids = [scheduler.add_token_request(prompt, budget, sampling=SamplingParams(max_new_tokens=budget))
+               for prompt, budget in zip(prompts, budgets)]
+        streamed = {rid: [] for rid in ids}
+        while scheduler.has_work():
+            for rid, token in scheduler.step().items():
+                streamed[rid].append(token)
+        got = [scheduler.finished[rid].generated_token_ids for rid in ids]
+        assert got == expected, run_ahead
+        assert [streamed[rid] for rid in ids] == expected
+        reasons = [scheduler.finished[rid].finish_reason for rid in ids]
+        assert reasons == ["stop" if e[-1] == end_token else "length" for e in expected]
+        engine.cache.check_invariants()
+        assert not engine.cache.requests and scheduler.reserved_blocks == [0]
+        results[run_ahead] = scheduler.steps_run_ahead
+    assert results[False] == 0 and results[True] > 10
+
+
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 def test_long_decoding(folders, dtype):
     """Two prompt tokens, then 250 tokens decoded one by one up to the last position."""
