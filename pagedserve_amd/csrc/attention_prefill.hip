@@ -1,40 +1,58 @@
 // Tiled paged attention for prompt portions on the matrix cores (bfloat16).
 //
-// One 256-thread block per (tile of 64 queries of one request, head); each of the four waves
-// owns 16 consecutive queries.  Keys and values are visited 64 at a time through the request's
-// block table, from the first key any query of the tile may see to the tile's last position
-// (the portion's own keys are already in the pages, so a whole prompt, a later portion and a
-// portion that starts in the middle of a page are one case).  Per key tile:
+// One block per (tile of 64 queries of one request, head).  Its 2 KS waves are arranged as
+// 2 x KS: a wave owns 32 consecutive queries and every KS-th run of 32 keys, with an
+// online-softmax state of its own; the KS states of a query are merged through LDS at the end.
+// A request's longest tile decides how long the launch takes, and splitting its keys over
+// waves shortens exactly that.  Keys and values are visited 32 KS at a time through the
+// request's block table, from the first key any query of the tile may see to the tile's last
+// position (the portion's own keys are already in the pages, so a whole prompt, a later
+// portion and a portion that starts in the middle of a page are one case).
 //
-//   * all threads copy the K tile [64 keys][head_dim] into LDS as it lies in the pages, and
-//     the V tile transposed to [head_dim][64 keys], so that both products find their reduction
-//     dimension contiguous;
-//   * S^T = K Q^T with v_mfma_f32_16x16x32_bf16: keys are the rows, queries the columns, so a
-//     lane ends up with 4 keys x its own query per 16-key block — the same (query, key-group)
-//     ownership that the second product needs for its column operand;
-//   * scale, causal/window mask, online softmax in float per query (running max and sum, as
-//     src/kernels/triton_paged_attention.py:275-331), probabilities rounded to bfloat16;
-//   * O^T += V^T P^T with the same instruction: head dimensions are the rows, queries the
-//     columns, 32 keys per instruction.
+// Loads.  The rows of the block table that the tile needs are copied into LDS once.  K and V
+// tiles then go from the pages straight into LDS (global_load_lds_dwordx4), several tiles
+// ahead of the one being multiplied, into a ring of stages; a tile lies there as in the
+// pages, [64 keys][head_dim], with the 16-byte pieces of a row rotated by the key's number
+// so that the operand reads below spread over the LDS banks.  Per tile there is one wait
+// (own loads of that tile have landed) and one barrier.
 //
-// head_dim is any multiple of 16 up to 128 (odd multiples are zero-padded to 32 for the first
-// product); other sizes run on the row-wise kernel.
+// Per key tile and wave:
+//   * S^T = K Q^T with v_mfma_f32_32x32x16_bf16: keys are the rows, queries the columns, so
+//     a lane holds 16 keys of its own query per block of 32 keys;
+//   * scale, causal/window mask (skipped where the whole tile is visible), online softmax in
+//     float per query (running max and sum, as src/kernels/triton_paged_attention.py:275-331)
+//     in units of log 2, probabilities rounded to bfloat16;
+//   * O^T += V^T P^T with the same instruction: head dimensions are the rows.  The row operand
+//     needs, per lane, consecutive keys of one head dimension, which ds_read_b64_tr_b16
+//     delivers from the row-major tile: within 16 lanes, lane r points at 4 dimensions of key
+//     r / 4 and receives dimension r of four keys.
+//
+// head_dim is any multiple of 16 up to 128; other sizes, and block tables wider than
+// AP_TABLE_MAX pages, run on the row-wise kernel.
 #include <math.h>
 
 #include "common.h"
 #include "pagedserve_hip.h"
 
 typedef __attribute__((__vector_size__(8 * sizeof(__bf16)))) __bf16 bf16x8;
-typedef __attribute__((__vector_size__(4 * sizeof(float)))) float f32x4;
+typedef __attribute__((__vector_size__(16 * sizeof(float)))) float f32x16;
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
 
-#define AP_KEYS 64      // keys per tile
-#define AP_QUERIES 64   // queries per block
-#define AP_V_STRIDE (AP_KEYS * 2 + 16)
+#define AP_QUERIES 64      // queries per block
+#define AP_KS 2             // waves along the keys
+#define AP_TABLE_MAX 2048  // block-table entries that a tile may need
 
-__device__ inline uint32_t pack_bf16(float lo, float hi) { return pack2_bf16(lo, hi); }
+typedef const __attribute__((address_space(1))) void* ap_global_ptr;
+typedef __attribute__((address_space(3))) void* ap_lds_ptr;
 
-template <int NDB>  // head_dim / 16
-__global__ __launch_bounds__(256) void attention_prefill_kernel(
+template <int PENDING>
+__device__ inline void ap_wait_loads_and_sync() {
+  asm volatile("s_waitcnt vmcnt(%0)\n\ts_barrier" ::"n"(PENDING) : "memory");
+}
+
+template <int NDB, int KS>  // head_dim / 16; waves along the keys
+__global__ __launch_bounds__(128 * KS) void attention_prefill_kernel(
     const bf16_t* __restrict__ q, int64_t q_stride, const bf16_t* __restrict__ k_pool,
     const bf16_t* __restrict__ v_pool, bf16_t* __restrict__ out, int64_t out_stride,
     const int* __restrict__ tile_item, const int* __restrict__ tile_q0,
@@ -42,17 +60,32 @@ __global__ __launch_bounds__(256) void attention_prefill_kernel(
     const int* __restrict__ tables, int table_width, int heads, int kv_heads, int page_size,
     int page_shift, int num_pages, float scale, int window) {
   constexpr int HD = NDB * 16;
-  constexpr int NDQ = (NDB + 1) / 2;   // 32-wide steps over the head dimension
-  constexpr int HDP = NDQ * 32;
-  constexpr int K_STRIDE = HDP * 2 + 16;
-  __shared__ __attribute__((aligned(16))) unsigned char k_lds[AP_KEYS * K_STRIDE];
-  __shared__ __attribute__((aligned(16))) unsigned char v_lds[HD * AP_V_STRIDE];
+  constexpr int ROW = HD * 2;                    // bytes of one key in a tile
+  constexpr int CH = HD / 8;                     // 16-byte pieces per row
+  constexpr int SPREAD = ROW <= 256 ? 256 / ROW : 1;   // keys that share one pass over the banks
+  constexpr int AP_KEYS = 32 * KS;               // keys per tile
+  constexpr int AP_WAVES = 2 * KS;
+  constexpr int TILE_BYTES = AP_KEYS * ROW;
+  constexpr int STAGE_BYTES = 2 * TILE_BYTES;    // K tile, then V tile
+  constexpr int FIT = 98304 / STAGE_BYTES;
+  constexpr int STAGES = FIT >= 4 ? 4 : (FIT >= 2 ? FIT : 2);
+  constexpr int INSTRUCTIONS = KS * NDB;         // load instructions per operand and stage
+  // every wave issues the same number of loads (the counter of loads in flight is per wave):
+  // where they do not divide evenly the last ones are issued twice
+  constexpr int PER_OPERAND = (NDB + 1) / 2;
+  constexpr int LOADS = 2 * PER_OPERAND;
+  constexpr int NDB32 = (NDB + 1) / 2;           // blocks of 32 head dimensions
+  static_assert(LOADS * 2 < 64, "the load counter has six bits");
+  __shared__ __attribute__((aligned(1024))) unsigned char stages[STAGES * STAGE_BYTES];
+  __shared__ int s_table[AP_TABLE_MAX];
 
   const int tid = threadIdx.x;
   const int lane = tid & 63;
   const int wave = tid >> 6;
-  const int sub = lane & 15;     // query of this lane within the wave
-  const int group = lane >> 4;   // which quarter of a reduction dimension
+  const int wave_q = wave & 1;   // which 32 queries
+  const int wave_k = wave >> 1;  // which run of 32 keys of every tile
+  const int sub = lane & 31;     // query of this lane within the wave; key or dimension row
+  const int half = lane >> 5;    // which half of a step's reduction dimension
   const int head = blockIdx.y;
   const int kv_head = head / (heads / kv_heads);
 
@@ -65,204 +98,274 @@ __global__ __launch_bounds__(256) void attention_prefill_kernel(
   const int start = kv_lens[item] - count;   // position of the portion's first token
   const int* table = tables + (int64_t)item * table_width;
 
-  const int qi = q0 + wave * 16 + sub;
+  const int qi = q0 + wave_q * 32 + sub;
   const bool q_valid = qi < count;
   const int q_pos = q_valid ? start + qi : -1;
-  const int wave_first = start + q0 + wave * 16;
-  const int wave_last_q = q0 + wave * 16 + 15 < count ? q0 + wave * 16 + 15 : count - 1;
+  const int wave_first = start + q0 + wave_q * 32;
+  const int wave_last_q = q0 + wave_q * 32 + 31 < count ? q0 + wave_q * 32 + 31 : count - 1;
   const int wave_last = start + wave_last_q;
-  const bool wave_active = q0 + wave * 16 < count;
+  const bool wave_active = q0 + wave_q * 32 < count;
   const int tile_last_q = q0 + AP_QUERIES - 1 < count ? q0 + AP_QUERIES - 1 : count - 1;
   const int key_end = start + tile_last_q + 1;
   int key_begin = 0;
   if (window > 0 && start + q0 - window + 1 > 0) key_begin = start + q0 - window + 1;
 
-  // zero the padding columns of the K tile once (odd NDB)
-  if (HDP > HD) {
-    for (int i = tid; i < AP_KEYS * (HDP - HD) / 8; i += 256) {
-      const int key = i / ((HDP - HD) / 8);
-      const int chunk = i % ((HDP - HD) / 8);
-      *reinterpret_cast<uint4*>(&k_lds[key * K_STRIDE + (HD + chunk * 8) * 2]) = uint4{0u, 0u, 0u, 0u};
-    }
+  // the block-table entries of keys key_begin .. key_end - 1
+  const int first_logical = page_shift >= 0 ? (key_begin >> page_shift) : key_begin / page_size;
+  const int last_logical = page_shift >= 0 ? ((key_end - 1) >> page_shift) : (key_end - 1) / page_size;
+  for (int i = tid; i <= last_logical - first_logical && i < AP_TABLE_MAX; i += 128 * KS) {
+    const int logical = first_logical + i;
+    const int page = logical < table_width ? table[logical] : 0;
+    s_table[i] = (page >= 0 && page < num_pages) ? page : 0;   // never an address outside the pool
   }
 
-  // queries as column operand of the first product: lane (query sub, dims dq*32 + group*8 ..)
-  uint4 qf[NDQ];
+  // queries as column operand of the first product: lane (query sub, dims step*16 + half*8 ..)
+  bf16x8 qf[NDB];
 #pragma unroll
-  for (int dq = 0; dq < NDQ; ++dq) {
-    const int d = dq * 32 + group * 8;
-    qf[dq] = (q_valid && d < HD)
-                 ? *reinterpret_cast<const uint4*>(q + (int64_t)(tok0 + qi) * q_stride +
-                                                   (int64_t)head * HD + d)
-                 : uint4{0u, 0u, 0u, 0u};
+  for (int step = 0; step < NDB; ++step) {
+    const uint4 zero = {0u, 0u, 0u, 0u};
+    const uint4 raw = q_valid ? *reinterpret_cast<const uint4*>(
+                                    q + (int64_t)(tok0 + qi) * q_stride + (int64_t)head * HD +
+                                    step * 16 + half * 8)
+                              : zero;
+    qf[step] = *reinterpret_cast<const bf16x8*>(&raw);
   }
+
+  // ---- loads.  Lane l of load instruction j of an operand fills bytes j*1024 + l*16 of the
+  // tile: piece (l*16 % ROW) / 16 of key (j*1024 + l*16) / ROW, which holds the key's piece
+  // number (slot - key / SPREAD) mod CH.
+  int load_key[PER_OPERAND], load_piece[PER_OPERAND];
+#pragma unroll
+  for (int j = 0; j < PER_OPERAND; ++j) {
+    const int number = wave * PER_OPERAND + j < INSTRUCTIONS ? wave * PER_OPERAND + j : INSTRUCTIONS - 1;
+    const int offset = number * 1024 + lane * 16;
+    const int key_local = offset / ROW;
+    const int slot = (offset - key_local * ROW) / 16;
+    load_key[j] = key_local;
+    load_piece[j] = (slot + CH - (key_local / SPREAD) % CH) % CH;
+  }
+  const int64_t head_offset = (int64_t)kv_head * page_size * HD;
+  const int64_t page_elems = (int64_t)kv_heads * page_size * HD;
+  auto issue = [&](int tile_number, int k0) {
+    unsigned char* stage = stages + (tile_number % STAGES) * STAGE_BYTES;
+#pragma unroll
+    for (int j = 0; j < PER_OPERAND; ++j) {
+      // keys outside the tile's visible range are fetched from a visible key instead: they
+      // are masked below, and whatever lies in pages that were given back is never read
+      int key = k0 + load_key[j];
+      key = key < key_begin ? key_begin : (key >= key_end ? key_end - 1 : key);
+      const int logical = page_shift >= 0 ? (key >> page_shift) : key / page_size;
+      const int page = s_table[logical - first_logical];
+      const int64_t offset = (int64_t)page * page_elems + head_offset +
+                             (int64_t)(key - logical * page_size) * HD + load_piece[j] * 8;
+      const int number = wave * PER_OPERAND + j < INSTRUCTIONS ? wave * PER_OPERAND + j : INSTRUCTIONS - 1;
+      const int dst = number * 1024;
+      __builtin_amdgcn_global_load_lds((ap_global_ptr)(k_pool + offset), (ap_lds_ptr)(stage + dst),
+                                       16, 0, 0);
+      __builtin_amdgcn_global_load_lds((ap_global_ptr)(v_pool + offset),
+                                       (ap_lds_ptr)(stage + TILE_BYTES + dst), 16, 0, 0);
+    }
+  };
 
   // Scores are kept in units of log 2 (scale * log2(e) folded into one factor), so that
   // every exponential is one v_exp_f32; probabilities are rounded to bfloat16 right after.
   const float scale_log2 = scale * 1.4426950408889634f;
   float m = -INFINITY, l = 0.f;
-  f32x4 acc[NDB];
+  f32x16 acc[NDB32];
 #pragma unroll
-  for (int db = 0; db < NDB; ++db) acc[db] = f32x4{0.f, 0.f, 0.f, 0.f};
+  for (int db = 0; db < NDB32; ++db)
+#pragma unroll
+    for (int e = 0; e < 16; ++e) acc[db][e] = 0.f;
 
-  // Each thread moves CHUNKS 16-byte pieces of a K tile and of a V tile; the next tile's
-  // pieces are loaded into registers while the current tile is being multiplied.
-  constexpr int CHUNKS = (AP_KEYS * NDB * 2 + 255) / 256;
-  uint4 k_next[CHUNKS], v_next[CHUNKS];
-  int page_next[CHUNKS];
-  // The address of a key needs its page, which is a load of its own: pages are fetched one
-  // tile further ahead than keys, so neither trip to memory is waited for.
-  auto fetch_pages = [&](int k0) {
-#pragma unroll
-    for (int i = 0; i < CHUNKS; ++i) {
-      const int c = tid + i * 256;
-      const int key_local = c % AP_KEYS;
-      const int key = k0 + key_local;
-      const int safe_key = key < key_end ? key : key_end - 1;
-      const int logical = page_shift >= 0 ? (safe_key >> page_shift) : safe_key / page_size;
-      page_next[i] = logical < table_width ? table[logical] : -1;
-    }
-  };
-  auto fetch_tile = [&](int k0) {
-#pragma unroll
-    for (int i = 0; i < CHUNKS; ++i) {
-      // piece c = (8 head dimensions dc, key c % 64): the lanes of a wave hold 64 consecutive
-      // keys of the same dimensions, so the transposed V stores below do not collide in LDS
-      const int c = tid + i * 256;
-      const int dc = c / AP_KEYS;
-      const int key_local = c - dc * AP_KEYS;
-      const int key = k0 + key_local;
-      // unconditional loads from clamped addresses, zeroed afterwards
-      const int safe_key = key < key_end ? key : key_end - 1;
-      const int logical = page_shift >= 0 ? (safe_key >> page_shift) : safe_key / page_size;
-      const int page = page_next[i];
-      const bool ok = key < key_end && dc < NDB * 2 && page >= 0 && page < num_pages;
-      const int64_t offset =
-          (((int64_t)(ok ? page : 0) * kv_heads + kv_head) * page_size +
-           (safe_key - logical * page_size)) * HD + (dc < NDB * 2 ? dc : 0) * 8;
-      k_next[i] = *reinterpret_cast<const uint4*>(k_pool + offset);
-      v_next[i] = *reinterpret_cast<const uint4*>(v_pool + offset);
-      if (!ok) {
-        k_next[i] = uint4{0u, 0u, 0u, 0u};
-        v_next[i] = uint4{0u, 0u, 0u, 0u};
-      }
-    }
-  };
-  auto store_tile = [&]() {
-#pragma unroll
-    for (int i = 0; i < CHUNKS; ++i) {
-      const int c = tid + i * 256;
-      const int dc = c / AP_KEYS;
-      const int key_local = c - dc * AP_KEYS;
-      if (dc >= NDB * 2) continue;
-      *reinterpret_cast<uint4*>(&k_lds[key_local * K_STRIDE + dc * 16]) = k_next[i];
-      const uint32_t words[4] = {v_next[i].x, v_next[i].y, v_next[i].z, v_next[i].w};
-#pragma unroll
-      for (int j = 0; j < 8; ++j) {
-        const uint16_t value = (uint16_t)(words[j >> 1] >> ((j & 1) * 16));
-        *reinterpret_cast<uint16_t*>(&v_lds[(dc * 8 + j) * AP_V_STRIDE + key_local * 2]) = value;
-      }
-    }
-  };
+  // ---- operand addresses inside a tile
+  // K row operand: lane (key sub, half) reads piece 2*step + half of key wave_k*32 + sub
+  const int k_row = (wave_k * 32 + sub) * ROW;
+  const int k_turn = ((wave_k * 32 + sub) / SPREAD) % CH;
+  // V row operand through the transposing read: in the 16 lanes of group g = lane / 16, lane r
+  // points at dimensions d0 + 4 (r % 4) .. + 3 of key base + half*4 + r / 4 (+ 8 for the second
+  // read) and receives dimension d0 + r of four keys, d0 = db*32 + (g & 1) * 16.
+  const int r16 = lane & 15;
+  const int v_dim = ((lane >> 4) & 1) * 16 + 4 * (r16 & 3);   // within the block of 32 dims
+  const int v_key = wave_k * 32 + half * 4 + (r16 >> 2);       // first run of 16 keys of the wave
 
   const int k_first = key_begin / AP_KEYS * AP_KEYS;
-  fetch_pages(k_first);
-  fetch_tile(k_first);
-  if (k_first + AP_KEYS < key_end) fetch_pages(k_first + AP_KEYS);
-  for (int k0 = k_first; k0 < key_end; k0 += AP_KEYS) {
-    __syncthreads();   // the previous tile has been consumed
-    store_tile();
-    __syncthreads();
-    if (k0 + AP_KEYS < key_end) {
-      fetch_tile(k0 + AP_KEYS);   // in flight during the products
-      if (k0 + 2 * AP_KEYS < key_end) fetch_pages(k0 + 2 * AP_KEYS);
-    }
-    // skip tiles that no query of this wave can see
-    if (!wave_active || k0 > wave_last) continue;
-    if (window > 0 && k0 + AP_KEYS - 1 < wave_first - window + 1) continue;
+  const int tiles = (key_end - k_first + AP_KEYS - 1) / AP_KEYS;
+  asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)\n\ts_barrier" ::: "memory");   // the table is in LDS
+  // the queries have arrived with that; a use here keeps the compiler from waiting for them
+  // (and with them for every tile in flight) inside the loop
+#pragma unroll
+  for (int step = 0; step < NDB; ++step) asm volatile("" : "+v"(qf[step]));
+#pragma unroll
+  for (int d = 0; d < STAGES - 1; ++d)
+    if (d < tiles) issue(d, k_first + d * AP_KEYS);
 
-    // S^T: 4 blocks of 16 keys; lane holds keys kb*16 + group*4 + i of its own query
-    float s[4][4];
+  for (int t = 0; t < tiles; ++t) {
+    const int k0 = k_first + t * AP_KEYS;
+    const int ahead = tiles - 1 - t < STAGES - 2 ? tiles - 1 - t : STAGES - 2;
+    if (ahead <= 0) ap_wait_loads_and_sync<0>();
+    else if (ahead == 1) ap_wait_loads_and_sync<LOADS>();
+    else ap_wait_loads_and_sync<2 * LOADS>();
+    if (t + STAGES - 1 < tiles) issue(t + STAGES - 1, k0 + (STAGES - 1) * AP_KEYS);
+    // this wave's run of 32 keys; skip it where no query of the wave can see it
+    const int kw = k0 + wave_k * 32;
+    if (!wave_active || kw > wave_last || kw >= key_end) continue;
+    if (window > 0 && kw + 31 < wave_first - window + 1) continue;
+    const unsigned char* k_tile = stages + (t % STAGES) * STAGE_BYTES;
+    const unsigned char* v_tile = k_tile + TILE_BYTES;
+
+    // S^T: element e is key (e/4)*8 + half*4 + e%4 of the run.  The operand reads are written
+    // as assembly (see the reads of V below).
+    const uint32_t k_base = (uint32_t)(uintptr_t)(ap_lds_ptr)k_tile;
+    u32x4 kr[NDB];
+#pragma unroll
+    for (int step = 0; step < NDB; ++step) {
+      const int slot = (2 * step + half + k_turn) % CH;
+      const uint32_t address = k_base + k_row + slot * 16;
+      asm volatile("ds_read_b128 %0, %1" : "=v"(kr[step]) : "v"(address) : "memory");
+    }
+    // the transposing reads of V are issued right behind: they arrive while S is computed
+    // (as assembly: the compiler would otherwise wait for every tile in flight before each)
+    const uint32_t v_base = (uint32_t)(uintptr_t)(ap_lds_ptr)v_tile;
+    u32x2 vr[2][NDB32][2];
+#pragma unroll
+    for (int run = 0; run < 2; ++run)
+#pragma unroll
+      for (int db = 0; db < NDB32; ++db) {
+        int dim = db * 32 + v_dim;
+        if (dim >= HD) dim -= 16;       // the padded half of the last block: any valid piece
+#pragma unroll
+        for (int second = 0; second < 2; ++second) {
+          const int key_local = v_key + run * 16 + second * 8;
+          const int slot = ((dim >> 3) + (key_local / SPREAD)) % CH;
+          const uint32_t address = v_base + key_local * ROW + slot * 16 + (dim & 7) * 2;
+          asm volatile("ds_read_b64_tr_b16 %0, %1" : "=v"(vr[run][db][second]) : "v"(address) : "memory");
+        }
+      }
+    constexpr int V_READS = 4 * NDB32;
+    // LDS reads return in order: all but the reads of V have arrived
+    asm volatile("s_waitcnt lgkmcnt(%0)" ::"n"(V_READS < 15 ? V_READS : 15) : "memory");
+    f32x16 s;
+#pragma unroll
+    for (int e = 0; e < 16; ++e) s[e] = 0.f;
+#pragma unroll
+    for (int step = 0; step < NDB; ++step) {
+      asm volatile("" : "+v"(kr[step]));   // used only behind the wait
+      s = __builtin_amdgcn_mfma_f32_32x32x16_bf16(*reinterpret_cast<const bf16x8*>(&kr[step]),
+                                                qf[step], s, 0, 0, 0);
+    }
+    // the whole run is visible to every query of the wave: no mask
+    const bool masked = kw + 31 > wave_first || kw + 32 > key_end ||
+                        (window > 0 && kw < wave_last - window + 1) || !q_valid;
+    // scores stay unscaled until the exponential: p = 2^(s c - m), with m kept in scaled units
     float tile_max = -INFINITY;
+    if (__builtin_amdgcn_readfirstlane(__any(masked) ? 1 : 0)) {
 #pragma unroll
-    for (int kb = 0; kb < 4; ++kb) {
-      f32x4 sacc = {0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-      for (int dq = 0; dq < NDQ; ++dq) {
-        const uint4 kf = *reinterpret_cast<const uint4*>(
-            &k_lds[(kb * 16 + sub) * K_STRIDE + (dq * 32 + group * 8) * 2]);
-        sacc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(*reinterpret_cast<const bf16x8*>(&kf),
-                                                       *reinterpret_cast<const bf16x8*>(&qf[dq]),
-                                                       sacc, 0, 0, 0);
+      for (int e = 0; e < 16; ++e) {
+        const int key = kw + (e >> 2) * 8 + half * 4 + (e & 3);
+        const bool visible = (key <= q_pos) & (window <= 0 || q_pos - key < window);
+        s[e] = visible ? s[e] : -INFINITY;
+        tile_max = fmaxf(tile_max, s[e]);
       }
+    } else {
 #pragma unroll
-      for (int i = 0; i < 4; ++i) {
-        const int key = k0 + kb * 16 + group * 4 + i;
-        const bool visible = key <= q_pos && (window <= 0 || q_pos - key < window);
-        s[kb][i] = visible ? sacc[i] * scale_log2 : -INFINITY;
-        tile_max = fmaxf(tile_max, s[kb][i]);
-      }
+      for (int e = 0; e < 16; ++e) tile_max = fmaxf(tile_max, s[e]);
     }
-    tile_max = fmaxf(tile_max, __shfl_xor(tile_max, 16, 64));
-    tile_max = fmaxf(tile_max, __shfl_xor(tile_max, 32, 64));
+    tile_max = fmaxf(tile_max, __shfl_xor(tile_max, 32, 64)) * scale_log2;   // scale > 0
     const float m_new = fmaxf(m, tile_max);
-    if (m_new == -INFINITY) {
-      // nothing visible to this query so far; other lanes of the wave may differ, so the
-      // products below still run with zero probabilities
-    }
-    const float correction =
-        (m == -INFINITY || m_new == -INFINITY) ? 0.f : __builtin_amdgcn_exp2f(m - m_new);
+    // A query that has seen nothing yet (m_new = -inf) takes 0 as its reference: its scores
+    // are all -inf and their exponentials 0.  Other lanes of the wave may differ, so the
+    // products below run in any case.
+    const float reference = (m_new == -INFINITY) ? 0.f : m_new;
     float tile_sum = 0.f;
-    uint32_t pw[4][2];
+    uint32_t words[8];
 #pragma unroll
-    for (int kb = 0; kb < 4; ++kb) {
-      float p[4];
-#pragma unroll
-      for (int i = 0; i < 4; ++i) {
-        p[i] = (s[kb][i] == -INFINITY) ? 0.f : __builtin_amdgcn_exp2f(s[kb][i] - m_new);
-        tile_sum += p[i];
-      }
-      pw[kb][0] = pack_bf16(p[0], p[1]);
-      pw[kb][1] = pack_bf16(p[2], p[3]);
+    for (int e = 0; e < 16; e += 2) {
+      const float p0 = __builtin_amdgcn_exp2f(fmaf(s[e], scale_log2, -reference));
+      const float p1 = __builtin_amdgcn_exp2f(fmaf(s[e + 1], scale_log2, -reference));
+      tile_sum += p0 + p1;
+      words[e >> 1] = pack2_bf16(p0, p1);
     }
-    tile_sum += __shfl_xor(tile_sum, 16, 64);
+    const u32x4 p_lo = {words[0], words[1], words[2], words[3]};
+    const u32x4 p_hi = {words[4], words[5], words[6], words[7]};
     tile_sum += __shfl_xor(tile_sum, 32, 64);
-    l = l * correction + tile_sum;
-    m = m_new;
+    // the running maximum rarely moves after the first tiles: rescale only where it did
+    if (__builtin_amdgcn_readfirstlane(__any(m_new != m) ? 1 : 0)) {
+      const float correction = (m == -INFINITY) ? 0.f : __builtin_amdgcn_exp2f(m - reference);
+      l *= correction;
 #pragma unroll
-    for (int db = 0; db < NDB; ++db)
+      for (int db = 0; db < NDB32; ++db)
 #pragma unroll
-      for (int i = 0; i < 4; ++i) acc[db][i] *= correction;
+        for (int e = 0; e < 16; ++e) acc[db][e] *= correction;
+      m = m_new;
+    }
+    l += tile_sum;
 
-    // O^T += V^T P^T, 32 keys per instruction: keys {kp*32 + group*4 + i} and
-    // {kp*32 + 16 + group*4 + i}, the same eight for both operands
+    // O^T += V^T P^T, 16 keys per instruction: slots 0..3 are keys base + half*4 + 0..3,
+    // slots 4..7 keys base + 8 + half*4 + 0..3, in both operands
+    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
 #pragma unroll
-    for (int kp = 0; kp < 2; ++kp) {
-      const uint4 pf = {pw[2 * kp][0], pw[2 * kp][1], pw[2 * kp + 1][0], pw[2 * kp + 1][1]};
+    for (int run = 0; run < 2; ++run)
 #pragma unroll
-      for (int db = 0; db < NDB; ++db) {
-        const unsigned char* v_row = &v_lds[(db * 16 + sub) * AP_V_STRIDE];
-        const uint2 lo = *reinterpret_cast<const uint2*>(v_row + (kp * 32 + group * 4) * 2);
-        const uint2 hi = *reinterpret_cast<const uint2*>(v_row + (kp * 32 + 16 + group * 4) * 2);
-        const uint4 vf = {lo.x, lo.y, hi.x, hi.y};
-        acc[db] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(*reinterpret_cast<const bf16x8*>(&vf),
-                                                         *reinterpret_cast<const bf16x8*>(&pf),
-                                                         acc[db], 0, 0, 0);
+      for (int db = 0; db < NDB32; ++db) {
+        asm volatile("" : "+v"(vr[run][db][0]), "+v"(vr[run][db][1]));   // used only behind the wait
+        const u32x4 raw = {vr[run][db][0].x, vr[run][db][0].y, vr[run][db][1].x, vr[run][db][1].y};
+        acc[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(
+            *reinterpret_cast<const bf16x8*>(&raw),
+            *reinterpret_cast<const bf16x8*>(run == 0 ? &p_lo : &p_hi), acc[db], 0, 0, 0);
       }
+  }
+
+  // ---- the KS states of a query are merged by the wave with the first run of keys.  The
+  // accumulators of waves with the same queries have the same layout, so lane meets lane.
+  if (KS > 1) {
+    constexpr int STATE = NDB32 * 16 + 2;      // floats per lane
+    static_assert((AP_WAVES - 2) * 64 * STATE * 4 <= STAGES * STAGE_BYTES, "the merge reuses the stages");
+    ap_wait_loads_and_sync<0>();               // every wave is past its last operand reads
+    float* states = reinterpret_cast<float*>(stages);
+    if (wave_k > 0) {
+      float* mine = states + ((wave_k - 1) * 2 + wave_q) * 64 * STATE + lane;
+      mine[0] = m;
+      mine[64] = l;
+#pragma unroll
+      for (int db = 0; db < NDB32; ++db)
+#pragma unroll
+        for (int e = 0; e < 16; ++e) mine[(2 + db * 16 + e) * 64] = acc[db][e];
+    }
+    __syncthreads();
+    if (wave_k > 0) return;
+#pragma unroll 1
+    for (int other = 1; other < KS; ++other) {
+      const float* theirs = states + ((other - 1) * 2 + wave_q) * 64 * STATE + lane;
+      const float m_o = theirs[0];
+      const float l_o = theirs[64];
+      const float m_n = fmaxf(m, m_o);
+      const float c_mine = (m == -INFINITY) ? 0.f : __builtin_amdgcn_exp2f(m - m_n);
+      const float c_theirs = (m_o == -INFINITY) ? 0.f : __builtin_amdgcn_exp2f(m_o - m_n);
+      l = l * c_mine + l_o * c_theirs;
+      m = m_n;
+#pragma unroll
+      for (int db = 0; db < NDB32; ++db)
+#pragma unroll
+        for (int e = 0; e < 16; ++e)
+          acc[db][e] = acc[db][e] * c_mine + theirs[(2 + db * 16 + e) * 64] * c_theirs;
     }
   }
 
-  // element i of an accumulator: head dimension db*16 + group*4 + i of query `sub`
+  // element e of an accumulator: head dimension db*32 + (e/4)*8 + half*4 + e%4 of query `sub`
   if (q_valid && l > 0.f) {
     const float inv = 1.0f / l;
     bf16_t* dst = out + (int64_t)(tok0 + qi) * out_stride + (int64_t)head * HD;
 #pragma unroll
-    for (int db = 0; db < NDB; ++db) {
-      uint2 packed;
-      packed.x = pack_bf16(acc[db][0] * inv, acc[db][1] * inv);
-      packed.y = pack_bf16(acc[db][2] * inv, acc[db][3] * inv);
-      *reinterpret_cast<uint2*>(dst + db * 16 + group * 4) = packed;
-    }
+    for (int db = 0; db < NDB32; ++db)
+#pragma unroll
+      for (int quad = 0; quad < 4; ++quad) {
+        const int dim = db * 32 + quad * 8 + half * 4;
+        if (dim >= HD) continue;
+        uint2 packed;
+        packed.x = pack2_bf16(acc[db][quad * 4] * inv, acc[db][quad * 4 + 1] * inv);
+        packed.y = pack2_bf16(acc[db][quad * 4 + 2] * inv, acc[db][quad * 4 + 3] * inv);
+        *reinterpret_cast<uint2*>(dst + dim) = packed;
+      }
   }
 }
 
@@ -282,6 +385,10 @@ extern "C" int ps_attention_prefill(const void* q, int64_t q_stride, const void*
   PS_REQUIRE(head_dim > 0 && head_dim % 16 == 0 && head_dim <= 128,
              "ps_attention_prefill: head_dim %d must be a multiple of 16 up to 128", head_dim);
   PS_REQUIRE(window >= 0 && heads <= 65535, "ps_attention_prefill: bad window or head count");
+  PS_REQUIRE(scale > 0.f, "ps_attention_prefill: the score scale must be positive, got %g", scale);
+  PS_REQUIRE(table_width <= AP_TABLE_MAX,
+             "ps_attention_prefill: block tables of %d pages exceed the %d that a tile keeps",
+             table_width, AP_TABLE_MAX);
   PS_REQUIRE((q_stride % 8) == 0 && ((uintptr_t)q % 16) == 0 && (out_stride % 4) == 0 &&
                  ((uintptr_t)out % 8) == 0,
              "ps_attention_prefill: q and out rows must allow 16- and 8-byte accesses");
@@ -294,7 +401,7 @@ extern "C" int ps_attention_prefill(const void* q, int64_t q_stride, const void*
   hipStream_t s = (hipStream_t)stream;
   dim3 grid(tiles, heads);
 #define PS_LAUNCH_AP(NDB)                                                                       \
-  hipLaunchKernelGGL((attention_prefill_kernel<NDB>), grid, dim3(256), 0, s, (const bf16_t*)q,  \
+  hipLaunchKernelGGL((attention_prefill_kernel<NDB, AP_KS>), grid, dim3(128 * AP_KS), 0, s, (const bf16_t*)q,  \
                      q_stride, (const bf16_t*)k_pool, (const bf16_t*)v_pool, (bf16_t*)out,      \
                      out_stride, tile_item, tile_q0, cu_tokens, kv_lens, tables, table_width,   \
                      heads, kv_heads, page_size, page_shift, num_pages, scale, window)

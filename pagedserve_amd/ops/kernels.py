@@ -404,9 +404,14 @@ def attention_decode(q, k_pool, v_pool, out, tok_item, tok_pos, tables, heads, s
 PREFILL_TILE = 64
 
 
-def prefill_supported(dtype, head_dim) -> bool:
-    """Whether the tiled matrix-core kernel takes this storage type and head size."""
-    return dtype == torch.bfloat16 and head_dim % 16 == 0 and head_dim <= 128
+PREFILL_TABLE_MAX = 2048
+
+
+def prefill_supported(dtype, head_dim, table_width=0) -> bool:
+    """Whether the tiled matrix-core kernel takes this storage type, head size and width of
+    the block tables (it keeps a tile's table entries in LDS)."""
+    return (dtype == torch.bfloat16 and head_dim % 16 == 0 and head_dim <= 128
+            and table_width <= PREFILL_TABLE_MAX)
 
 
 def attention_prefill(q, k_pool, v_pool, out, tile_item, tile_q0, cu_tokens, kv_lens, tables,

@@ -97,7 +97,7 @@ class Attention(Mixer):
                                      ctx.positions, tables, self.heads, self.scale, splits,
                                      partial=partial, window=self.window, waves=waves,
                                      tok_list=None if singles == tokens else ctx.single_tokens)
-        if singles < tokens and kernels.prefill_supported(self.dtype, self.head_dim):
+        if singles < tokens and kernels.prefill_supported(self.dtype, self.head_dim, tables.shape[1]):
             kernels.attention_prefill(q, cache.k_pool, cache.v_pool, context, ctx.tile_item,
                                       ctx.tile_q0, ctx.cu_tokens, ctx.kv_lens, tables,
                                       self.heads, self.scale, self.window)
