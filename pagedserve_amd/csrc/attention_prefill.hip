@@ -40,7 +40,6 @@ typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
 
 #define AP_QUERIES 64      // queries per block
-#define AP_KS 2             // waves along the keys
 #define AP_TABLE_MAX 2048  // block-table entries that a tile may need
 
 typedef const __attribute__((address_space(1))) void* ap_global_ptr;
@@ -144,8 +143,11 @@ __global__ __launch_bounds__(128 * KS) void attention_prefill_kernel(
     load_key[j] = key_local;
     load_piece[j] = (slot + CH - (key_local / SPREAD) % CH) % CH;
   }
-  const int64_t head_offset = (int64_t)kv_head * page_size * HD;
+  const int head_offset = kv_head * page_size * HD;   // inside a page: fits an int
   const int64_t page_elems = (int64_t)kv_heads * page_size * HD;
+  int load_fixed[PER_OPERAND];
+#pragma unroll
+  for (int j = 0; j < PER_OPERAND; ++j) load_fixed[j] = head_offset + load_piece[j] * 8;
   auto issue = [&](int tile_number, int k0) {
     unsigned char* stage = stages + (tile_number % STAGES) * STAGE_BYTES;
 #pragma unroll
@@ -156,8 +158,8 @@ __global__ __launch_bounds__(128 * KS) void attention_prefill_kernel(
       key = key < key_begin ? key_begin : (key >= key_end ? key_end - 1 : key);
       const int logical = page_shift >= 0 ? (key >> page_shift) : key / page_size;
       const int page = s_table[logical - first_logical];
-      const int64_t offset = (int64_t)page * page_elems + head_offset +
-                             (int64_t)(key - logical * page_size) * HD + load_piece[j] * 8;
+      const int64_t offset =
+          (int64_t)page * page_elems + (load_fixed[j] + (key - logical * page_size) * HD);
       const int number = wave * PER_OPERAND + j < INSTRUCTIONS ? wave * PER_OPERAND + j : INSTRUCTIONS - 1;
       const int dst = number * 1024;
       __builtin_amdgcn_global_load_lds((ap_global_ptr)(k_pool + offset), (ap_lds_ptr)(stage + dst),
@@ -179,14 +181,36 @@ __global__ __launch_bounds__(128 * KS) void attention_prefill_kernel(
 
   // ---- operand addresses inside a tile
   // K row operand: lane (key sub, half) reads piece 2*step + half of key wave_k*32 + sub
-  const int k_row = (wave_k * 32 + sub) * ROW;
-  const int k_turn = ((wave_k * 32 + sub) / SPREAD) % CH;
+  int k_off[NDB];
+  {
+    const int key_local = wave_k * 32 + sub;
+    const int turn = (key_local / SPREAD) % CH;
+#pragma unroll
+    for (int step = 0; step < NDB; ++step)
+      k_off[step] = key_local * ROW + ((2 * step + half + turn) % CH) * 16;
+  }
   // V row operand through the transposing read: in the 16 lanes of group g = lane / 16, lane r
   // points at dimensions d0 + 4 (r % 4) .. + 3 of key base + half*4 + r / 4 (+ 8 for the second
   // read) and receives dimension d0 + r of four keys, d0 = db*32 + (g & 1) * 16.
-  const int r16 = lane & 15;
-  const int v_dim = ((lane >> 4) & 1) * 16 + 4 * (r16 & 3);   // within the block of 32 dims
-  const int v_key = wave_k * 32 + half * 4 + (r16 >> 2);       // first run of 16 keys of the wave
+  int v_off[2][NDB32][2];
+  {
+    const int r16 = lane & 15;
+    const int v_dim = ((lane >> 4) & 1) * 16 + 4 * (r16 & 3);   // within the block of 32 dims
+    const int v_key = wave_k * 32 + half * 4 + (r16 >> 2);       // first run of 16 keys of the wave
+#pragma unroll
+    for (int run = 0; run < 2; ++run)
+#pragma unroll
+      for (int db = 0; db < NDB32; ++db) {
+        int dim = db * 32 + v_dim;
+        if (dim >= HD) dim -= 16;       // the padded half of the last block: any valid piece
+#pragma unroll
+        for (int second = 0; second < 2; ++second) {
+          const int key_local = v_key + run * 16 + second * 8;
+          const int slot = ((dim >> 3) + (key_local / SPREAD)) % CH;
+          v_off[run][db][second] = TILE_BYTES + key_local * ROW + slot * 16 + (dim & 7) * 2;
+        }
+      }
+  }
 
   const int k_first = key_begin / AP_KEYS * AP_KEYS;
   const int tiles = (key_end - k_first + AP_KEYS - 1) / AP_KEYS;
@@ -210,37 +234,26 @@ __global__ __launch_bounds__(128 * KS) void attention_prefill_kernel(
     const int kw = k0 + wave_k * 32;
     if (!wave_active || kw > wave_last || kw >= key_end) continue;
     if (window > 0 && kw + 31 < wave_first - window + 1) continue;
-    const unsigned char* k_tile = stages + (t % STAGES) * STAGE_BYTES;
-    const unsigned char* v_tile = k_tile + TILE_BYTES;
-
     // S^T: element e is key (e/4)*8 + half*4 + e%4 of the run.  The operand reads are written
-    // as assembly (see the reads of V below).
-    const uint32_t k_base = (uint32_t)(uintptr_t)(ap_lds_ptr)k_tile;
+    // as assembly: the compiler would otherwise wait for every tile in flight before each.
+    // The transposing reads of V are issued right behind: they arrive while S is computed.
+    const uint32_t stage_base =
+        (uint32_t)(uintptr_t)(ap_lds_ptr)stages + (uint32_t)((t % STAGES) * STAGE_BYTES);
     u32x4 kr[NDB];
 #pragma unroll
-    for (int step = 0; step < NDB; ++step) {
-      const int slot = (2 * step + half + k_turn) % CH;
-      const uint32_t address = k_base + k_row + slot * 16;
-      asm volatile("ds_read_b128 %0, %1" : "=v"(kr[step]) : "v"(address) : "memory");
-    }
-    // the transposing reads of V are issued right behind: they arrive while S is computed
-    // (as assembly: the compiler would otherwise wait for every tile in flight before each)
-    const uint32_t v_base = (uint32_t)(uintptr_t)(ap_lds_ptr)v_tile;
+    for (int step = 0; step < NDB; ++step)
+      asm volatile("ds_read_b128 %0, %1" : "=v"(kr[step]) : "v"(stage_base + k_off[step]) : "memory");
     u32x2 vr[2][NDB32][2];
 #pragma unroll
     for (int run = 0; run < 2; ++run)
 #pragma unroll
-      for (int db = 0; db < NDB32; ++db) {
-        int dim = db * 32 + v_dim;
-        if (dim >= HD) dim -= 16;       // the padded half of the last block: any valid piece
+      for (int db = 0; db < NDB32; ++db)
 #pragma unroll
-        for (int second = 0; second < 2; ++second) {
-          const int key_local = v_key + run * 16 + second * 8;
-          const int slot = ((dim >> 3) + (key_local / SPREAD)) % CH;
-          const uint32_t address = v_base + key_local * ROW + slot * 16 + (dim & 7) * 2;
-          asm volatile("ds_read_b64_tr_b16 %0, %1" : "=v"(vr[run][db][second]) : "v"(address) : "memory");
-        }
-      }
+        for (int second = 0; second < 2; ++second)
+          asm volatile("ds_read_b64_tr_b16 %0, %1"
+                       : "=v"(vr[run][db][second])
+                       : "v"(stage_base + v_off[run][db][second])
+                       : "memory");
     constexpr int V_READS = 4 * NDB32;
     // LDS reads return in order: all but the reads of V have arrived
     asm volatile("s_waitcnt lgkmcnt(%0)" ::"n"(V_READS < 15 ? V_READS : 15) : "memory");
@@ -400,11 +413,24 @@ extern "C" int ps_attention_prefill(const void* q, int64_t q_stride, const void*
   }
   hipStream_t s = (hipStream_t)stream;
   dim3 grid(tiles, heads);
+  // With few blocks each takes a compute unit for itself, and four waves along the keys
+  // shorten the longest block; with many, smaller blocks that share a unit balance better.
+  const bool wide = (int64_t)tiles * heads <= 256;
 #define PS_LAUNCH_AP(NDB)                                                                       \
-  hipLaunchKernelGGL((attention_prefill_kernel<NDB, AP_KS>), grid, dim3(128 * AP_KS), 0, s, (const bf16_t*)q,  \
-                     q_stride, (const bf16_t*)k_pool, (const bf16_t*)v_pool, (bf16_t*)out,      \
-                     out_stride, tile_item, tile_q0, cu_tokens, kv_lens, tables, table_width,   \
-                     heads, kv_heads, page_size, page_shift, num_pages, scale, window)
+  do {                                                                                          \
+    if (wide)                                                                                   \
+      hipLaunchKernelGGL((attention_prefill_kernel<NDB, 4>), grid, dim3(512), 0, s,             \
+                         (const bf16_t*)q, q_stride, (const bf16_t*)k_pool,                     \
+                         (const bf16_t*)v_pool, (bf16_t*)out, out_stride, tile_item, tile_q0,   \
+                         cu_tokens, kv_lens, tables, table_width, heads, kv_heads, page_size,   \
+                         page_shift, num_pages, scale, window);                                 \
+    else                                                                                        \
+      hipLaunchKernelGGL((attention_prefill_kernel<NDB, 2>), grid, dim3(256), 0, s,             \
+                         (const bf16_t*)q, q_stride, (const bf16_t*)k_pool,                     \
+                         (const bf16_t*)v_pool, (bf16_t*)out, out_stride, tile_item, tile_q0,   \
+                         cu_tokens, kv_lens, tables, table_width, heads, kv_heads, page_size,   \
+                         page_shift, num_pages, scale, window);                                 \
+  } while (0)
   switch (head_dim / 16) {
     case 1: PS_LAUNCH_AP(1); break;
     case 2: PS_LAUNCH_AP(2); break;

@@ -423,7 +423,9 @@ def test_kernels_refuse_bad_sizes():
                         torch.zeros(2, 3, device="cuda"))
 
 
-@pytest.mark.parametrize("heads,kv_heads,head_dim,page_size", [(1, 1, 32, 16), (4, 4, 16, 8), (6, 2, 48, 16), (2, 2, 128, 4), (12, 12, 64, 16), (3, 1, 80, 12)])
+@pytest.mark.parametrize("heads,kv_heads,head_dim,page_size", [(1, 1, 32, 16), (4, 4, 16, 8), (6, 2, 48, 16), (2, 2, 128, 4), (12, 12, 64, 16), (3, 1, 80, 12),
+                                                                # more than 256 blocks: the kernel's other arrangement of waves
+                                                                (24, 8, 64, 16), (20, 20, 48, 8), (18, 18, 112, 16)])
 @pytest.mark.parametrize("window", [0, 37])
 def test_attention_prefill_tiles(heads, kv_heads, head_dim, page_size, window):
     """The tiled kernel against the row-wise one: fresh prompts and later portions of many
