@@ -140,6 +140,8 @@ def main(argv=None):
     parser.add_argument("--dtype", default="bfloat16", choices=("bfloat16", "float32"))
     parser.add_argument("--layers", type=int, default=None, help="fewer layers than the configuration")
     parser.add_argument("--no-points", action="store_true", help="skip batch 1 / 64 and prefill")
+    parser.add_argument("--prefill-only", action="store_true",
+                        help="only the 2,048-token prefill step, --steps times (for profiles)")
     args = parser.parse_args(argv)
     if args.gpus != 1:
         print(f"bench.py measures one GPU; --gpus {args.gpus} is not supported by this engine")
@@ -153,6 +155,14 @@ def main(argv=None):
     engine, sampler, config = _build(args.dtype, max_requests=64, max_step_tokens=PREFILL_TOKENS,
                                      layers=args.layers)
     context = config.n_positions
+    if args.prefill_only:
+        seconds = prefill_run(engine, config, reps=args.steps, warmup=min(args.warmup, 2))
+        flops = step_flops(config, [PREFILL_TOKENS // 2] * 2, 2)
+        print(json.dumps({"prefill": {
+            "value": round(PREFILL_TOKENS / seconds, 1), "tokens": PREFILL_TOKENS,
+            "ms": round(seconds * 1e3, 4),
+            "frac": round(flops / seconds / (PEAK_TFLOPS[short] * 1e12), 4)}}), flush=True)
+        return 0
     elapsed, mean_context = decode_run(engine, sampler, config, args.batch, context, args.steps,
                                        args.warmup)
     ms_per_step = elapsed / args.steps * 1e3
