@@ -3,6 +3,7 @@ and lets a call read another call's cache, and a toy mixer with state of its own
 registered, built and stepped from here without touching the framework's files."""
 
 import math
+import os
 
 import pytest
 import torch
@@ -301,3 +302,188 @@ def test_toy_mixer_with_state_of_its_own(tmp_path):
     engine.finish("a")
     again = engine.step([StepEntry("c", a, list(range(len(a))))]).logits.double().cpu()
     assert float((again - expected_a).abs().max()) <= 2e-5 * float(expected_a.abs().max())
+
+
+def test_toy_feed_forward_with_routing(tmp_path):
+    """A routed feed-forward defined here: router logits in float, the best of four experts
+    per token, its output scaled by the router's probability.  Layer 0 keeps the dense
+    feed-forward, layer 1 gets the routed one: parts are chosen layer by layer, and the
+    framework's files know nothing of this kind."""
+    import dataclasses
+
+    from pagedserve_amd.config import GPT2Config, PartSpec, resolve_architecture
+    from pagedserve_amd.engine import Engine, StepEntry
+    from pagedserve_amd.model import DecoderModel
+    from pagedserve_amd.parts import FEED_FORWARDS, FeedForward, register_feed_forward
+    from pagedserve_amd.weights import MATRIX, ParamSpec, WeightSource, load_parameters
+
+    experts = 4
+    if "toy_routed" not in FEED_FORWARDS:
+        @register_feed_forward("toy_routed")
+        class Routed(FeedForward):
+            def __init__(self, width, dtype, experts, inner):
+                self.width, self.dtype, self.experts, self.inner = width, dtype, experts, inner
+
+            def parameters(self):
+                return {"router.weight": ParamSpec((self.experts, self.width), MATRIX),
+                        "up.weight": ParamSpec((self.experts * self.inner, self.width), MATRIX),
+                        "down.weight": ParamSpec((self.width, self.experts * self.inner), MATRIX)}
+
+            def forward(self, x, residual, ctx):
+                rows = x[:ctx.tokens].float()
+                probabilities = torch.softmax(rows @ self.router_weight.float().t(), dim=-1)
+                weight, choice = probabilities.max(dim=-1)
+                for expert in range(self.experts):           # host loop: a toy, not a kernel
+                    mine = (choice == expert).nonzero().flatten()
+                    if mine.numel() == 0:
+                        continue
+                    cut = slice(expert * self.inner, (expert + 1) * self.inner)
+                    hidden = torch.nn.functional.gelu(rows[mine] @ self.up_weight[cut].float().t(),
+                                                      approximate="tanh")
+                    residual[mine] += weight[mine, None] * (hidden @ self.down_weight[:, cut].float().t())
+
+    config, page_size, seed, prefix = helpers.TINY["A"]
+    tensors = helpers.lively_tensors(config, seed)
+    generator = torch.Generator().manual_seed(77)
+    tensors["h.1.mlp.router.weight"] = torch.randn(experts, config["n_embd"], generator=generator) * 0.5
+    folder = helpers.write_folder(os.path.join(str(tmp_path), "routed"), config, tensors, prefix)
+    arch = resolve_architecture(config)
+    typed = GPT2Config.from_dict(config)
+    base = arch.build_spec(typed)
+    inner = config["n_inner"] // experts
+    routed = dataclasses.replace(base.blocks[1], feed_forward=PartSpec.make("toy_routed", experts=experts, inner=inner))
+    spec = dataclasses.replace(base, blocks=(base.blocks[0], routed))
+    model = DecoderModel(spec, torch.float32, "cuda")
+    sources = {k: v for k, v in arch.weight_sources(typed, base).items()
+               if not k.startswith("blocks.1.feed_forward.")}
+    sources["blocks.1.feed_forward.router.weight"] = WeightSource("h.1.mlp.router.weight")
+    sources["blocks.1.feed_forward.up.weight"] = WeightSource("h.1.mlp.c_fc.weight", transpose=True)
+    sources["blocks.1.feed_forward.down.weight"] = WeightSource("h.1.mlp.c_proj.weight", transpose=True)
+    loaded = load_parameters(folder, model.parameters(), sources, torch.float32, "cuda",
+                             ignorable=lambda name: name.startswith("h.1.mlp.c_") and name.endswith(".bias"))
+    model.bind(loaded)
+    engine = Engine(model, num_pages=16, page_size=page_size, max_requests=3, max_step_tokens=64)
+
+    raw, weights = P.read_model_folder(folder)
+
+    def plain(ids):
+        h = P.embed(weights["wte.weight"], weights["wpe.weight"], torch.tensor(ids), torch.arange(len(ids)))
+        h = P.block(h, weights, raw, 0)
+        eps = raw["layer_norm_epsilon"]
+        normed = P.layer_norm(h, weights["h.1.ln_1.weight"], weights["h.1.ln_1.bias"], eps)
+        h = h + P.attention_sublayer(normed, weights, "h.1.", raw["n_head"], P.attention_scale(raw, 1))
+        normed = P.layer_norm(h, weights["h.1.ln_2.weight"], weights["h.1.ln_2.bias"], eps)
+        probabilities = torch.softmax(normed @ weights["h.1.mlp.router.weight"].t(), dim=-1)
+        out = torch.zeros_like(h)
+        for t in range(len(ids)):
+            e = int(probabilities[t].argmax())
+            cut = slice(e * inner, (e + 1) * inner)
+            hidden = P.gelu_tanh(normed[t] @ weights["h.1.mlp.c_fc.weight"][:, cut])
+            out[t] = probabilities[t, e] * (hidden @ weights["h.1.mlp.c_proj.weight"][cut])
+        return P.lm_head(h + out, weights, raw), probabilities.argmax(-1)
+
+    ids = helpers.random_tokens(40, config["vocab_size"], 810)
+    expected, chosen = plain(ids)
+    assert len(set(chosen.tolist())) >= 3            # the tokens really go to different experts
+    rows = {}
+    for start, size in ((0, 13), (13, 1), (14, 2), (16, 24)):
+        out = engine.step([StepEntry("r", ids[start:start + size], list(range(size)))]).logits.double().cpu()
+        for i in range(size):
+            rows[start + i] = out[i]
+    error = max(float((rows[p] - expected[p]).abs().max()) for p in rows)
+    assert len(rows) == len(ids) and error <= 2e-5 * float(expected.abs().max()), error
+
+
+def _rotate(values, positions, head_dim, base=100.0):
+    """Pairs (2i, 2i+1) of every head turned by the angle position * base^(-2i/head_dim)."""
+    heads = values.shape[-1] // head_dim
+    shaped = values.reshape(values.shape[0], heads, head_dim // 2, 2).double()
+    inverse = base ** (-torch.arange(0, head_dim, 2, dtype=torch.float64, device=values.device) / head_dim)
+    angle = positions.double()[:, None, None] * inverse[None, None, :]
+    cos, sin = torch.cos(angle), torch.sin(angle)
+    first = shaped[..., 0] * cos - shaped[..., 1] * sin
+    second = shaped[..., 0] * sin + shaped[..., 1] * cos
+    return torch.stack((first, second), dim=-1).reshape(values.shape)
+
+
+def test_toy_rotation_is_a_function_of_distances():
+    """The toy rotation below is pinned by what a rotary encoding is for: scores of rotated
+    queries and keys depend on the distance of their positions only."""
+    generator = torch.Generator().manual_seed(5)
+    q = torch.randn(6, 32, generator=generator, dtype=torch.float64)
+    k = torch.randn(6, 32, generator=generator, dtype=torch.float64)
+    positions = torch.tensor([0, 1, 2, 5, 9, 10])
+    scores = _rotate(q, positions, 16) @ _rotate(k, positions, 16).t()
+    shifted = _rotate(q, positions + 37, 16) @ _rotate(k, positions + 37, 16).t()
+    torch.testing.assert_close(scores, shifted, atol=1e-10, rtol=0)
+    assert float((scores - q @ k.t()).abs().max()) > 0.1      # and it does turn something
+
+
+def test_toy_position_encoding_that_rotates_queries_and_keys(tmp_path):
+    """Another position encoding, registered here: nothing is added to the embedding, queries
+    and keys are rotated before the keys are cached (the hook that the attention part offers).
+    Whole prompt, portions and decoded tokens against a plain computation."""
+    import dataclasses
+
+    from pagedserve_amd.config import GPT2Config, PartSpec, resolve_architecture
+    from pagedserve_amd.engine import Engine, StepEntry
+    from pagedserve_amd.model import DecoderModel
+    from pagedserve_amd.parts import POSITIONS, PositionEncoding, register_position
+    from pagedserve_amd.weights import load_parameters
+
+    if "toy_rotary" not in POSITIONS:
+        @register_position("toy_rotary")
+        class ToyRotary(PositionEncoding):
+            transforms_qk = True
+
+            def __init__(self, width, dtype, head_dim, max_positions=0):
+                self.width, self.dtype, self.head_dim, self.max_positions = width, dtype, head_dim, max_positions
+
+            def apply_to_qk(self, q, k, ctx):
+                positions = ctx.positions[:q.shape[0]]
+                q.copy_(_rotate(q, positions, self.head_dim).to(q.dtype))
+                k.copy_(_rotate(k, positions, self.head_dim).to(k.dtype))
+
+    folder, config, page_size = helpers.tiny_folder(tmp_path, "A")
+    arch = resolve_architecture(config)
+    typed = GPT2Config.from_dict(config)
+    base = arch.build_spec(typed)
+    head_dim = config["n_embd"] // config["n_head"]
+    spec = dataclasses.replace(base, position=PartSpec.make("toy_rotary", head_dim=head_dim,
+                                                            max_positions=config["n_positions"]))
+    model = DecoderModel(spec, torch.float32, "cuda")
+    sources = {k: v for k, v in arch.weight_sources(typed, base).items() if not k.startswith("position.")}
+    loaded = load_parameters(folder, model.parameters(), sources, torch.float32, "cuda",
+                             ignorable=lambda name: name == "wpe.weight")
+    model.bind(loaded)
+    engine = Engine(model, num_pages=16, page_size=page_size, max_requests=3, max_step_tokens=64)
+
+    raw, weights = P.read_model_folder(folder)
+    heads = config["n_head"]
+
+    def plain(ids):
+        positions = torch.arange(len(ids))
+        h = weights["wte.weight"][torch.tensor(ids)].double()
+        eps = raw["layer_norm_epsilon"]
+        for layer in range(config["n_layer"]):
+            prefix = f"h.{layer}."
+            normed = P.layer_norm(h, weights[prefix + "ln_1.weight"], weights[prefix + "ln_1.bias"], eps)
+            qkv = P.conv1d(normed, weights[prefix + "attn.c_attn.weight"], weights[prefix + "attn.c_attn.bias"])
+            q, k, v = qkv.split(config["n_embd"], dim=-1)
+            q, k = _rotate(q, positions, head_dim), _rotate(k, positions, head_dim)
+            context = P.merge_heads(P.causal_attention(P.split_heads(q, heads), P.split_heads(k, heads),
+                                                       P.split_heads(v, heads), P.attention_scale(raw, layer)))
+            h = h + P.conv1d(context, weights[prefix + "attn.c_proj.weight"], weights[prefix + "attn.c_proj.bias"])
+            normed = P.layer_norm(h, weights[prefix + "ln_2.weight"], weights[prefix + "ln_2.bias"], eps)
+            h = h + P.mlp_sublayer(normed, weights, prefix, raw["activation_function"])
+        return P.lm_head(h, weights, raw)
+
+    ids = helpers.random_tokens(45, config["vocab_size"], 820)
+    expected = plain(ids)
+    rows = {}
+    for start, size in ((0, 11), (11, 1), (12, 1), (13, 2), (15, 30)):
+        out = engine.step([StepEntry("r", ids[start:start + size], list(range(size)))]).logits.double().cpu()
+        for i in range(size):
+            rows[start + i] = out[i]
+    error = max(float((rows[p] - expected[p]).abs().max()) for p in rows)
+    assert len(rows) == len(ids) and error <= 2e-5 * float(expected.abs().max()), error
