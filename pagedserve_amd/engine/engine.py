@@ -32,7 +32,7 @@ class StepEntry:
     tokens: Sequence[int]
     want: Sequence[int] = field(default_factory=list)
     # The one token of this entry is not known to the host yet: it is the token that the last
-    # step (a greedy one) chose for its row ``carry``.  ``tokens`` then holds a placeholder.
+    # step chose on the device for its row ``carry``.  ``tokens`` then holds a placeholder.
     carry: Optional[int] = None
 
 
@@ -42,7 +42,7 @@ class StepOutput:
     rows: List[tuple]               # (request_id, position) of each row
     tokens: Optional[torch.Tensor] = None   # int32 [wanted]: argmax of each row, if asked for
     # a copy of ``tokens`` in pinned host memory, complete once ``ready`` has happened; it is
-    # overwritten by the second next greedy step
+    # overwritten by the second next step that chooses tokens
     host_tokens: Optional[torch.Tensor] = None
     ready: Optional[torch.cuda.Event] = None
 
@@ -90,7 +90,7 @@ class Engine:
         self.views = model.cache_views(self.cache)
         self.workspace = Workspace(max_step_tokens, self.device)
         self.table_width = -(-self.spec.max_positions // page_size)
-        capacity = (7 * max_step_tokens + 5 * max_requests + 1
+        capacity = (9 * max_step_tokens + 5 * max_requests + 1
                     + len(groups) * max_requests * self.table_width + 16)
         self._meta_device = torch.empty(capacity, dtype=torch.int32, device=self.device)
         self._meta_host = [torch.empty(capacity, dtype=torch.int32, pin_memory=True) for _ in range(2)]
@@ -180,12 +180,20 @@ class Engine:
         if len(self.cache.requests) + new > self.max_requests:
             raise StepError(f"more than {self.max_requests} live requests")
 
-    def step(self, entries: Sequence[StepEntry], greedy: bool = False) -> StepOutput:
+    supports_draws = True
+
+    def step(self, entries: Sequence[StepEntry], greedy: bool = False, draws=None) -> StepOutput:
         """Run one batch.  With ``greedy`` the argmax of every wanted row is computed on the
         GPU as part of the step (inside the graph of a replayed decode step) and returned as
-        ``StepOutput.tokens``."""
+        ``StepOutput.tokens``.  With ``draws``, one ``(1 / temperature, uniform number)`` per
+        wanted row, each row's token is drawn there instead (argmax where the first is 0)."""
         entries = list(entries)
         self._validate(entries)
+        if draws is not None:
+            draws = [(float(a), float(b)) for a, b in draws]
+            if len(draws) != sum(len(entry.want) for entry in entries):
+                raise StepError(f"{len(draws)} draws for {sum(len(e.want) for e in entries)} wanted rows")
+            greedy = draws
         admitted = []
         cache = self.cache
         try:
@@ -216,7 +224,7 @@ class Engine:
         self.steps += 1
         return output
 
-    def _pack(self, entries):
+    def _pack(self, entries, select=None):
         """Fill the packed index buffer on the host, copy it, and return the step context.
 
         The layout depends only on (tokens, items, wanted rows, one-token items)."""
@@ -236,7 +244,8 @@ class Engine:
         for name, size in (("token_ids", tokens), ("token_src", tokens), ("positions", tokens),
                            ("tok_item", tokens),
                            ("cu_tokens", items + 1), ("kv_lens", items), ("slots", items),
-                           ("rows", wanted), ("single_tokens", singles),
+                           ("rows", wanted), ("inv_temperature", wanted), ("uniform", wanted),
+                           ("single_tokens", singles),
                            ("portion_tokens", tokens - singles), ("tile_item", tiles),
                            ("tile_q0", tiles)):
             offsets[name] = (cursor, size)
@@ -316,6 +325,9 @@ class Engine:
                 step_items.append(StepItem(entry.request_id, record.slot, start, count, flat))
                 flat += count
             cu[items] = flat
+        if isinstance(select, list):
+            section("inv_temperature").view(np.float32)[:] = [a for a, _ in select]
+            section("uniform").view(np.float32)[:] = [b for _, b in select]
         slot_index = np.asarray(slot_list, dtype=np.int64)
         for group in range(groups):
             section(f"tables{group}").reshape(items, width)[:] = cache.table_arrays[group][slot_index]
@@ -340,6 +352,8 @@ class Engine:
             max_positions=self.spec.max_positions,
             tile_item=view("tile_item"), tile_q0=view("tile_q0"),
             token_src=view("token_src"), carried_tokens=self._tokens)
+        self._draw_views = (view("inv_temperature").view(torch.float32),
+                            view("uniform").view(torch.float32))
         return ctx, view("rows"), row_keys
 
     def _forward(self, ctx, rows, logits, wanted, greedy):
@@ -348,7 +362,11 @@ class Engine:
         if greedy and wanted:
             from ..ops import kernels
 
-            tokens = kernels.sample(out, None, None, self._tokens[:wanted])
+            if isinstance(greedy, list):
+                inv_temperature, uniform = self._draw_views
+                tokens = kernels.sample(out, inv_temperature, uniform, self._tokens[:wanted])
+            else:
+                tokens = kernels.sample(out, None, None, self._tokens[:wanted])
         return out, tokens
 
     def _run(self, entries, greedy=False) -> StepOutput:
@@ -369,26 +387,27 @@ class Engine:
 
     def _run_step(self, entries, greedy=False) -> StepOutput:
         items = len(entries)
+        mode = 2 if isinstance(greedy, list) else int(bool(greedy))   # how tokens are chosen
         if self.use_graphs and self._graphs:
             # a captured step: every entry brings one token and wants its logits
-            plan = self._graphs.get((items, greedy))
+            plan = self._graphs.get((items, mode))
             if (plan is not None and plan.logits.data_ptr() == self._logit_buffer(items).data_ptr()
                     and all(len(e.tokens) == 1 and len(e.want) == 1 for e in entries)):
-                return self._replay(plan, entries)
-        ctx, rows, row_keys = self._pack(entries)
+                return self._replay(plan, entries, greedy)
+        ctx, rows, row_keys = self._pack(entries, greedy)
         wanted = len(row_keys)
         logits = self._logit_buffer(wanted)
         graph_key = None
         if self.use_graphs and ctx.decode_only and wanted == ctx.tokens:
             # A step of single tokens that all want their logits.  Every launch argument is
             # then a function of the number of items (and of buffer addresses).
-            graph_key = (items, greedy)
+            graph_key = (items, mode)
         if graph_key is None or graph_key in self._graph_failures:
             out, tokens = self._forward(ctx, rows, logits, wanted, greedy)
             return StepOutput(logits=out, rows=row_keys, tokens=tokens)
         # launch shapes inside a graph must not depend on this step's lengths
         ctx.max_kv_len = self.spec.max_positions
-        seen_key = (items, greedy, logits.data_ptr())
+        seen_key = (items, mode, logits.data_ptr())
         if seen_key not in self._graph_seen:
             # first time: run directly, so that every buffer exists before a capture
             self._graph_seen.add(seen_key)
@@ -422,7 +441,7 @@ class Engine:
         graph.launch()
         return StepOutput(logits=out, rows=row_keys, tokens=tokens)
 
-    def _replay(self, plan, entries) -> StepOutput:
+    def _replay(self, plan, entries, select=None) -> StepOutput:
         """A captured decode step: refresh the per-step indices, copy them, launch the graph."""
         cache = self.cache
         turn = self._meta_turn
@@ -447,6 +466,9 @@ class Engine:
         sections["positions"][:] = starts
         sections["kv_lens"][:] = [start + 1 for start in starts]
         sections["slots"][:] = slots
+        if isinstance(select, list):
+            sections["inv_temperature"].view(np.float32)[:] = [a for a, _ in select]
+            sections["uniform"].view(np.float32)[:] = [b for _, b in select]
         for group in range(len(cache.groups)):
             sections[f"tables{group}"][:] = cache.table_arrays[group][slots]
         self._meta_device[:plan.used].copy_(self._meta_host[turn][:plan.used], non_blocking=True)

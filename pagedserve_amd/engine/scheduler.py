@@ -23,7 +23,7 @@ requests have reserved (``:119-122,138-142``); otherwise it and everything behin
 nothing is preempted.  A request whose worst case exceeds the whole pool is refused when
 it is added.
 
-**Running ahead.**  While every running request decodes greedily and nobody waits, the
+**Running ahead.**  While every running request decodes and nobody waits, the
 iteration after the current one is launched before the current one's tokens have reached
 the host: its entries say "the token that the last step chose for row r" instead of a token
 id, and the host's work for an iteration overlaps the GPU's work for the next.  A request
@@ -71,7 +71,7 @@ class _Pending:
     entries: list
     producers: list           # requests that receive a token from it, in row order
     output: object
-    can_carry: bool           # greedy single-token rows: the next iteration may carry them on
+    can_carry: bool           # single-token rows chosen on the device: the next iteration may carry them on
 
 
 class ContinuousBatchScheduler:
@@ -299,8 +299,14 @@ class ContinuousBatchScheduler:
         # greedy rows are picked on the GPU inside the step (one launch less, and part of the
         # captured graph of a decode step)
         greedy = bool(producers) and all(r.sampling.temperature == 0 for r in producers)
+        draws = None
+        if producers and not greedy and getattr(self.engine, "supports_draws", False):
+            draws = self._draws(producers, 0)
         try:
-            output = self.engine.step(entries, greedy=greedy)
+            if draws is not None:
+                output = self.engine.step(entries, draws=draws)
+            else:
+                output = self.engine.step(entries, greedy=greedy)
         except Exception:
             for request in new_requests:
                 for g, pages in enumerate(request.reserved_blocks):
@@ -308,7 +314,18 @@ class ContinuousBatchScheduler:
                 request.reserved_blocks = []
             raise
         decode_only = all(not request.is_prefilling for request, _ in selected)
-        return _Pending(selected, entries, producers, output, greedy and decode_only)
+        return _Pending(selected, entries, producers, output,
+                        (greedy or draws is not None) and decode_only)
+
+    @staticmethod
+    def _draws(producers, ahead):
+        """(1 / temperature, uniform number) of the next token of each request; ``ahead`` = 1
+        when the request's last token is still on its way to the host."""
+        from ..sampling.params import uniform_for
+
+        return [(0.0 if r.sampling.temperature == 0 else 1.0 / r.sampling.temperature,
+                 uniform_for(r.seed, r.request_id, len(r.generated_token_ids) + ahead))
+                for r in producers]
 
     def _launch_ahead(self, pending) -> Optional["_Pending"]:
         """Start the iteration after ``pending`` before ``pending``'s tokens are known, if
@@ -328,12 +345,16 @@ class ContinuousBatchScheduler:
             entries.append(StepEntry(request.request_id, [0], [0], carry=row))
         if not selected:
             return None
+        producers = [request for request, _ in selected]
         try:
-            output = self.engine.step(entries, greedy=True)
+            if all(r.sampling.temperature == 0 for r in producers):
+                output = self.engine.step(entries, greedy=True)
+            else:
+                output = self.engine.step(entries, draws=self._draws(producers, 1))
         except ValueError:
             return None       # the ordinary launch of the next iteration reports it
         self.steps_run_ahead += 1
-        return _Pending(selected, entries, [request for request, _ in selected], output, True)
+        return _Pending(selected, entries, producers, output, True)
 
     def _resolve(self, pending) -> Dict[int, int]:
         """Read the tokens of a launched iteration and move its requests on."""

@@ -98,6 +98,40 @@ def test_running_ahead_gives_the_same_tokens_and_stops_at_the_end_token(folders)
     assert results[False] == 0 and results[True] > 10
 
 
+def test_running_ahead_with_temperature_draws_the_same_tokens(folders):
+    """Drawn tokens (seeded) are the same whether the host's sampler picks them from the
+    logits after each step, the step picks them on the device, or steps run ahead."""
+    from pagedserve_amd.engine import ContinuousBatchScheduler, Engine
+    from pagedserve_amd.model import load_model
+    from pagedserve_amd.sampling import Sampler, SamplingParams
+
+    folder, config, page_size = folders["B"]
+    prompts = [helpers.random_tokens(n, config["vocab_size"], 950 + i) for i, n in enumerate([4, 21, 9])]
+    budgets = [30, 18, 25]
+    temperatures = [6.0, 0.0, 12.0]
+    model, _ = load_model(folder, dtype="float32")
+    results = []
+    for on_device, run_ahead in ((False, False), (True, False), (True, True)):
+        engine = Engine(model, num_pages=32, page_size=page_size, max_requests=4, max_step_tokens=64)
+        engine.supports_draws = on_device
+        scheduler = ContinuousBatchScheduler(engine, Sampler(engine.device, 4), max_batch_size=4,
+                                             eos_token_id=None, run_ahead=run_ahead)
+        ids = [scheduler.add_token_request(prompt, budget, sampling=SamplingParams(
+                   max_new_tokens=budget, temperature=temperature, seed=11 + i))
+               for i, (prompt, budget, temperature) in enumerate(zip(prompts, budgets, temperatures))]
+        scheduler.run_until_complete()
+        results.append([scheduler.finished[rid].generated_token_ids for rid in ids])
+        assert [len(tokens) for tokens in results[-1]] == budgets
+        if run_ahead:
+            assert scheduler.steps_run_ahead > 10
+        engine.cache.check_invariants()
+    assert results[0] == results[1] == results[2]
+    # the draws are no argmax in disguise
+    raw, weights = plain_gpt2.read_model_folder(folder)
+    assert results[0][0] != plain_gpt2.greedy_generate(raw, weights, prompts[0], budgets[0])
+    assert results[0][1] == plain_gpt2.greedy_generate(raw, weights, prompts[1], budgets[1])
+
+
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 def test_long_decoding(folders, dtype):
     """Two prompt tokens, then 250 tokens decoded one by one up to the last position."""
