@@ -31,6 +31,13 @@ HIPCC_FLAGS = [
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
     "-Wno-unused-command-line-argument",
 ]
+# Per source: matrix products that accumulate in ordinary vector registers.  Kernels that go on
+# computing with the results (softmax, wide epilogues) then need no copies from the
+# accumulation registers; the skinny decode products are better off without.
+EXTRA_FLAGS = {
+    "attention_prefill.hip": ["-mllvm", "-amdgpu-mfma-vgpr-form"],
+    "gemm_tiled_bf16.hip": ["-mllvm", "-amdgpu-mfma-vgpr-form"],
+}
 
 
 class KernelLibraryError(RuntimeError):
@@ -51,6 +58,7 @@ def source_hash() -> str:
         with open(os.path.join(SOURCE_DIR, name), "rb") as handle:
             digest.update(handle.read())
     digest.update(" ".join(HIPCC_FLAGS).encode())
+    digest.update(repr(sorted(EXTRA_FLAGS.items())).encode())
     return digest.hexdigest()[:16]
 
 
@@ -110,7 +118,7 @@ def build(target_dir=None, verbose=True, jobs=None) -> str:
             name = pending.pop(0)
             obj = os.path.join(object_dir, name[:-4] + ".o")
             objects.append(obj)
-            command = [hipcc] + HIPCC_FLAGS + ["-I", SOURCE_DIR, "-c",
+            command = [hipcc] + HIPCC_FLAGS + EXTRA_FLAGS.get(name, []) + ["-I", SOURCE_DIR, "-c",
                                               os.path.join(SOURCE_DIR, name), "-o", obj]
             running[name] = subprocess.Popen(command, stdout=subprocess.PIPE,
                                              stderr=subprocess.STDOUT, text=True)
