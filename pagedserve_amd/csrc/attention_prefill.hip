@@ -75,7 +75,10 @@ __global__ __launch_bounds__(128 * KS) void attention_prefill_kernel(
   constexpr int LOADS = 2 * PER_OPERAND;
   constexpr int NDB32 = (NDB + 1) / 2;           // blocks of 32 head dimensions
   static_assert(LOADS * 2 < 64, "the load counter has six bits");
-  __shared__ __attribute__((aligned(1024))) unsigned char stages[STAGES * STAGE_BYTES];
+  // the states that the waves merge at the end lie where the stages were
+  constexpr int MERGE_BYTES = (AP_WAVES - 2) * 64 * (NDB32 * 16 + 2) * 4;
+  constexpr int LDS_BYTES = STAGES * STAGE_BYTES > MERGE_BYTES ? STAGES * STAGE_BYTES : MERGE_BYTES;
+  __shared__ __attribute__((aligned(1024))) unsigned char stages[LDS_BYTES];
   __shared__ int s_table[AP_TABLE_MAX];
 
   const int tid = threadIdx.x;
@@ -229,43 +232,49 @@ __global__ __launch_bounds__(128 * KS) void attention_prefill_kernel(
     if (ahead <= 0) ap_wait_loads_and_sync<0>();
     else if (ahead == 1) ap_wait_loads_and_sync<LOADS>();
     else ap_wait_loads_and_sync<2 * LOADS>();
-    if (t + STAGES - 1 < tiles) issue(t + STAGES - 1, k0 + (STAGES - 1) * AP_KEYS);
-    // this wave's run of 32 keys; skip it where no query of the wave can see it
+    // this wave's run of 32 keys; it is skipped where no query of the wave can see it
     const int kw = k0 + wave_k * 32;
-    if (!wave_active || kw > wave_last || kw >= key_end) continue;
-    if (window > 0 && kw + 31 < wave_first - window + 1) continue;
+    const bool active = wave_active && kw <= wave_last && kw < key_end &&
+                        !(window > 0 && kw + 31 < wave_first - window + 1);
     // S^T: element e is key (e/4)*8 + half*4 + e%4 of the run.  The operand reads are written
     // as assembly: the compiler would otherwise wait for every tile in flight before each.
-    // The transposing reads of V are issued right behind: they arrive while S is computed.
+    // The transposing reads of V are issued right behind them.
     const uint32_t stage_base =
         (uint32_t)(uintptr_t)(ap_lds_ptr)stages + (uint32_t)((t % STAGES) * STAGE_BYTES);
     u32x4 kr[NDB];
-#pragma unroll
-    for (int step = 0; step < NDB; ++step)
-      asm volatile("ds_read_b128 %0, %1" : "=v"(kr[step]) : "v"(stage_base + k_off[step]) : "memory");
     u32x2 vr[2][NDB32][2];
+    if (active) {
 #pragma unroll
-    for (int run = 0; run < 2; ++run)
+      for (int step = 0; step < NDB; ++step)
+        asm volatile("ds_read_b128 %0, %1" : "=v"(kr[step]) : "v"(stage_base + k_off[step]) : "memory");
 #pragma unroll
-      for (int db = 0; db < NDB32; ++db)
+      for (int run = 0; run < 2; ++run)
 #pragma unroll
-        for (int second = 0; second < 2; ++second)
-          asm volatile("ds_read_b64_tr_b16 %0, %1"
-                       : "=v"(vr[run][db][second])
-                       : "v"(stage_base + v_off[run][db][second])
-                       : "memory");
-    constexpr int V_READS = 4 * NDB32;
-    // LDS reads return in order: all but the reads of V have arrived
-    asm volatile("s_waitcnt lgkmcnt(%0)" ::"n"(V_READS < 15 ? V_READS : 15) : "memory");
-    f32x16 s;
+        for (int db = 0; db < NDB32; ++db)
 #pragma unroll
-    for (int e = 0; e < 16; ++e) s[e] = 0.f;
-#pragma unroll
-    for (int step = 0; step < NDB; ++step) {
-      asm volatile("" : "+v"(kr[step]));   // used only behind the wait
-      s = __builtin_amdgcn_mfma_f32_32x32x16_bf16(*reinterpret_cast<const bf16x8*>(&kr[step]),
-                                                qf[step], s, 0, 0, 0);
+          for (int second = 0; second < 2; ++second)
+            asm volatile("ds_read_b64_tr_b16 %0, %1"
+                         : "=v"(vr[run][db][second])
+                         : "v"(stage_base + v_off[run][db][second])
+                         : "memory");
     }
+    // Everything read by assembly is waited for before the compiler's own code goes on (it
+    // does not know that those registers are still on their way).
+    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+    f32x16 s;
+    if (active) {
+#pragma unroll
+      for (int e = 0; e < 16; ++e) s[e] = 0.f;
+#pragma unroll
+      for (int step = 0; step < NDB; ++step) {
+        asm volatile("" : "+v"(kr[step]));   // used only behind the wait
+        s = __builtin_amdgcn_mfma_f32_32x32x16_bf16(*reinterpret_cast<const bf16x8*>(&kr[step]),
+                                                  qf[step], s, 0, 0, 0);
+      }
+    }
+    // the tile that is STAGES - 1 ahead is asked for while the matrix cores work on S
+    if (t + STAGES - 1 < tiles) issue(t + STAGES - 1, k0 + (STAGES - 1) * AP_KEYS);
+    if (!active) continue;
     // the whole run is visible to every query of the wave: no mask
     const bool masked = kw + 31 > wave_first || kw + 32 > key_end ||
                         (window > 0 && kw < wave_last - window + 1) || !q_valid;
@@ -315,7 +324,6 @@ __global__ __launch_bounds__(128 * KS) void attention_prefill_kernel(
 
     // O^T += V^T P^T, 16 keys per instruction: slots 0..3 are keys base + half*4 + 0..3,
     // slots 4..7 keys base + 8 + half*4 + 0..3, in both operands
-    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
 #pragma unroll
     for (int run = 0; run < 2; ++run)
 #pragma unroll
@@ -332,7 +340,7 @@ __global__ __launch_bounds__(128 * KS) void attention_prefill_kernel(
   // accumulators of waves with the same queries have the same layout, so lane meets lane.
   if (KS > 1) {
     constexpr int STATE = NDB32 * 16 + 2;      // floats per lane
-    static_assert((AP_WAVES - 2) * 64 * STATE * 4 <= STAGES * STAGE_BYTES, "the merge reuses the stages");
+    static_assert((AP_WAVES - 2) * 64 * STATE * 4 == MERGE_BYTES, "the merge reuses the stages");
     ap_wait_loads_and_sync<0>();               // every wave is past its last operand reads
     float* states = reinterpret_cast<float*>(stages);
     if (wave_k > 0) {
