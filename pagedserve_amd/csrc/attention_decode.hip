@@ -139,8 +139,12 @@ __global__ __launch_bounds__(64 * AD_WAVES) void attention_decode_kernel(
 #pragma unroll
       for (int i = 0; i < 8; ++i) dot = fmaf(qf[i], kf[i], dot);
       if (!has_dims) dot = 0.f;
-#pragma unroll
-      for (int offset = LPK / 2; offset > 0; offset >>= 1) dot += __shfl_xor(dot, offset, 64);
+      if (LPK <= 16) {
+        dot = lanes_sum<(LPK <= 16 ? LPK : 16)>(dot);
+      } else {
+        dot = lanes_sum<16>(dot);
+        dot += __shfl_xor(dot, 16, 64);
+      }
       s[u] = valid[u] ? dot * scale : -INFINITY;
       m_new = fmaxf(m_new, s[u]);
     }

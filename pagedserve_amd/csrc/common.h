@@ -84,16 +84,50 @@ __device__ inline bf16_t from_float<bf16_t>(float v) {
   return float_to_bf16(v);
 }
 
-__device__ inline float wave_sum(float v) {
-#pragma unroll
-  for (int offset = PS_WAVE / 2; offset > 0; offset >>= 1) v += __shfl_xor(v, offset, PS_WAVE);
+// Lane exchanges inside a row of 16 lanes run on the vector unit itself (DPP), not through
+// the LDS crossbar that __shfl_xor uses: a reduction over a wave is four such steps, then the
+// four row results are read as scalars.  CTRL: 0xB1 / 0x4E swap neighbours / pairs inside a
+// quad, 0x141 / 0x140 mirror a half row / a row.
+template <int CTRL>
+__device__ inline float lane_exchange(float v) {
+  return __builtin_bit_cast(
+      float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), CTRL, 0xF, 0xF, true));
+}
+
+// Sum over aligned groups of N lanes (N = 2, 4, 8 or 16); every lane receives its group's sum.
+template <int N>
+__device__ inline float lanes_sum(float v) {
+  static_assert(N == 1 || N == 2 || N == 4 || N == 8 || N == 16, "groups inside a row of 16 lanes");
+  if (N >= 2) v += lane_exchange<0xB1>(v);
+  if (N >= 4) v += lane_exchange<0x4E>(v);
+  if (N >= 8) v += lane_exchange<0x141>(v);
+  if (N >= 16) v += lane_exchange<0x140>(v);
   return v;
 }
 
-__device__ inline float wave_max(float v) {
-#pragma unroll
-  for (int offset = PS_WAVE / 2; offset > 0; offset >>= 1) v = fmaxf(v, __shfl_xor(v, offset, PS_WAVE));
+template <int N>
+__device__ inline float lanes_max(float v) {
+  static_assert(N == 1 || N == 2 || N == 4 || N == 8 || N == 16, "groups inside a row of 16 lanes");
+  if (N >= 2) v = fmaxf(v, lane_exchange<0xB1>(v));
+  if (N >= 4) v = fmaxf(v, lane_exchange<0x4E>(v));
+  if (N >= 8) v = fmaxf(v, lane_exchange<0x141>(v));
+  if (N >= 16) v = fmaxf(v, lane_exchange<0x140>(v));
   return v;
+}
+
+__device__ inline float read_lane(float v, int lane) {
+  return __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), lane));
+}
+
+// Every lane receives the sum / the maximum over the wave.
+__device__ inline float wave_sum(float v) {
+  v = lanes_sum<16>(v);
+  return (read_lane(v, 0) + read_lane(v, 16)) + (read_lane(v, 32) + read_lane(v, 48));
+}
+
+__device__ inline float wave_max(float v) {
+  v = lanes_max<16>(v);
+  return fmaxf(fmaxf(read_lane(v, 0), read_lane(v, 16)), fmaxf(read_lane(v, 32), read_lane(v, 48)));
 }
 
 // Sum over a block of up to 1024 threads; every thread receives the total.
