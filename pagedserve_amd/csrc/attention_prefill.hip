@@ -292,7 +292,7 @@ __global__ __launch_bounds__(128 * KS) void attention_prefill_kernel(
 #pragma unroll
       for (int e = 0; e < 16; ++e) tile_max = fmaxf(tile_max, s[e]);
     }
-    tile_max = fmaxf(tile_max, __shfl_xor(tile_max, 32, 64)) * scale_log2;   // scale > 0
+    tile_max = halves_max(tile_max) * scale_log2;   // scale > 0
     const float m_new = fmaxf(m, tile_max);
     // A query that has seen nothing yet (m_new = -inf) takes 0 as its reference: its scores
     // are all -inf and their exponentials 0.  Other lanes of the wave may differ, so the
@@ -309,7 +309,7 @@ __global__ __launch_bounds__(128 * KS) void attention_prefill_kernel(
     }
     const u32x4 p_lo = {words[0], words[1], words[2], words[3]};
     const u32x4 p_hi = {words[4], words[5], words[6], words[7]};
-    tile_sum += __shfl_xor(tile_sum, 32, 64);
+    tile_sum = halves_sum(tile_sum);
     // the running maximum rarely moves after the first tiles: rescale only where it did
     if (__builtin_amdgcn_readfirstlane(__any(m_new != m) ? 1 : 0)) {
       const float correction = (m == -INFINITY) ? 0.f : __builtin_amdgcn_exp2f(m - reference);

@@ -115,6 +115,20 @@ __device__ inline float lanes_max(float v) {
   return v;
 }
 
+// The sum / maximum of a lane's value and that of the lane 32 further (or back): one swap of
+// the wave's halves (v_permlane32_swap) instead of a trip through LDS.
+__device__ inline float halves_sum(float v) {
+  const int bits = __builtin_bit_cast(int, v);
+  const auto both = __builtin_amdgcn_permlane32_swap(bits, bits, false, false);
+  return __builtin_bit_cast(float, (int)both[0]) + __builtin_bit_cast(float, (int)both[1]);
+}
+
+__device__ inline float halves_max(float v) {
+  const int bits = __builtin_bit_cast(int, v);
+  const auto both = __builtin_amdgcn_permlane32_swap(bits, bits, false, false);
+  return fmaxf(__builtin_bit_cast(float, (int)both[0]), __builtin_bit_cast(float, (int)both[1]));
+}
+
 __device__ inline float read_lane(float v, int lane) {
   return __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), lane));
 }
