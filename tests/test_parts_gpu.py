@@ -487,3 +487,90 @@ def test_toy_position_encoding_that_rotates_queries_and_keys(tmp_path):
             rows[start + i] = out[i]
     error = max(float((rows[p] - expected[p]).abs().max()) for p in rows)
     assert len(rows) == len(ids) and error <= 2e-5 * float(expected.abs().max()), error
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_a_windowed_layer_has_pages_of_its_own_and_gives_them_back(tmp_path, dtype):
+    """Layer 0 sees all keys, layer 1 the last 20 of them (the attention part's window): two
+    cache groups with pools of their own.  Two requests advance in portions and single
+    tokens far beyond the window, so pages of the windowed group go back and are used again
+    while the requests run; logits against a plain computation with the same window."""
+    import dataclasses
+
+    from pagedserve_amd.config import GPT2Config, resolve_architecture
+    from pagedserve_amd.engine import Engine, StepEntry
+    from pagedserve_amd.model import DecoderModel
+    from pagedserve_amd.weights import load_parameters
+
+    window = 20
+    folder, config, page_size = helpers.tiny_folder(tmp_path, "A")
+    arch = resolve_architecture(config)
+    typed = GPT2Config.from_dict(config)
+    base = arch.build_spec(typed)
+    mixer = base.blocks[1].mixer
+    from pagedserve_amd.config import PartSpec
+    windowed = dataclasses.replace(base.blocks[1], mixer=PartSpec.make(mixer.kind, **{**mixer.as_dict(), "window": window}))
+    spec = dataclasses.replace(base, blocks=(base.blocks[0], windowed))
+    torch_dtype = torch.float32 if dtype == "float32" else torch.bfloat16
+    model = DecoderModel(spec, torch_dtype, "cuda")
+    model.bind(load_parameters(folder, model.parameters(), arch.weight_sources(typed, spec), torch_dtype, "cuda"))
+    groups, _ = model.cache_requirements()
+    assert sorted(g.window for g in groups) == [0, window]
+    # so few pages that the windowed group must reuse what it gave back: two requests of up to
+    # 110 tokens need 28 pages of 8 in the full group, the windowed group gets by with far less
+    engine = Engine(model, num_pages=30, page_size=page_size, max_requests=2, max_step_tokens=64)
+
+    raw, weights = P.read_model_folder(folder)
+    if dtype == "bfloat16":
+        weights = P.round_weights_to_bfloat16(weights)
+    heads = raw["n_head"]
+
+    def plain(ids):
+        h = P.embed(weights["wte.weight"], weights["wpe.weight"], torch.tensor(ids), torch.arange(len(ids)))
+        h = P.block(h, weights, raw, 0)
+        eps = raw["layer_norm_epsilon"]
+        normed = P.layer_norm(h, weights["h.1.ln_1.weight"], weights["h.1.ln_1.bias"], eps)
+        qkv = P.conv1d(normed, weights["h.1.attn.c_attn.weight"], weights["h.1.attn.c_attn.bias"])
+        q, k, v = qkv.split(raw["n_embd"], dim=-1)
+        context = P.causal_attention(P.split_heads(q, heads), P.split_heads(k, heads), P.split_heads(v, heads),
+                                     P.attention_scale(raw, 1), window=window)
+        h = h + P.conv1d(P.merge_heads(context), weights["h.1.attn.c_proj.weight"], weights["h.1.attn.c_proj.bias"])
+        normed = P.layer_norm(h, weights["h.1.ln_2.weight"], weights["h.1.ln_2.bias"], eps)
+        h = h + P.mlp_sublayer(normed, weights, "h.1.", raw["activation_function"])
+        return P.lm_head(h, weights, raw)
+
+    requests = {"a": helpers.random_tokens(110, config["vocab_size"], 830),
+                "b": helpers.random_tokens(97, config["vocab_size"], 831)}
+    expected = {rid: plain(ids) for rid, ids in requests.items()}
+    # the window really matters for these weights
+    unwindowed = helpers.plain_logits(folder, requests["a"], bfloat16=dtype == "bfloat16")
+    assert float((unwindowed[-1] - expected["a"][-1]).abs().max()) > 1e-3 * float(expected["a"].abs().max())
+
+    plan = [[("a", 33)], [("a", 1), ("b", 41)], [("a", 7), ("b", 1)], [("a", 1), ("b", 1)], [("a", 30), ("b", 2)],
+            [("b", 37)], [("a", 1), ("b", 1)], [("a", 2), ("b", 13)], [("a", 35), ("b", 1)]]
+    done = {"a": 0, "b": 0}
+    got = {"a": {}, "b": {}}
+    windowed_group = [g for g, spec_ in enumerate(engine.cache.groups) if spec_.window == window][0]
+    most_pages = 0
+    for step in plan:
+        entries = []
+        for rid, size in step:
+            start = done[rid]
+            entries.append(StepEntry(rid, requests[rid][start:start + size], list(range(size))))
+        out = engine.step(entries).logits.double().cpu()
+        row = 0
+        for rid, size in step:
+            for i in range(size):
+                got[rid][done[rid] + i] = out[row]
+                row += 1
+            done[rid] += size
+        engine.cache.check_invariants()
+        most_pages = max(most_pages, engine.cache.pools[windowed_group].num_allocated)
+    assert done == {"a": 110, "b": 97}
+    # a request holds about window / page pages there, whatever its length
+    assert most_pages <= 2 * (-(-window // page_size) + 9)
+    tolerance = helpers.TOLERANCE[dtype]
+    for rid in requests:
+        scale = float(expected[rid].abs().max())
+        error = max(float((got[rid][p] - expected[rid][p]).abs().max()) for p in got[rid])
+        assert len(got[rid]) == len(requests[rid]) and error <= tolerance * scale, (rid, error, scale)
