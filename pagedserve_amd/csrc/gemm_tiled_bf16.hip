@@ -11,8 +11,10 @@
 //
 // Four waves in a 2 x 2 arrangement; a wave owns WM x WN accumulators of 32 x 32
 // (v_mfma_f32_32x32x16_bf16, float accumulation), so a block makes 64 WM x 64 WN outputs.
-// Per k tile there is one wait (own loads of that tile have landed; later tiles stay in
-// flight) and one barrier, after which the stage that was multiplied last is refilled.
+// Per k tile there is one wait (own loads of the next tile have landed; later tiles stay in
+// flight) and one barrier, placed before the tile's last k step so that three steps' products
+// are queued in the matrix core meanwhile; after it the stage that was multiplied before is
+// refilled and the next tile's first operands are fetched.
 //
 // Rows beyond m or n are fetched from the last valid row instead (they only feed outputs that
 // are never stored).  The epilogue is the one of the other products: bias, GELU, residual
@@ -76,7 +78,7 @@ __global__ __launch_bounds__(256) void gemm_nt_bf16_tiled_kernel(
   constexpr int LOADS_W = BN / 32;
   constexpr int LOADS = LOADS_A + LOADS_W;
   static_assert(STAGES >= 2 && STAGES <= 4, "two to four stages");
-  static_assert(LOADS * (STAGES - 2) < 64, "the load counter has six bits");
+  static_assert(LOADS * (STAGES - 1) < 64, "the load counter has six bits");
   __shared__ __attribute__((aligned(1024))) unsigned char lds[STAGES * STAGE_BYTES];
 
   const int tid = threadIdx.x;
@@ -141,23 +143,53 @@ __global__ __launch_bounds__(256) void gemm_nt_bf16_tiled_kernel(
   const int key = (lane >> 1) & 7;   // ((row >> 1) & 7) of every row this lane reads
   const int a_row = (wave_m * WM * 32 + (lane & 31)) * TB_ROW;
   const int w_row = (BM + wave_n * WN * 32 + (lane & 31)) * TB_ROW;
-  auto compute = [&](int kt) {
+  // The operands of k step s + 1 are fetched before the products of step s are issued, also
+  // across tiles: before the last step of a tile the wave waits for the next tile's loads
+  // and meets the other waves, with three steps' products already queued in the matrix core,
+  // then fetches the next tile's first operands.
+  bf16x8 fa[2][WM], fw[2][WN];
+  auto fetch = [&](int kt, int s, bf16x8* da, bf16x8* dw) {
     const unsigned char* stage = lds + (kt % STAGES) * STAGE_BYTES;
-    // the operands of step s + 1 are fetched before the products of step s are issued
-    bf16x8 fa[2][WM], fw[2][WN];
-    auto fetch = [&](int s, bf16x8* da, bf16x8* dw) {
-      const int slot = ((2 * s + (lane >> 5)) ^ key) << 4;
+    const int slot = ((2 * s + (lane >> 5)) ^ key) << 4;
 #pragma unroll
-      for (int i = 0; i < WM; ++i)
-        da[i] = *reinterpret_cast<const bf16x8*>(stage + a_row + i * 32 * TB_ROW + slot);
+    for (int i = 0; i < WM; ++i)
+      da[i] = *reinterpret_cast<const bf16x8*>(stage + a_row + i * 32 * TB_ROW + slot);
 #pragma unroll
-      for (int j = 0; j < WN; ++j)
-        dw[j] = *reinterpret_cast<const bf16x8*>(stage + w_row + j * 32 * TB_ROW + slot);
-    };
-    fetch(0, fa[0], fw[0]);
+    for (int j = 0; j < WN; ++j)
+      dw[j] = *reinterpret_cast<const bf16x8*>(stage + w_row + j * 32 * TB_ROW + slot);
+  };
+  constexpr int STEPS = TB_BK / 16;
+  static_assert(STEPS % 2 == 0, "the operand buffers alternate per step");
+
 #pragma unroll
-    for (int s = 0; s < TB_BK / 16; ++s) {
-      if (s + 1 < TB_BK / 16) fetch(s + 1, fa[(s + 1) & 1], fw[(s + 1) & 1]);
+  for (int d = 0; d < STAGES - 1; ++d)
+    if (d < k_tiles) issue(d);
+  {
+    // tile 0 has landed; tiles 1 .. STAGES - 2 may stay in flight, as far as they exist
+    const int ahead = k_tiles - 1 < STAGES - 2 ? k_tiles - 1 : STAGES - 2;
+    if (ahead <= 0) wait_loads_and_sync<0>();
+    else if (ahead == 1) wait_loads_and_sync<LOADS>();
+    else wait_loads_and_sync<2 * LOADS>();
+  }
+  fetch(0, 0, fa[0], fw[0]);
+  for (int kt = 0; kt < k_tiles; ++kt) {
+    // the stage of tile kt - 1 is free: every wave met the others after its last read of it
+    if (kt + STAGES - 1 < k_tiles) issue(kt + STAGES - 1);
+#pragma unroll
+    for (int s = 0; s < STEPS; ++s) {
+      if (s + 1 < STEPS) {
+        fetch(kt, s + 1, fa[(s + 1) & 1], fw[(s + 1) & 1]);
+      } else if (kt + 1 < k_tiles) {
+        // own reads of this tile are complete before the others may overwrite its stage
+        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+        // tiles kt + 2 .. kt + STAGES - 1 may stay in flight, as far as they exist
+        const int last = k_tiles - 1 < kt + STAGES - 1 ? k_tiles - 1 : kt + STAGES - 1;
+        const int ahead = last - (kt + 1);
+        if (ahead <= 0) wait_loads_and_sync<0>();
+        else if (ahead == 1) wait_loads_and_sync<LOADS>();
+        else wait_loads_and_sync<2 * LOADS>();
+        fetch(kt + 1, 0, fa[0], fw[0]);
+      }
 #pragma unroll
       for (int i = 0; i < WM; ++i)
 #pragma unroll
@@ -165,20 +197,6 @@ __global__ __launch_bounds__(256) void gemm_nt_bf16_tiled_kernel(
           acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa[s & 1][i], fw[s & 1][j],
                                                               acc[i][j], 0, 0, 0);
     }
-  };
-
-#pragma unroll
-  for (int d = 0; d < STAGES - 1; ++d)
-    if (d < k_tiles) issue(d);
-  for (int kt = 0; kt < k_tiles; ++kt) {
-    // tiles kt + 1 .. kt + STAGES - 2 may stay in flight, as far as they exist
-    const int ahead = k_tiles - 1 - kt < STAGES - 2 ? k_tiles - 1 - kt : STAGES - 2;
-    if (ahead <= 0) wait_loads_and_sync<0>();
-    else if (ahead == 1) wait_loads_and_sync<LOADS>();
-    else wait_loads_and_sync<2 * LOADS>();
-    // the stage of tile kt - 1 is free now: every wave is past its reads
-    if (kt + STAGES - 1 < k_tiles) issue(kt + STAGES - 1);
-    compute(kt);
   }
 
   // ---- epilogue.  Element e of a 32 x 32 accumulator is row (e / 4) * 8 + (lane / 32) * 4 +
