@@ -108,9 +108,11 @@ class Engine:
         # The engine's work runs on a stream of its own (default priority): a capture cannot
         # record from the default stream.
         self.stream = torch.cuda.Stream(device=self.device)
-        self.use_graphs = use_graphs
+        # a part that looks at host values of a step cannot be replayed
+        self.use_graphs = use_graphs and getattr(model, "graph_safe", False)
+        self.max_graphs = 48     # recorded layouts kept; the least recently made goes first
         self._graphs = {}        # key -> StepGraph
-        self._graph_seen = set()  # keys that ran once without a graph (buffers exist now)
+        self._graph_seen = {}     # layout -> steps that ran without a graph (buffers exist now)
         self._graph_failures = {}
         self.steps = 0
 
@@ -386,31 +388,42 @@ class Engine:
         return output
 
     def _run_step(self, entries, greedy=False) -> StepOutput:
+        """Steps of one layout (numbers of tokens, items, wanted rows, one-token items and
+        query tiles, and how tokens are chosen) issue the same launches with the same
+        arguments: everything else lies in the packed index buffer.  The first step of a
+        layout runs directly (buffers get allocated), the second is recorded as a HIP graph,
+        later ones copy their indices and replay it."""
         items = len(entries)
         mode = 2 if isinstance(greedy, list) else int(bool(greedy))   # how tokens are chosen
         if self.use_graphs and self._graphs:
-            # a captured step: every entry brings one token and wants its logits
-            plan = self._graphs.get((items, mode))
+            # every entry brings one token and wants its logits: the lean path
+            plan = self._graphs.get((items, items, items, items, 0, mode))
             if (plan is not None and plan.logits.data_ptr() == self._logit_buffer(items).data_ptr()
                     and all(len(e.tokens) == 1 and len(e.want) == 1 for e in entries)):
                 return self._replay(plan, entries, greedy)
         ctx, rows, row_keys = self._pack(entries, greedy)
         wanted = len(row_keys)
         logits = self._logit_buffer(wanted)
-        graph_key = None
-        if self.use_graphs and ctx.decode_only and wanted == ctx.tokens:
-            # A step of single tokens that all want their logits.  Every launch argument is
-            # then a function of the number of items (and of buffer addresses).
-            graph_key = (items, mode)
-        if graph_key is None or graph_key in self._graph_failures:
+        singles = ctx.single_tokens.numel()
+        graph_key = (ctx.tokens, items, wanted, singles, ctx.tile_item.numel(), mode)
+        if not self.use_graphs or graph_key in self._graph_failures:
             out, tokens = self._forward(ctx, rows, logits, wanted, greedy)
             return StepOutput(logits=out, rows=row_keys, tokens=tokens)
         # launch shapes inside a graph must not depend on this step's lengths
+        exact_kv_len = ctx.max_kv_len
         ctx.max_kv_len = self.spec.max_positions
-        seen_key = (items, mode, logits.data_ptr())
-        if seen_key not in self._graph_seen:
-            # first time: run directly, so that every buffer exists before a capture
-            self._graph_seen.add(seen_key)
+        plan = self._graphs.get(graph_key)
+        if plan is not None and plan.logits.data_ptr() == logits.data_ptr():
+            # recorded: the indices are on their way already (``_pack`` copied them)
+            plan.graph.launch()
+            return StepOutput(logits=plan.logits[:wanted], rows=row_keys, tokens=plan.tokens)
+        # The first step of a layout runs directly, so that every buffer exists before a
+        # capture.  Recording costs about as much as a few steps: decode layouts come back
+        # at once and are recorded at their second step, others when they keep coming back.
+        seen_key = graph_key + (logits.data_ptr(),)
+        seen = self._graph_seen.get(seen_key, 0)
+        if seen < (1 if singles == ctx.tokens else 3):
+            self._graph_seen[seen_key] = seen + 1
             out, tokens = self._forward(ctx, rows, logits, wanted, greedy)
             return StepOutput(logits=out, rows=row_keys, tokens=tokens)
         from ..ops.kernels import StepGraph
@@ -423,7 +436,7 @@ class Engine:
         except Exception as error:       # the capture is abandoned, the step runs directly
             StepGraph.abort()
             self._graph_failures[graph_key] = f"{type(error).__name__}: {error}"
-            ctx.max_kv_len = max(item.start + 1 for item in ctx.items)
+            ctx.max_kv_len = exact_kv_len
             out, tokens = self._forward(ctx, rows, logits, wanted, greedy)
             return StepOutput(logits=out, rows=row_keys, tokens=tokens)
         offsets, used = self._last_layout
@@ -434,9 +447,12 @@ class Engine:
             for group in range(len(self.cache.groups)):
                 views[f"tables{group}"] = views[f"tables{group}"].reshape(items, self.table_width)
             sections.append(views)
-        old = self._graphs.get(graph_key)
+        old = self._graphs.pop(graph_key, None)
         if old is not None:
             old.graph.destroy()
+        while len(self._graphs) >= self.max_graphs:
+            oldest = next(iter(self._graphs))
+            self._graphs.pop(oldest).graph.destroy()
         self._graphs[graph_key] = _ReplayPlan(graph, used, sections, out, tokens, items)
         graph.launch()
         return StepOutput(logits=out, rows=row_keys, tokens=tokens)

@@ -118,6 +118,13 @@ class DecoderModel:
         return views
 
     # ---------------------------------------------------------------- forward
+    @property
+    def graph_safe(self) -> bool:
+        """Whether a step of this model may be recorded and replayed as a graph: every part
+        says so of itself."""
+        parts = [self.position, self.final_norm] + list(self.blocks)
+        return all(getattr(part, "graph_safe", False) for part in parts)
+
     def forward(self, ctx, views, logit_rows, logits_out):
         """Run the step's tokens; write logits of ``logit_rows`` (int32 indices into the
         step's tokens) into the float tensor ``logits_out``."""

@@ -21,6 +21,8 @@ class Attention(Mixer):
     ``scale`` multiplies the scores (``head_dim**-0.5`` in src/model/paged_attention.py:27).
     """
 
+    graph_safe = True
+
     accepts_pending_norm = True
 
     def __init__(self, width: int, dtype, heads: int, kv_heads: int, head_dim: int, scale: float,

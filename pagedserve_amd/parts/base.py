@@ -61,6 +61,12 @@ class CacheView:
 
 
 class Part:
+    # True when ``forward`` issues the same launches with the same arguments for every step
+    # of one layout (it reads what differs between steps from the step's device tensors
+    # only): such a step may be recorded once and replayed as a graph.  A part that looks at
+    # host values of the step (``ctx.items``, lengths) must leave this False.
+    graph_safe = False
+
     def parameters(self) -> Dict[str, ParamSpec]:
         return {}
 

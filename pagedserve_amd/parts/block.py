@@ -16,6 +16,11 @@ class PreNormBlock:
         self.norm2 = norm2
         self.feed_forward = feed_forward
 
+    @property
+    def graph_safe(self):
+        """The arrangement itself looks at no host value of the step; its parts decide."""
+        return all(getattr(part, "graph_safe", False) for part in self.parts().values())
+
     def parts(self):
         return {"norm1": self.norm1, "mixer": self.mixer, "norm2": self.norm2,
                 "feed_forward": self.feed_forward}

@@ -13,6 +13,8 @@ class DenseFeedForward(FeedForward):
     """``residual += act(x W_up + b_up) W_down + b_down``
     (src/model/paged_decoder.py:178-179,224-228; activations ``:273-280``)."""
 
+    graph_safe = True
+
     accepts_pending_norm = True
 
     def __init__(self, width: int, dtype, inner: int, activation: str, bias: bool = True):

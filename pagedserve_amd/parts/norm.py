@@ -11,6 +11,8 @@ class LayerNorm(Norm):
     """(h - mean) / sqrt(var + eps) * gamma + beta with the biased variance
     (src/model/paged_decoder.py:170-177; src/kernels/triton_residual_layernorm.py:25-39)."""
 
+    graph_safe = True
+
     def __init__(self, width: int, dtype, eps: float):
         self.width = width
         self.dtype = dtype
@@ -29,6 +31,8 @@ class LayerNorm(Norm):
 @register_norm("rmsnorm")
 class RMSNorm(Norm):
     """h / sqrt(mean(h^2) + eps) * gamma.  Not used by GPT-2; the kernel's second mode."""
+
+    graph_safe = True
 
     def __init__(self, width: int, dtype, eps: float):
         self.width = width

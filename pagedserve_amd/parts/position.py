@@ -11,6 +11,8 @@ class LearnedAbsolutePositions(PositionEncoding):
     (src/model/paged_decoder.py:289,311-313).  Positions must lie in ``[0, max_positions)``
     (src/model/paged_decoder.py:519-522)."""
 
+    graph_safe = True
+
     def __init__(self, width: int, dtype, max_positions: int):
         self.width = width
         self.dtype = dtype
@@ -26,6 +28,8 @@ class LearnedAbsolutePositions(PositionEncoding):
 @register_position("none")
 class NoPositions(PositionEncoding):
     """Nothing is added and nothing is rotated."""
+
+    graph_safe = True
 
     def __init__(self, width: int, dtype, max_positions: int = 0):
         self.width = width

@@ -169,3 +169,50 @@ def test_graph_replay_matches_direct_launches(folders, references, dtype):
     assert outputs[True].keys() == outputs[False].keys()
     worst = max(float((outputs[True][key] - outputs[False][key]).abs().max()) for key in outputs[True])
     assert worst <= helpers.TOLERANCE[dtype] * 0.2 * float(reference["r4"].abs().max())
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_graph_replay_of_mixed_steps(folders, references, dtype):
+    """Steps of one layout that are no pure decode steps (a prompt portion beside a decoded
+    token and a two-token portion) are recorded after they have come back a few times; every
+    replay gives the logits of the plain computation, with other layouts and a finished
+    request's reused pages between the replays."""
+    from pagedserve_amd.engine import Engine, StepEntry
+    from pagedserve_amd.model import load_model
+
+    folder, config, page_size = folders["B"]
+    requests = _requests("B", config)
+    model, _ = load_model(folder, dtype=dtype)
+    engine = Engine(model, num_pages=30, page_size=page_size, max_requests=4, max_step_tokens=128)
+    rows = {}
+
+    def run(entries):
+        out = engine.step(entries)
+        values = out.logits.double().cpu()
+        for index, key in enumerate(out.rows):
+            rows[key] = values[index]
+
+    cursor = {"r4": 0, "r3": 0, "r2": 0}
+    run([StepEntry("r3", requests["r3"][:11], list(range(11)))])
+    cursor["r3"] = 11
+    replays_before = 0
+    for turn in range(12):
+        # the same layout every turn: 7 tokens of r4's prompt, 1 token of r3, 2 tokens of r2
+        entries = [StepEntry("r4", requests["r4"][cursor["r4"]:cursor["r4"] + 7], [0, 6]),
+                   StepEntry("r3", [requests["r3"][cursor["r3"]]], [0]),
+                   StepEntry("r2", requests["r2"][cursor["r2"]:cursor["r2"] + 2], [1])]
+        run(entries)
+        cursor["r4"] += 7
+        cursor["r3"] += 1
+        cursor["r2"] += 2
+        if turn == 6:    # another layout, and pages that change hands, between two replays
+            run([StepEntry("r1", requests["r1"][:9], list(range(9)))])
+            engine.finish("r1")
+            run([StepEntry("r0", requests["r0"][:1], [0])])
+            engine.finish("r0")
+    summary = engine.graph_summary()
+    assert summary["captured_graphs"] >= 1 and summary["graph_replays"] >= 6, summary
+    assert not summary["capture_failures"], summary
+    error, scale, where = helpers.max_error(rows, references[("B", dtype == "bfloat16")])
+    assert error <= helpers.TOLERANCE[dtype] * scale, (error, scale, where)
+    engine.cache.check_invariants()
