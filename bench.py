@@ -87,8 +87,10 @@ def decode_run(engine, sampler, config, batch, context_end, steps, warmup, seed=
     return elapsed, mean_context
 
 
-def prefill_run(engine, config, reps=5, warmup=2, seed=1):
-    """Seconds per step of 2 x 1024 prompt tokens (logits at each prompt's last token)."""
+def prefill_run(engine, config, reps=8, warmup=5, seed=1):
+    """Seconds per step of 2 x 1024 prompt tokens (logits at each prompt's last token), in the
+    steady state: the warm-up covers the steps that allocate buffers and record the layout's
+    graph."""
     import torch
 
     from pagedserve_amd.engine import StepEntry
@@ -156,7 +158,7 @@ def main(argv=None):
                                      layers=args.layers)
     context = config.n_positions
     if args.prefill_only:
-        seconds = prefill_run(engine, config, reps=args.steps, warmup=min(args.warmup, 2))
+        seconds = prefill_run(engine, config, reps=args.steps, warmup=max(min(args.warmup, 8), 5))
         flops = step_flops(config, [PREFILL_TOKENS // 2] * 2, 2)
         print(json.dumps({"prefill": {
             "value": round(PREFILL_TOKENS / seconds, 1), "tokens": PREFILL_TOKENS,

@@ -83,6 +83,19 @@ class PagePool:
         self.peak_allocated = max(self.peak_allocated, self.num_allocated)
         return page
 
+    def allocate_many(self, count: int) -> List[int]:
+        """``count`` pages in the order that ``allocate`` would hand them out."""
+        if count > len(self.free_pages):
+            raise CacheFull("KV cache full")
+        pages = self.free_pages[len(self.free_pages) - count:][::-1]
+        del self.free_pages[len(self.free_pages) - count:]
+        for page in pages:
+            if self._held[page]:
+                raise AssertionError(f"page {page} was on the free list while held")
+            self._held[page] = True
+        self.peak_allocated = max(self.peak_allocated, self.num_allocated)
+        return pages
+
     def free(self, page: int):
         if not 0 <= page < self.num_pages:
             raise ValueError(f"page {page} does not exist")
@@ -223,19 +236,21 @@ class CacheManager:
         if self.max_positions is not None and new_length > self.max_positions:
             raise ValueError(
                 f"request {request_id!r} would reach {new_length} positions, the model has {self.max_positions}")
-        taken: List[Tuple[int, int]] = []
-        try:
-            for group_index, missing in enumerate(self.pages_missing(request_id, new_length)):
-                for _ in range(missing):
-                    taken.append((group_index, self.pools[group_index].allocate()))
-        except CacheFull:
-            for group_index, page in reversed(taken):
-                self.pools[group_index].free(page)
-            raise
-        for group_index, page in taken:
-            record.tables[group_index].append(page)
+        missing = self.pages_missing(request_id, new_length)
+        if not any(missing):
+            return
+        for group_index, count in enumerate(missing):
+            if count > self.pools[group_index].num_free:
+                raise CacheFull("KV cache full")      # nothing has been taken yet
+        for group_index, count in enumerate(missing):
+            if count == 0:
+                continue
+            pages = self.pools[group_index].allocate_many(count)
+            table = record.tables[group_index]
+            first = len(table)
+            table.extend(pages)
             if self.table_arrays is not None:
-                self.table_arrays[group_index][record.slot, len(record.tables[group_index]) - 1] = page
+                self.table_arrays[group_index][record.slot, first:first + count] = pages
 
     def commit(self, request_id: Hashable, new_length: int):
         """The step that wrote positions ``< new_length`` succeeded."""

@@ -160,7 +160,14 @@ class Engine:
             count = len(entry.tokens)
             if count == 0:
                 raise StepError(f"request {entry.request_id!r} brings no tokens")
-            if min(entry.tokens) < 0 or max(entry.tokens) >= vocab:
+            if count > 16:
+                # long portions are checked (and later packed) as arrays, converted once
+                if not isinstance(entry.tokens, np.ndarray):
+                    entry.tokens = np.asarray(entry.tokens, dtype=np.int64)
+                low, high = int(entry.tokens.min()), int(entry.tokens.max())
+            else:
+                low, high = min(entry.tokens), max(entry.tokens)
+            if low < 0 or high >= vocab:
                 raise StepError(f"a token of request {entry.request_id!r} is outside "
                                 f"the vocabulary of {vocab}")
             if entry.carry is not None and (count != 1 or not 0 <= entry.carry < self._carried_rows):
