@@ -1,14 +1,16 @@
 // Matrix products on the matrix cores (MFMA) of gfx950:  C[m, n] = epi(sum_k A[m, k] W[n, k] + b[n]).
 //
-// Two kernels.
+// Three kernels (the tiled bfloat16 product for many rows with k a multiple of 64 is a file of
+// its own, gemm_tiled_bf16.hip; this file dispatches to it).
 //
-// gemm_nt_tiled_kernel — many rows (prompt portions).  128 x 128 outputs per 256-thread block,
-//   four waves in a 2 x 2 arrangement, each wave 2 x 2 tiles of 32 x 32.  A and W tiles of 64
-//   bytes of k per row go global -> registers -> LDS (two buffers, one barrier per k tile);
-//   every lane reads 16 bytes of k for its row from LDS.  For bfloat16 that is the operand of
-//   one v_mfma_f32_32x32x16_bf16; for float the four values feed four v_mfma_f32_32x32x2_f32
-//   (both operands use the same assignment of k to lanes and instructions, which is all a dot
-//   product needs).  The float instantiation multiplies true 32-bit inputs.
+// gemm_nt_tiled_kernel — many rows in float32, and bfloat16 shapes the other tiled kernel does
+//   not take.  128 x 128 outputs per 256-thread block, four waves in a 2 x 2 arrangement, each
+//   wave 2 x 2 tiles of 32 x 32.  A and W tiles of 64 bytes of k per row go global ->
+//   registers -> LDS (two buffers, one barrier per k tile); every lane reads 16 bytes of k for
+//   its row from LDS.  For bfloat16 that is the operand of one v_mfma_f32_32x32x16_bf16; for
+//   float the four values feed four v_mfma_f32_32x32x2_f32 (both operands use the same
+//   assignment of k to lanes and instructions, which is all a dot product needs).  The float
+//   instantiation multiplies true 32-bit inputs.
 //
 // gemm_nt_skinny_kernel — up to 64 rows (decode), bfloat16.  The product is bound by reading W
 //   once, and at these sizes by the latency of that one trip to memory, so weights go straight
@@ -22,11 +24,11 @@
 //
 // gemm_nt_skinny_norm_kernel — the skinny kernel for up to 16 rows with the norm of its input
 //   fused in front: while the block's weight loads are in flight, each wave normalises four of
-//   the float input rows in registers (statistics by shuffles, as the norm kernel) and leaves
+//   the float input rows in registers (statistics by lane exchanges, as the norm kernel) and leaves
 //   them in LDS as bfloat16; the product then reads its column operand from LDS.  One launch
 //   and one trip to memory instead of two launches.
 //
-// Both kernels can also store the key and value columns of a [q | k | v] output into cache
+// All of them can also store the key and value columns of a [q | k | v] output into cache
 // pages from their epilogue (KvScatter).
 //
 // Accumulation is float in all cases.  Shapes that the kernels cannot take (k not a multiple
