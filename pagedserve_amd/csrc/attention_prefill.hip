@@ -88,11 +88,12 @@ __global__ __launch_bounds__(128 * KS) void attention_prefill_kernel(
   const int wave_k = wave >> 1;  // which run of 32 keys of every tile
   const int sub = lane & 31;     // query of this lane within the wave; key or dimension row
   const int half = lane >> 5;    // which half of a step's reduction dimension
-  const int head = blockIdx.y;
+  const int head = blockIdx.x;
   const int kv_head = head / (heads / kv_heads);
 
-  // later tiles of a request see more keys: start them first
-  const int tile_index = gridDim.x - 1 - blockIdx.x;
+  // blocks start in the order of their numbers, heads fastest: the caller lists the tiles that
+  // see the most keys first, so the longest blocks start first and the shortest fill the gaps
+  const int tile_index = blockIdx.y;
   const int item = tile_item[tile_index];
   const int q0 = tile_q0[tile_index];
   const int tok0 = cu_tokens[item];
@@ -396,7 +397,7 @@ extern "C" int ps_attention_prefill(const void* q, int64_t q_stride, const void*
                                     const int* cu_tokens, const int* kv_lens, const int* tables,
                                     int table_width, int heads, int kv_heads, int head_dim,
                                     int page_size, int num_pages, float scale, int window,
-                                    int dtype, void* stream) {
+                                    int max_kv_len, int dtype, void* stream) {
   PS_REQUIRE(tiles >= 0 && heads > 0 && kv_heads > 0 && page_size > 0 && num_pages > 0 &&
                  table_width > 0,
              "ps_attention_prefill: bad sizes");
@@ -405,7 +406,7 @@ extern "C" int ps_attention_prefill(const void* q, int64_t q_stride, const void*
              "ps_attention_prefill: heads (%d) must be a multiple of kv_heads (%d)", heads, kv_heads);
   PS_REQUIRE(head_dim > 0 && head_dim % 16 == 0 && head_dim <= 128,
              "ps_attention_prefill: head_dim %d must be a multiple of 16 up to 128", head_dim);
-  PS_REQUIRE(window >= 0 && heads <= 65535, "ps_attention_prefill: bad window or head count");
+  PS_REQUIRE(window >= 0 && tiles <= 65535, "ps_attention_prefill: bad window or too many tiles (%d)", tiles);
   PS_REQUIRE(scale > 0.f, "ps_attention_prefill: the score scale must be positive, got %g", scale);
   PS_REQUIRE(table_width <= AP_TABLE_MAX,
              "ps_attention_prefill: block tables of %d pages exceed the %d that a tile keeps",
@@ -420,10 +421,11 @@ extern "C" int ps_attention_prefill(const void* q, int64_t q_stride, const void*
     while ((1 << page_shift) < page_size) ++page_shift;
   }
   hipStream_t s = (hipStream_t)stream;
-  dim3 grid(tiles, heads);
+  dim3 grid(heads, tiles);
   // With few blocks each takes a compute unit for itself, and four waves along the keys
-  // shorten the longest block; with many, smaller blocks that share a unit balance better.
-  const bool wide = (int64_t)tiles * heads <= 256;
+  // shorten the longest block (if the caller knows of no long context, that does not pay);
+  // with many, smaller blocks that share a unit balance better.
+  const bool wide = (int64_t)tiles * heads <= 256 && (max_kv_len <= 0 || max_kv_len >= 512);
 #define PS_LAUNCH_AP(NDB)                                                                       \
   do {                                                                                          \
     if (wide)                                                                                   \

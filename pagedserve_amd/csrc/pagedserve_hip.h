@@ -97,12 +97,15 @@ int ps_attention_decode(const void* q, int64_t q_stride, const void* k_pool, con
 
 // Tiled attention on the matrix cores for items that bring several tokens (bfloat16, head_dim a
 // multiple of 16 up to 128).  Tile i covers queries tile_q0[i] .. tile_q0[i] + 63 of item
-// tile_item[i]; cu_tokens and kv_lens describe the step's items.
+// tile_item[i]; cu_tokens and kv_lens describe the step's items.  Blocks start in the order of
+// the list (all heads of tile 0, then of tile 1, ...): list the tiles that see the most keys first.
+// max_kv_len: no query sees more keys than that (0: unknown); it only steers the launch shape.
 int ps_attention_prefill(const void* q, int64_t q_stride, const void* k_pool, const void* v_pool,
                          void* out, int64_t out_stride, const int* tile_item, const int* tile_q0,
                          int tiles, const int* cu_tokens, const int* kv_lens, const int* tables,
                          int table_width, int heads, int kv_heads, int head_dim, int page_size,
-                         int num_pages, float scale, int window, int dtype, void* stream);
+                         int num_pages, float scale, int window, int max_kv_len, int dtype,
+                         void* stream);
 
 // tokens[r] = argmax (inv_temperature[r] == 0) or a draw from softmax(logits * inv_temperature[r])
 // by inverse CDF at uniform[r] in [0, 1).

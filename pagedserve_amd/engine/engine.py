@@ -334,6 +334,13 @@ class Engine:
                 step_items.append(StepItem(entry.request_id, record.slot, start, count, flat))
                 flat += count
             cu[items] = flat
+            if tile_cursor > 1:
+                # tiles that see the most keys first: the kernel's blocks start in this order,
+                # and the longest should not be the last to start
+                keys = np.asarray(starts, dtype=np.int64)[tile_item] + tile_q0
+                order = np.argsort(-keys, kind="stable")
+                tile_item[:] = tile_item[order]
+                tile_q0[:] = tile_q0[order]
         if isinstance(select, list):
             section("inv_temperature").view(np.float32)[:] = [a for a, _ in select]
             section("uniform").view(np.float32)[:] = [b for _, b in select]

@@ -37,7 +37,7 @@ _SIGNATURES = {
                             c_void_p],
     "ps_attention_prefill": [c_void_p, c_int64, c_void_p, c_void_p, c_void_p, c_int64, c_void_p,
                              c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int,
-                             c_int, c_int, c_int, c_float, c_int, c_int, c_void_p],
+                             c_int, c_int, c_int, c_float, c_int, c_int, c_int, c_void_p],
     "ps_sample": [c_void_p, c_int64, c_void_p, c_void_p, c_void_p, c_int, c_int, c_void_p],
 }
 
@@ -415,8 +415,10 @@ def prefill_supported(dtype, head_dim, table_width=0) -> bool:
 
 
 def attention_prefill(q, k_pool, v_pool, out, tile_item, tile_q0, cu_tokens, kv_lens, tables,
-                      heads, scale, window=0):
-    """Attention of items with several tokens, 64 queries per block, on the matrix cores."""
+                      heads, scale, window=0, max_kv_len=0):
+    """Attention of items with several tokens, 64 queries per block, on the matrix cores.
+    Blocks start in the order of the tile list: the tiles that see the most keys belong first.
+    ``max_kv_len`` (no query sees more keys; 0 = unknown) only steers the launch shape."""
     _check(q, "q", torch.bfloat16, 2)
     _check(out, "out", torch.bfloat16, 2)
     pages, kv_heads, page_size, head_dim = _check_pools(k_pool, v_pool, q.dtype)
@@ -438,8 +440,8 @@ def attention_prefill(q, k_pool, v_pool, out, tile_item, tile_q0, cu_tokens, kv_
     _call("ps_attention_prefill", q.data_ptr(), q_stride, k_pool.data_ptr(), v_pool.data_ptr(),
           out.data_ptr(), out_stride, tile_item.data_ptr(), tile_q0.data_ptr(), tiles,
           cu_tokens.data_ptr(), kv_lens.data_ptr(), tables.data_ptr(), tables.shape[1], heads,
-          kv_heads, head_dim, page_size, pages, float(scale), int(window), dtype_code(q.dtype),
-          _stream())
+          kv_heads, head_dim, page_size, pages, float(scale), int(window), int(max_kv_len),
+          dtype_code(q.dtype), _stream())
     return out
 
 

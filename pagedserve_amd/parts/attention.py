@@ -102,7 +102,8 @@ class Attention(Mixer):
         if singles < tokens and kernels.prefill_supported(self.dtype, self.head_dim, tables.shape[1]):
             kernels.attention_prefill(q, cache.k_pool, cache.v_pool, context, ctx.tile_item,
                                       ctx.tile_q0, ctx.cu_tokens, ctx.kv_lens, tables,
-                                      self.heads, self.scale, self.window)
+                                      self.heads, self.scale, self.window,
+                                      max_kv_len=ctx.max_kv_len)
         elif singles < tokens:
             kernels.attention_rowwise(q, cache.k_pool, cache.v_pool, context, ctx.tok_item,
                                       ctx.positions, tables, self.heads, self.scale, self.window,
