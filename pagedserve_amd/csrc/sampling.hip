@@ -3,7 +3,8 @@
 // softmax(logits / temperature) by inverse CDF.  The uniform number of a row is made by the
 // host from (seed, request, step), so a draw does not depend on what else is in the batch.
 //
-// One 1024-thread block per row.  The maximum is found with coalesced strided reads.  For a
+// One 1024-thread block per row.  The maximum is found with coalesced strided reads, sixteen
+// of them in flight per thread.  For a
 // draw, wave w owns the contiguous id range [w * seg, (w + 1) * seg): it sums
 // exp((l - max) / T) over its range 64 ids at a time, thread 0 picks the range that holds
 // uniform * total, and that wave walks its range again with a prefix sum over each 64 ids to
@@ -15,6 +16,7 @@
 
 #define SM_THREADS 1024
 #define SM_WAVES (SM_THREADS / 64)
+#define SM_LOADS 16   // a row of 16,384 logits is one trip to memory for the maximum
 
 __global__ __launch_bounds__(SM_THREADS) void sample_kernel(
     const float* __restrict__ logits, int64_t ld, const float* __restrict__ inv_temperature,
@@ -35,15 +37,15 @@ __global__ __launch_bounds__(SM_THREADS) void sample_kernel(
   // maximum and its first index
   float best = -INFINITY;
   int best_idx = vocab;
-  for (int i0 = tid; i0 < vocab; i0 += 4 * SM_THREADS) {
-    float v[4];
+  for (int i0 = tid; i0 < vocab; i0 += SM_LOADS * SM_THREADS) {
+    float v[SM_LOADS];
 #pragma unroll
-    for (int u = 0; u < 4; ++u) {   // four loads in flight, index clamped, masked below
+    for (int u = 0; u < SM_LOADS; ++u) {   // all loads in flight, index clamped, masked below
       const int i = i0 + u * SM_THREADS;
       v[u] = row[i < vocab ? i : vocab - 1];
     }
 #pragma unroll
-    for (int u = 0; u < 4; ++u) {
+    for (int u = 0; u < SM_LOADS; ++u) {
       const int i = i0 + u * SM_THREADS;
       if (i < vocab && v[u] > best) {
         best = v[u];
