@@ -288,3 +288,78 @@ def test_uniform_numbers_are_a_function_of_seed_request_and_index():
     assert float(torch.tensor(values, dtype=torch.float32).max()) < 1.0
     with pytest.raises(ValueError):
         SamplingParams(temperature=-1)
+
+
+class ChoosingEngine(FakeEngine):
+    """The stand-in with what running ahead needs: it chooses tokens itself, hands them over
+    only when asked (as a copy that is "on its way"), and resolves entries that carry on a
+    row of the last step instead of a token id."""
+
+    supports_draws = True
+
+    def __init__(self, **kwargs):
+        super().__init__(**kwargs)
+        self.last_tokens = []
+        self.outstanding = 0      # steps whose tokens nobody has read yet
+        self.most_outstanding = 0
+
+    def step(self, entries, greedy=False, draws=None):
+        assert greedy or draws is not None
+        for entry in entries:
+            if entry.carry is not None:
+                assert len(entry.tokens) == 1 and 0 <= entry.carry < len(self.last_tokens)
+                entry.tokens = [self.last_tokens[entry.carry]]
+        output = super().step(entries)
+        tokens = output.logits.argmax(-1)
+        self.last_tokens = tokens.tolist()
+        self.outstanding += 1
+        self.most_outstanding = max(self.most_outstanding, self.outstanding)
+        engine = self
+
+        class Ready:
+            def synchronize(self_inner):
+                engine.outstanding -= 1
+
+        output.tokens = tokens
+        output.host_tokens = tokens.clone()
+        output.ready = Ready()
+        return output
+
+
+@pytest.mark.parametrize("run_ahead", [False, True])
+def test_running_ahead_decisions(run_ahead):
+    """While all requests decode and nobody waits, the next iteration is launched before the
+    last one's tokens are read: requests that end by length are left out of it, one that meets
+    the end token gets its extra token dropped, a newcomer stops it until its prompt is in.
+    Tokens and finish reasons are those of the step-by-step run."""
+    end_token = expected_tokens([3, 1, 4], 9)[5]
+    prompts = {"a": [3, 1, 4], "b": [2, 7], "c": [9, 9, 9, 9], "late": [5, 6]}
+    budgets = {"a": 9, "b": 4, "c": 12, "late": 6}
+    engine = ChoosingEngine()
+    scheduler = ContinuousBatchScheduler(engine, ArgmaxSampler(), tokenizer=None, max_batch_size=8,
+                                         eos_token_id=end_token, run_ahead=run_ahead)
+    ids = {name: scheduler.add_token_request(prompts[name], budgets[name]) for name in ("a", "b", "c")}
+    streamed = {}
+    steps = 0
+    while scheduler.has_work():
+        if steps == 6:
+            ids["late"] = scheduler.add_token_request(prompts["late"], budgets["late"])
+        for rid, token in scheduler.step().items():
+            streamed.setdefault(rid, []).append(token)
+        steps += 1
+    for name, rid in ids.items():
+        free_run = expected_tokens(prompts[name], budgets[name])
+        cut = free_run.index(end_token) + 1 if end_token in free_run else len(free_run)
+        request = scheduler.finished[rid]
+        assert request.generated_token_ids == free_run[:cut], name
+        assert streamed[rid] == free_run[:cut]
+        assert request.finish_reason == ("stop" if cut < len(free_run) or free_run[-1] == end_token else "length")
+    assert scheduler.finished[ids["a"]].finish_reason == "stop"      # the end token really came
+    assert not engine.cache.requests and scheduler.reserved_blocks == [0]
+    if run_ahead:
+        assert scheduler.steps_run_ahead >= 5 and engine.most_outstanding == 2
+        # no step carried a request on after its last token by length
+        for step in engine.steps:
+            assert len(step) <= 4
+    else:
+        assert scheduler.steps_run_ahead == 0 and engine.most_outstanding == 1
