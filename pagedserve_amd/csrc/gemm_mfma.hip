@@ -241,8 +241,8 @@ __global__ __launch_bounds__(256) void gemm_nt_tiled_kernel(
 // Sum the four waves' partial tiles and finish element (row sub, column n0 + group*4 + wave).
 template <typename TOut, int EPI, int MB>
 __device__ inline void skinny_epilogue(float (*partial)[MB][4][64], const float* bias, TOut* c,
-                                       int m, int n, int ldc, int n0, int split, int k_splits,
-                                       const KvScatter& scatter) {
+                                       int m, int n, int ldc, int n0, int row0, int split,
+                                       int k_splits, const KvScatter& scatter) {
   const int lane = threadIdx.x & 63;
   const int i = threadIdx.x >> 6;
   const int sub = lane & 15;
@@ -251,7 +251,7 @@ __device__ inline void skinny_epilogue(float (*partial)[MB][4][64], const float*
   if (col >= n) return;
 #pragma unroll
   for (int b = 0; b < MB; ++b) {
-    const int row = b * 16 + sub;
+    const int row = row0 + b * 16 + sub;
     if (row >= m) continue;
     float v = partial[0][b][i][lane] + partial[1][b][i][lane] + partial[2][b][i][lane] +
               partial[3][b][i][lane];
@@ -281,6 +281,7 @@ __global__ __launch_bounds__(64 * SK_WAVES) void gemm_nt_skinny_kernel(
   const int wave = threadIdx.x >> 6;
   const int n0 = blockIdx.x * 16;
   const int split = blockIdx.y;
+  const int row0 = blockIdx.z * (MB * 16);
   const int k_begin = split * k_chunk;
   const int k_end = k_begin + k_chunk < k ? k_begin + k_chunk : k;
   const int sub = lane & 15;
@@ -290,7 +291,7 @@ __global__ __launch_bounds__(64 * SK_WAVES) void gemm_nt_skinny_kernel(
   const bf16_t* a_ptr[MB];
 #pragma unroll
   for (int b = 0; b < MB; ++b) {
-    const int row = b * 16 + sub < m ? b * 16 + sub : m - 1;
+    const int row = row0 + b * 16 + sub < m ? row0 + b * 16 + sub : m - 1;
     a_ptr[b] = a + (int64_t)row * lda + group * 16;
   }
   f32x4 acc[MB];
@@ -346,7 +347,7 @@ __global__ __launch_bounds__(64 * SK_WAVES) void gemm_nt_skinny_kernel(
     for (int i = 0; i < 4; ++i) partial[wave][b][i][lane] = acc[b][i];
   __syncthreads();
   // element i of a 16 x 16 accumulator: weight row (lane / 16) * 4 + i, activation row lane % 16
-  skinny_epilogue<TOut, EPI, MB>(partial, bias, c, m, n, ldc, n0, split, k_splits, scatter);
+  skinny_epilogue<TOut, EPI, MB>(partial, bias, c, m, n, ldc, n0, row0, split, k_splits, scatter);
 }
 
 // ---------------------------------------------------------------- skinny with fused norm
@@ -488,7 +489,7 @@ __global__ __launch_bounds__(64 * SK_WAVES) void gemm_nt_skinny_norm_kernel(
 #pragma unroll
   for (int i = 0; i < 4; ++i) partial[wave][0][i][lane] = acc[i];
   __syncthreads();
-  skinny_epilogue<TOut, EPI, 1>(partial, bias, c, m, n, ldc, n0, 0, 1, scatter);
+  skinny_epilogue<TOut, EPI, 1>(partial, bias, c, m, n, ldc, n0, 0, 0, 1, scatter);
 }
 
 // --------------------------------------------------------------------------------- host
@@ -551,16 +552,24 @@ template <typename TOut, int EPI>
 static void launch_skinny_mb(const void* a, const void* w, const float* bias, void* c, int m,
                              int n, int k, int lda, int ldc, int k_chunk, int k_splits,
                              const KvScatter& scatter, hipStream_t s) {
-  dim3 grid((n + 15) / 16, k_splits);
+  // Rows go 16 to an accumulator, up to four accumulators to a block.  Where the columns and
+  // the k ranges give few blocks, the rows are spread over more of them (every one reads the
+  // same weights, which the L2 absorbs; blocks that differ only in z run on one XCD when the
+  // number of column blocks is a multiple of 8).
+  const int row_blocks = (m + 15) / 16;
+  const int grid_xy = ((n + 15) / 16) * k_splits;
+  int z = 256 / grid_xy;
+  z = z < 1 ? 1 : (z > row_blocks ? row_blocks : z);
+  const int per = (row_blocks + z - 1) / z;
+  dim3 grid((n + 15) / 16, k_splits, (row_blocks + per - 1) / per);
   dim3 block(64 * SK_WAVES);
 #define PS_LAUNCH_SK(MB)                                                                       \
   hipLaunchKernelGGL((gemm_nt_skinny_kernel<TOut, EPI, MB>), grid, block, 0, s,                \
                      (const bf16_t*)a, (const bf16_t*)w, bias, (TOut*)c, m, n, k, lda, ldc,    \
                      k_chunk, k_splits, scatter)
-  const int blocks = (m + 15) / 16;
-  if (blocks <= 1) PS_LAUNCH_SK(1);
-  else if (blocks == 2) PS_LAUNCH_SK(2);
-  else if (blocks == 3) PS_LAUNCH_SK(3);
+  if (per <= 1) PS_LAUNCH_SK(1);
+  else if (per == 2) PS_LAUNCH_SK(2);
+  else if (per == 3) PS_LAUNCH_SK(3);
   else PS_LAUNCH_SK(4);
 #undef PS_LAUNCH_SK
 }
@@ -629,7 +638,10 @@ int ps_gemm_nt_mfma(const void* a, const void* w, const float* bias, void* c, in
   // Up to 64 rows the skinny kernel has every load of a block in flight at once, which counts
   // when the weights come from memory and not from a cache; the tiled kernel walks k tile by
   // tile and wins only where there are tiles enough to fill the chip (the output head).
-  const bool skinny_k = m <= 64 && n < 64 * 256;
+  // A k beyond one round of the skinny kernel's loads makes it loop; there the tiled kernel
+  // with its deep ring of stages is ahead, except where partial sums of a split k can be
+  // added in place (residual epilogue), which keeps every block at one round.
+  const bool skinny_k = m <= 64 && n < 64 * 256 && (epilogue == PS_EPI_RESIDUAL || k <= 1024);
   if (dtype == PS_BF16 && m <= 64 && (skinny_k || !ps_gemm_nt_bf16_tiled_supported(a, w, m, k, lda))) {
     if (c_dtype == PS_F32)
       return launch_skinny<float>(a, w, bias, c, m, n, k, lda, ldc, epilogue, scatter, s);

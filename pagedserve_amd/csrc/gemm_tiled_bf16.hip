@@ -67,6 +67,18 @@ __device__ inline void wait_loads_and_sync() {
   asm volatile("s_waitcnt vmcnt(%0)\n\ts_barrier" ::"n"(PENDING) : "memory");
 }
 
+// The same with `ahead` tiles (known only at run time) of LOADS loads each left in flight.
+template <int LOADS, int MOST>
+__device__ inline void wait_ahead_and_sync(int ahead) {
+  if (ahead <= 0) wait_loads_and_sync<0>();
+  else if (ahead == 1 || MOST == 1) wait_loads_and_sync<LOADS>();
+  else if (ahead == 2 || MOST == 2) wait_loads_and_sync<2 * LOADS>();
+  else if (ahead == 3 || MOST == 3) wait_loads_and_sync<(MOST >= 3 ? 3 : 0) * LOADS>();
+  else if (ahead == 4 || MOST == 4) wait_loads_and_sync<(MOST >= 4 ? 4 : 0) * LOADS>();
+  else if (ahead == 5 || MOST == 5) wait_loads_and_sync<(MOST >= 5 ? 5 : 0) * LOADS>();
+  else wait_loads_and_sync<(MOST >= 6 ? 6 : 0) * LOADS>();
+}
+
 template <int WM, int WN, int STAGES, typename TOut, int EPI>
 __global__ __launch_bounds__(256) void gemm_nt_bf16_tiled_kernel(
     const bf16_t* __restrict__ a, const bf16_t* __restrict__ w, const float* __restrict__ bias,
@@ -77,7 +89,7 @@ __global__ __launch_bounds__(256) void gemm_nt_bf16_tiled_kernel(
   constexpr int LOADS_A = BM / 32;   // load instructions per wave and stage (8 rows each)
   constexpr int LOADS_W = BN / 32;
   constexpr int LOADS = LOADS_A + LOADS_W;
-  static_assert(STAGES >= 2 && STAGES <= 4, "two to four stages");
+  static_assert(STAGES >= 2 && STAGES <= 8, "two to eight stages");
   static_assert(LOADS * (STAGES - 1) < 64, "the load counter has six bits");
   __shared__ __attribute__((aligned(1024))) unsigned char lds[STAGES * STAGE_BYTES];
 
@@ -167,9 +179,7 @@ __global__ __launch_bounds__(256) void gemm_nt_bf16_tiled_kernel(
   {
     // tile 0 has landed; tiles 1 .. STAGES - 2 may stay in flight, as far as they exist
     const int ahead = k_tiles - 1 < STAGES - 2 ? k_tiles - 1 : STAGES - 2;
-    if (ahead <= 0) wait_loads_and_sync<0>();
-    else if (ahead == 1) wait_loads_and_sync<LOADS>();
-    else wait_loads_and_sync<2 * LOADS>();
+    wait_ahead_and_sync<LOADS, STAGES - 2>(ahead);
   }
   fetch(0, 0, fa[0], fw[0]);
   for (int kt = 0; kt < k_tiles; ++kt) {
@@ -184,10 +194,7 @@ __global__ __launch_bounds__(256) void gemm_nt_bf16_tiled_kernel(
         asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
         // tiles kt + 2 .. kt + STAGES - 1 may stay in flight, as far as they exist
         const int last = k_tiles - 1 < kt + STAGES - 1 ? k_tiles - 1 : kt + STAGES - 1;
-        const int ahead = last - (kt + 1);
-        if (ahead <= 0) wait_loads_and_sync<0>();
-        else if (ahead == 1) wait_loads_and_sync<LOADS>();
-        else wait_loads_and_sync<2 * LOADS>();
+        wait_ahead_and_sync<LOADS, STAGES - 2>(last - (kt + 1));
         fetch(kt + 1, 0, fa[0], fw[0]);
       }
 #pragma unroll
@@ -358,7 +365,10 @@ static int launch_variant(const void* a, const void* w, const float* bias, void*
 
 // Tile shapes by the number of blocks they give: the chip has 256 compute units, and a product
 // of this size is over in a few microseconds, so filling them counts for more than the reuse
-// inside a large tile.  Long k with few tiles takes deeper prefetch instead.
+// inside a large tile.  Long k with few tiles takes deeper prefetch instead: a block that is
+// alone on its compute unit needs many tiles in flight to keep its share of the memory
+// system busy (eight stages for one row of tiles over a long k, which is a decode step of a
+// wide model).
 template <typename TOut>
 static int launch_tiled_bf16(const void* a, const void* w, const float* bias, void* c, int m,
                              int n, int k, int lda, int ldc, int epilogue,
@@ -369,6 +379,8 @@ static int launch_tiled_bf16(const void* a, const void* w, const float* bias, vo
     return launch_variant<2, 2, 2, TOut>(a, w, bias, c, m, n, k, lda, ldc, epilogue, scatter, s);
   if (m > 64 && tiles_128_64 >= 384)
     return launch_variant<2, 1, 2, TOut>(a, w, bias, c, m, n, k, lda, ldc, epilogue, scatter, s);
+  if (m <= 64 && k > 1024 && (int64_t)((n + 63) / 64) <= 256)
+    return launch_variant<1, 1, 8, TOut>(a, w, bias, c, m, n, k, lda, ldc, epilogue, scatter, s);
   if (k >= 2048)
     return launch_variant<1, 1, 4, TOut>(a, w, bias, c, m, n, k, lda, ldc, epilogue, scatter, s);
   return launch_variant<1, 1, 2, TOut>(a, w, bias, c, m, n, k, lda, ldc, epilogue, scatter, s);
