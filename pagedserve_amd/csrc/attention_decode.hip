@@ -50,15 +50,29 @@ struct Raw8<bf16_t> {
   }
 };
 
-// Merge the online-softmax state (m, l, acc) with another one.
-__device__ inline void merge_state(float& m, float& l, float* acc, float m_o, float l_o,
-                                   const float* acc_o, int n) {
-  const float m_n = fmaxf(m, m_o);
-  const float c1 = (m == -INFINITY) ? 0.f : expf(m - m_n);
-  const float c2 = (m_o == -INFINITY) ? 0.f : expf(m_o - m_n);
-  l = l * c1 + l_o * c2;
-  for (int i = 0; i < n; ++i) acc[i] = acc[i] * c1 + acc_o[i] * c2;
-  m = m_n;
+// 2^x by the hardware instruction (one ulp; the arguments here are never positive).  Scores
+// are kept in units of log 2, so that no multiplication precedes it.
+__device__ inline float exp2_fast(float x) { return __builtin_amdgcn_exp2f(x); }
+
+// Over the lanes that hold the same head dimensions (l ^ LPK, l ^ 2 LPK, ... l ^ 32): the
+// maximum, then the sums of the states scaled to it.
+template <int LPK>
+__device__ inline float groups_max(float v) {
+  if (LPK <= 1) v = xor_max<1>(v);
+  if (LPK <= 2) v = xor_max<2>(v);
+  if (LPK <= 4) v = xor_max<4>(v);
+  if (LPK <= 8) v = xor_max<8>(v);
+  if (LPK <= 16) v = xor_max<16>(v);
+  return xor_max<32>(v);
+}
+template <int LPK>
+__device__ inline float groups_sum(float v) {
+  if (LPK <= 1) v = xor_sum<1>(v);
+  if (LPK <= 2) v = xor_sum<2>(v);
+  if (LPK <= 4) v = xor_sum<4>(v);
+  if (LPK <= 8) v = xor_sum<8>(v);
+  if (LPK <= 16) v = xor_sum<16>(v);
+  return xor_sum<32>(v);
 }
 
 template <typename T, int LPK, int AD_WAVES, int AD_UNROLL>
@@ -68,7 +82,7 @@ __global__ __launch_bounds__(64 * AD_WAVES) void attention_decode_kernel(
     float* __restrict__ partial, const int* __restrict__ tok_list,
     const int* __restrict__ tok_item, const int* __restrict__ tok_pos,
     const int* __restrict__ tables, int table_width, int heads, int kv_heads, int head_dim,
-    int page_size, int page_shift, int num_pages, float scale, int window, int splits) {
+    int page_size, int page_shift, int num_pages, float scale_log2, int window, int splits) {
   constexpr int GROUPS = 64 / LPK;               // keys per wave load
   constexpr int KEYS_PER_WAVE = GROUPS * AD_UNROLL;
   __shared__ float s_acc[AD_WAVES][256];
@@ -145,17 +159,17 @@ __global__ __launch_bounds__(64 * AD_WAVES) void attention_decode_kernel(
         dot = lanes_sum<16>(dot);
         dot += __shfl_xor(dot, 16, 64);
       }
-      s[u] = valid[u] ? dot * scale : -INFINITY;
+      s[u] = valid[u] ? dot * scale_log2 : -INFINITY;
       m_new = fmaxf(m_new, s[u]);
     }
     if (m_new != -INFINITY) {
-      const float correction = (m == -INFINITY) ? 0.f : expf(m - m_new);
+      const float correction = (m == -INFINITY) ? 0.f : exp2_fast(m - m_new);
       l *= correction;
 #pragma unroll
       for (int i = 0; i < 8; ++i) acc[i] *= correction;
 #pragma unroll
       for (int u = 0; u < AD_UNROLL; ++u) {
-        const float p = valid[u] ? expf(s[u] - m_new) : 0.f;
+        const float p = valid[u] ? exp2_fast(s[u] - m_new) : 0.f;
         l += p;
         float vf[8];
         vr[u].widen(vf);
@@ -171,15 +185,15 @@ __global__ __launch_bounds__(64 * AD_WAVES) void attention_decode_kernel(
     for (int i = 0; i < 8; ++i) acc[i] = 0.f;
   }
 
-  // merge the lane groups of this wave
+  // merge the lane groups of this wave: every state is scaled to the wave's maximum, then
+  // the sums run over the lanes that hold the same head dimensions
+  {
+    const float wave_m = groups_max<LPK>(m);
+    const float c = (m == -INFINITY) ? 0.f : exp2_fast(m - wave_m);
+    l = groups_sum<LPK>(l * c);
 #pragma unroll
-  for (int offset = LPK; offset < 64; offset <<= 1) {
-    const float m_o = __shfl_xor(m, offset, 64);
-    const float l_o = __shfl_xor(l, offset, 64);
-    float acc_o[8];
-#pragma unroll
-    for (int i = 0; i < 8; ++i) acc_o[i] = __shfl_xor(acc[i], offset, 64);
-    merge_state(m, l, acc, m_o, l_o, acc_o, 8);
+    for (int i = 0; i < 8; ++i) acc[i] = groups_sum<LPK>(acc[i] * c);
+    m = wave_m;
   }
   if (group == 0 && has_dims) {
 #pragma unroll
@@ -200,7 +214,7 @@ __global__ __launch_bounds__(64 * AD_WAVES) void attention_decode_kernel(
   float block_l = 0.f, value = 0.f;
 #pragma unroll
   for (int w = 0; w < AD_WAVES; ++w) {
-    const float c = (s_ml[w][0] == -INFINITY) ? 0.f : expf(s_ml[w][0] - block_m);
+    const float c = (s_ml[w][0] == -INFINITY) ? 0.f : exp2_fast(s_ml[w][0] - block_m);
     block_l += s_ml[w][1] * c;
     if (d < head_dim) value += s_acc[w][d] * c;
   }
@@ -217,7 +231,7 @@ __global__ __launch_bounds__(64 * AD_WAVES) void attention_decode_kernel(
   }
 }
 
-// out = sum_s acc_s e^{m_s - M} / sum_s l_s e^{m_s - M}.  One wave per (token, head); lane s
+// out = sum_s acc_s 2^{m_s - M} / sum_s l_s 2^{m_s - M} (the maxima are in units of log 2).  One wave per (token, head); lane s
 // first fetches (m_s, l_s) of split s (splits <= 64), so the weights cost one trip to memory.
 template <typename T>
 __global__ __launch_bounds__(64) void attention_reduce_kernel(
@@ -232,7 +246,7 @@ __global__ __launch_bounds__(64) void attention_reduce_kernel(
   const float m_s = lane < splits ? src[lane * stride + head_dim] : -INFINITY;
   const float l_s = lane < splits ? src[lane * stride + head_dim + 1] : 0.f;
   const float total_m = wave_max(m_s);
-  const float weight = (m_s == -INFINITY) ? 0.f : expf(m_s - total_m);
+  const float weight = (m_s == -INFINITY) ? 0.f : exp2_fast(m_s - total_m);
   const float total_l = wave_sum(l_s * weight);
   for (int d = lane; d < head_dim; d += 64) {
     float value = 0.f;
@@ -259,8 +273,8 @@ static int launch_decode(const void* q, int64_t q_stride, const void* k_pool, co
                      dim3(64 * WAVES), 0, s,                                                     \
                      (const T*)q, q_stride, (const T*)k_pool, (const T*)v_pool, (T*)out,         \
                      out_stride, partial, tok_list, tok_item, tok_pos, tables, table_width,      \
-                     heads, kv_heads, head_dim, page_size, page_shift, num_pages, scale, window, \
-                     splits)
+                     heads, kv_heads, head_dim, page_size, page_shift, num_pages,                \
+                     scale * 1.4426950408889634f, window, splits)
 #define PS_LAUNCH_AD(LPK)            \
   do {                               \
     if (waves == 16) {               \

@@ -129,6 +129,36 @@ __device__ inline float halves_max(float v) {
   return fmaxf(__builtin_bit_cast(float, (int)both[0]), __builtin_bit_cast(float, (int)both[1]));
 }
 
+// The sum / maximum of a lane's value and that of lane (l ^ OFFSET), for OFFSET = 8, 16 or 32
+// without a trip through LDS (a rotation inside the row of 16 lanes, a swap of rows, a swap of
+// the wave's halves); other offsets go through the shuffle.
+template <int OFFSET>
+__device__ inline float lane_xor(float v) {
+  return __shfl_xor(v, OFFSET, 64);
+}
+template <int OFFSET>
+__device__ inline float xor_sum(float v) {
+  if (OFFSET == 8) return v + lane_exchange<0x128>(v);
+  if (OFFSET == 16) {
+    const int bits = __builtin_bit_cast(int, v);
+    const auto both = __builtin_amdgcn_permlane16_swap(bits, bits, false, false);
+    return __builtin_bit_cast(float, (int)both[0]) + __builtin_bit_cast(float, (int)both[1]);
+  }
+  if (OFFSET == 32) return halves_sum(v);
+  return v + lane_xor<OFFSET>(v);
+}
+template <int OFFSET>
+__device__ inline float xor_max(float v) {
+  if (OFFSET == 8) return fmaxf(v, lane_exchange<0x128>(v));
+  if (OFFSET == 16) {
+    const int bits = __builtin_bit_cast(int, v);
+    const auto both = __builtin_amdgcn_permlane16_swap(bits, bits, false, false);
+    return fmaxf(__builtin_bit_cast(float, (int)both[0]), __builtin_bit_cast(float, (int)both[1]));
+  }
+  if (OFFSET == 32) return halves_max(v);
+  return fmaxf(v, lane_xor<OFFSET>(v));
+}
+
 __device__ inline float read_lane(float v, int lane) {
   return __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), lane));
 }
