@@ -369,20 +369,9 @@ __global__ __launch_bounds__(64 * SK_WAVES) void gemm_nt_skinny_norm_kernel(
   const bf16_t* w_ptr = w + (int64_t)w_row * k + group * 16;
   const uint4 zero = {0u, 0u, 0u, 0u};
 
-  // 1. this wave's weights: all loads leave now and arrive while the rows are normalised
   uint4 wf[SK_UNROLL][2];
   bool first[SK_UNROLL], second[SK_UNROLL];
-#pragma unroll
-  for (int u = 0; u < SK_UNROLL; ++u) {
-    const int ku = wave * 64 + u * SK_WAVES * 64;
-    const int kk = ku + group * 16;
-    first[u] = kk < k;
-    second[u] = kk + 8 < k;
-    wf[u][0] = *reinterpret_cast<const uint4*>(w_ptr + (first[u] ? ku : -group * 16));
-    wf[u][1] = *reinterpret_cast<const uint4*>(w_ptr + (second[u] ? ku + 8 : -group * 16));
-  }
-
-  // 2. rows wave, wave + 4, wave + 8, wave + 12: statistics and normalisation in registers
+  // 1. rows wave, wave + 4, wave + 8, wave + 12: statistics and normalisation in registers
   //    (mean, centred values, biased variance, rsqrt(var + eps), scale, shift; reference:
   //    src/kernels/triton_residual_layernorm.py:25-39), result to LDS as bfloat16.  A lane
   //    owns columns 4 * lane + 256 * i (one 16-byte load each); all loads of the four rows and
@@ -410,6 +399,19 @@ __global__ __launch_bounds__(64 * SK_WAVES) void gemm_nt_skinny_norm_kernel(
                   : zero4;
 #pragma unroll
       for (int j = 0; j < 4; ++j) v[j][i] = *reinterpret_cast<const float4*>(src[j] + safe);
+    }
+    // 2. this wave's weights.  A wave's loads come back in the order in which they left, so
+    //    these leave after the loads of the rows (which come from the L2 and are there first)
+    //    and travel while the rows are normalised; issued before them they would hold the
+    //    rows back for the whole trip to memory.
+#pragma unroll
+    for (int u = 0; u < SK_UNROLL; ++u) {
+      const int ku = wave * 64 + u * SK_WAVES * 64;
+      const int kk = ku + group * 16;
+      first[u] = kk < k;
+      second[u] = kk + 8 < k;
+      wf[u][0] = *reinterpret_cast<const uint4*>(w_ptr + (first[u] ? ku : -group * 16));
+      wf[u][1] = *reinterpret_cast<const uint4*>(w_ptr + (second[u] ? ku + 8 : -group * 16));
     }
     // rows beyond m (the same for the whole wave) are not worked on
     bool live_row[4];
