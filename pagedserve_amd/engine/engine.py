@@ -21,6 +21,7 @@ import numpy as np
 import torch
 
 from ..cache.manager import CacheFull, CacheManager
+from ..ops import kernels
 from ..parts.base import StepContext, StepItem, Workspace
 
 
@@ -215,11 +216,12 @@ class Engine:
                 cache.grow(entry.request_id, record.length + len(entry.tokens))
             caller = torch.cuda.current_stream(self.device)
             if caller.cuda_stream == self.stream.cuda_stream:
-                output = self._run(entries, greedy)
+                with kernels.on_stream(self.stream):
+                    output = self._run(entries, greedy)
             else:
                 # the caller may still be reading the last step's logits
                 self.stream.wait_stream(caller)
-                with torch.cuda.stream(self.stream):
+                with torch.cuda.stream(self.stream), kernels.on_stream(self.stream):
                     output = self._run(entries, greedy)
                 caller.wait_stream(self.stream)
         except Exception:

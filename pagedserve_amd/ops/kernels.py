@@ -65,8 +65,33 @@ def _call(name, *args):
         raise KernelError(f"{name} failed ({status}): {message}")
 
 
+_STREAM_HANDLE = None
+
+
 def _stream():
+    if _STREAM_HANDLE is not None:
+        return _STREAM_HANDLE
     return torch.cuda.current_stream().cuda_stream
+
+
+class on_stream:
+    """While active, every kernel of this module is launched on ``stream`` (which must be
+    torch's current stream, so that torch's own work keeps its order with them) without asking
+    torch for it at each launch: that question costs as much as the rest of a launch."""
+
+    def __init__(self, stream: "torch.cuda.Stream"):
+        self.handle = stream.cuda_stream
+
+    def __enter__(self):
+        global _STREAM_HANDLE
+        self.previous = _STREAM_HANDLE
+        _STREAM_HANDLE = self.handle
+        return self
+
+    def __exit__(self, *exc):
+        global _STREAM_HANDLE
+        _STREAM_HANDLE = self.previous
+        return False
 
 
 def dtype_code(dtype: torch.dtype) -> int:
@@ -505,7 +530,7 @@ class StepGraph:
             fn.argtypes = [c_void_p, c_void_p]
             fn.restype = c_int
             _BOUND["ps_graph_launch"] = fn
-        if fn(self.handle, torch.cuda.current_stream().cuda_stream) != 0:
+        if fn(self.handle, _stream()) != 0:
             raise KernelError(load_library().ps_last_error().decode())
         self.replays += 1
 
