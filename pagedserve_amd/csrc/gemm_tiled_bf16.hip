@@ -340,7 +340,7 @@ static int launch_variant(const void* a, const void* w, const float* bias, void*
   // place (residual epilogue) k is split over blocks.  Float atomics are slow, so this pays
   // only while the output is small.
   int k_splits = 1;
-  if (epilogue == PS_EPI_RESIDUAL && tiles_m * tiles_n <= 64 && k >= 1024) {
+  if (epilogue == PS_EPI_RESIDUAL && tiles_m * tiles_n <= 64 && k >= 2048) {
     k_splits = 256 / (tiles_m * tiles_n);
     if (k_splits > k / 256) k_splits = k / 256;
   }
@@ -365,10 +365,7 @@ static int launch_variant(const void* a, const void* w, const float* bias, void*
 
 // Tile shapes by the number of blocks they give: the chip has 256 compute units, and a product
 // of this size is over in a few microseconds, so filling them counts for more than the reuse
-// inside a large tile.  Long k with few tiles takes deeper prefetch instead: a block that is
-// alone on its compute unit needs many tiles in flight to keep its share of the memory
-// system busy (eight stages for one row of tiles over a long k, which is a decode step of a
-// wide model).
+// inside a large tile.
 template <typename TOut>
 static int launch_tiled_bf16(const void* a, const void* w, const float* bias, void* c, int m,
                              int n, int k, int lda, int ldc, int epilogue,
@@ -379,9 +376,18 @@ static int launch_tiled_bf16(const void* a, const void* w, const float* bias, vo
     return launch_variant<2, 2, 2, TOut>(a, w, bias, c, m, n, k, lda, ldc, epilogue, scatter, s);
   if (m > 64 && tiles_128_64 >= 384)
     return launch_variant<2, 1, 2, TOut>(a, w, bias, c, m, n, k, lda, ldc, epilogue, scatter, s);
-  if (m <= 64 && k > 1024 && (int64_t)((n + 63) / 64) <= 256)
+  // 64 x 64 tiles.  What a compute unit has in flight decides how long a k tile takes to
+  // arrive from memory.  Many blocks fill a unit by their number and keep two stages, which
+  // lets five of them in; up to two blocks per unit get four stages each; a single row of
+  // tiles over a long k (a decode step of a wide model) leaves most units empty and the
+  // others with one block, whose ring is made as deep as LDS allows (eight stages).  Eight
+  // stages for every launch of at most one block per unit measured slower than four: a block
+  // that takes most of the LDS keeps the next launch's blocks out until it has ended.
+  const int64_t tiles_64 = (int64_t)((m + 63) / 64) * ((n + 63) / 64);
+  const int k_tiles = k / TB_BK;
+  if (m <= 64 && tiles_64 <= 256 && k > 1024)
     return launch_variant<1, 1, 8, TOut>(a, w, bias, c, m, n, k, lda, ldc, epilogue, scatter, s);
-  if (k >= 2048)
+  if ((tiles_64 <= 512 && k_tiles > 2) || k >= 2048)
     return launch_variant<1, 1, 4, TOut>(a, w, bias, c, m, n, k, lda, ldc, epilogue, scatter, s);
   return launch_variant<1, 1, 2, TOut>(a, w, bias, c, m, n, k, lda, ldc, epilogue, scatter, s);
 }
