@@ -238,24 +238,27 @@ __global__ __launch_bounds__(256) void gemm_nt_tiled_kernel(
 #define SK_WAVES 4
 #define SK_UNROLL 4   // 64-k steps whose loads are issued together
 
-// Sum the four waves' partial tiles and finish element (row sub, column n0 + group*4 + wave).
+// Sum the four waves' partial tiles and finish the block's 16 columns of MB x 16 rows.
+// Element i of lane l of an accumulator is column (l / 16) * 4 + i of row l % 16; thread t
+// finishes column t % 16 of row t / 16 of each accumulator, so that 16 consecutive threads
+// store one run of 16 columns.
 template <typename TOut, int EPI, int MB>
 __device__ inline void skinny_epilogue(float (*partial)[MB][4][64], const float* bias, TOut* c,
                                        int m, int n, int ldc, int n0, int row0, int split,
                                        int k_splits, const KvScatter& scatter) {
-  const int lane = threadIdx.x & 63;
-  const int i = threadIdx.x >> 6;
-  const int sub = lane & 15;
-  const int group = lane >> 4;
-  const int col = n0 + group * 4 + i;
+  const int col_in = threadIdx.x & 15;
+  const int row_in = threadIdx.x >> 4;
+  const int col = n0 + col_in;
   if (col >= n) return;
+  const int i = col_in & 3;
+  const int lane = (col_in >> 2) * 16 + row_in;
+  const float bias_here = (bias != nullptr && split == 0) ? bias[col] : 0.f;
 #pragma unroll
   for (int b = 0; b < MB; ++b) {
-    const int row = row0 + b * 16 + sub;
+    const int row = row0 + b * 16 + row_in;
     if (row >= m) continue;
     float v = partial[0][b][i][lane] + partial[1][b][i][lane] + partial[2][b][i][lane] +
-              partial[3][b][i][lane];
-    if (bias != nullptr && split == 0) v += bias[col];
+              partial[3][b][i][lane] + bias_here;
     TOut* dst = c + (int64_t)row * ldc + col;
     if (EPI == PS_EPI_RESIDUAL) {
       if (k_splits > 1) {
@@ -271,37 +274,46 @@ __device__ inline void skinny_epilogue(float (*partial)[MB][4][64], const float*
   }
 }
 
-template <typename TOut, int EPI, int MB>
+template <typename TOut, int EPI, int MB, int NT>
 __global__ __launch_bounds__(64 * SK_WAVES) void gemm_nt_skinny_kernel(
     const bf16_t* __restrict__ a, const bf16_t* __restrict__ w, const float* __restrict__ bias,
     TOut* __restrict__ c, int m, int n, int k, int lda, int ldc, int k_chunk, int k_splits,
     KvScatter scatter) {
-  __shared__ float partial[SK_WAVES][MB][4][64];
+  // NT tiles of 16 columns per block share the loads of the rows of A: with very many
+  // columns (the output head) those loads, though they come from the L2, are as many bytes
+  // as the weights themselves.
+  __shared__ float partial[NT][SK_WAVES][MB][4][64];
   const int lane = threadIdx.x & 63;
   const int wave = threadIdx.x >> 6;
-  const int n0 = blockIdx.x * 16;
+  const int n0 = blockIdx.x * 16 * NT;
   const int split = blockIdx.y;
   const int row0 = blockIdx.z * (MB * 16);
   const int k_begin = split * k_chunk;
   const int k_end = k_begin + k_chunk < k ? k_begin + k_chunk : k;
   const int sub = lane & 15;
   const int group = lane >> 4;
-  const int w_row = n0 + sub < n ? n0 + sub : n - 1;
-  const bf16_t* w_ptr = w + (int64_t)w_row * k + group * 16;
+  const bf16_t* w_ptr[NT];
+#pragma unroll
+  for (int j = 0; j < NT; ++j) {
+    const int w_row = n0 + j * 16 + sub < n ? n0 + j * 16 + sub : n - 1;
+    w_ptr[j] = w + (int64_t)w_row * k + group * 16;
+  }
   const bf16_t* a_ptr[MB];
 #pragma unroll
   for (int b = 0; b < MB; ++b) {
     const int row = row0 + b * 16 + sub < m ? row0 + b * 16 + sub : m - 1;
     a_ptr[b] = a + (int64_t)row * lda + group * 16;
   }
-  f32x4 acc[MB];
+  f32x4 acc[NT][MB];
 #pragma unroll
-  for (int b = 0; b < MB; ++b) acc[b] = f32x4{0.f, 0.f, 0.f, 0.f};
+  for (int j = 0; j < NT; ++j)
+#pragma unroll
+    for (int b = 0; b < MB; ++b) acc[j][b] = f32x4{0.f, 0.f, 0.f, 0.f};
 
   const uint4 zero = {0u, 0u, 0u, 0u};
   // wave `wave` takes the 64-k steps wave, wave + 4, ... of the block's range
   for (int k0 = k_begin + wave * 64; k0 < k_end; k0 += SK_WAVES * SK_UNROLL * 64) {
-    uint4 wf[SK_UNROLL][2], xf[SK_UNROLL][MB][2];
+    uint4 wf[SK_UNROLL][NT][2], xf[SK_UNROLL][MB][2];
 #pragma unroll
     for (int u = 0; u < SK_UNROLL; ++u) {
       const int ku = k0 + u * SK_WAVES * 64;
@@ -312,20 +324,25 @@ __global__ __launch_bounds__(64 * SK_WAVES) void gemm_nt_skinny_kernel(
       // would not be issued together
       const int o0 = first ? ku : k_begin - group * 16;
       const int o1 = second ? ku + 8 : k_begin - group * 16;
-      wf[u][0] = *reinterpret_cast<const uint4*>(w_ptr + o0);
-      wf[u][1] = *reinterpret_cast<const uint4*>(w_ptr + o1);
+#pragma unroll
+      for (int j = 0; j < NT; ++j) {
+        wf[u][j][0] = *reinterpret_cast<const uint4*>(w_ptr[j] + o0);
+        wf[u][j][1] = *reinterpret_cast<const uint4*>(w_ptr[j] + o1);
+      }
 #pragma unroll
       for (int b = 0; b < MB; ++b) {
         xf[u][b][0] = *reinterpret_cast<const uint4*>(a_ptr[b] + o0);
         xf[u][b][1] = *reinterpret_cast<const uint4*>(a_ptr[b] + o1);
       }
       if (!first) {
-        wf[u][0] = zero;
+#pragma unroll
+        for (int j = 0; j < NT; ++j) wf[u][j][0] = zero;
 #pragma unroll
         for (int b = 0; b < MB; ++b) xf[u][b][0] = zero;
       }
       if (!second) {
-        wf[u][1] = zero;
+#pragma unroll
+        for (int j = 0; j < NT; ++j) wf[u][j][1] = zero;
 #pragma unroll
         for (int b = 0; b < MB; ++b) xf[u][b][1] = zero;
       }
@@ -333,21 +350,28 @@ __global__ __launch_bounds__(64 * SK_WAVES) void gemm_nt_skinny_kernel(
 #pragma unroll
     for (int u = 0; u < SK_UNROLL; ++u)
 #pragma unroll
-      for (int b = 0; b < MB; ++b)
+      for (int j = 0; j < NT; ++j)
 #pragma unroll
-        for (int h = 0; h < 2; ++h)
-          acc[b] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(
-              *reinterpret_cast<const bf16x8*>(&wf[u][h]),
-              *reinterpret_cast<const bf16x8*>(&xf[u][b][h]), acc[b], 0, 0, 0);
+        for (int b = 0; b < MB; ++b)
+#pragma unroll
+          for (int h = 0; h < 2; ++h)
+            acc[j][b] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(
+                *reinterpret_cast<const bf16x8*>(&wf[u][j][h]),
+                *reinterpret_cast<const bf16x8*>(&xf[u][b][h]), acc[j][b], 0, 0, 0);
   }
 
 #pragma unroll
-  for (int b = 0; b < MB; ++b)
+  for (int j = 0; j < NT; ++j)
 #pragma unroll
-    for (int i = 0; i < 4; ++i) partial[wave][b][i][lane] = acc[b][i];
+    for (int b = 0; b < MB; ++b)
+#pragma unroll
+      for (int i = 0; i < 4; ++i) partial[j][wave][b][i][lane] = acc[j][b][i];
   __syncthreads();
   // element i of a 16 x 16 accumulator: weight row (lane / 16) * 4 + i, activation row lane % 16
-  skinny_epilogue<TOut, EPI, MB>(partial, bias, c, m, n, ldc, n0, row0, split, k_splits, scatter);
+#pragma unroll
+  for (int j = 0; j < NT; ++j)
+    skinny_epilogue<TOut, EPI, MB>(partial[j], bias, c, m, n, ldc, n0 + j * 16, row0, split,
+                                   k_splits, scatter);
 }
 
 // ---------------------------------------------------------------- skinny with fused norm
@@ -566,10 +590,16 @@ static void launch_skinny_mb(const void* a, const void* w, const float* bias, vo
   dim3 grid((n + 15) / 16, k_splits, (row_blocks + per - 1) / per);
   dim3 block(64 * SK_WAVES);
 #define PS_LAUNCH_SK(MB)                                                                       \
-  hipLaunchKernelGGL((gemm_nt_skinny_kernel<TOut, EPI, MB>), grid, block, 0, s,                \
+  hipLaunchKernelGGL((gemm_nt_skinny_kernel<TOut, EPI, MB, 1>), grid, block, 0, s,             \
                      (const bf16_t*)a, (const bf16_t*)w, bias, (TOut*)c, m, n, k, lda, ldc,    \
                      k_chunk, k_splits, scatter)
-  if (per <= 1) PS_LAUNCH_SK(1);
+  if (per <= 1 && k_splits == 1 && n >= 16 * 1024) {
+    // the output head: two tiles of columns per block
+    grid.x = (n + 31) / 32;
+    hipLaunchKernelGGL((gemm_nt_skinny_kernel<TOut, EPI, 1, 2>), grid, block, 0, s,
+                       (const bf16_t*)a, (const bf16_t*)w, bias, (TOut*)c, m, n, k, lda, ldc,
+                       k_chunk, k_splits, scatter);
+  } else if (per <= 1) PS_LAUNCH_SK(1);
   else if (per == 2) PS_LAUNCH_SK(2);
   else if (per == 3) PS_LAUNCH_SK(3);
   else PS_LAUNCH_SK(4);
