@@ -113,7 +113,9 @@ class Attention(Mixer):
     def _splits(self, count: int, max_kv_len: int):
         """(ranges per request, waves per block).  Many (token, head) pairs fill the chip with
         one block of 4 waves each; with fewer pairs and long contexts one block of 16 waves
-        takes a whole request's keys, so that no second launch is needed to merge ranges; few
+        takes a whole request's keys, so that no second launch is needed to merge ranges
+        (1024 keys and more per block: what one compute unit can pull is the limit then, and
+        ranges go to further units); few
         pairs are cut into ranges so that the chip is filled, never into more than the keys
         of the longest request can feed."""
         visible = max_kv_len if self.window <= 0 else min(max_kv_len, self.window)
@@ -121,7 +123,9 @@ class Attention(Mixer):
         if pairs >= 384:
             return 1, 4
         if pairs >= 64 and visible > kernels.decode_keys_per_block(self.head_dim, 4):
-            return 1, 16
+            # contexts of several thousand keys: two or three such blocks per request, as
+            # long as every block still has a compute unit of its own
+            return max(1, min(256 // pairs, visible // 1024)), 16
         most = max(1, -(-visible // kernels.decode_keys_per_block(self.head_dim, 4)))
         wanted = max(1, -(-1024 // pairs))
         return min(most, wanted, 64), 4

@@ -593,3 +593,10 @@ def test_attention_decode_sixteen_waves(dtype):
     kernels.attention_decode(q, k_pool, v_pool, out, tok_item, tok_pos, tables, heads, 0.125, 1, waves=16)
     atol, rtol = (3e-5, 3e-5) if dtype == torch.float32 else (2e-2, 2e-2)
     torch.testing.assert_close(out.double(), expected.double(), atol=atol, rtol=rtol)
+    # two and three ranges per request, merged by the reduce kernel
+    for splits in (2, 3):
+        partial = torch.full((len(contexts) * heads * splits * (head_dim + 2),), float("nan"), device="cuda")
+        out = torch.full_like(q, float("nan"))
+        kernels.attention_decode(q, k_pool, v_pool, out, tok_item, tok_pos, tables, heads, 0.125, splits,
+                                 partial=partial, waves=16)
+        torch.testing.assert_close(out.double(), expected.double(), atol=atol, rtol=rtol)
