@@ -269,7 +269,7 @@ static int launch_decode(const void* q, int64_t q_stride, const void* k_pool, co
   }
   dim3 grid(count, heads, splits);
 #define PS_LAUNCH_ADW(LPK, WAVES)                                                                \
-  hipLaunchKernelGGL((attention_decode_kernel<T, LPK, WAVES, (WAVES == 16 ? 8 : 4)>), grid,      \
+  hipLaunchKernelGGL((attention_decode_kernel<T, LPK, WAVES, (WAVES == 16 && sizeof(T) == 2 ? 8 : 4)>), grid, \
                      dim3(64 * WAVES), 0, s,                                                     \
                      (const T*)q, q_stride, (const T*)k_pool, (const T*)v_pool, (T*)out,         \
                      out_stride, partial, tok_list, tok_item, tok_pos, tables, table_width,      \
