@@ -9,10 +9,10 @@ int ps_gemm_nt_simple(const void* a, const void* w, const float* bias, void* c, 
                       hipStream_t s);
 int ps_gemm_nt_mfma(const void* a, const void* w, const float* bias, void* c, int m, int n, int k,
                     int lda, int ldc, int dtype, int c_dtype, int epilogue,
-                    const KvScatter& scatter, hipStream_t s);
+                    const KvScatter& scatter, const void* w_packed, hipStream_t s);
 int ps_norm_gemm_fused(const NormPrologue& norm, const void* w, const float* bias, void* c, int m,
                        int n, int k, int ldc, int c_dtype, int epilogue, const KvScatter& scatter,
-                       hipStream_t s);
+                       const void* w_packed, hipStream_t s);
 bool ps_gemm_nt_mfma_supported(const void* a, const void* w, int k, int lda, int dtype);
 bool ps_norm_gemm_fusable(const void* w, const NormPrologue& norm, int m, int n, int k, int dtype);
 
@@ -74,7 +74,7 @@ extern "C" int ps_linear(const PsLinearArgs* p, void* stream) {
     NormPrologue norm = {p->norm_h, p->norm_rows, p->gamma, p->beta, p->eps, p->rms, p->ldh};
     if (ps_norm_gemm_fusable(p->w, norm, m, n, k, p->dtype)) {
       return ps_norm_gemm_fused(norm, p->w, p->bias, p->c, m, n, k, p->ldc, p->c_dtype,
-                                p->epilogue, scatter, s);
+                                p->epilogue, scatter, p->w_packed, s);
     }
     PS_REQUIRE(p->norm_out != nullptr, "ps_linear: scratch for the normed rows is needed");
     PS_REQUIRE(p->ldh == k, "ps_linear: unfused norm needs dense rows (ldh %d, k %d)", p->ldh, k);
@@ -90,7 +90,7 @@ extern "C" int ps_linear(const PsLinearArgs* p, void* stream) {
                     (p->dtype == PS_BF16 || m >= 96);
   if (mfma)
     return ps_gemm_nt_mfma(a, p->w, p->bias, p->c, m, n, k, lda, p->ldc, p->dtype, p->c_dtype,
-                           p->epilogue, scatter, s);
+                           p->epilogue, scatter, p->dtype == PS_BF16 ? p->w_packed : nullptr, s);
   int status = ps_gemm_nt_simple(a, p->w, p->bias, p->c, m, n, k, lda, p->ldc, p->dtype,
                                  p->c_dtype, p->epilogue, s);
   if (status != 0 || scatter.k_pool == nullptr) return status;

@@ -274,11 +274,11 @@ __device__ inline void skinny_epilogue(float (*partial)[MB][4][64], const float*
   }
 }
 
-template <typename TOut, int EPI, int MB, int NT>
+template <typename TOut, int EPI, int MB, int NT, int UNROLL>
 __global__ __launch_bounds__(64 * SK_WAVES) void gemm_nt_skinny_kernel(
     const bf16_t* __restrict__ a, const bf16_t* __restrict__ w, const float* __restrict__ bias,
     TOut* __restrict__ c, int m, int n, int k, int lda, int ldc, int k_chunk, int k_splits,
-    KvScatter scatter) {
+    KvScatter scatter, const bf16_t* __restrict__ wp) {
   // NT tiles of 16 columns per block share the loads of the rows of A: with very many
   // columns (the output head) those loads, though they come from the L2, are as many bytes
   // as the weights themselves.
@@ -297,6 +297,13 @@ __global__ __launch_bounds__(64 * SK_WAVES) void gemm_nt_skinny_kernel(
   for (int j = 0; j < NT; ++j) {
     const int w_row = n0 + j * 16 + sub < n ? n0 + j * 16 + sub : n - 1;
     w_ptr[j] = w + (int64_t)w_row * k + group * 16;
+    if (wp != nullptr) {
+      // packed copy: the 16 x 64 tile of step s lies in the order in which the lanes hold it,
+      // first the halves of the first product, then those of the second (1 KB each)
+      const int tiles = (n + 15) / 16;
+      const int tile = n0 / 16 + j < tiles ? n0 / 16 + j : tiles - 1;
+      w_ptr[j] = wp + (int64_t)tile * (k / 64) * 1024 + lane * 8;
+    }
   }
   const bf16_t* a_ptr[MB];
 #pragma unroll
@@ -312,10 +319,10 @@ __global__ __launch_bounds__(64 * SK_WAVES) void gemm_nt_skinny_kernel(
 
   const uint4 zero = {0u, 0u, 0u, 0u};
   // wave `wave` takes the 64-k steps wave, wave + 4, ... of the block's range
-  for (int k0 = k_begin + wave * 64; k0 < k_end; k0 += SK_WAVES * SK_UNROLL * 64) {
-    uint4 wf[SK_UNROLL][NT][2], xf[SK_UNROLL][MB][2];
+  for (int k0 = k_begin + wave * 64; k0 < k_end; k0 += SK_WAVES * UNROLL * 64) {
+    uint4 wf[UNROLL][NT][2], xf[UNROLL][MB][2];
 #pragma unroll
-    for (int u = 0; u < SK_UNROLL; ++u) {
+    for (int u = 0; u < UNROLL; ++u) {
       const int ku = k0 + u * SK_WAVES * 64;
       const int kk = ku + group * 16;
       const bool first = kk < k_end;
@@ -324,10 +331,13 @@ __global__ __launch_bounds__(64 * SK_WAVES) void gemm_nt_skinny_kernel(
       // would not be issued together
       const int o0 = first ? ku : k_begin - group * 16;
       const int o1 = second ? ku + 8 : k_begin - group * 16;
+      // (packed: k is a multiple of 64, so a step is whole or absent)
+      const int p0 = wp != nullptr ? (first ? (ku / 64) * 1024 : 0) : o0;
+      const int p1 = wp != nullptr ? p0 + 512 : o1;
 #pragma unroll
       for (int j = 0; j < NT; ++j) {
-        wf[u][j][0] = *reinterpret_cast<const uint4*>(w_ptr[j] + o0);
-        wf[u][j][1] = *reinterpret_cast<const uint4*>(w_ptr[j] + o1);
+        wf[u][j][0] = *reinterpret_cast<const uint4*>(w_ptr[j] + p0);
+        wf[u][j][1] = *reinterpret_cast<const uint4*>(w_ptr[j] + p1);
       }
 #pragma unroll
       for (int b = 0; b < MB; ++b) {
@@ -348,7 +358,7 @@ __global__ __launch_bounds__(64 * SK_WAVES) void gemm_nt_skinny_kernel(
       }
     }
 #pragma unroll
-    for (int u = 0; u < SK_UNROLL; ++u)
+    for (int u = 0; u < UNROLL; ++u)
 #pragma unroll
       for (int j = 0; j < NT; ++j)
 #pragma unroll
@@ -381,7 +391,8 @@ __global__ __launch_bounds__(64 * SK_WAVES) void gemm_nt_skinny_kernel(
 template <typename TOut, int EPI>
 __global__ __launch_bounds__(64 * SK_WAVES) void gemm_nt_skinny_norm_kernel(
     NormPrologue norm, const bf16_t* __restrict__ w, const float* __restrict__ bias,
-    TOut* __restrict__ c, int m, int n, int k, int ldc, KvScatter scatter) {
+    TOut* __restrict__ c, int m, int n, int k, int ldc, KvScatter scatter,
+    const bf16_t* __restrict__ wp) {
   __shared__ float partial[SK_WAVES][1][4][64];
   __shared__ __attribute__((aligned(16))) bf16_t xs[16 * SN_STRIDE];
   const int lane = threadIdx.x & 63;
@@ -391,6 +402,7 @@ __global__ __launch_bounds__(64 * SK_WAVES) void gemm_nt_skinny_norm_kernel(
   const int group = lane >> 4;
   const int w_row = n0 + sub < n ? n0 + sub : n - 1;
   const bf16_t* w_ptr = w + (int64_t)w_row * k + group * 16;
+  if (wp != nullptr) w_ptr = wp + (int64_t)(n0 / 16) * (k / 64) * 1024 + lane * 8;   // packed copy
   const uint4 zero = {0u, 0u, 0u, 0u};
 
   uint4 wf[SK_UNROLL][2];
@@ -434,8 +446,10 @@ __global__ __launch_bounds__(64 * SK_WAVES) void gemm_nt_skinny_norm_kernel(
       const int kk = ku + group * 16;
       first[u] = kk < k;
       second[u] = kk + 8 < k;
-      wf[u][0] = *reinterpret_cast<const uint4*>(w_ptr + (first[u] ? ku : -group * 16));
-      wf[u][1] = *reinterpret_cast<const uint4*>(w_ptr + (second[u] ? ku + 8 : -group * 16));
+      const int p0 = wp != nullptr ? (first[u] ? (ku / 64) * 1024 : 0) : (first[u] ? ku : -group * 16);
+      const int p1 = wp != nullptr ? p0 + 512 : (second[u] ? ku + 8 : -group * 16);
+      wf[u][0] = *reinterpret_cast<const uint4*>(w_ptr + p0);
+      wf[u][1] = *reinterpret_cast<const uint4*>(w_ptr + p1);
     }
     // rows beyond m (the same for the whole wave) are not worked on
     bool live_row[4];
@@ -577,7 +591,7 @@ static int launch_tiled(const void* a, const void* w, const float* bias, void* c
 template <typename TOut, int EPI>
 static void launch_skinny_mb(const void* a, const void* w, const float* bias, void* c, int m,
                              int n, int k, int lda, int ldc, int k_chunk, int k_splits,
-                             const KvScatter& scatter, hipStream_t s) {
+                             const KvScatter& scatter, const bf16_t* wp, hipStream_t s) {
   // Rows go 16 to an accumulator, up to four accumulators to a block.  Where the columns and
   // the k ranges give few blocks, the rows are spread over more of them (every one reads the
   // same weights, which the L2 absorbs; blocks that differ only in z run on one XCD when the
@@ -590,15 +604,20 @@ static void launch_skinny_mb(const void* a, const void* w, const float* bias, vo
   dim3 grid((n + 15) / 16, k_splits, (row_blocks + per - 1) / per);
   dim3 block(64 * SK_WAVES);
 #define PS_LAUNCH_SK(MB)                                                                       \
-  hipLaunchKernelGGL((gemm_nt_skinny_kernel<TOut, EPI, MB, 1>), grid, block, 0, s,             \
+  hipLaunchKernelGGL((gemm_nt_skinny_kernel<TOut, EPI, MB, 1, SK_UNROLL>), grid, block, 0, s,  \
                      (const bf16_t*)a, (const bf16_t*)w, bias, (TOut*)c, m, n, k, lda, ldc,    \
-                     k_chunk, k_splits, scatter)
+                     k_chunk, k_splits, scatter, wp)
   if (per <= 1 && k_splits == 1 && n >= 16 * 1024) {
     // the output head: two tiles of columns per block
     grid.x = (n + 31) / 32;
-    hipLaunchKernelGGL((gemm_nt_skinny_kernel<TOut, EPI, 1, 2>), grid, block, 0, s,
+    hipLaunchKernelGGL((gemm_nt_skinny_kernel<TOut, EPI, 1, 2, SK_UNROLL>), grid, block, 0, s,
                        (const bf16_t*)a, (const bf16_t*)w, bias, (TOut*)c, m, n, k, lda, ldc,
-                       k_chunk, k_splits, scatter);
+                       k_chunk, k_splits, scatter, wp);
+  } else if (per <= 1 && k_chunk > SK_WAVES * SK_UNROLL * 64) {
+    // up to 16 rows leave registers for twice the loads: a k of up to 2048 in one round
+    hipLaunchKernelGGL((gemm_nt_skinny_kernel<TOut, EPI, 1, 1, 2 * SK_UNROLL>), grid, block, 0, s,
+                       (const bf16_t*)a, (const bf16_t*)w, bias, (TOut*)c, m, n, k, lda, ldc,
+                       k_chunk, k_splits, scatter, wp);
   } else if (per <= 1) PS_LAUNCH_SK(1);
   else if (per == 2) PS_LAUNCH_SK(2);
   else if (per == 3) PS_LAUNCH_SK(3);
@@ -609,7 +628,8 @@ static void launch_skinny_mb(const void* a, const void* w, const float* bias, vo
 template <typename TOut>
 static int launch_skinny(const void* a, const void* w, const float* bias, void* c, int m, int n,
                          int k, int lda, int ldc, int epilogue, const KvScatter& scatter,
-                         hipStream_t s) {
+                         const bf16_t* wp, hipStream_t s) {
+  if (k % 64 != 0) wp = nullptr;   // the packed copy exists for whole steps of 64 only
   // A block covers 1024 k with one round of loads.  Longer k is split over blocks where the
   // partial sums can be added in place (residual epilogue), else the block loops.
   int k_splits = 1;
@@ -619,7 +639,7 @@ static int launch_skinny(const void* a, const void* w, const float* bias, void* 
   k_splits = (k + k_chunk - 1) / k_chunk;
 #define PS_SKINNY_CASE(EPI)                                                                      \
   case EPI:                                                                                      \
-    launch_skinny_mb<TOut, EPI>(a, w, bias, c, m, n, k, lda, ldc, k_chunk, k_splits, scatter, s); \
+    launch_skinny_mb<TOut, EPI>(a, w, bias, c, m, n, k, lda, ldc, k_chunk, k_splits, scatter, wp, s); \
     break
   switch (epilogue) {
     PS_SKINNY_CASE(PS_EPI_NONE);
@@ -636,13 +656,14 @@ static int launch_skinny(const void* a, const void* w, const float* bias, void* 
 template <typename TOut>
 static int launch_skinny_norm(const NormPrologue& norm, const void* w, const float* bias, void* c,
                               int m, int n, int k, int ldc, int epilogue, const KvScatter& scatter,
-                              hipStream_t s) {
+                              const bf16_t* wp, hipStream_t s) {
+  if (k % 64 != 0) wp = nullptr;
   dim3 grid((n + 15) / 16);
   dim3 block(64 * SK_WAVES);
 #define PS_NORM_CASE(EPI)                                                                     \
   case EPI:                                                                                   \
     hipLaunchKernelGGL((gemm_nt_skinny_norm_kernel<TOut, EPI>), grid, block, 0, s, norm,       \
-                       (const bf16_t*)w, bias, (TOut*)c, m, n, k, ldc, scatter);              \
+                       (const bf16_t*)w, bias, (TOut*)c, m, n, k, ldc, scatter, wp);          \
     break
   switch (epilogue) {
     PS_NORM_CASE(PS_EPI_NONE);
@@ -658,15 +679,17 @@ static int launch_skinny_norm(const NormPrologue& norm, const void* w, const flo
 
 int ps_norm_gemm_fused(const NormPrologue& norm, const void* w, const float* bias, void* c, int m,
                        int n, int k, int ldc, int c_dtype, int epilogue, const KvScatter& scatter,
-                       hipStream_t s) {
+                       const void* w_packed, hipStream_t s) {
+  const bf16_t* wp = (const bf16_t*)w_packed;
   if (c_dtype == PS_F32)
-    return launch_skinny_norm<float>(norm, w, bias, c, m, n, k, ldc, epilogue, scatter, s);
-  return launch_skinny_norm<bf16_t>(norm, w, bias, c, m, n, k, ldc, epilogue, scatter, s);
+    return launch_skinny_norm<float>(norm, w, bias, c, m, n, k, ldc, epilogue, scatter, wp, s);
+  return launch_skinny_norm<bf16_t>(norm, w, bias, c, m, n, k, ldc, epilogue, scatter, wp, s);
 }
 
 int ps_gemm_nt_mfma(const void* a, const void* w, const float* bias, void* c, int m, int n, int k,
                     int lda, int ldc, int dtype, int c_dtype, int epilogue,
-                    const KvScatter& scatter, hipStream_t s) {
+                    const KvScatter& scatter, const void* w_packed, hipStream_t s) {
+  const bf16_t* wp = (const bf16_t*)w_packed;
   // Up to 64 rows the skinny kernel has every load of a block in flight at once, which counts
   // when the weights come from memory and not from a cache; the tiled kernel walks k tile by
   // tile and wins only where there are tiles enough to fill the chip (the output head).
@@ -676,8 +699,8 @@ int ps_gemm_nt_mfma(const void* a, const void* w, const float* bias, void* c, in
   const bool skinny_k = m <= 64 && n < 64 * 256 && (epilogue == PS_EPI_RESIDUAL || k <= 1024);
   if (dtype == PS_BF16 && m <= 64 && (skinny_k || !ps_gemm_nt_bf16_tiled_supported(a, w, m, k, lda))) {
     if (c_dtype == PS_F32)
-      return launch_skinny<float>(a, w, bias, c, m, n, k, lda, ldc, epilogue, scatter, s);
-    return launch_skinny<bf16_t>(a, w, bias, c, m, n, k, lda, ldc, epilogue, scatter, s);
+      return launch_skinny<float>(a, w, bias, c, m, n, k, lda, ldc, epilogue, scatter, wp, s);
+    return launch_skinny<bf16_t>(a, w, bias, c, m, n, k, lda, ldc, epilogue, scatter, wp, s);
   }
   if (dtype == PS_BF16 && !skinny_k && ps_gemm_nt_bf16_tiled_supported(a, w, m, k, lda))
     return ps_gemm_nt_bf16_tiled(a, w, bias, c, m, n, k, lda, ldc, c_dtype, epilogue, scatter, s);

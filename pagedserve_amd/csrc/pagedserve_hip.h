@@ -42,6 +42,13 @@ int ps_gemm_nt(const void* a, const void* w, const float* bias, void* c, int m, 
 //   * k_pool != null: the output is [q | k | v] columns (q_cols, then kv_cols twice); besides
 //     being written to c, the k and v columns of row t are stored in the cache at the page
 //     slot of position tok_pos[t] of item tok_item[t] (what ps_kv_write does).
+//   * w_packed != null (bfloat16, k a multiple of 64): a second copy of w for the products of
+//     few rows, which stream the weights once and are bound by how they read them.  Rows are
+//     padded to a multiple of 16; the 16 x 64 tile of rows 16 t .. 16 t + 15 and columns
+//     64 s .. 64 s + 63 lies at element ((t * (k / 64) + s) * 1024 as two runs of 512: run h
+//     holds, for lane = g * 16 + r (g = 0..3, r = 0..15), the 8 values w[16 t + r][64 s + 16 g +
+//     8 h ..]: the order in which a wave's lanes hold the operand of v_mfma_f32_16x16x32_bf16,
+//     so that one load of a wave is 1 KB of consecutive memory.
 typedef struct PsLinearArgs {
   const void* a;
   const void* w;
@@ -63,6 +70,7 @@ typedef struct PsLinearArgs {
   const int* tok_pos;
   const int* tables;
   int table_width, q_cols, kv_cols, head_dim, kv_heads, page_size, num_pages;
+  const void* w_packed;   // null, or the copy of w that ps_pack_weight_layout describes
 } PsLinearArgs;
 
 int ps_linear(const PsLinearArgs* args, void* stream);

@@ -43,6 +43,7 @@ class DecoderModel:
         self.final_norm = build_part(NORMS, "norm", spec.final_norm, **common)
         self.embedding_table = None
         self.head_weight = None
+        self.head_packed = None
         # the mixer of the call that writes a cache entry decides what the entry holds
         self._entry_spec = {}
         for call in spec.schedule:
@@ -83,6 +84,7 @@ class DecoderModel:
         # the tied head is the embedding table itself, not a copy
         # (src/model/paged_decoder.py:300-301)
         self.head_weight = self.embedding_table if self.spec.tie_head else tensors["head.weight"]
+        self.head_packed = kernels.pack_decode_weight(self.head_weight)
         self.parameter_bytes = sum(t.numel() * t.element_size() for t in tensors.values())
         self.parameter_count = sum(t.numel() for t in tensors.values())
 
@@ -144,5 +146,5 @@ class DecoderModel:
         # logits = f @ table^T without bias, always float
         # (src/model/paged_decoder.py:295-301,605)
         out = logits_out[:wanted]
-        kernels.linear(pending, self.head_weight, None, out)
+        kernels.linear(pending, self.head_weight, None, out, packed=self.head_packed)
         return out

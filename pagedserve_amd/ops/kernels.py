@@ -223,6 +223,7 @@ class _LinearArgs(ctypes.Structure):
         ("tables", c_void_p),
         ("table_width", c_int), ("q_cols", c_int), ("kv_cols", c_int), ("head_dim", c_int),
         ("kv_heads", c_int), ("page_size", c_int), ("num_pages", c_int),
+        ("w_packed", c_void_p),
     ]
 
 
@@ -250,11 +251,27 @@ class PendingNorm:
                     rms=self.rms)[:count]
 
 
-def linear(x, w, bias, out, epilogue="none", scatter=None):
+def pack_decode_weight(w):
+    """A second copy of the bfloat16 matrix ``w [n, k]`` (k a multiple of 64, else None) for
+    the products of few rows: rows padded to a multiple of 16, every 16 x 64 tile laid out in
+    the order in which a wave's lanes hold the MFMA operand (``csrc/pagedserve_hip.h`` gives the
+    formula), so that a wave's load is 1 KB of consecutive memory.  Made once when weights are
+    bound; it doubles the memory of the matrices it is made for."""
+    if w.dtype != torch.bfloat16 or w.ndim != 2 or w.shape[1] % 64 != 0 or not w.is_cuda:
+        return None
+    n, k = w.shape
+    padded_rows = -(-n // 16) * 16
+    source = w if padded_rows == n else torch.cat([w, w.new_zeros((padded_rows - n, k))])
+    # [tile, row in tile, step, lane group, half, 8] -> [tile, step, half, lane group, row, 8]
+    return source.view(padded_rows // 16, 16, k // 64, 4, 2, 8).permute(0, 2, 4, 3, 1, 5).contiguous()
+
+
+def linear(x, w, bias, out, epilogue="none", scatter=None, packed=None):
     """out = epilogue(x w^T + bias) where ``x`` is a tensor or a ``PendingNorm``.
 
     ``scatter = (k_pool, v_pool, tok_item, tok_pos, tables, q_cols, kv_cols)`` also stores the
-    key and value columns of a ``[q | k | v]`` output into their cache pages."""
+    key and value columns of a ``[q | k | v]`` output into their cache pages.  ``packed`` is
+    ``pack_decode_weight(w)`` or None; the kernels for few rows read it instead of ``w``."""
     _check(w, "w", ndim=2)
     _check(out, "out", ndim=2)
     n, k = w.shape
@@ -299,6 +316,12 @@ def linear(x, w, bias, out, epilogue="none", scatter=None):
     if epilogue not in EPILOGUES:
         raise KernelError(f"linear: unknown epilogue {epilogue!r}")
     args.w = w.data_ptr()
+    if packed is not None:
+        if (packed.dtype != torch.bfloat16 or w.dtype != torch.bfloat16 or not packed.is_cuda
+                or not packed.is_contiguous() or k % 64 != 0
+                or packed.numel() != -(-n // 16) * 16 * k):
+            raise KernelError(f"linear: the packed copy does not belong to w {tuple(w.shape)}")
+        args.w_packed = packed.data_ptr()
     args.bias = _ptr(bias)
     args.c = out.data_ptr()
     args.m, args.n, args.k = m, n, k

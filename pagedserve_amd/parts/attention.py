@@ -59,6 +59,9 @@ class Attention(Mixer):
         self.out_weight = tensors["out.weight"]
         self.qkv_bias = tensors.get("qkv.bias")
         self.out_bias = tensors.get("out.bias")
+        # copies in the layout that the products of few rows (decode steps) read fastest
+        self.qkv_packed = kernels.pack_decode_weight(self.qkv_weight)
+        self.out_packed = kernels.pack_decode_weight(self.out_weight)
 
     def cache_spec(self):
         return PagedKVSpec(self.kv_heads, self.head_dim, self.window)
@@ -76,9 +79,9 @@ class Attention(Mixer):
             # keys and values go to their pages from the product's own epilogue
             kernels.linear(x, self.qkv_weight, self.qkv_bias, qkv,
                            scatter=(cache.k_pool, cache.v_pool, ctx.tok_item, ctx.positions, tables,
-                                    self.q_cols, self.kv_cols))
+                                    self.q_cols, self.kv_cols), packed=self.qkv_packed)
         else:
-            kernels.linear(x, self.qkv_weight, self.qkv_bias, qkv)
+            kernels.linear(x, self.qkv_weight, self.qkv_bias, qkv, packed=self.qkv_packed)
             if rotates:
                 self.position.apply_to_qk(q, k, ctx)
             if cache.writes:
@@ -108,7 +111,8 @@ class Attention(Mixer):
             kernels.attention_rowwise(q, cache.k_pool, cache.v_pool, context, ctx.tok_item,
                                       ctx.positions, tables, self.heads, self.scale, self.window,
                                       tok_list=None if singles == 0 else ctx.portion_tokens)
-        kernels.linear(context, self.out_weight, self.out_bias, residual, epilogue="residual")
+        kernels.linear(context, self.out_weight, self.out_bias, residual, epilogue="residual",
+                       packed=self.out_packed)
 
     def _splits(self, count: int, max_kv_len: int):
         """(ranges per request, waves per block).  Many (token, head) pairs fill the chip with

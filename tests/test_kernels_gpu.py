@@ -600,3 +600,59 @@ def test_attention_decode_sixteen_waves(dtype):
         kernels.attention_decode(q, k_pool, v_pool, out, tok_item, tok_pos, tables, heads, 0.125, splits,
                                  partial=partial, waves=16)
         torch.testing.assert_close(out.double(), expected.double(), atol=atol, rtol=rtol)
+
+
+PACKED_SHAPES = [(1, 50, 64), (8, 768, 3072), (8, 2304, 768), (16, 3072, 768), (17, 768, 768), (5, 1000, 320),
+                 (64, 2304, 768), (48, 100, 3072), (9, 16411, 320), (16, 330, 1600), (40, 400, 1600), (300, 1000, 320)]
+
+
+@pytest.mark.parametrize("m,n,k", PACKED_SHAPES)
+@pytest.mark.parametrize("epilogue", ["none", "gelu_tanh", "residual"])
+def test_linear_with_packed_weights(m, n, k, epilogue):
+    """The copy of a weight matrix in the lanes' operand order gives the product that the
+    matrix itself gives, bit for bit where partial sums are not added atomically: plain, with
+    a pending norm, and with the key/value scatter; a row count that is no multiple of 16, a k
+    beyond one round of loads, many rows (where the copy is not used)."""
+    from pagedserve_amd.ops import kernels
+
+    dtype = torch.bfloat16
+    a = _rand((m, k), dtype, 210, 1.0)
+    w = _rand((n, k), dtype, 211, 1.0 / math.sqrt(k))
+    bias = _rand((n,), torch.float32, 212)
+    packed = kernels.pack_decode_weight(w)
+    assert packed is not None and packed.numel() == -(-n // 16) * 16 * k
+    # the layout: row r, column c of w
+    for r, c in ((0, 0), (n - 1, k - 1), (min(n - 1, 17), 37)):
+        tile, row = divmod(r, 16)
+        step, rest = divmod(c, 64)
+        group, rest = divmod(rest, 16)
+        half, e = divmod(rest, 8)
+        assert packed[tile, step, half, group, row, e] == w[r, c]
+    start = _rand((m, n), torch.float32, 213)
+
+    def run(x, use_packed):
+        out = start.clone() if epilogue == "residual" else torch.full((m, n), float("nan"), dtype=dtype, device="cuda")
+        kernels.linear(x, w, bias, out, epilogue=epilogue, packed=packed if use_packed else None)
+        return out
+
+    plain, with_copy = run(a, False), run(a, True)
+    atomic = epilogue == "residual" and k > 1024 and m <= 64
+    if atomic:
+        torch.testing.assert_close(with_copy, plain, atol=1e-4, rtol=1e-5)
+    else:
+        assert torch.equal(with_copy, plain)
+    if m <= 64:
+        h = _rand((m, k), torch.float32, 214, 2.0)
+        gamma = 1.0 + _rand((k,), torch.float32, 215, 0.2)
+        beta = _rand((k,), torch.float32, 216, 0.2)
+        scratch = torch.empty((m, k), dtype=dtype, device="cuda")
+        pending = lambda: kernels.PendingNorm(h, gamma, beta, 1e-5, False, scratch, None)
+        plain, with_copy = run(pending(), False), run(pending(), True)
+        if atomic:
+            torch.testing.assert_close(with_copy, plain, atol=1e-4, rtol=1e-5)
+        else:
+            assert torch.equal(with_copy, plain)
+    assert kernels.pack_decode_weight(_rand((32, 100), dtype, 217)) is None
+    assert kernels.pack_decode_weight(_rand((32, 128), torch.float32, 218)) is None
+    with pytest.raises(kernels.KernelError, match="packed copy"):
+        kernels.linear(a, w, bias, run(a, False), epilogue=epilogue, packed=packed[:-1].contiguous() if packed.shape[0] > 1 else packed.float())
