@@ -71,6 +71,9 @@ class Part:
         return {}
 
     def bind(self, tensors: Dict[str, torch.Tensor]):
+        """Receive the tensors that ``parameters`` named.  A part may derive further tensors
+        from them here (the built-in ones keep a second copy of their matrices in a layout for
+        decode steps): whoever changes a weight afterwards binds again."""
         for name in self.parameters():
             setattr(self, name.replace(".", "_"), tensors[name])
 
