@@ -61,7 +61,12 @@ def decode_run(engine, sampler, config, batch, context_end, steps, warmup, seed=
     from pagedserve_amd.sampling import SamplingParams
 
     generator = torch.Generator().manual_seed(seed)
-    new_tokens = steps + warmup + 1
+    # Prompts are prefilled a few per iteration while the requests that are through decode
+    # on: the first request is that many tokens ahead of the last.  Every request gets room
+    # for it, so that none ends (and the batch stays whole) inside the timed steps; the first
+    # one's context ends at ``context_end``, the last one's that many tokens earlier.
+    ahead = -(-batch * context_end // engine.max_step_tokens)
+    new_tokens = steps + warmup + 1 + ahead
     prompt_len = context_end - new_tokens
     if prompt_len < 1:
         raise ValueError("steps + warmup leave no room for a prompt")
@@ -81,7 +86,7 @@ def decode_run(engine, sampler, config, batch, context_end, steps, warmup, seed=
         scheduler.step()
     torch.cuda.synchronize()
     elapsed = time.perf_counter() - started
-    mean_context = context_end - 1 - (steps - 1) / 2.0
+    mean_context = context_end - 1 - (steps - 1) / 2.0 - ahead / 2.0
     while scheduler.has_work():
         scheduler.step()
     return elapsed, mean_context

@@ -5,6 +5,7 @@
 #include <string.h>
 
 #include "common.h"
+#include "linear.h"
 #include "pagedserve_hip.h"
 
 // ---------------------------------------------------------------- error channel
@@ -94,7 +95,8 @@ extern "C" int ps_embed(const void* table, const void* pos_table, const int* ids
 template <typename T, bool RMS, int VPT>
 __global__ __launch_bounds__(256) void norm_wave_kernel(
     const float* __restrict__ x, const int* __restrict__ rows, const float* __restrict__ gamma,
-    const float* __restrict__ beta, T* __restrict__ out, int n_rows, int width, float eps) {
+    const float* __restrict__ beta, T* __restrict__ out, int n_rows, int width, float eps,
+    int packed) {
   const int lane = threadIdx.x & 63;
   const int r = blockIdx.x * 4 + (threadIdx.x >> 6);
   if (r >= n_rows) return;
@@ -131,7 +133,10 @@ __global__ __launch_bounds__(256) void norm_wave_kernel(
 #pragma unroll
   for (int i = 0; i < VPT; ++i) {
     const int col = lane + i * 64;
-    if (col < width) dst[col] = from_float<T>(v[i] * inv_std * g[i] + b[i]);
+    if (col >= width) continue;
+    const T y = from_float<T>(v[i] * inv_std * g[i] + b[i]);
+    if (packed) out[packed_offset(r, col, width)] = y;
+    else dst[col] = y;
   }
 }
 
@@ -165,12 +170,12 @@ __global__ void norm_block_kernel(const float* __restrict__ x, const int* __rest
 
 template <typename T, bool RMS>
 static void launch_norm(const float* x, const int* rows, const float* gamma, const float* beta,
-                        void* out, int n_rows, int width, float eps, hipStream_t s) {
+                        void* out, int n_rows, int width, float eps, int packed, hipStream_t s) {
   const int per_lane = (width + 63) / 64;
   const dim3 grid((n_rows + 3) / 4);
 #define PS_LAUNCH_NW(VPT)                                                                       \
   hipLaunchKernelGGL((norm_wave_kernel<T, RMS, VPT>), grid, dim3(256), 0, s, x, rows, gamma, beta, \
-                     (T*)out, n_rows, width, eps)
+                     (T*)out, n_rows, width, eps, packed)
   if (per_lane <= 2) PS_LAUNCH_NW(2);
   else if (per_lane <= 4) PS_LAUNCH_NW(4);
   else if (per_lane <= 8) PS_LAUNCH_NW(8);
@@ -183,23 +188,34 @@ static void launch_norm(const float* x, const int* rows, const float* gamma, con
 #undef PS_LAUNCH_NW
 }
 
-extern "C" int ps_norm(const float* x, const int* rows, const float* gamma, const float* beta,
-                       void* out, int n_rows, int width, float eps, int rms, int out_dtype,
-                       void* stream) {
+// The norm with its rows written row by row (packed == 0) or in the operand order of the
+// skinny product (packed_offset in linear.h; needs width a multiple of 64 up to 2048 and room
+// for the row count rounded up to 16).
+int ps_norm_layout(const float* x, const int* rows, const float* gamma, const float* beta,
+                   void* out, int n_rows, int width, float eps, int rms, int out_dtype,
+                   int packed, hipStream_t s) {
   PS_REQUIRE(n_rows >= 0 && width > 0, "ps_norm: bad sizes (rows %d, width %d)", n_rows, width);
   PS_REQUIRE(out_dtype == PS_F32 || out_dtype == PS_BF16, "ps_norm: unknown dtype %d", out_dtype);
   PS_REQUIRE(eps > 0.f, "ps_norm: eps must be positive");
+  PS_REQUIRE(!packed || (width % 64 == 0 && width <= 2048),
+             "ps_norm: the packed layout needs a width that is a multiple of 64 up to 2048");
   if (n_rows == 0) return 0;
-  hipStream_t s = (hipStream_t)stream;
   if (out_dtype == PS_F32) {
-    if (rms) launch_norm<float, true>(x, rows, gamma, beta, out, n_rows, width, eps, s);
-    else launch_norm<float, false>(x, rows, gamma, beta, out, n_rows, width, eps, s);
+    if (rms) launch_norm<float, true>(x, rows, gamma, beta, out, n_rows, width, eps, packed, s);
+    else launch_norm<float, false>(x, rows, gamma, beta, out, n_rows, width, eps, packed, s);
   } else {
-    if (rms) launch_norm<bf16_t, true>(x, rows, gamma, beta, out, n_rows, width, eps, s);
-    else launch_norm<bf16_t, false>(x, rows, gamma, beta, out, n_rows, width, eps, s);
+    if (rms) launch_norm<bf16_t, true>(x, rows, gamma, beta, out, n_rows, width, eps, packed, s);
+    else launch_norm<bf16_t, false>(x, rows, gamma, beta, out, n_rows, width, eps, packed, s);
   }
   PS_CHECK_LAUNCH("ps_norm");
   return 0;
+}
+
+extern "C" int ps_norm(const float* x, const int* rows, const float* gamma, const float* beta,
+                       void* out, int n_rows, int width, float eps, int rms, int out_dtype,
+                       void* stream) {
+  return ps_norm_layout(x, rows, gamma, beta, out, n_rows, width, eps, rms, out_dtype, 0,
+                        (hipStream_t)stream);
 }
 
 // ---------------------------------------------------------------- key/value scatter

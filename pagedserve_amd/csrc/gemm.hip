@@ -9,7 +9,12 @@ int ps_gemm_nt_simple(const void* a, const void* w, const float* bias, void* c, 
                       hipStream_t s);
 int ps_gemm_nt_mfma(const void* a, const void* w, const float* bias, void* c, int m, int n, int k,
                     int lda, int ldc, int dtype, int c_dtype, int epilogue,
-                    const KvScatter& scatter, const void* w_packed, hipStream_t s);
+                    const KvScatter& scatter, const void* w_packed, int layouts, hipStream_t s);
+bool ps_gemm_nt_mfma_skinny(const void* a, const void* w, int m, int n, int k, int lda, int dtype,
+                            int epilogue);
+int ps_norm_layout(const float* x, const int* rows, const float* gamma, const float* beta,
+                   void* out, int n_rows, int width, float eps, int rms, int out_dtype,
+                   int packed, hipStream_t s);
 int ps_norm_gemm_fused(const NormPrologue& norm, const void* w, const float* bias, void* c, int m,
                        int n, int k, int ldc, int c_dtype, int epilogue, const KvScatter& scatter,
                        const void* w_packed, hipStream_t s);
@@ -70,6 +75,16 @@ extern "C" int ps_linear(const PsLinearArgs* p, void* stream) {
 
   const void* a = p->a;
   int lda = p->lda;
+  if (p->c_layout != nullptr) *p->c_layout = 0;
+  // 17 to 64 rows of bfloat16: activations may travel in the packed order (linear.h)
+  const bool decode_rows = p->dtype == PS_BF16 && m > 16 && m <= 64;
+  const int padded_rows = (m + 15) / 16 * 16;
+  int layouts = 0;
+  if (p->a_packed) {
+    PS_REQUIRE(!has_norm && decode_rows && k % 64 == 0,
+               "ps_linear: packed input rows go with 17 to 64 bfloat16 rows and k a multiple of 64");
+    layouts |= 1;
+  }
   if (has_norm) {
     NormPrologue norm = {p->norm_h, p->norm_rows, p->gamma, p->beta, p->eps, p->rms, p->ldh};
     if (ps_norm_gemm_fusable(p->w, norm, m, n, k, p->dtype)) {
@@ -78,19 +93,33 @@ extern "C" int ps_linear(const PsLinearArgs* p, void* stream) {
     }
     PS_REQUIRE(p->norm_out != nullptr, "ps_linear: scratch for the normed rows is needed");
     PS_REQUIRE(p->ldh == k, "ps_linear: unfused norm needs dense rows (ldh %d, k %d)", p->ldh, k);
-    int status = ps_norm(p->norm_h, p->norm_rows, p->gamma, p->beta, p->norm_out, m, k, p->eps,
-                         p->rms, p->dtype, stream);
+    const bool pack_norm = decode_rows && k % 64 == 0 && k <= 2048 &&
+                           p->norm_out_rows >= padded_rows &&
+                           ps_gemm_nt_mfma_skinny(p->norm_out, p->w, m, n, k, k, p->dtype, p->epilogue);
+    int status = ps_norm_layout(p->norm_h, p->norm_rows, p->gamma, p->beta, p->norm_out, m, k,
+                                p->eps, p->rms, p->dtype, pack_norm ? 1 : 0, s);
     if (status != 0) return status;
     a = p->norm_out;
     lda = k;
+    if (pack_norm) layouts |= 1;
   }
   // Matrix cores when the operands allow 16-byte loads; in float only for many rows (the
   // tile is 128 rows high), else the plain kernel.
   const bool mfma = ps_gemm_nt_mfma_supported(a, p->w, k, lda, p->dtype) &&
                     (p->dtype == PS_BF16 || m >= 96);
-  if (mfma)
+  if (mfma) {
+    if (p->c_packed_request && decode_rows && p->c_dtype == PS_BF16 && n % 64 == 0 &&
+        p->epilogue != PS_EPI_RESIDUAL && scatter.k_pool == nullptr && p->c_rows >= padded_rows &&
+        p->ldc == n && p->c_layout != nullptr &&
+        ps_gemm_nt_mfma_skinny(a, p->w, m, n, k, lda, p->dtype, p->epilogue)) {
+      layouts |= 2;
+      *p->c_layout = 1;
+    }
     return ps_gemm_nt_mfma(a, p->w, p->bias, p->c, m, n, k, lda, p->ldc, p->dtype, p->c_dtype,
-                           p->epilogue, scatter, p->dtype == PS_BF16 ? p->w_packed : nullptr, s);
+                           p->epilogue, scatter, p->dtype == PS_BF16 ? p->w_packed : nullptr,
+                           layouts, s);
+  }
+  PS_REQUIRE(layouts == 0, "ps_linear: packed input rows need operands that the matrix-core kernels take");
   int status = ps_gemm_nt_simple(a, p->w, p->bias, p->c, m, n, k, lda, p->ldc, p->dtype,
                                  p->c_dtype, p->epilogue, s);
   if (status != 0 || scatter.k_pool == nullptr) return status;

@@ -245,7 +245,7 @@ __global__ __launch_bounds__(256) void gemm_nt_tiled_kernel(
 template <typename TOut, int EPI, int MB>
 __device__ inline void skinny_epilogue(float (*partial)[MB][4][64], const float* bias, TOut* c,
                                        int m, int n, int ldc, int n0, int row0, int split,
-                                       int k_splits, const KvScatter& scatter) {
+                                       int k_splits, const KvScatter& scatter, int c_packed = 0) {
   const int col_in = threadIdx.x & 15;
   const int row_in = threadIdx.x >> 4;
   const int col = n0 + col_in;
@@ -259,7 +259,9 @@ __device__ inline void skinny_epilogue(float (*partial)[MB][4][64], const float*
     if (row >= m) continue;
     float v = partial[0][b][i][lane] + partial[1][b][i][lane] + partial[2][b][i][lane] +
               partial[3][b][i][lane] + bias_here;
-    TOut* dst = c + (int64_t)row * ldc + col;
+    // (c_packed: the output is the operand of another skinny product and is written in the
+    // order in which that one reads it)
+    TOut* dst = c_packed ? c + packed_offset(row, col, n) : c + (int64_t)row * ldc + col;
     if (EPI == PS_EPI_RESIDUAL) {
       if (k_splits > 1) {
         unsafeAtomicAdd(reinterpret_cast<float*>(dst), v);
@@ -278,7 +280,9 @@ template <typename TOut, int EPI, int MB, int NT, int UNROLL>
 __global__ __launch_bounds__(64 * SK_WAVES) void gemm_nt_skinny_kernel(
     const bf16_t* __restrict__ a, const bf16_t* __restrict__ w, const float* __restrict__ bias,
     TOut* __restrict__ c, int m, int n, int k, int lda, int ldc, int k_chunk, int k_splits,
-    KvScatter scatter, const bf16_t* __restrict__ wp) {
+    KvScatter scatter, const bf16_t* __restrict__ wp, int layouts) {
+  // layouts: bit 0, the rows of A lie in the packed order (packed_offset); bit 1, C is to be
+  // written in it.
   // NT tiles of 16 columns per block share the loads of the rows of A: with very many
   // columns (the output head) those loads, though they come from the L2, are as many bytes
   // as the weights themselves.
@@ -310,6 +314,7 @@ __global__ __launch_bounds__(64 * SK_WAVES) void gemm_nt_skinny_kernel(
   for (int b = 0; b < MB; ++b) {
     const int row = row0 + b * 16 + sub < m ? row0 + b * 16 + sub : m - 1;
     a_ptr[b] = a + (int64_t)row * lda + group * 16;
+    if (layouts & 1) a_ptr[b] = a + (int64_t)(row >> 4) * (k / 64) * 1024 + lane * 8;
   }
   f32x4 acc[NT][MB];
 #pragma unroll
@@ -339,10 +344,12 @@ __global__ __launch_bounds__(64 * SK_WAVES) void gemm_nt_skinny_kernel(
         wf[u][j][0] = *reinterpret_cast<const uint4*>(w_ptr[j] + p0);
         wf[u][j][1] = *reinterpret_cast<const uint4*>(w_ptr[j] + p1);
       }
+      const int q0 = (layouts & 1) ? (first ? (ku / 64) * 1024 : 0) : o0;
+      const int q1 = (layouts & 1) ? q0 + 512 : o1;
 #pragma unroll
       for (int b = 0; b < MB; ++b) {
-        xf[u][b][0] = *reinterpret_cast<const uint4*>(a_ptr[b] + o0);
-        xf[u][b][1] = *reinterpret_cast<const uint4*>(a_ptr[b] + o1);
+        xf[u][b][0] = *reinterpret_cast<const uint4*>(a_ptr[b] + q0);
+        xf[u][b][1] = *reinterpret_cast<const uint4*>(a_ptr[b] + q1);
       }
       if (!first) {
 #pragma unroll
@@ -381,7 +388,7 @@ __global__ __launch_bounds__(64 * SK_WAVES) void gemm_nt_skinny_kernel(
 #pragma unroll
   for (int j = 0; j < NT; ++j)
     skinny_epilogue<TOut, EPI, MB>(partial[j], bias, c, m, n, ldc, n0 + j * 16, row0, split,
-                                   k_splits, scatter);
+                                   k_splits, scatter, layouts & 2);
 }
 
 // ---------------------------------------------------------------- skinny with fused norm
@@ -591,7 +598,8 @@ static int launch_tiled(const void* a, const void* w, const float* bias, void* c
 template <typename TOut, int EPI>
 static void launch_skinny_mb(const void* a, const void* w, const float* bias, void* c, int m,
                              int n, int k, int lda, int ldc, int k_chunk, int k_splits,
-                             const KvScatter& scatter, const bf16_t* wp, hipStream_t s) {
+                             const KvScatter& scatter, const bf16_t* wp, int layouts,
+                             hipStream_t s) {
   // Rows go 16 to an accumulator, up to four accumulators to a block.  Where the columns and
   // the k ranges give few blocks, the rows are spread over more of them (every one reads the
   // same weights, which the L2 absorbs; blocks that differ only in z run on one XCD when the
@@ -606,18 +614,18 @@ static void launch_skinny_mb(const void* a, const void* w, const float* bias, vo
 #define PS_LAUNCH_SK(MB)                                                                       \
   hipLaunchKernelGGL((gemm_nt_skinny_kernel<TOut, EPI, MB, 1, SK_UNROLL>), grid, block, 0, s,  \
                      (const bf16_t*)a, (const bf16_t*)w, bias, (TOut*)c, m, n, k, lda, ldc,    \
-                     k_chunk, k_splits, scatter, wp)
+                     k_chunk, k_splits, scatter, wp, layouts)
   if (per <= 1 && k_splits == 1 && n >= 16 * 1024) {
     // the output head: two tiles of columns per block
     grid.x = (n + 31) / 32;
     hipLaunchKernelGGL((gemm_nt_skinny_kernel<TOut, EPI, 1, 2, SK_UNROLL>), grid, block, 0, s,
                        (const bf16_t*)a, (const bf16_t*)w, bias, (TOut*)c, m, n, k, lda, ldc,
-                       k_chunk, k_splits, scatter, wp);
+                       k_chunk, k_splits, scatter, wp, layouts);
   } else if (per <= 1 && k_chunk > SK_WAVES * SK_UNROLL * 64) {
     // up to 16 rows leave registers for twice the loads: a k of up to 2048 in one round
     hipLaunchKernelGGL((gemm_nt_skinny_kernel<TOut, EPI, 1, 1, 2 * SK_UNROLL>), grid, block, 0, s,
                        (const bf16_t*)a, (const bf16_t*)w, bias, (TOut*)c, m, n, k, lda, ldc,
-                       k_chunk, k_splits, scatter, wp);
+                       k_chunk, k_splits, scatter, wp, layouts);
   } else if (per <= 1) PS_LAUNCH_SK(1);
   else if (per == 2) PS_LAUNCH_SK(2);
   else if (per == 3) PS_LAUNCH_SK(3);
@@ -628,7 +636,7 @@ static void launch_skinny_mb(const void* a, const void* w, const float* bias, vo
 template <typename TOut>
 static int launch_skinny(const void* a, const void* w, const float* bias, void* c, int m, int n,
                          int k, int lda, int ldc, int epilogue, const KvScatter& scatter,
-                         const bf16_t* wp, hipStream_t s) {
+                         const bf16_t* wp, int layouts, hipStream_t s) {
   if (k % 64 != 0) wp = nullptr;   // the packed copy exists for whole steps of 64 only
   // A block covers 1024 k with one round of loads.  Longer k is split over blocks where the
   // partial sums can be added in place (residual epilogue), else the block loops.
@@ -639,7 +647,8 @@ static int launch_skinny(const void* a, const void* w, const float* bias, void* 
   k_splits = (k + k_chunk - 1) / k_chunk;
 #define PS_SKINNY_CASE(EPI)                                                                      \
   case EPI:                                                                                      \
-    launch_skinny_mb<TOut, EPI>(a, w, bias, c, m, n, k, lda, ldc, k_chunk, k_splits, scatter, wp, s); \
+    launch_skinny_mb<TOut, EPI>(a, w, bias, c, m, n, k, lda, ldc, k_chunk, k_splits, scatter, wp, \
+                                layouts, s);                                                     \
     break
   switch (epilogue) {
     PS_SKINNY_CASE(PS_EPI_NONE);
@@ -686,23 +695,35 @@ int ps_norm_gemm_fused(const NormPrologue& norm, const void* w, const float* bia
   return launch_skinny_norm<bf16_t>(norm, w, bias, c, m, n, k, ldc, epilogue, scatter, wp, s);
 }
 
+// Whether ps_gemm_nt_mfma takes the skinny kernel for this product.
+// Up to 64 rows the skinny kernel has every load of a block in flight at once, which counts
+// when the weights come from memory and not from a cache; the tiled kernel walks k tile by
+// tile and wins only where there are tiles enough to fill the chip (the output head).
+// A k beyond one round of the skinny kernel's loads makes it loop; there the tiled kernel
+// with its deep ring of stages is ahead, except where partial sums of a split k can be
+// added in place (residual epilogue), which keeps every block at one round.
+bool ps_gemm_nt_mfma_skinny(const void* a, const void* w, int m, int n, int k, int lda, int dtype,
+                            int epilogue) {
+  if (dtype != PS_BF16 || m > 64) return false;
+  const bool skinny_k = n < 64 * 256 && (epilogue == PS_EPI_RESIDUAL || k <= 1024 || m <= 16);
+  return skinny_k || !ps_gemm_nt_bf16_tiled_supported(a, w, m, k, lda);
+}
+
 int ps_gemm_nt_mfma(const void* a, const void* w, const float* bias, void* c, int m, int n, int k,
                     int lda, int ldc, int dtype, int c_dtype, int epilogue,
-                    const KvScatter& scatter, const void* w_packed, hipStream_t s) {
+                    const KvScatter& scatter, const void* w_packed, int layouts, hipStream_t s) {
   const bf16_t* wp = (const bf16_t*)w_packed;
-  // Up to 64 rows the skinny kernel has every load of a block in flight at once, which counts
-  // when the weights come from memory and not from a cache; the tiled kernel walks k tile by
-  // tile and wins only where there are tiles enough to fill the chip (the output head).
-  // A k beyond one round of the skinny kernel's loads makes it loop; there the tiled kernel
-  // with its deep ring of stages is ahead, except where partial sums of a split k can be
-  // added in place (residual epilogue), which keeps every block at one round.
-  const bool skinny_k = m <= 64 && n < 64 * 256 && (epilogue == PS_EPI_RESIDUAL || k <= 1024);
-  if (dtype == PS_BF16 && m <= 64 && (skinny_k || !ps_gemm_nt_bf16_tiled_supported(a, w, m, k, lda))) {
+  if (ps_gemm_nt_mfma_skinny(a, w, m, n, k, lda, dtype, epilogue)) {
     if (c_dtype == PS_F32)
-      return launch_skinny<float>(a, w, bias, c, m, n, k, lda, ldc, epilogue, scatter, wp, s);
-    return launch_skinny<bf16_t>(a, w, bias, c, m, n, k, lda, ldc, epilogue, scatter, wp, s);
+      return launch_skinny<float>(a, w, bias, c, m, n, k, lda, ldc, epilogue, scatter, wp, layouts, s);
+    return launch_skinny<bf16_t>(a, w, bias, c, m, n, k, lda, ldc, epilogue, scatter, wp, layouts, s);
   }
-  if (dtype == PS_BF16 && !skinny_k && ps_gemm_nt_bf16_tiled_supported(a, w, m, k, lda))
+  if (layouts != 0) {
+    ps_set_error("ps_linear: packed activations go with the skinny product only (m %d, n %d, k %d)",
+                 m, n, k);
+    return 1;
+  }
+  if (dtype == PS_BF16 && ps_gemm_nt_bf16_tiled_supported(a, w, m, k, lda))
     return ps_gemm_nt_bf16_tiled(a, w, bias, c, m, n, k, lda, ldc, c_dtype, epilogue, scatter, s);
   if (dtype == PS_F32 && c_dtype == PS_F32)
     return launch_tiled<float, float>(a, w, bias, c, m, n, k, lda, ldc, epilogue, scatter, s);

@@ -13,6 +13,16 @@ struct KvScatter {
   int table_width, q_cols, kv_cols, head_dim, kv_heads, page_size, page_shift, num_pages;
 };
 
+// Activations of a decode step (17 to 64 rows) may lie in the order in which the lanes of the
+// skinny product hold their operand, like the packed weight copies: rows in blocks of 16, the
+// 16 x 64 tile of row block t and columns 64 s .. 64 s + 63 at element (t * (cols / 64) + s) *
+// 1024 as two runs of 512, run h holding for lane = g * 16 + r the 8 values of row 16 t + r,
+// columns 64 s + 16 g + 8 h ...  A producer writes element (row, col) at this offset.
+__host__ __device__ inline int64_t packed_offset(int row, int col, int cols) {
+  return ((((int64_t)(row >> 4) * (cols >> 6) + (col >> 6)) * 2 + ((col >> 3) & 1)) * 64 +
+          (((col >> 4) & 3) * 16 + (row & 15))) * 8 + (col & 7);
+}
+
 struct NormPrologue {
   const float* h;        // null: no norm
   const int* rows;

@@ -49,6 +49,13 @@ int ps_gemm_nt(const void* a, const void* w, const float* bias, void* c, int m, 
 //     holds, for lane = g * 16 + r (g = 0..3, r = 0..15), the 8 values w[16 t + r][64 s + 16 g +
 //     8 h ..]: the order in which a wave's lanes hold the operand of v_mfma_f32_16x16x32_bf16,
 //     so that one load of a wave is 1 KB of consecutive memory.
+//   * packed activations: between two products of 17 to 64 rows (a decode step of a larger
+//     batch) the rows may be kept in the order in which the second product's lanes hold their
+//     operand, rows in blocks of 16 and tiles of 16 x 64 as for w_packed; it is bound by the
+//     loads of its activations as much as of its weights.  The norm in front of a product is
+//     written that way by ps_linear itself; for c the caller asks (c_packed_request, bfloat16
+//     output, n a multiple of 64, no residual epilogue, no scatter), is told through c_layout,
+//     and passes a_packed to the call that reads the buffer.
 typedef struct PsLinearArgs {
   const void* a;
   const void* w;
@@ -70,7 +77,12 @@ typedef struct PsLinearArgs {
   const int* tok_pos;
   const int* tables;
   int table_width, q_cols, kv_cols, head_dim, kv_heads, page_size, num_pages;
-  const void* w_packed;   // null, or the copy of w that ps_pack_weight_layout describes
+  const void* w_packed;   // null, or the copy of w described above
+  int a_packed;           // the rows of a lie in the packed activation order (see below)
+  int c_packed_request;   // c may be written in that order if the kernel chosen can
+  int c_rows;             // rows that c has room for (the packed order rounds m up to 16)
+  int norm_out_rows;      // rows that norm_out has room for
+  int* c_layout;          // null, or where ps_linear says how it wrote c: 0 rows, 1 packed
 } PsLinearArgs;
 
 int ps_linear(const PsLinearArgs* args, void* stream);

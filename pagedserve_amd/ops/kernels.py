@@ -224,6 +224,8 @@ class _LinearArgs(ctypes.Structure):
         ("table_width", c_int), ("q_cols", c_int), ("kv_cols", c_int), ("head_dim", c_int),
         ("kv_heads", c_int), ("page_size", c_int), ("num_pages", c_int),
         ("w_packed", c_void_p),
+        ("a_packed", c_int), ("c_packed_request", c_int), ("c_rows", c_int),
+        ("norm_out_rows", c_int), ("c_layout", ctypes.POINTER(c_int)),
     ]
 
 
@@ -266,12 +268,28 @@ def pack_decode_weight(w):
     return source.view(padded_rows // 16, 16, k // 64, 4, 2, 8).permute(0, 2, 4, 3, 1, 5).contiguous()
 
 
-def linear(x, w, bias, out, epilogue="none", scatter=None, packed=None):
+def _row_capacity(tensor, columns: int) -> int:
+    """Rows of ``columns`` values that fit from the tensor's first element to the end of its
+    storage (a workspace slice ``buffer[:tokens]`` has room for the whole buffer)."""
+    if tensor.ndim != 2 or tensor.shape[1] != columns or not tensor.is_contiguous():
+        return 0
+    elements = tensor.untyped_storage().nbytes() // tensor.element_size() - tensor.storage_offset()
+    return int(elements // columns)
+
+
+def linear(x, w, bias, out, epilogue="none", scatter=None, packed=None, a_packed=False,
+           packed_out=False):
     """out = epilogue(x w^T + bias) where ``x`` is a tensor or a ``PendingNorm``.
 
     ``scatter = (k_pool, v_pool, tok_item, tok_pos, tables, q_cols, kv_cols)`` also stores the
     key and value columns of a ``[q | k | v]`` output into their cache pages.  ``packed`` is
-    ``pack_decode_weight(w)`` or None; the kernels for few rows read it instead of ``w``."""
+    ``pack_decode_weight(w)`` or None; the kernels for few rows read it instead of ``w``.
+
+    Between two products of 17 to 64 rows the activations may travel in the order in which the
+    second one's lanes hold them (``csrc/linear.h: packed_offset``).  ``packed_out=True`` allows
+    that for ``out`` (whose storage must have room for the rows rounded up to 16) and makes the
+    call return ``(out, written_packed)``; the buffer then goes to the next call with
+    ``a_packed=written_packed`` and means nothing to anyone else."""
     _check(w, "w", ndim=2)
     _check(out, "out", ndim=2)
     n, k = w.shape
@@ -300,6 +318,9 @@ def linear(x, w, bias, out, epilogue="none", scatter=None, packed=None):
         args.rms = 1 if x.rms else 0
         args.ldh = k
         args.lda = k
+        args.norm_out_rows = _row_capacity(x.scratch, k)
+        if a_packed:
+            raise KernelError("linear: a pending norm has no packed rows")
     else:
         _check(x, "x", w.dtype, 2)
         if x.shape[1] != k:
@@ -307,6 +328,11 @@ def linear(x, w, bias, out, epilogue="none", scatter=None, packed=None):
         m = x.shape[0]
         args.a = x.data_ptr()
         args.lda = _rows(x, "x")
+        if a_packed:
+            if _row_capacity(x, k) < -(-m // 16) * 16:
+                raise KernelError("linear: packed input rows need a dense buffer with room for "
+                                  "the row count rounded up to 16")
+            args.a_packed = 1
     if out.shape[0] != m or out.shape[1] != n:
         raise KernelError(f"linear: out {tuple(out.shape)} must be [{m}, {n}]")
     if bias is not None:
@@ -342,6 +368,11 @@ def linear(x, w, bias, out, epilogue="none", scatter=None, packed=None):
         args.q_cols, args.kv_cols = int(q_cols), int(kv_cols)
         args.head_dim, args.kv_heads = head_dim, kv_heads
         args.page_size, args.num_pages = page_size, pages
+    layout = c_int(0)
+    if packed_out:
+        args.c_packed_request = 1
+        args.c_rows = _row_capacity(out, n)
+        args.c_layout = ctypes.pointer(layout)
     lib = load_library()
     fn = _BOUND.get("ps_linear")
     if fn is None:
@@ -352,6 +383,8 @@ def linear(x, w, bias, out, epilogue="none", scatter=None, packed=None):
     status = fn(ctypes.byref(args), _stream())
     if status != 0:
         raise KernelError(f"ps_linear failed ({status}): {lib.ps_last_error().decode('utf-8', 'replace')}")
+    if packed_out:
+        return out, bool(layout.value)
     return out
 
 

@@ -47,7 +47,10 @@ class DenseFeedForward(FeedForward):
 
     def forward(self, x, residual, ctx):
         hidden = ctx.workspace.rows("ffn", self.inner, self.dtype)[:ctx.tokens]
-        kernels.linear(x, self.up_weight, self.up_bias, hidden, epilogue=self.activation,
-                       packed=self.up_packed)
+        # (the hidden rows belong to these two calls alone: at 17 to 64 rows the first may leave
+        # them in the order in which the second reads them)
+        _, hidden_packed = kernels.linear(x, self.up_weight, self.up_bias, hidden,
+                                          epilogue=self.activation, packed=self.up_packed,
+                                          packed_out=True)
         kernels.linear(hidden, self.down_weight, self.down_bias, residual, epilogue="residual",
-                       packed=self.down_packed)
+                       packed=self.down_packed, a_packed=hidden_packed)

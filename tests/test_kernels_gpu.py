@@ -656,3 +656,48 @@ def test_linear_with_packed_weights(m, n, k, epilogue):
     assert kernels.pack_decode_weight(_rand((32, 128), torch.float32, 218)) is None
     with pytest.raises(kernels.KernelError, match="packed copy"):
         kernels.linear(a, w, bias, run(a, False), epilogue=epilogue, packed=packed[:-1].contiguous() if packed.shape[0] > 1 else packed.float())
+
+
+@pytest.mark.parametrize("m", [17, 32, 47, 64])
+@pytest.mark.parametrize("inner,width", [(3072, 768), (320, 128), (1600, 1600)])
+def test_linear_chain_with_packed_activations(m, inner, width):
+    """Norm, product, activation, product as a decode step of 17 to 64 rows runs them: the
+    normed rows and the hidden rows may travel in the lanes' operand order.  The result equals
+    the chain with every buffer row by row, bit for bit up to the order of atomic adds."""
+    from pagedserve_amd.ops import kernels
+
+    dtype = torch.bfloat16
+    h = _rand((m, width), torch.float32, 230, 2.0)
+    gamma = 1.0 + _rand((width,), torch.float32, 231, 0.2)
+    beta = _rand((width,), torch.float32, 232, 0.2)
+    up = _rand((inner, width), dtype, 233, 1.0 / math.sqrt(width))
+    down = _rand((width, inner), dtype, 234, 1.0 / math.sqrt(inner))
+    up_bias, down_bias = _rand((inner,), torch.float32, 235), _rand((width,), torch.float32, 236)
+    start = _rand((m, width), torch.float32, 237)
+    workspace_rows = 80                      # room for the rows rounded up to 16
+
+    def chain(allow_packed):
+        scratch = torch.full((workspace_rows, width), float("nan"), dtype=dtype, device="cuda")
+        hidden = torch.full((workspace_rows, inner), float("nan"), dtype=dtype, device="cuda")[:m]
+        # a scratch slice without room behind it keeps the norm row by row
+        normed = scratch[:m] if allow_packed else scratch[:m].clone()
+        pending = kernels.PendingNorm(h, gamma, beta, 1e-5, False, normed, None)
+        if allow_packed:
+            _, was_packed = kernels.linear(pending, up, up_bias, hidden, epilogue="gelu_tanh", packed_out=True)
+        else:
+            kernels.linear(pending, up, up_bias, hidden, epilogue="gelu_tanh")
+            was_packed = False
+        out = start.clone()
+        kernels.linear(hidden, down, down_bias, out, epilogue="residual", a_packed=was_packed)
+        return out, was_packed
+
+    plain, _ = chain(False)
+    fast, was_packed = chain(True)
+    # the first product is skinny when k <= 1024 or the rows are too few for the tiled kernel:
+    # then its output travels packed
+    assert was_packed == ((width <= 1024 or m <= 32) and inner % 64 == 0)
+    torch.testing.assert_close(fast, plain, atol=1e-4, rtol=1e-5)
+    reference = start.double() + F.gelu(
+        (F.layer_norm(h.double(), (width,), gamma.double(), beta.double(), 1e-5).to(dtype).double()
+         @ up.double().t() + up_bias.double()), approximate="tanh").to(dtype).double() @ down.double().t() + down_bias.double()
+    assert (fast.double() - reference).abs().max().item() <= 2e-2 * reference.abs().max().item()
