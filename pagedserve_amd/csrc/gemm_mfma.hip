@@ -459,55 +459,40 @@ __global__ __launch_bounds__(64 * SK_WAVES) void gemm_nt_skinny_norm_kernel(
       wf[u][1] = *reinterpret_cast<const uint4*>(w_ptr + p1);
     }
     // rows beyond m (the same for the whole wave) are not worked on
-    bool live_row[4];
-#pragma unroll
-    for (int j = 0; j < 4; ++j) live_row[j] = wave + j * SK_WAVES < m;
-    float sum[4], sq[4], mean[4], inv_std[4];
-#pragma unroll
-    for (int j = 0; j < 4; ++j) {
-      sum[j] = 0.f;
-      if (!live_row[j]) continue;
-#pragma unroll
-      for (int i = 0; i < V4; ++i) {
-        if (!in_row[i]) v[j][i] = zero4;
-        sum[j] += (v[j][i].x + v[j][i].y) + (v[j][i].z + v[j][i].w);
-      }
-    }
-#pragma unroll
-    for (int j = 0; j < 4; ++j)
-      mean[j] = (norm.rms || !live_row[j]) ? 0.f : wave_sum(sum[j]) / (float)k;
-#pragma unroll
-    for (int j = 0; j < 4; ++j) {
-      sq[j] = 0.f;
-      if (!live_row[j]) continue;
-#pragma unroll
-      for (int i = 0; i < V4; ++i) {
-        if (in_row[i]) {
-          v[j][i].x -= mean[j];
-          v[j][i].y -= mean[j];
-          v[j][i].z -= mean[j];
-          v[j][i].w -= mean[j];
-        }
-        sq[j] += (v[j][i].x * v[j][i].x + v[j][i].y * v[j][i].y) +
-                 (v[j][i].z * v[j][i].z + v[j][i].w * v[j][i].w);
-      }
-    }
-#pragma unroll
-    for (int j = 0; j < 4; ++j)
-      inv_std[j] = live_row[j] ? 1.0f / sqrtf(wave_sum(sq[j]) / (float)k + norm.eps) : 0.f;
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
       const int token = wave + j * SK_WAVES;
       const bool live = token < m;
+      float sum = 0.f, sq = 0.f, mean = 0.f, inv_std = 0.f;
+      if (live) {
+#pragma unroll
+        for (int i = 0; i < V4; ++i) {
+          if (!in_row[i]) v[j][i] = zero4;
+          sum += (v[j][i].x + v[j][i].y) + (v[j][i].z + v[j][i].w);
+        }
+        mean = norm.rms ? 0.f : wave_sum(sum) / (float)k;
+#pragma unroll
+        for (int i = 0; i < V4; ++i) {
+          if (in_row[i]) {
+            v[j][i].x -= mean;
+            v[j][i].y -= mean;
+            v[j][i].z -= mean;
+            v[j][i].w -= mean;
+          }
+          sq += (v[j][i].x * v[j][i].x + v[j][i].y * v[j][i].y) +
+                (v[j][i].z * v[j][i].z + v[j][i].w * v[j][i].w);
+        }
+        inv_std = 1.0f / sqrtf(wave_sum(sq) / (float)k + norm.eps);
+      }
 #pragma unroll
       for (int i = 0; i < V4; ++i) {
         if (!in_row[i]) continue;
         uint2 packed = {0u, 0u};
         if (live) {
-          const float y0 = v[j][i].x * inv_std[j] * g[i].x + bt[i].x;
-          const float y1 = v[j][i].y * inv_std[j] * g[i].y + bt[i].y;
-          const float y2 = v[j][i].z * inv_std[j] * g[i].z + bt[i].z;
-          const float y3 = v[j][i].w * inv_std[j] * g[i].w + bt[i].w;
+          const float y0 = v[j][i].x * inv_std * g[i].x + bt[i].x;
+          const float y1 = v[j][i].y * inv_std * g[i].y + bt[i].y;
+          const float y2 = v[j][i].z * inv_std * g[i].z + bt[i].z;
+          const float y3 = v[j][i].w * inv_std * g[i].w + bt[i].w;
           packed.x = pack2_bf16(y0, y1);
           packed.y = pack2_bf16(y2, y3);
         }
