@@ -395,7 +395,9 @@ __global__ __launch_bounds__(64 * SK_WAVES) void gemm_nt_skinny_kernel(
 #define SN_MAX_K 1024              // one round of loads covers it: 4 waves x 4 steps x 64
 #define SN_STRIDE (SN_MAX_K + 8)   // LDS row stride in elements (16-byte aligned, skewed)
 
-template <typename TOut, int EPI>
+// NR: rows that a wave normalises (rows wave, wave + 4, ...: 4 NR >= m).  Rows of LDS beyond
+// them stay as they are: they only feed outputs that are never stored.
+template <typename TOut, int EPI, int NR>
 __global__ __launch_bounds__(64 * SK_WAVES) void gemm_nt_skinny_norm_kernel(
     NormPrologue norm, const bf16_t* __restrict__ w, const float* __restrict__ bias,
     TOut* __restrict__ c, int m, int n, int k, int ldc, KvScatter scatter,
@@ -422,11 +424,11 @@ __global__ __launch_bounds__(64 * SK_WAVES) void gemm_nt_skinny_norm_kernel(
   {
     constexpr int V4 = SN_MAX_K / 256;
     const float4 zero4 = {0.f, 0.f, 0.f, 0.f};
-    float4 g[V4], bt[V4], v[4][V4];
+    float4 g[V4], bt[V4], v[NR][V4];
     bool in_row[V4];
-    const float* src[4];
+    const float* src[NR];
 #pragma unroll
-    for (int j = 0; j < 4; ++j) {
+    for (int j = 0; j < NR; ++j) {
       const int token = wave + j * SK_WAVES;
       const int t = token < m ? token : m - 1;
       src[j] = norm.h + (int64_t)(norm.rows ? norm.rows[t] : t) * norm.ldh;
@@ -441,7 +443,7 @@ __global__ __launch_bounds__(64 * SK_WAVES) void gemm_nt_skinny_norm_kernel(
                   ? *reinterpret_cast<const float4*>(norm.beta + safe)
                   : zero4;
 #pragma unroll
-      for (int j = 0; j < 4; ++j) v[j][i] = *reinterpret_cast<const float4*>(src[j] + safe);
+      for (int j = 0; j < NR; ++j) v[j][i] = *reinterpret_cast<const float4*>(src[j] + safe);
     }
     // 2. this wave's weights.  A wave's loads come back in the order in which they left, so
     //    these leave after the loads of the rows (which come from the L2 and are there first)
@@ -460,7 +462,7 @@ __global__ __launch_bounds__(64 * SK_WAVES) void gemm_nt_skinny_norm_kernel(
     }
     // rows beyond m (the same for the whole wave) are not worked on
 #pragma unroll
-    for (int j = 0; j < 4; ++j) {
+    for (int j = 0; j < NR; ++j) {
       const int token = wave + j * SK_WAVES;
       const bool live = token < m;
       float sum = 0.f, sq = 0.f, mean = 0.f, inv_std = 0.f;
@@ -654,10 +656,15 @@ static int launch_skinny_norm(const NormPrologue& norm, const void* w, const flo
   if (k % 64 != 0) wp = nullptr;
   dim3 grid((n + 15) / 16);
   dim3 block(64 * SK_WAVES);
+#define PS_NORM_LAUNCH(EPI, NR)                                                               \
+  hipLaunchKernelGGL((gemm_nt_skinny_norm_kernel<TOut, EPI, NR>), grid, block, 0, s, norm,    \
+                     (const bf16_t*)w, bias, (TOut*)c, m, n, k, ldc, scatter, wp)
 #define PS_NORM_CASE(EPI)                                                                     \
   case EPI:                                                                                   \
-    hipLaunchKernelGGL((gemm_nt_skinny_norm_kernel<TOut, EPI>), grid, block, 0, s, norm,       \
-                       (const bf16_t*)w, bias, (TOut*)c, m, n, k, ldc, scatter, wp);          \
+    if (m <= 4) PS_NORM_LAUNCH(EPI, 1);                                                       \
+    else if (m <= 8) PS_NORM_LAUNCH(EPI, 2);                                                  \
+    else if (m <= 12) PS_NORM_LAUNCH(EPI, 3);                                                 \
+    else PS_NORM_LAUNCH(EPI, 4);                                                              \
     break
   switch (epilogue) {
     PS_NORM_CASE(PS_EPI_NONE);
@@ -667,6 +674,7 @@ static int launch_skinny_norm(const NormPrologue& norm, const void* w, const flo
     default: ps_set_error("ps_linear: unknown epilogue %d", epilogue); return 1;
   }
 #undef PS_NORM_CASE
+#undef PS_NORM_LAUNCH
   PS_CHECK_LAUNCH("ps_linear(skinny, fused norm)");
   return 0;
 }
