@@ -397,7 +397,7 @@ __global__ __launch_bounds__(64 * SK_WAVES) void gemm_nt_skinny_kernel(
 
 // NR: rows that a wave normalises (rows wave, wave + 4, ...: 4 NR >= m).  Rows of LDS beyond
 // them stay as they are: they only feed outputs that are never stored.
-template <typename TOut, int EPI, int NR>
+template <typename TOut, int EPI, int NR, int UNROLL>
 __global__ __launch_bounds__(64 * SK_WAVES) void gemm_nt_skinny_norm_kernel(
     NormPrologue norm, const bf16_t* __restrict__ w, const float* __restrict__ bias,
     TOut* __restrict__ c, int m, int n, int k, int ldc, KvScatter scatter,
@@ -414,8 +414,8 @@ __global__ __launch_bounds__(64 * SK_WAVES) void gemm_nt_skinny_norm_kernel(
   if (wp != nullptr) w_ptr = wp + (int64_t)(n0 / 16) * (k / 64) * 1024 + lane * 8;   // packed copy
   const uint4 zero = {0u, 0u, 0u, 0u};
 
-  uint4 wf[SK_UNROLL][2];
-  bool first[SK_UNROLL], second[SK_UNROLL];
+  uint4 wf[UNROLL][2];
+  bool first[UNROLL], second[UNROLL];
   // 1. rows wave, wave + 4, wave + 8, wave + 12: statistics and normalisation in registers
   //    (mean, centred values, biased variance, rsqrt(var + eps), scale, shift; reference:
   //    src/kernels/triton_residual_layernorm.py:25-39), result to LDS as bfloat16.  A lane
@@ -450,7 +450,7 @@ __global__ __launch_bounds__(64 * SK_WAVES) void gemm_nt_skinny_norm_kernel(
     //    and travel while the rows are normalised; issued before them they would hold the
     //    rows back for the whole trip to memory.
 #pragma unroll
-    for (int u = 0; u < SK_UNROLL; ++u) {
+    for (int u = 0; u < UNROLL; ++u) {
       const int ku = wave * 64 + u * SK_WAVES * 64;
       const int kk = ku + group * 16;
       first[u] = kk < k;
@@ -507,7 +507,7 @@ __global__ __launch_bounds__(64 * SK_WAVES) void gemm_nt_skinny_norm_kernel(
   // 3. the product: column operand from LDS
   f32x4 acc = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-  for (int u = 0; u < SK_UNROLL; ++u) {
+  for (int u = 0; u < UNROLL; ++u) {
     const int ku = wave * 64 + u * SK_WAVES * 64;
     const int kk = ku + group * 16;
     uint4 x0 = zero, x1 = zero;
@@ -598,16 +598,23 @@ static void launch_skinny_mb(const void* a, const void* w, const float* bias, vo
   const int per = (row_blocks + z - 1) / z;
   dim3 grid((n + 15) / 16, k_splits, (row_blocks + per - 1) / per);
   dim3 block(64 * SK_WAVES);
-#define PS_LAUNCH_SK(MB)                                                                       \
-  hipLaunchKernelGGL((gemm_nt_skinny_kernel<TOut, EPI, MB, 1, SK_UNROLL>), grid, block, 0, s,  \
+  // a k range of up to 768 (GPT-2's width) needs three steps per wave, not four: a step that
+  // is not there would still be fetched from a clamped address
+  const bool three = k_chunk <= SK_WAVES * 3 * 64;
+#define PS_LAUNCH_SKU(MB, NT, UNROLL)                                                          \
+  hipLaunchKernelGGL((gemm_nt_skinny_kernel<TOut, EPI, MB, NT, UNROLL>), grid, block, 0, s,    \
                      (const bf16_t*)a, (const bf16_t*)w, bias, (TOut*)c, m, n, k, lda, ldc,    \
                      k_chunk, k_splits, scatter, wp, layouts)
+#define PS_LAUNCH_SK(MB)                                                                       \
+  do {                                                                                         \
+    if (three) PS_LAUNCH_SKU(MB, 1, 3);                                                        \
+    else PS_LAUNCH_SKU(MB, 1, SK_UNROLL);                                                      \
+  } while (0)
   if (per <= 1 && k_splits == 1 && n >= 16 * 1024) {
     // the output head: two tiles of columns per block
     grid.x = (n + 31) / 32;
-    hipLaunchKernelGGL((gemm_nt_skinny_kernel<TOut, EPI, 1, 2, SK_UNROLL>), grid, block, 0, s,
-                       (const bf16_t*)a, (const bf16_t*)w, bias, (TOut*)c, m, n, k, lda, ldc,
-                       k_chunk, k_splits, scatter, wp, layouts);
+    if (three) PS_LAUNCH_SKU(1, 2, 3);
+    else PS_LAUNCH_SKU(1, 2, SK_UNROLL);
   } else if (per <= 1 && k_chunk > SK_WAVES * SK_UNROLL * 64) {
     // up to 16 rows leave registers for twice the loads: a k of up to 2048 in one round
     hipLaunchKernelGGL((gemm_nt_skinny_kernel<TOut, EPI, 1, 1, 2 * SK_UNROLL>), grid, block, 0, s,
@@ -618,6 +625,7 @@ static void launch_skinny_mb(const void* a, const void* w, const float* bias, vo
   else if (per == 3) PS_LAUNCH_SK(3);
   else PS_LAUNCH_SK(4);
 #undef PS_LAUNCH_SK
+#undef PS_LAUNCH_SKU
 }
 
 template <typename TOut>
@@ -657,8 +665,15 @@ static int launch_skinny_norm(const NormPrologue& norm, const void* w, const flo
   dim3 grid((n + 15) / 16);
   dim3 block(64 * SK_WAVES);
 #define PS_NORM_LAUNCH(EPI, NR)                                                               \
-  hipLaunchKernelGGL((gemm_nt_skinny_norm_kernel<TOut, EPI, NR>), grid, block, 0, s, norm,    \
-                     (const bf16_t*)w, bias, (TOut*)c, m, n, k, ldc, scatter, wp)
+  do {                                                                                        \
+    if (k <= SK_WAVES * 3 * 64)                                                               \
+      hipLaunchKernelGGL((gemm_nt_skinny_norm_kernel<TOut, EPI, NR, 3>), grid, block, 0, s,   \
+                         norm, (const bf16_t*)w, bias, (TOut*)c, m, n, k, ldc, scatter, wp);  \
+    else                                                                                      \
+      hipLaunchKernelGGL((gemm_nt_skinny_norm_kernel<TOut, EPI, NR, SK_UNROLL>), grid, block, \
+                         0, s, norm, (const bf16_t*)w, bias, (TOut*)c, m, n, k, ldc, scatter, \
+                         wp);                                                                 \
+  } while (0)
 #define PS_NORM_CASE(EPI)                                                                     \
   case EPI:                                                                                   \
     if (m <= 4) PS_NORM_LAUNCH(EPI, 1);                                                       \
