@@ -216,3 +216,34 @@ def test_graph_replay_of_mixed_steps(folders, references, dtype):
     error, scale, where = helpers.max_error(rows, references[("B", dtype == "bfloat16")])
     assert error <= helpers.TOLERANCE[dtype] * scale, (error, scale, where)
     engine.cache.check_invariants()
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_many_live_requests_match_plain(tmp_path, dtype):
+    """Up to 24 live requests with portions of 1 to 23 tokens: steps of 17 to 64 tokens and
+    more, where the bfloat16 path keeps activations in the skinny products' operand order
+    (widths that are multiples of 64, unlike the two tiny configurations), against the plain
+    implementation like every other cut."""
+    from pagedserve_amd.engine import Engine
+    from pagedserve_amd.model import load_model
+
+    config = {"architectures": ["GPT2LMHeadModel"], "model_type": "gpt2", "layer_norm_epsilon": 1e-5,
+              "activation_function": "gelu", "tie_word_embeddings": True, "n_layer": 2, "n_embd": 128,
+              "n_head": 2, "n_inner": 320, "vocab_size": 1000, "n_positions": 256}
+    folder = str(tmp_path / "wide")
+    helpers.write_folder(folder, config, helpers.lively_tensors(config, 301))
+    g = torch.Generator().manual_seed(11)
+    requests = {f"m{i}": helpers.random_tokens(int(torch.randint(3, 90, (1,), generator=g)), 1000, 4000 + i)
+                for i in range(30)}
+    reference = {rid: helpers.plain_logits(folder, tokens, bfloat16=dtype == "bfloat16")
+                 for rid, tokens in requests.items()}
+    model, _ = load_model(folder, dtype=dtype)
+    steps = helpers.trace_mixed(requests, max_live=24, portion=(5, 23, 1, 9, 17), decode_tail=7, seed=5)
+    sizes = {sum(len(e["tokens"]) for e in step["entries"]) for step in steps}
+    assert any(17 <= size <= 64 for size in sizes) and any(size <= 16 for size in sizes)
+    pages = -(-helpers.live_token_budget(steps) // 16)
+    engine = Engine(model, num_pages=pages, page_size=16, max_requests=24, max_step_tokens=512)
+    rows = helpers.replay_in_process(engine, steps)
+    error, scale, where = helpers.max_error(rows, reference)
+    assert error <= helpers.TOLERANCE[dtype] * scale, (dtype, error, scale, where)
+    engine.cache.check_invariants()
