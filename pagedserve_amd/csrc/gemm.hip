@@ -21,6 +21,10 @@ int ps_norm_gemm_fused(const NormPrologue& norm, const void* w, const float* bia
 bool ps_gemm_nt_mfma_supported(const void* a, const void* w, int k, int lda, int dtype);
 bool ps_norm_gemm_fusable(const void* w, const NormPrologue& norm, int m, int n, int k, int dtype);
 
+// The size of the argument block, so that a caller that lays it out by hand can check that
+// it agrees with this library.
+extern "C" int ps_linear_args_size(void) { return (int)sizeof(PsLinearArgs); }
+
 extern "C" int ps_linear(const PsLinearArgs* p, void* stream) {
   PS_REQUIRE(p != nullptr, "ps_linear: no arguments");
   const int m = p->m, n = p->n, k = p->k;

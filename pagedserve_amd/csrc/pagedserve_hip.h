@@ -86,6 +86,7 @@ typedef struct PsLinearArgs {
 } PsLinearArgs;
 
 int ps_linear(const PsLinearArgs* args, void* stream);
+int ps_linear_args_size(void);   // sizeof(PsLinearArgs) as this library was built
 
 // Store keys and values of the step's tokens into their pages.
 //   k, v: [tokens, kv_heads * head_dim] with row stride `stride`;

@@ -376,6 +376,11 @@ def linear(x, w, bias, out, epilogue="none", scatter=None, packed=None, a_packed
     lib = load_library()
     fn = _BOUND.get("ps_linear")
     if fn is None:
+        lib.ps_linear_args_size.restype = c_int
+        if lib.ps_linear_args_size() != ctypes.sizeof(_LinearArgs):
+            raise KernelError("ps_linear: the argument block of this module "
+                              f"({ctypes.sizeof(_LinearArgs)} bytes) is not the library's "
+                              f"({lib.ps_linear_args_size()} bytes); rebuild the library")
         fn = lib.ps_linear
         fn.argtypes = [ctypes.POINTER(_LinearArgs), c_void_p]
         fn.restype = c_int
