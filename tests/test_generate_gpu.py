@@ -272,3 +272,31 @@ def test_smoke_entry():
     import __graft_entry__
 
     __graft_entry__.smoke()
+
+
+@pytest.mark.parametrize("strategy", ["orca", "sarathi"])
+def test_many_requests_under_page_pressure_match_plain(folders, strategy):
+    """Twenty requests of random lengths through the scheduler with pages for a few of them
+    at a time: requests wait, run, end and give their pages to the next ones; every output
+    equals the plain implementation's greedy continuation, and nothing is left behind."""
+    from pagedserve_amd.engine.llm import LLM
+    from pagedserve_amd.sampling import SamplingParams
+
+    folder, config, page_size = folders["A"]
+    g = torch.Generator().manual_seed(23)
+    lengths = [int(torch.randint(1, 60, (1,), generator=g)) for _ in range(20)]
+    budgets = [int(torch.randint(2, 14, (1,), generator=g)) for _ in range(20)]
+    prompts = [helpers.random_tokens(n, config["vocab_size"], 800 + i) for i, n in enumerate(lengths)]
+    raw, weights = plain_gpt2.read_model_folder(folder)
+    expected = [plain_gpt2.greedy_generate(raw, weights, prompt, budget) for prompt, budget in zip(prompts, budgets)]
+    options = dict(scheduling_strategy=strategy)
+    if strategy == "sarathi":
+        options.update(prefill_chunk_size=16, max_prefill_requests=2)
+    # 30 pages of 8 tokens: the longest request needs 10 of them, so three to six run at a time
+    llm = LLM(folder, dtype="float32", block_size=page_size, num_kv_pages=30, max_batch_size=6,
+              eos_token_id=None, **options)
+    outputs = llm.generate(prompts, [SamplingParams(max_new_tokens=budget) for budget in budgets])
+    assert [o.token_ids for o in outputs] == expected
+    llm.engine.cache.check_invariants()
+    assert not llm.engine.cache.requests
+    assert llm.scheduler.iterations > 20       # they did not all fit at once
