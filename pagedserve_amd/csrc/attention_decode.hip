@@ -14,6 +14,8 @@
 // attention_reduce_kernel merges the splits.
 #include <math.h>
 
+#include <mutex>
+
 #include "common.h"
 #include "pagedserve_hip.h"
 
@@ -300,6 +302,94 @@ static int launch_decode(const void* q, int64_t q_stride, const void* k_pool, co
   return 0;
 }
 
+static int check_decode_sizes(const char* who, int count, int heads, int kv_heads, int head_dim,
+                              int page_size, int num_pages, int table_width, int window,
+                              int splits, int waves, int dtype) {
+  PS_REQUIRE(count >= 0 && heads > 0 && kv_heads > 0 && page_size > 0 && num_pages > 0 &&
+                 table_width > 0,
+             "%s: bad sizes", who);
+  PS_REQUIRE(heads % kv_heads == 0, "%s: heads (%d) must be a multiple of kv_heads (%d)", who,
+             heads, kv_heads);
+  PS_REQUIRE(head_dim > 0 && head_dim % 16 == 0 && head_dim <= 256,
+             "%s: head_dim %d must be a multiple of 16 up to 256", who, head_dim);
+  PS_REQUIRE(window >= 0, "%s: negative window", who);
+  PS_REQUIRE(splits >= 1 && splits <= 64 && heads <= 65535,
+             "%s: splits %d / heads %d out of range", who, splits, heads);
+  PS_REQUIRE(dtype == PS_F32 || dtype == PS_BF16, "%s: unknown dtype %d", who, dtype);
+  PS_REQUIRE(waves == 4 || waves == 16, "%s: blocks have 4 or 16 waves, not %d", who, waves);
+  return 0;
+}
+
+// ---- the variant that allocates nothing ------------------------------------------------------
+// The partial results of the key ranges live in a file-scope device array instead of a buffer
+// that the caller allocates.  Every GPU holds its own copy of the array at its own address;
+// the name below is only the host's handle for hipGetSymbolAddress, never a kernel argument.
+static __device__ __align__(256) float scratch[PS_DECODE_STATIC_SCRATCH_FLOATS];
+
+#define PS_MAX_DEVICES 64
+static std::mutex g_scratch_mutex;
+static float* g_scratch_ptr[PS_MAX_DEVICES];   // per device: where its copy of `scratch` lies
+
+// The address of the current device's copy (looked up once per device), or null with the
+// error set.
+static float* static_scratch_of_current_device() {
+  int device = -1;
+  hipError_t status = hipGetDevice(&device);
+  if (status != hipSuccess || device < 0 || device >= PS_MAX_DEVICES) {
+    ps_set_error("ps_attention_decode_static: no current device (%s)",
+                 status == hipSuccess ? "index out of range" : hipGetErrorString(status));
+    return nullptr;
+  }
+  std::lock_guard<std::mutex> lock(g_scratch_mutex);
+  if (g_scratch_ptr[device] == nullptr) {
+    void* address = nullptr;
+    status = hipGetSymbolAddress(&address, HIP_SYMBOL(scratch));
+    if (status != hipSuccess || address == nullptr) {
+      ps_set_error("ps_attention_decode_static: hipGetSymbolAddress failed on device %d: %s",
+                   device, hipGetErrorString(status));
+      return nullptr;
+    }
+    g_scratch_ptr[device] = static_cast<float*>(address);
+  }
+  return g_scratch_ptr[device];
+}
+
+extern "C" int ps_attention_decode_static(const void* q, int64_t q_stride, const void* k_pool,
+                                          const void* v_pool, void* out, int64_t out_stride,
+                                          const int* tok_list, const int* tok_item,
+                                          const int* tok_pos, const int* tables, int table_width,
+                                          int count, int heads, int kv_heads, int head_dim,
+                                          int page_size, int num_pages, float scale, int window,
+                                          int splits, int waves, int dtype, void* stream) {
+  if (check_decode_sizes("ps_attention_decode_static", count, heads, kv_heads, head_dim, page_size,
+                         num_pages, table_width, window, splits, waves, dtype))
+    return 1;
+  float* partial = nullptr;
+  if (splits > 1) {
+    const int64_t need = (int64_t)count * heads * splits * (head_dim + 2);
+    PS_REQUIRE(need <= (int64_t)PS_DECODE_STATIC_SCRATCH_FLOATS,
+               "ps_attention_decode_static: %d tokens x %d heads x %d splits x (%d + 2) = %lld "
+               "floats of partial results exceed the static scratch of %lld floats; use fewer "
+               "splits or ps_attention_decode with a buffer of the caller",
+               count, heads, splits, head_dim, (long long)need,
+               (long long)PS_DECODE_STATIC_SCRATCH_FLOATS);
+    partial = static_scratch_of_current_device();
+    if (partial == nullptr) return 3;
+  }
+  if (count == 0) return 0;
+  // Nothing in the scratch has to start at zero: every (token, head, range) block writes its
+  // whole record (accumulators, maximum, sum) before the merge kernel reads it, also when its
+  // range holds no key.
+  hipStream_t s = (hipStream_t)stream;
+  if (dtype == PS_F32)
+    return launch_decode<float>(q, q_stride, k_pool, v_pool, out, out_stride, partial, tok_list,
+                                tok_item, tok_pos, tables, table_width, count, heads, kv_heads,
+                                head_dim, page_size, num_pages, scale, window, splits, waves, s);
+  return launch_decode<bf16_t>(q, q_stride, k_pool, v_pool, out, out_stride, partial, tok_list,
+                               tok_item, tok_pos, tables, table_width, count, heads, kv_heads,
+                               head_dim, page_size, num_pages, scale, window, splits, waves, s);
+}
+
 extern "C" int ps_attention_decode(const void* q, int64_t q_stride, const void* k_pool,
                                    const void* v_pool, void* out, int64_t out_stride,
                                    float* partial, int64_t partial_floats, const int* tok_list,
@@ -307,19 +397,9 @@ extern "C" int ps_attention_decode(const void* q, int64_t q_stride, const void* 
                                    int table_width, int count, int heads, int kv_heads,
                                    int head_dim, int page_size, int num_pages, float scale,
                                    int window, int splits, int waves, int dtype, void* stream) {
-  PS_REQUIRE(count >= 0 && heads > 0 && kv_heads > 0 && page_size > 0 && num_pages > 0 &&
-                 table_width > 0,
-             "ps_attention_decode: bad sizes");
-  PS_REQUIRE(heads % kv_heads == 0,
-             "ps_attention_decode: heads (%d) must be a multiple of kv_heads (%d)", heads, kv_heads);
-  PS_REQUIRE(head_dim > 0 && head_dim % 16 == 0 && head_dim <= 256,
-             "ps_attention_decode: head_dim %d must be a multiple of 16 up to 256", head_dim);
-  PS_REQUIRE(window >= 0, "ps_attention_decode: negative window");
-  PS_REQUIRE(splits >= 1 && splits <= 64 && heads <= 65535,
-             "ps_attention_decode: splits %d / heads %d out of range", splits, heads);
-  PS_REQUIRE(dtype == PS_F32 || dtype == PS_BF16, "ps_attention_decode: unknown dtype %d", dtype);
-  PS_REQUIRE(waves == 4 || waves == 16, "ps_attention_decode: blocks have 4 or 16 waves, not %d",
-             waves);
+  if (check_decode_sizes("ps_attention_decode", count, heads, kv_heads, head_dim, page_size,
+                         num_pages, table_width, window, splits, waves, dtype))
+    return 1;
   if (splits > 1) {
     const int64_t need = (int64_t)count * heads * splits * (head_dim + 2);
     PS_REQUIRE(partial != nullptr && partial_floats >= need,

@@ -116,6 +116,24 @@ int ps_attention_decode(const void* q, int64_t q_stride, const void* k_pool, con
                         int head_dim, int page_size, int num_pages, float scale, int window,
                         int splits, int waves, int dtype, void* stream);
 
+// ps_attention_decode for callers that cannot allocate device memory: code under HIP graph
+// capture, tight serving loops, harnesses that forbid hipMalloc.  It has no counterpart in the
+// reference.  The partial results of the key ranges go into a device array that is part of the
+// library (PS_DECODE_STATIC_SCRATCH_FLOATS floats = 8 MiB, held by every GPU the library runs
+// on until the process ends) instead of a buffer of the caller; the call allocates and frees
+// nothing.  count * heads * splits * (head_dim + 2) beyond that size is refused with an error.
+// All calls on one GPU share that GPU's array: calls that overlap in time on one GPU (different
+// streams, or threads) race on it and give wrong results; calls on one stream are ordered and
+// safe.  Nothing in the array has to be cleared between calls.
+#define PS_DECODE_STATIC_SCRATCH_FLOATS (2 * 1024 * 1024)
+int ps_attention_decode_static(const void* q, int64_t q_stride, const void* k_pool,
+                               const void* v_pool, void* out, int64_t out_stride,
+                               const int* tok_list, const int* tok_item, const int* tok_pos,
+                               const int* tables, int table_width, int count, int heads,
+                               int kv_heads, int head_dim, int page_size, int num_pages,
+                               float scale, int window, int splits, int waves, int dtype,
+                               void* stream);
+
 // Tiled attention on the matrix cores for items that bring several tokens (bfloat16, head_dim a
 // multiple of 16 up to 128).  Tile i covers queries tile_q0[i] .. tile_q0[i] + 63 of item
 // tile_item[i]; cu_tokens and kv_lens describe the step's items.  Blocks start in the order of
