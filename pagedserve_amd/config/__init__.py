@@ -1,4 +1,5 @@
-from .gpt2 import ConfigError, GPT2Config, read_config_json
+from .base import ConfigError, read_config_json
+from .gpt2 import GPT2Config
 from .registry import ARCHITECTURES, Architecture, register_architecture, resolve_architecture
 from .spec import BlockSpec, LayerCall, ModelSpec, PartSpec
 

@@ -6,28 +6,13 @@ what it cannot run (src/model/gpt2.py:23-30).  Here the JSON file itself is the
 source, and no size or constant that it gives is repeated in code.
 """
 
-import json
-import os
 from dataclasses import dataclass
 from typing import Optional
 
+from .base import ConfigError, require_int as _require_int
+
 _TANH_GELU = ("gelu_new", "gelu_pytorch_tanh")
 _ERF_GELU = ("gelu",)
-
-
-class ConfigError(ValueError):
-    """A config.json that this engine cannot run, with the reason."""
-
-
-def _require_int(raw, key, default=None, minimum=1):
-    value = raw.get(key, default)
-    if value is None:
-        raise ConfigError(f"config.json lacks '{key}'")
-    if isinstance(value, bool) or not isinstance(value, int):
-        raise ConfigError(f"config.json '{key}' must be an integer, got {value!r}")
-    if value < minimum:
-        raise ConfigError(f"config.json '{key}' must be >= {minimum}, got {value}")
-    return value
 
 
 @dataclass(frozen=True)
@@ -125,14 +110,3 @@ class GPT2Config:
             "tie_word_embeddings": self.tie_word_embeddings,
             "eos_token_id": self.eos_token_id,
         }
-
-
-def read_config_json(folder) -> dict:
-    path = os.path.join(folder, "config.json")
-    if not os.path.isfile(path):
-        raise ConfigError(f"{folder!r} holds no config.json")
-    with open(path) as handle:
-        raw = json.load(handle)
-    if not isinstance(raw, dict):
-        raise ConfigError(f"{path} does not hold a JSON object")
-    return raw

@@ -4,13 +4,14 @@ The reference picks a model by a fixed tuple of names and an if/elif chain
 (main.py:22-25,104-130).  Here ``config.json``'s ``architectures[0]`` is the key.
 An entry bundles the typed configuration class, the function that turns it into a
 ``ModelSpec`` (parts, run order), the map from checkpoint tensor names to the
-parts' parameters, and the random initialiser of the random-weights mode.
+parts' parameters, how the checkpoint's names are prefixed, and the random initialiser of
+the random-weights mode.
 """
 
 from dataclasses import dataclass
 from typing import Any, Callable, Dict
 
-from .gpt2 import ConfigError
+from .base import ConfigError
 from .spec import ModelSpec
 
 
@@ -27,6 +28,10 @@ class Architecture:
     # names of checkpoint tensors that may be present and are not weights
     ignorable: Callable[[Any, str], bool] = lambda config, name: False
     model_type: str = ""
+    # prefixes under which checkpoints of this architecture may store their tensors
+    strip_prefixes: tuple = ()
+    # (config, canonical tensor name) -> the name under which the random-weights mode stores it
+    stored_name: Callable[[Any, str], str] = lambda config, name: name
 
 
 ARCHITECTURES: Dict[str, Architecture] = {}

@@ -1,7 +1,7 @@
 """Architecture-neutral description of a model as data.
 
 A model is an embedding, a list of blocks, an order in which the blocks run, a final
-norm and an output head.  Every block names its parts by *kind* with the sizes and
+norm and an output head, each of them a part chosen by kind.  Every block names its parts by *kind* with the sizes and
 constants they need, so two layers of one model may use different mixers or
 feed-forwards, and nothing in a part knows which model it belongs to.
 
@@ -37,15 +37,41 @@ class PartSpec:
 class BlockSpec:
     """One layer: how its parts are arranged and which parts they are.
 
-    ``arrangement`` names a block class (``"pre_norm"``: ``h += mixer(norm1(h))``
-    then ``h += feed_forward(norm2(h))``).
+    ``arrangement`` names a block class; the class says which named parts it is made of and
+    what role each plays (``"pre_norm"``: ``norm1``, ``mixer``, ``norm2``, ``feed_forward``,
+    run as ``h += mixer(norm1(h))`` then ``h += feed_forward(norm2(h))``).  ``parts`` gives a
+    ``PartSpec`` for each of those names, so an arrangement with another number of parts needs
+    no other record.
     """
 
     arrangement: str
-    norm1: PartSpec
-    mixer: PartSpec
-    norm2: PartSpec
-    feed_forward: PartSpec
+    parts: Tuple[Tuple[str, PartSpec], ...]
+
+    @staticmethod
+    def make(arrangement: str, **parts: PartSpec) -> "BlockSpec":
+        return BlockSpec(arrangement, tuple(parts.items()))
+
+    def with_part(self, name: str, spec: PartSpec) -> "BlockSpec":
+        """This block with the part ``name`` replaced (or added)."""
+        parts = dict(self.parts)
+        parts[name] = spec
+        return BlockSpec(self.arrangement, tuple(parts.items()))
+
+    def part(self, name: str) -> PartSpec:
+        for key, spec in self.parts:
+            if key == name:
+                return spec
+        raise KeyError(f"block of arrangement {self.arrangement!r} has no part {name!r}; "
+                       f"it has: {', '.join(key for key, _ in self.parts)}")
+
+    def __getattr__(self, name):
+        # block.mixer, block.norm1, ...: the named part
+        if name.startswith("__") or name in ("arrangement", "parts"):
+            raise AttributeError(name)
+        try:
+            return self.part(name)
+        except KeyError as error:
+            raise AttributeError(str(error)) from None
 
 
 @dataclass(frozen=True)
@@ -77,6 +103,9 @@ class ModelSpec:
     tie_head: bool
     eos_token_id: Optional[int] = None
     extra: Tuple[Tuple[str, Any], ...] = field(default=())
+    # how token ids become rows of the stream, and how the last rows become logits
+    embedding: PartSpec = PartSpec("lookup")
+    head: PartSpec = PartSpec("linear")
 
     def __post_init__(self):
         if not self.blocks:

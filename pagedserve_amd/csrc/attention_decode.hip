@@ -52,9 +52,15 @@ struct Raw8<bf16_t> {
   }
 };
 
-// 2^x by the hardware instruction (one ulp; the arguments here are never positive).  Scores
-// are kept in units of log 2, so that no multiplication precedes it.
-__device__ inline float exp2_fast(float x) { return __builtin_amdgcn_exp2f(x); }
+// 2^x (the arguments here are never positive).  Scores are kept in units of log 2, so that no
+// multiplication precedes it.  The 32-bit path takes the library's exp2f, which is exact to an
+// ulp over the whole range, tiny results included; bfloat16 storage takes the bare hardware
+// instruction.
+template <typename T>
+__device__ inline float exp2_fast(float x) {
+  if constexpr (sizeof(T) == 4) return exp2f(x);
+  else return __builtin_amdgcn_exp2f(x);
+}
 
 // Over the lanes that hold the same head dimensions (l ^ LPK, l ^ 2 LPK, ... l ^ 32): the
 // maximum, then the sums of the states scaled to it.
@@ -165,13 +171,13 @@ __global__ __launch_bounds__(64 * AD_WAVES) void attention_decode_kernel(
       m_new = fmaxf(m_new, s[u]);
     }
     if (m_new != -INFINITY) {
-      const float correction = (m == -INFINITY) ? 0.f : exp2_fast(m - m_new);
+      const float correction = (m == -INFINITY) ? 0.f : exp2_fast<T>(m - m_new);
       l *= correction;
 #pragma unroll
       for (int i = 0; i < 8; ++i) acc[i] *= correction;
 #pragma unroll
       for (int u = 0; u < AD_UNROLL; ++u) {
-        const float p = valid[u] ? exp2_fast(s[u] - m_new) : 0.f;
+        const float p = valid[u] ? exp2_fast<T>(s[u] - m_new) : 0.f;
         l += p;
         float vf[8];
         vr[u].widen(vf);
@@ -191,7 +197,7 @@ __global__ __launch_bounds__(64 * AD_WAVES) void attention_decode_kernel(
   // the sums run over the lanes that hold the same head dimensions
   {
     const float wave_m = groups_max<LPK>(m);
-    const float c = (m == -INFINITY) ? 0.f : exp2_fast(m - wave_m);
+    const float c = (m == -INFINITY) ? 0.f : exp2_fast<T>(m - wave_m);
     l = groups_sum<LPK>(l * c);
 #pragma unroll
     for (int i = 0; i < 8; ++i) acc[i] = groups_sum<LPK>(acc[i] * c);
@@ -216,7 +222,7 @@ __global__ __launch_bounds__(64 * AD_WAVES) void attention_decode_kernel(
   float block_l = 0.f, value = 0.f;
 #pragma unroll
   for (int w = 0; w < AD_WAVES; ++w) {
-    const float c = (s_ml[w][0] == -INFINITY) ? 0.f : exp2_fast(s_ml[w][0] - block_m);
+    const float c = (s_ml[w][0] == -INFINITY) ? 0.f : exp2_fast<T>(s_ml[w][0] - block_m);
     block_l += s_ml[w][1] * c;
     if (d < head_dim) value += s_acc[w][d] * c;
   }
@@ -248,12 +254,19 @@ __global__ __launch_bounds__(64) void attention_reduce_kernel(
   const float m_s = lane < splits ? src[lane * stride + head_dim] : -INFINITY;
   const float l_s = lane < splits ? src[lane * stride + head_dim + 1] : 0.f;
   const float total_m = wave_max(m_s);
-  const float weight = (m_s == -INFINITY) ? 0.f : exp2_fast(m_s - total_m);
+  const float weight = (m_s == -INFINITY) ? 0.f : exp2_fast<T>(m_s - total_m);
   const float total_l = wave_sum(l_s * weight);
-  for (int d = lane; d < head_dim; d += 64) {
+  // Every lane takes part in every round, also where head_dim leaves it no dimension: the
+  // weights travel by shuffles, and a shuffle only reads lanes that execute it.
+  for (int d0 = 0; d0 < head_dim; d0 += 64) {
+    const int d = d0 + lane;
+    const bool mine = d < head_dim;
+    const int safe_d = mine ? d : 0;
     float value = 0.f;
-    for (int s = 0; s < splits; ++s) value = fmaf(src[s * stride + d], __shfl(weight, s, 64), value);
-    out[(int64_t)t * out_stride + (int64_t)head * head_dim + d] = from_float<T>(value / total_l);
+    for (int s = 0; s < splits; ++s)
+      value = fmaf(src[s * stride + safe_d], __shfl(weight, s, 64), value);
+    if (mine)
+      out[(int64_t)t * out_stride + (int64_t)head * head_dim + d] = from_float<T>(value / total_l);
   }
 }
 
@@ -310,8 +323,10 @@ static int check_decode_sizes(const char* who, int count, int heads, int kv_head
              "%s: bad sizes", who);
   PS_REQUIRE(heads % kv_heads == 0, "%s: heads (%d) must be a multiple of kv_heads (%d)", who,
              heads, kv_heads);
-  PS_REQUIRE(head_dim > 0 && head_dim % 16 == 0 && head_dim <= 256,
-             "%s: head_dim %d must be a multiple of 16 up to 256", who, head_dim);
+  // a lane fetches eight consecutive head dimensions of a key in one piece
+  PS_REQUIRE(head_dim > 0 && head_dim % 8 == 0 && head_dim <= 256,
+             "%s: head_dim %d must be a multiple of 8 up to 256 (ps_attention_rowwise takes "
+             "every head size)", who, head_dim);
   PS_REQUIRE(window >= 0, "%s: negative window", who);
   PS_REQUIRE(splits >= 1 && splits <= 64 && heads <= 65535,
              "%s: splits %d / heads %d out of range", who, splits, heads);

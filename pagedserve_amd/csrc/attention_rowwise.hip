@@ -106,9 +106,8 @@ extern "C" int ps_attention_rowwise(const void* q, int64_t q_stride, const void*
              "ps_attention_rowwise: bad sizes");
   PS_REQUIRE(heads % kv_heads == 0, "ps_attention_rowwise: heads (%d) must be a multiple of kv_heads (%d)",
              heads, kv_heads);
-  PS_REQUIRE(head_dim > 0 && head_dim % 16 == 0 && head_dim <= 64 * AR_MAX_DIMS,
-             "ps_attention_rowwise: head_dim %d must be a multiple of 16 up to %d", head_dim,
-             64 * AR_MAX_DIMS);
+  PS_REQUIRE(head_dim > 0 && head_dim <= 64 * AR_MAX_DIMS,
+             "ps_attention_rowwise: head_dim %d must lie in 1..%d", head_dim, 64 * AR_MAX_DIMS);
   PS_REQUIRE(window >= 0, "ps_attention_rowwise: negative window");
   PS_REQUIRE(heads <= 65535, "ps_attention_rowwise: too many heads");
   PS_REQUIRE(dtype == PS_F32 || dtype == PS_BF16, "ps_attention_rowwise: unknown dtype %d", dtype);

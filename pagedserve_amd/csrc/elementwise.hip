@@ -37,14 +37,15 @@ extern "C" int ps_device_info(int* compute_units, int* lds_bytes, char* arch, in
 }
 
 // ---------------------------------------------------------------- embedding
-// h0[t] = wte[id[t]] + wpe[pos[t]]  (reference: src/model/paged_decoder.py:306-314).
+// h0[t] = scale * wte[id[t]] + wpe[pos[t]]  (reference: src/model/paged_decoder.py:306-314,
+// where the scale is 1).
 // The id of token t is ids[t], or carried[src[t]] where src[t] >= 0: a token that an earlier
 // step chose on the device and that the host has not seen yet.
 template <typename T>
 __global__ void embed_kernel(const T* __restrict__ table, const T* __restrict__ pos_table,
                              const int* __restrict__ ids, const int* __restrict__ src,
                              const int* __restrict__ carried, const int* __restrict__ positions,
-                             float* __restrict__ out, int width, int vocab) {
+                             float* __restrict__ out, int width, int vocab, float scale) {
   const int t = blockIdx.x;
   int id = ids[t];
   if (src != nullptr) {
@@ -57,15 +58,16 @@ __global__ void embed_kernel(const T* __restrict__ table, const T* __restrict__ 
   if (pos_table != nullptr) {
     const T* prow = pos_table + (int64_t)positions[t] * width;
     for (int i = threadIdx.x; i < width; i += blockDim.x)
-      dst[i] = to_float<T>(row[i]) + to_float<T>(prow[i]);
+      dst[i] = to_float<T>(row[i]) * scale + to_float<T>(prow[i]);
   } else {
-    for (int i = threadIdx.x; i < width; i += blockDim.x) dst[i] = to_float<T>(row[i]);
+    for (int i = threadIdx.x; i < width; i += blockDim.x) dst[i] = to_float<T>(row[i]) * scale;
   }
 }
 
 extern "C" int ps_embed(const void* table, const void* pos_table, const int* ids, const int* src,
                         const int* carried, const int* positions, float* out, int tokens,
-                        int width, int vocab, int max_positions, int dtype, void* stream) {
+                        int width, int vocab, int max_positions, float scale, int dtype,
+                        void* stream) {
   PS_REQUIRE(tokens >= 0 && width > 0 && vocab > 0, "ps_embed: bad sizes (tokens %d, width %d)",
              tokens, width);
   PS_REQUIRE(dtype == PS_F32 || dtype == PS_BF16, "ps_embed: unknown dtype %d", dtype);
@@ -76,11 +78,12 @@ extern "C" int ps_embed(const void* table, const void* pos_table, const int* ids
   hipStream_t s = (hipStream_t)stream;
   if (dtype == PS_F32)
     hipLaunchKernelGGL(embed_kernel<float>, dim3(tokens), dim3(threads), 0, s, (const float*)table,
-                       (const float*)pos_table, ids, src, carried, positions, out, width, vocab);
+                       (const float*)pos_table, ids, src, carried, positions, out, width, vocab,
+                       scale);
   else
     hipLaunchKernelGGL(embed_kernel<bf16_t>, dim3(tokens), dim3(threads), 0, s,
                        (const bf16_t*)table, (const bf16_t*)pos_table, ids, src, carried,
-                       positions, out, width, vocab);
+                       positions, out, width, vocab, scale);
   PS_CHECK_LAUNCH("ps_embed");
   return 0;
 }

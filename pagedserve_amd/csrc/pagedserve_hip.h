@@ -20,11 +20,11 @@ extern "C" {
 const char* ps_last_error(void);
 int ps_device_info(int* compute_units, int* lds_bytes, char* arch, int arch_len);
 
-// out[t, :] = table[id(t), :] + (pos_table ? pos_table[positions[t], :] : 0), in float, where
-// id(t) = ids[t], or carried[src[t]] if src is given and src[t] >= 0.
+// out[t, :] = scale * table[id(t), :] + (pos_table ? pos_table[positions[t], :] : 0), in float,
+// where id(t) = ids[t], or carried[src[t]] if src is given and src[t] >= 0.
 int ps_embed(const void* table, const void* pos_table, const int* ids, const int* src,
              const int* carried, const int* positions, float* out, int tokens, int width,
-             int vocab, int max_positions, int dtype, void* stream);
+             int vocab, int max_positions, float scale, int dtype, void* stream);
 
 // out[r, :] = norm(x[rows ? rows[r] : r, :]) * gamma (+ beta).  rms != 0: no mean, no beta.
 int ps_norm(const float* x, const int* rows, const float* gamma, const float* beta, void* out,
@@ -98,8 +98,7 @@ int ps_kv_write(const void* k, const void* v, int64_t stride, void* k_pool, void
 
 // Attention of `tokens` tokens of the step (those listed in tok_list, or all when it is
 // null) over their requests' cached keys 0..position (or the last `window` of them), one
-// wave per (token, head).  Any head_dim that is a multiple of 16 up to 256; heads must be a
-// multiple of kv_heads.
+// wave per (token, head).  Any head_dim from 1 to 256; heads must be a multiple of kv_heads.
 int ps_attention_rowwise(const void* q, int64_t q_stride, const void* k_pool, const void* v_pool,
                          void* out, int64_t out_stride, const int* tok_list, const int* tok_item,
                          const int* tok_pos, const int* tables, int table_width, int tokens,
@@ -108,7 +107,8 @@ int ps_attention_rowwise(const void* q, int64_t q_stride, const void* k_pool, co
 
 // The same result for single queries, with each token's keys cut into `splits` ranges that
 // run as separate blocks of `waves` (4 or 16) waves; `partial` is scratch of
-// count * heads * splits * (head_dim + 2) floats (unused when splits == 1).
+// count * heads * splits * (head_dim + 2) floats (unused when splits == 1).  head_dim is a
+// multiple of 8 up to 256.
 int ps_attention_decode(const void* q, int64_t q_stride, const void* k_pool, const void* v_pool,
                         void* out, int64_t out_stride, float* partial, int64_t partial_floats,
                         const int* tok_list, const int* tok_item, const int* tok_pos,

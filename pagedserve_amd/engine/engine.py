@@ -91,6 +91,9 @@ class Engine:
         self.views = model.cache_views(self.cache)
         self.workspace = Workspace(max_step_tokens, self.device)
         self.table_width = -(-self.spec.max_positions // page_size)
+        # queries of an item with several tokens are listed in tiles of the size that the
+        # model's mixers ask for (None: no mixer wants tiles)
+        self.query_tile = getattr(model, "query_tile", None)
         capacity = (9 * max_step_tokens + 5 * max_requests + 1
                     + len(groups) * max_requests * self.table_width + 16)
         self._meta_device = torch.empty(capacity, dtype=torch.int32, device=self.device)
@@ -100,8 +103,10 @@ class Engine:
         self._meta_owner = [None, None]   # replay plan whose constant arrays a buffer holds
         self._meta_turn = 0
         self._logits = None
-        self._tokens = torch.zeros(max(max_requests, 64), dtype=torch.int32, device=self.device)
-        self._tokens_host = [torch.zeros(max(max_requests, 64), dtype=torch.int32, pin_memory=True)
+        # chosen tokens: one per wanted row, and a step wants at most one row per token
+        self._tokens = torch.zeros(max(max_requests, max_step_tokens), dtype=torch.int32,
+                                   device=self.device)
+        self._tokens_host = [torch.zeros(self._tokens.numel(), dtype=torch.int32, pin_memory=True)
                              for _ in range(2)]
         self._tokens_ready = [torch.cuda.Event(), torch.cuda.Event()]
         self._tokens_turn = 0
@@ -112,9 +117,15 @@ class Engine:
         # a part that looks at host values of a step cannot be replayed
         self.use_graphs = use_graphs and getattr(model, "graph_safe", False)
         self.max_graphs = 48     # recorded layouts kept; the least recently made goes first
+        self.max_layouts_remembered = 512
         self._graphs = {}        # key -> StepGraph
         self._graph_seen = {}     # layout -> steps that ran without a graph (buffers exist now)
         self._graph_failures = {}
+        self._graph_retired = []  # (event, graph): dropped, destroyed once the event has happened
+        self.graphs_captured = 0
+        self.graphs_evicted = 0
+        self._replays_of_dropped = 0
+        self.capture_seconds = 0.0
         self.steps = 0
 
     # ------------------------------------------------------------------ admin
@@ -131,7 +142,11 @@ class Engine:
     def graph_summary(self) -> dict:
         """Counters in the manner of src/model/paged_decoder.py:498-507."""
         return {"enabled": self.use_graphs, "captured_graphs": len(self._graphs),
-                "graph_replays": sum(plan.graph.replays for plan in self._graphs.values()),
+                "captures": self.graphs_captured, "evicted": self.graphs_evicted,
+                "capture_seconds": round(self.capture_seconds, 4),
+                "layouts_remembered": len(self._graph_seen),
+                "graph_replays": self._replays_of_dropped
+                + sum(plan.graph.replays for plan in self._graphs.values()),
                 "graph_nodes": {str(key): plan.graph.nodes for key, plan in self._graphs.items()},
                 "capture_failures": list(self._graph_failures.values())}
 
@@ -177,6 +192,9 @@ class Engine:
             if entry.want and (min(entry.want) < 0 or max(entry.want) >= count):
                 raise StepError(f"request {entry.request_id!r} wants logits at place "
                                 f"{max(entry.want)} of {count} tokens")
+            if len(set(entry.want)) != len(entry.want):
+                # (the index buffers hold one wanted row per token at most)
+                raise StepError(f"request {entry.request_id!r} wants logits at the same place twice")
             record = self.cache.requests.get(entry.request_id)
             have = record.length if record is not None else 0
             new += record is None
@@ -246,8 +264,9 @@ class Engine:
         wants = [len(entry.want) for entry in entries]
         wanted = sum(wants)
         singles = counts.count(1)
-        # items with several tokens are cut into tiles of 64 queries for the tiled kernel
-        tiles = sum(-(-count // 64) for count in counts if count > 1)
+        # items with several tokens are cut into tiles of queries for the mixers' tiled kernels
+        tile = self.query_tile
+        tiles = sum(-(-count // tile) for count in counts if count > 1) if tile else 0
         groups = len(cache.groups)
         width = self.table_width
         offsets = {}
@@ -325,7 +344,7 @@ class Engine:
                     portion_tokens[portion_cursor:portion_cursor + count] = np.arange(
                         flat, flat + count, dtype=np.int32)
                     portion_cursor += count
-                    for q0 in range(0, count, 64):
+                    for q0 in range(0, count, tile) if tile else ():
                         tile_item[tile_cursor] = index
                         tile_q0[tile_cursor] = q0
                         tile_cursor += 1
@@ -439,11 +458,18 @@ class Engine:
         seen_key = graph_key + (logits.data_ptr(),)
         seen = self._graph_seen.get(seen_key, 0)
         if seen < (1 if singles == ctx.tokens else 3):
+            # (re-inserted at the end: the layouts that have not come back for longest go first)
+            self._graph_seen.pop(seen_key, None)
             self._graph_seen[seen_key] = seen + 1
+            while len(self._graph_seen) > self.max_layouts_remembered:
+                del self._graph_seen[next(iter(self._graph_seen))]
             out, tokens = self._forward(ctx, rows, logits, wanted, greedy)
             return StepOutput(logits=out, rows=row_keys, tokens=tokens)
+        import time
+
         from ..ops.kernels import StepGraph
 
+        capture_started = time.perf_counter()
         graph = StepGraph()
         StepGraph.begin()
         try:
@@ -465,13 +491,32 @@ class Engine:
             sections.append(views)
         old = self._graphs.pop(graph_key, None)
         if old is not None:
-            old.graph.destroy()
+            self._retire_graph(old)
         while len(self._graphs) >= self.max_graphs:
             oldest = next(iter(self._graphs))
-            self._graphs.pop(oldest).graph.destroy()
+            self._retire_graph(self._graphs.pop(oldest))
+            self.graphs_evicted += 1
         self._graphs[graph_key] = _ReplayPlan(graph, used, sections, out, tokens, items)
+        self.graphs_captured += 1
+        self.capture_seconds += time.perf_counter() - capture_started
         graph.launch()
         return StepOutput(logits=out, rows=row_keys, tokens=tokens)
+
+    def _retire_graph(self, plan):
+        """A recorded layout is dropped.  Its last launch may still be running (the engine never
+        waits for its stream), so the executable graph is destroyed only after an event
+        recorded behind everything launched so far has happened."""
+        event = torch.cuda.Event()
+        event.record(self.stream)
+        self._graph_retired.append((event, plan.graph))
+        self._replays_of_dropped += plan.graph.replays
+        still_busy = []
+        for event, graph in self._graph_retired:
+            if event.query():
+                graph.destroy()
+            else:
+                still_busy.append((event, graph))
+        self._graph_retired = still_busy
 
     def _replay(self, plan, entries, select=None) -> StepOutput:
         """A captured decode step: refresh the per-step indices, copy them, launch the graph."""

@@ -96,8 +96,10 @@ def build_scheduler(model=REFERENCE_MODEL, scheduling_strategy=ORCA_STRATEGY, pr
     engine.memory_budget_source = source
     from ..sampling.sampler import Sampler
 
+    # "config": what config.json says (null there means that no token ends a request); an
+    # explicit value, None included, overrides it.  The scheduler never asks the tokenizer.
     eos = config.eos_token_id if eos_token_id == "config" else eos_token_id
-    tokenizer = load_tokenizer(folder if scratch is None else None, config.vocab_size, eos)
+    tokenizer = load_tokenizer(None if model == REFERENCE_MODEL else model, config.vocab_size, eos)
     scheduler = ContinuousBatchScheduler(
         engine, Sampler(device, max_batch_size), tokenizer=tokenizer,
         max_batch_size=max_batch_size, eos_token_id=eos,

@@ -1,12 +1,12 @@
 """Continuous batching above the step function.
 
-Queues and life cycle follow the reference's ``ContinuousBatchScheduler``
-(src/scheduler/orca_scheduler.py:32-303): requests wait until their whole prompt is
-cached, then decode one token per iteration until ``max_new_tokens`` or the end token,
-then give back what they hold.  Two selection strategies:
+What a request goes through is what the reference's ``ContinuousBatchScheduler`` puts it
+through (src/scheduler/orca_scheduler.py:32-303): it waits until its whole prompt is cached,
+then decodes one token per iteration until ``max_new_tokens`` or the end token, then gives
+back what it holds.  Two ways of choosing an iteration's work:
 
-* ``orca``: requests in arrival order, decoding ones with their single token and
-  waiting ones with their whole remaining prompt (``:128-146,187-188``);
+* ``orca``: requests in arrival order, decoding ones with their single token and waiting
+  ones with their whole remaining prompt (``:128-146,187-188``);
 * ``sarathi``: all decoding requests first, then prompt portions of at most
   ``prefill_chunk_size`` tokens (``:148-169,182-186``), one prefilling request per
   iteration as in the reference unless ``max_prefill_requests`` allows more.
@@ -23,6 +23,11 @@ requests have reserved (``:119-122,138-142``); otherwise it and everything behin
 nothing is preempted.  A request whose worst case exceeds the whole pool is refused when
 it is added.
 
+**More decoding requests than an iteration holds.**  The engine may have more request slots
+than ``max_batch_size``.  The decoding requests of an iteration are then those that were
+served least recently, so that every one advances at the same rate; the reference always
+takes the lowest ids (``:165-166``), and the others starve until those finish.
+
 **Running ahead.**  While every running request decodes and nobody waits, the
 iteration after the current one is launched before the current one's tokens have reached
 the host: its entries say "the token that the last step chose for row r" instead of a token
@@ -32,16 +37,19 @@ token too many computed, which is dropped.  The tokens that a request receives a
 either way.
 """
 
-from collections import deque
 from dataclasses import dataclass, field
 from typing import Dict, List, Optional
 
-from ..sampling.params import SamplingParams, fresh_seed
+from ..sampling.params import SamplingParams, fresh_seed, uniform_for
 from .engine import StepEntry
 
 ORCA_STRATEGY = "orca"
 SARATHI_STRATEGY = "sarathi"
 SUPPORTED_SCHEDULING_STRATEGIES = (ORCA_STRATEGY, SARATHI_STRATEGY)
+
+# ``eos_token_id`` of the constructor when the caller leaves the choice to the tokenizer; ``None``
+# means that no token ends a request.
+FROM_TOKENIZER = "tokenizer"
 
 
 @dataclass
@@ -53,71 +61,180 @@ class RequestState:
     sampling: SamplingParams
     seed: int
     generated_token_ids: List[int] = field(default_factory=list)
-    pending_token_id: Optional[int] = None
+    pending_token_id: Optional[int] = None      # the token that the next decode step brings
     reserved_blocks: List[int] = field(default_factory=list)   # per cache group; [] = not admitted
-    prefill_cursor: int = 0
+    prefill_cursor: int = 0                     # prompt tokens that are cached
     finish_reason: Optional[str] = None
+    last_served: int = -1                       # ticket of its last turn; tickets grow with time
 
     @property
     def is_prefilling(self) -> bool:
         return self.pending_token_id is None
 
+    @property
+    def prompt_left(self) -> int:
+        return len(self.prompt_token_ids) - self.prefill_cursor
+
+
+class _PageLedger:
+    """Pages promised to admitted requests, per cache group.  A promise covers the request's
+    worst case, so the sum never exceeds a pool and a running request never lacks a page."""
+
+    def __init__(self, cache, longest_step):
+        self.cache = cache
+        self.longest_step = longest_step
+        self.promised = [0] * len(cache.groups)
+
+    def worst_case(self, request) -> List[int]:
+        """Most pages per group that the request ever holds
+        (src/scheduler/orca_scheduler.py:119-122)."""
+        total = len(request.prompt_token_ids) + request.max_new_tokens
+        return [self.cache.pages_for_length(group, total, self.longest_step)
+                for group in range(len(self.cache.groups))]
+
+    def ever_fits(self, request) -> Optional[str]:
+        """None, or why no pool could ever hold the request."""
+        for group, (pages, pool) in enumerate(zip(self.worst_case(request), self.cache.pools)):
+            if pages > pool.num_pages:
+                return (f"the request needs {pages} pages of cache group {group}, the pool has "
+                        f"{pool.num_pages}: it could never be scheduled")
+        return None
+
+    def has_room(self, request, beside) -> bool:
+        """Whether the request's worst case fits beside all promises and ``beside`` (pages that
+        the iteration being planned is about to promise)."""
+        return all(promised + extra + need <= pool.num_pages
+                   for promised, extra, need, pool in zip(self.promised, beside,
+                                                          self.worst_case(request), self.cache.pools))
+
+    def promise(self, request):
+        request.reserved_blocks = self.worst_case(request)
+        for group, pages in enumerate(request.reserved_blocks):
+            self.promised[group] += pages
+
+    def withdraw(self, request):
+        for group, pages in enumerate(request.reserved_blocks):
+            self.promised[group] -= pages
+        request.reserved_blocks = []
+
+
+class _Plan:
+    """The work of one iteration while it is being chosen: (request, tokens) pairs under the
+    limits on requests, tokens and prompts, and the pages that newcomers among them need."""
+
+    def __init__(self, scheduler):
+        self.scheduler = scheduler
+        self.chosen = []                          # (request, tokens it brings)
+        self.tokens_left = scheduler.max_num_batched_tokens
+        self.prompts = 0
+        self.newcomers = 0
+        self.newcomer_pages = [0] * len(scheduler.ledger.promised)
+
+    @property
+    def full(self) -> bool:
+        return len(self.chosen) >= self.scheduler.max_batch_size or self.tokens_left == 0
+
+    def add_decode(self, request):
+        self.chosen.append((request, 1))
+        self.tokens_left -= 1
+
+    def admits(self, request) -> bool:
+        """Whether a request that holds no promise yet could get one in this iteration."""
+        scheduler = self.scheduler
+        if scheduler.admitted_requests() + self.newcomers >= scheduler.engine.max_requests:
+            return False
+        return scheduler.ledger.has_room(request, self.newcomer_pages)
+
+    def add_prompt(self, request, longest) -> bool:
+        """A portion of the request's prompt; False when the request has to wait for pages
+        or a slot (and with it everything behind it: first come, first served)."""
+        if not request.reserved_blocks:
+            if not self.admits(request):
+                return False
+            for group, pages in enumerate(self.scheduler.ledger.worst_case(request)):
+                self.newcomer_pages[group] += pages
+            self.newcomers += 1
+        size = min(request.prompt_left, self.tokens_left, longest)
+        self.chosen.append((request, size))
+        self.tokens_left -= size
+        self.prompts += 1
+        return True
+
 
 @dataclass
-class _Pending:
+class _Flight:
     """An iteration that runs on the GPU and whose tokens the host has not read yet."""
 
-    selected: list            # (request, number of tokens)
-    entries: list
-    producers: list           # requests that receive a token from it, in row order
+    chosen: list              # (request, number of tokens)
+    receivers: list           # requests that get a token from it, in the order of the logits rows
     output: object
-    can_carry: bool           # single-token rows chosen on the device: the next iteration may carry them on
+    can_carry: bool           # every row is a decoded token chosen on the device
 
 
 class ContinuousBatchScheduler:
     def __init__(self, engine, sampler, tokenizer=None, max_batch_size: int = 32,
-                 eos_token_id=None, scheduling_strategy: str = ORCA_STRATEGY,
+                 eos_token_id=FROM_TOKENIZER, scheduling_strategy: str = ORCA_STRATEGY,
                  prefill_chunk_size: int = 16, max_num_batched_tokens: Optional[int] = None,
                  max_prefill_requests: Optional[int] = None, run_ahead: bool = True):
-        if max_batch_size <= 0:
-            raise ValueError("max_batch_size must be positive")
         if scheduling_strategy not in SUPPORTED_SCHEDULING_STRATEGIES:
-            choices = ", ".join(SUPPORTED_SCHEDULING_STRATEGIES)
-            raise ValueError(f"Unknown scheduling strategy '{scheduling_strategy}'. "
-                             f"Choose one of: {choices}")
-        if prefill_chunk_size <= 0:
-            raise ValueError("prefill_chunk_size must be positive")
+            raise ValueError(f"Unknown scheduling strategy '{scheduling_strategy}'. Choose one of: "
+                             + ", ".join(SUPPORTED_SCHEDULING_STRATEGIES))
+        for name, value in (("max_batch_size", max_batch_size), ("prefill_chunk_size", prefill_chunk_size)):
+            if value <= 0:
+                raise ValueError(f"{name} must be positive")
         if max_batch_size > engine.max_requests:
             raise ValueError(f"max_batch_size {max_batch_size} exceeds the engine's "
                              f"{engine.max_requests} request slots")
         budget = engine.max_step_tokens if max_num_batched_tokens is None else max_num_batched_tokens
-        if budget <= 0:
-            raise ValueError("max_num_batched_tokens must be positive")
-        if budget > engine.max_step_tokens:
-            raise ValueError(f"max_num_batched_tokens {budget} exceeds the engine's "
-                             f"max_step_tokens {engine.max_step_tokens}")
+        if not 0 < budget <= engine.max_step_tokens:
+            raise ValueError(f"max_num_batched_tokens must lie in 1..{engine.max_step_tokens} "
+                             f"(the engine's max_step_tokens), got {budget}")
         self.engine = engine
         self.sampler = sampler
         self.tokenizer = tokenizer
         self.max_batch_size = max_batch_size
-        self.eos_token_id = (eos_token_id if eos_token_id is not None
-                             else getattr(tokenizer, "eos_token_id", None))
+        # "tokenizer": the tokenizer's end token, if it has one; None: nothing ends a request
+        if eos_token_id == FROM_TOKENIZER:
+            eos_token_id = getattr(tokenizer, "eos_token_id", None)
+        self.eos_token_id = eos_token_id
         self.scheduling_strategy = scheduling_strategy
         self.prefill_chunk_size = prefill_chunk_size
         self.max_num_batched_tokens = budget
         if max_prefill_requests is None:
             max_prefill_requests = 1 if scheduling_strategy == SARATHI_STRATEGY else max_batch_size
         self.max_prefill_requests = max_prefill_requests
-
-        self.waiting = deque()                       # prompt tokens still to cache
-        self.active: Dict[int, RequestState] = {}    # decoding
-        self.finished: Dict[int, RequestState] = {}  # done, nothing held
-        self.next_request_id = 0
-        self.reserved_blocks = [0] * len(engine.cache.groups)
-        self.iterations = 0
         self.run_ahead = run_ahead
+
+        # Every request that is not finished, in arrival order (ids grow with arrival).
+        self._live: Dict[int, RequestState] = {}
+        self.finished: Dict[int, RequestState] = {}
+        self.ledger = _PageLedger(engine.cache, budget)
+        self.next_request_id = 0
+        self.iterations = 0
+        self._tickets = 0
         self.steps_run_ahead = 0
-        self._inflight = None       # a launched iteration whose tokens the host has not read
+        self._inflight: Optional[_Flight] = None
+
+    # ----------------------------------------------------------------- views
+    @property
+    def waiting(self) -> List[RequestState]:
+        """Requests whose prompt is not wholly cached yet, in arrival order."""
+        return [request for request in self._live.values() if request.is_prefilling]
+
+    @property
+    def active(self) -> Dict[int, RequestState]:
+        """Decoding requests by id."""
+        return {rid: request for rid, request in self._live.items() if not request.is_prefilling}
+
+    @property
+    def reserved_blocks(self) -> List[int]:
+        return list(self.ledger.promised)
+
+    def admitted_requests(self) -> int:
+        return sum(1 for request in self._live.values() if request.reserved_blocks)
+
+    def _required_blocks(self, request) -> List[int]:
+        return self.ledger.worst_case(request)
 
     # ------------------------------------------------------------- admission
     def add_request(self, prompt, max_new_tokens=200, sampling: Optional[SamplingParams] = None):
@@ -131,284 +248,238 @@ class ContinuousBatchScheduler:
 
     def add_token_request(self, prompt_token_ids, max_new_tokens=200,
                           prompt="<tokenized prompt>", sampling: Optional[SamplingParams] = None):
-        """Add an already tokenized request (src/scheduler/orca_scheduler.py:85-116)."""
-        if max_new_tokens <= 0:
-            raise ValueError("max_new_tokens must be positive")
+        """Queue an already tokenized request; the checks of
+        src/scheduler/orca_scheduler.py:85-116, and one more: a request that no pool could
+        ever hold is refused here instead of waiting for ever."""
         if hasattr(prompt_token_ids, "tolist"):
             prompt_token_ids = prompt_token_ids.reshape(-1).tolist()
-        prompt_token_ids = list(prompt_token_ids)
-        if not prompt_token_ids:
-            raise ValueError("The tokenizer produced an empty prompt")
-        if any(isinstance(token, bool) or not isinstance(token, int) for token in prompt_token_ids):
-            raise ValueError("The tokenizer must produce integer token IDs")
-        if min(prompt_token_ids) < 0 or max(prompt_token_ids) >= self.engine.spec.vocab_size:
-            raise ValueError("A prompt token is outside the model vocabulary")
-        if len(prompt_token_ids) + max_new_tokens > self.engine.spec.max_positions:
-            raise ValueError("Prompt plus requested generation exceeds the model context limit")
-        sampling = sampling or SamplingParams(max_new_tokens=max_new_tokens)
+        tokens = list(prompt_token_ids)
+        spec = self.engine.spec
+        problem = None
+        if max_new_tokens <= 0:
+            problem = "max_new_tokens must be positive"
+        elif not tokens:
+            problem = "The tokenizer produced an empty prompt"
+        elif not all(type(token) is int for token in tokens):
+            problem = "The tokenizer must produce integer token IDs"
+        elif not all(0 <= token < spec.vocab_size for token in tokens):
+            problem = "A prompt token is outside the model vocabulary"
+        elif len(tokens) + max_new_tokens > spec.max_positions:
+            problem = "Prompt plus requested generation exceeds the model context limit"
+        if problem:
+            raise ValueError(problem)
+        if sampling is None:
+            sampling = SamplingParams(max_new_tokens=max_new_tokens)
         request = RequestState(
             request_id=self.next_request_id, prompt=prompt, max_new_tokens=max_new_tokens,
-            prompt_token_ids=prompt_token_ids, sampling=sampling,
-            seed=sampling.seed if sampling.seed is not None else fresh_seed())
-        need = self._required_blocks(request)
-        for group, (pages, pool) in enumerate(zip(need, self.engine.cache.pools)):
-            if pages > pool.num_pages:
-                raise ValueError(
-                    f"the request needs {pages} pages of cache group {group}, the pool has "
-                    f"{pool.num_pages}: it could never be scheduled")
+            prompt_token_ids=tokens, sampling=sampling,
+            seed=fresh_seed() if sampling.seed is None else sampling.seed)
+        problem = self.ledger.ever_fits(request)
+        if problem:
+            raise ValueError(problem)
         self.next_request_id += 1
-        self.waiting.append(request)
+        self._live[request.request_id] = request
         return request.request_id
 
-    def _required_blocks(self, request) -> List[int]:
-        """Worst-case pages per cache group (src/scheduler/orca_scheduler.py:119-122)."""
-        total = len(request.prompt_token_ids) + request.max_new_tokens
-        cache = self.engine.cache
-        return [cache.pages_for_length(group, total, self.max_num_batched_tokens)
-                for group in range(len(cache.groups))]
-
-    def _fits(self, request, newly_reserved, newly_admitted=0) -> bool:
-        """Worst-case pages fit beside all reservations, and a request slot is free."""
-        admitted = sum(1 for r in self.waiting if r.reserved_blocks) + len(self.active)
-        if admitted + newly_admitted >= self.engine.max_requests:
-            return False
-        need = self._required_blocks(request)
-        return all(self.reserved_blocks[g] + newly_reserved[g] + need[g] <= pool.num_pages
-                   for g, pool in enumerate(self.engine.cache.pools))
-
     # ------------------------------------------------------------- selection
+    def _decoding_in_turn(self, room: int) -> List[RequestState]:
+        """At most ``room`` decoding requests, in arrival order.  When there are more, those
+        that were served least recently are taken, so that all of them advance."""
+        decoding = [request for request in self._live.values() if not request.is_prefilling]
+        if len(decoding) > room:
+            decoding.sort(key=lambda request: (request.last_served, request.request_id))
+            decoding = sorted(decoding[:max(room, 0)], key=lambda request: request.request_id)
+        return decoding
+
     def select_requests(self):
         """[(request, tokens it brings)] for the next iteration."""
+        plan = _Plan(self)
         if self.scheduling_strategy == SARATHI_STRATEGY:
-            decoding = sorted(self.active.values(), key=lambda r: r.request_id)
-            prefilling = list(self.waiting)
-        else:
-            pool = sorted(list(self.active.values()) + list(self.waiting),
-                          key=lambda r: r.request_id)
-            decoding, prefilling = None, None
-        selected = []
-        budget = self.max_num_batched_tokens
-        newly = [0] * len(self.reserved_blocks)
-        admitted_now = 0
-        prefills = 0
-
-        def take_prefill(request) -> bool:
-            """False: this request and all behind it must wait (first come, first served)."""
-            nonlocal budget, prefills, admitted_now
-            if not request.reserved_blocks:
-                if not self._fits(request, newly, admitted_now):
-                    return False
-                for g, pages in enumerate(self._required_blocks(request)):
-                    newly[g] += pages
-                admitted_now += 1
-            remaining = len(request.prompt_token_ids) - request.prefill_cursor
-            size = min(remaining, budget)
-            if self.scheduling_strategy == SARATHI_STRATEGY:
-                size = min(size, self.prefill_chunk_size)
-            selected.append((request, size))
-            budget -= size
-            prefills += 1
-            return True
-
-        if self.scheduling_strategy == SARATHI_STRATEGY:
-            # room is kept for one prompt portion when a prompt is waiting
+            prompts = self.waiting
+            # room is kept for one prompt portion when a prompt can run
             # (src/scheduler/orca_scheduler.py:165)
-            head_fits = bool(prefilling) and (bool(prefilling[0].reserved_blocks)
-                                              or self._fits(prefilling[0], newly))
-            decode_capacity = self.max_batch_size - (1 if head_fits else 0)
-            for request in decoding[:max(decode_capacity, 0)]:
-                if budget == 0:
+            head_can_run = bool(prompts) and (bool(prompts[0].reserved_blocks) or plan.admits(prompts[0]))
+            for request in self._decoding_in_turn(self.max_batch_size - int(head_can_run)):
+                if plan.full:
                     break
-                selected.append((request, 1))
-                budget -= 1
-            for request in prefilling:
-                if (len(selected) >= self.max_batch_size or budget == 0
-                        or prefills >= self.max_prefill_requests):
+                plan.add_decode(request)
+            for request in prompts:
+                if plan.full or plan.prompts >= self.max_prefill_requests:
                     break
-                if not take_prefill(request):
+                if not plan.add_prompt(request, self.prefill_chunk_size):
                     break
         else:
-            for request in pool:
-                if len(selected) >= self.max_batch_size or budget == 0:
+            in_turn = {request.request_id for request in self._decoding_in_turn(self.max_batch_size)}
+            for request in self._live.values():
+                if plan.full:
                     break
-                if request.is_prefilling:
-                    if prefills >= self.max_prefill_requests:
-                        continue
-                    if not take_prefill(request):
+                if not request.is_prefilling:
+                    if request.request_id in in_turn:
+                        plan.add_decode(request)
+                elif plan.prompts < self.max_prefill_requests:
+                    if not plan.add_prompt(request, self.max_num_batched_tokens):
                         break
-                else:
-                    selected.append((request, 1))
-                    budget -= 1
-        return selected
+        return plan.chosen
 
     def build_step_entries(self, selected) -> List[StepEntry]:
         entries = []
         for request, size in selected:
             if request.is_prefilling:
                 start = request.prefill_cursor
-                tokens = request.prompt_token_ids[start:start + size]
-                last = start + size == len(request.prompt_token_ids)
-                # only the final portion of a prompt produces a token
+                # only the portion that ends the prompt produces a token
                 # (src/scheduler/orca_scheduler.py:191)
-                entries.append(StepEntry(request.request_id, tokens, [size - 1] if last else []))
+                want = [size - 1] if size == request.prompt_left else []
+                entries.append(StepEntry(request.request_id,
+                                         request.prompt_token_ids[start:start + size], want))
             else:
                 entries.append(StepEntry(request.request_id, [request.pending_token_id], [0]))
         return entries
 
     # ------------------------------------------------------------------ step
     def step(self) -> Dict[int, int]:
-        """One iteration.  With a real engine the whole iteration (step, token selection and
-        the copy of the tokens) runs on the engine's own stream, which saves the hand-over
-        between streams on every step."""
+        """One iteration: {request id: the token it received}.  With a real engine the whole
+        iteration (step, token selection and the copy of the tokens) runs on the engine's own
+        stream, which saves the hand-over between streams on every step."""
         stream = getattr(self.engine, "stream", None)
         if stream is None:
-            return self._step()
+            return self._iterate()
         import torch
 
         previous = torch.cuda.current_stream(stream.device)
         torch.cuda.set_stream(stream)
         try:
-            return self._step()
+            return self._iterate()
         finally:
             torch.cuda.set_stream(previous)
 
-    def _step(self) -> Dict[int, int]:
-        pending = self._inflight
-        self._inflight = None
-        if pending is None:
-            pending = self._launch()
-            if pending is None:
+    def _iterate(self) -> Dict[int, int]:
+        flight, self._inflight = self._inflight, None
+        if flight is None:
+            flight = self._take_off()
+            if flight is None:
                 return {}
-        self._inflight = self._launch_ahead(pending)
-        return self._resolve(pending)
+        self._inflight = self._take_off_ahead(flight)
+        return self._land(flight)
 
-    def _launch(self) -> Optional["_Pending"]:
-        """Select, reserve, and start one iteration on the GPU."""
-        selected = self.select_requests()
-        if not selected:
-            if self.waiting or self.active:
+    def _choose_on_device(self, receivers, ahead):
+        """How the engine should pick the tokens of ``receivers``: keyword arguments of
+        ``engine.step``.  Greedy rows are picked inside the step (one launch less, and part of
+        a decode step's graph); with temperatures each row gets ``(1 / temperature, uniform
+        number)``, if the engine draws; else the logits go to the sampler."""
+        if not receivers:
+            return {}
+        if all(request.sampling.temperature == 0 for request in receivers):
+            return {"greedy": True}
+        if not getattr(self.engine, "supports_draws", False):
+            return {}
+        # ``ahead`` = 1 when the request's last token is still on its way to the host
+        return {"draws": [(0.0 if r.sampling.temperature == 0 else 1.0 / r.sampling.temperature,
+                           uniform_for(r.seed, r.request_id, len(r.generated_token_ids) + ahead))
+                          for r in receivers]}
+
+    def _take_off(self) -> Optional[_Flight]:
+        """Choose an iteration's work, promise pages to its newcomers, start it on the GPU."""
+        chosen = self.select_requests()
+        if not chosen:
+            if self._live:
                 raise RuntimeError("No request can be scheduled with the available KV memory")
             return None
-        new_requests = [request for request, _ in selected if not request.reserved_blocks]
-        for request in new_requests:
-            request.reserved_blocks = self._required_blocks(request)
-            for g, pages in enumerate(request.reserved_blocks):
-                self.reserved_blocks[g] += pages
-        entries = self.build_step_entries(selected)
-        producers = [request for (request, size), entry in zip(selected, entries) if entry.want]
-        # greedy rows are picked on the GPU inside the step (one launch less, and part of the
-        # captured graph of a decode step)
-        greedy = bool(producers) and all(r.sampling.temperature == 0 for r in producers)
-        draws = None
-        if producers and not greedy and getattr(self.engine, "supports_draws", False):
-            draws = self._draws(producers, 0)
+        newcomers = [request for request, _ in chosen if not request.reserved_blocks]
+        for request in newcomers:
+            self.ledger.promise(request)
+        entries = self.build_step_entries(chosen)
+        receivers = [request for (request, _), entry in zip(chosen, entries) if entry.want]
+        how = self._choose_on_device(receivers, 0)
         try:
-            if draws is not None:
-                output = self.engine.step(entries, draws=draws)
-            else:
-                output = self.engine.step(entries, greedy=greedy)
+            output = self.engine.step(entries, **how)
         except Exception:
-            for request in new_requests:
-                for g, pages in enumerate(request.reserved_blocks):
-                    self.reserved_blocks[g] -= pages
-                request.reserved_blocks = []
+            # nothing ran: the newcomers' promises are withdrawn
+            # (src/scheduler/orca_scheduler.py:243-247)
+            for request in newcomers:
+                self.ledger.withdraw(request)
             raise
-        decode_only = all(not request.is_prefilling for request, _ in selected)
-        return _Pending(selected, entries, producers, output,
-                        (greedy or draws is not None) and decode_only)
+        only_decodes = all(not request.is_prefilling for request, _ in chosen)
+        return _Flight(chosen, receivers, output, bool(how) and only_decodes)
 
-    @staticmethod
-    def _draws(producers, ahead):
-        """(1 / temperature, uniform number) of the next token of each request; ``ahead`` = 1
-        when the request's last token is still on its way to the host."""
-        from ..sampling.params import uniform_for
-
-        return [(0.0 if r.sampling.temperature == 0 else 1.0 / r.sampling.temperature,
-                 uniform_for(r.seed, r.request_id, len(r.generated_token_ids) + ahead))
-                for r in producers]
-
-    def _launch_ahead(self, pending) -> Optional["_Pending"]:
-        """Start the iteration after ``pending`` before ``pending``'s tokens are known, if
-        it is certain which requests it holds: all of ``pending``'s that do not end by
-        length, each carrying on the token that ``pending`` chooses for it."""
-        if (not self.run_ahead or not pending.can_carry or self.waiting
-                or getattr(pending.output, "host_tokens", None) is None
-                or len(self.active) != len(pending.selected)):
+    def _take_off_ahead(self, flight) -> Optional[_Flight]:
+        """Start the iteration after ``flight`` before ``flight``'s tokens are known, if it is
+        certain which requests it holds: all of ``flight``'s that do not end by length, each
+        carrying on the token that ``flight`` chooses for it."""
+        if (not self.run_ahead or not flight.can_carry
+                or getattr(flight.output, "host_tokens", None) is None):
             return None
-        selected, entries = [], []
-        for row, (request, _) in enumerate(pending.selected):
+        if any(request.is_prefilling for request in self._live.values()):
+            return None         # a prompt waits: the next iteration is chosen in the ordinary way
+        if len(self._live) != len(flight.chosen):
+            return None         # a request sat ``flight`` out, or has just ended
+        chosen, entries = [], []
+        for row, (request, _) in enumerate(flight.chosen):
             if request.finish_reason is not None:
-                continue      # ended at the end token while ``pending`` was already running
+                continue        # ended at the end token while ``flight`` was already running
             if len(request.generated_token_ids) + 2 > request.max_new_tokens:
-                continue      # ``pending`` brings its last token
-            selected.append((request, 1))
+                continue        # ``flight`` brings its last token
+            chosen.append((request, 1))
             entries.append(StepEntry(request.request_id, [0], [0], carry=row))
-        if not selected:
+        if not chosen:
             return None
-        producers = [request for request, _ in selected]
+        receivers = [request for request, _ in chosen]
         try:
-            if all(r.sampling.temperature == 0 for r in producers):
-                output = self.engine.step(entries, greedy=True)
-            else:
-                output = self.engine.step(entries, draws=self._draws(producers, 1))
+            output = self.engine.step(entries, **self._choose_on_device(receivers, 1))
         except ValueError:
-            return None       # the ordinary launch of the next iteration reports it
+            return None         # the ordinary start of the next iteration reports it
         self.steps_run_ahead += 1
-        return _Pending(selected, entries, producers, output, True)
+        return _Flight(chosen, receivers, output, True)
 
-    def _resolve(self, pending) -> Dict[int, int]:
-        """Read the tokens of a launched iteration and move its requests on."""
-        selected, entries, producers, output = (pending.selected, pending.entries,
-                                                pending.producers, pending.output)
-        if output.logits.shape[0] != len(producers):
+    def _tokens_of(self, flight) -> List[int]:
+        output = flight.output
+        if output.logits.shape[0] != len(flight.receivers):
             raise RuntimeError("the engine returned a wrong number of logits rows")
-        if getattr(output, "tokens", None) is not None:
-            tokens = output.token_list() if hasattr(output, "token_list") else output.tokens.tolist()
-        else:
-            tokens = self.sampler.sample(
-                output.logits, [r.sampling for r in producers], [r.request_id for r in producers],
-                [len(r.generated_token_ids) for r in producers], [r.seed for r in producers])
+        if getattr(output, "tokens", None) is None:
+            receivers = flight.receivers
+            return self.sampler.sample(
+                output.logits, [r.sampling for r in receivers], [r.request_id for r in receivers],
+                [len(r.generated_token_ids) for r in receivers], [r.seed for r in receivers])
+        return output.token_list() if hasattr(output, "token_list") else output.tokens.tolist()
+
+    def _land(self, flight) -> Dict[int, int]:
+        """Read the tokens of a started iteration and move its requests on."""
+        tokens = dict(zip((id(request) for request in flight.receivers), self._tokens_of(flight)))
         emitted = {}
-        completed_prefill = set()
-        next_token = iter(tokens)
-        for (request, size), entry in zip(selected, entries):
+        served = []
+        for request, size in flight.chosen:
             if request.finish_reason is not None:
-                # ended at the end token after this iteration had been launched ahead: the
-                # token computed for it here is dropped
-                next(next_token)
-                continue
+                continue        # ended after this iteration had been started ahead: its token is dropped
+            served.append(request)
             if request.is_prefilling:
                 request.prefill_cursor += size
-                if request.prefill_cursor < len(request.prompt_token_ids):
+                if request.prompt_left:
                     continue
-                completed_prefill.add(request.request_id)
-            token = int(next(next_token))
+            token = int(tokens[id(request)])
             request.generated_token_ids.append(token)
             request.pending_token_id = token
             emitted[request.request_id] = token
-            reason = None
-            if len(request.generated_token_ids) >= request.max_new_tokens:
-                reason = "length"
-            if (self.eos_token_id is not None and token == self.eos_token_id
+            if (token == self.eos_token_id and self.eos_token_id is not None
                     and not request.sampling.ignore_eos):
-                reason = "stop"
-            if reason is not None:
-                request.finish_reason = reason
-                self.active.pop(request.request_id, None)
-                self.engine.finish(request.request_id)
-                for g, pages in enumerate(request.reserved_blocks):
-                    self.reserved_blocks[g] -= pages
-                request.reserved_blocks = []
-                self.finished[request.request_id] = request
-            else:
-                self.active[request.request_id] = request
-        if completed_prefill:
-            self.waiting = deque(r for r in self.waiting if r.request_id not in completed_prefill)
+                self._retire(request, "stop")
+            elif len(request.generated_token_ids) >= request.max_new_tokens:
+                self._retire(request, "length")
+        # those that had waited longest for this turn are also first in line for the next one
+        for request in sorted(served, key=lambda request: (request.last_served, request.request_id)):
+            request.last_served = self._tickets
+            self._tickets += 1
         self.iterations += 1
         return emitted
 
+    def _retire(self, request, reason):
+        """The request is over: pages, slot and promise go back."""
+        request.finish_reason = reason
+        del self._live[request.request_id]
+        self.engine.finish(request.request_id)
+        self.ledger.withdraw(request)
+        self.finished[request.request_id] = request
+
     def has_work(self) -> bool:
-        return bool(self.waiting or self.active or self._inflight is not None)
+        return bool(self._live) or self._inflight is not None
 
     def run_until_complete(self):
         while self.has_work():

@@ -13,9 +13,9 @@ import torch
 from ..cache.manager import CacheGroupSpec, StateSpec
 from ..config.spec import ModelSpec
 from ..ops import kernels
-from ..parts import (ARRANGEMENTS, FEED_FORWARDS, MIXERS, NORMS, POSITIONS, CacheView,
+from ..parts import (ARRANGEMENTS, EMBEDDINGS, HEADS, NORMS, POSITIONS, ROLES, CacheView,
                      PagedKVSpec, SlotStateSpec, build_part)
-from ..weights.loader import MATRIX, TABLE, ParamSpec
+from ..weights.loader import ParamSpec
 
 
 class DecoderModel:
@@ -25,25 +25,37 @@ class DecoderModel:
         self.device = torch.device(device)
         common = dict(width=spec.width, dtype=dtype)
         self.position = build_part(POSITIONS, "position encoding", spec.position, **common)
+        self.embedding = build_part(EMBEDDINGS, "embedding", spec.embedding,
+                                    vocab_size=spec.vocab_size, **common)
+        self.head = build_part(HEADS, "output head", spec.head, vocab_size=spec.vocab_size,
+                               tied=spec.tie_head, **common)
         self.blocks = []
         for block_spec in spec.blocks:
             if block_spec.arrangement not in ARRANGEMENTS:
                 raise KeyError(f"unknown block arrangement {block_spec.arrangement!r}; "
                                f"known: {', '.join(sorted(ARRANGEMENTS))}")
-            mixer = build_part(MIXERS, "mixer", block_spec.mixer, **common)
-            mixer.set_position(self.position)
-            block = ARRANGEMENTS[block_spec.arrangement](
-                width=spec.width, dtype=dtype,
-                norm1=build_part(NORMS, "norm", block_spec.norm1, **common),
-                mixer=mixer,
-                norm2=build_part(NORMS, "norm", block_spec.norm2, **common),
-                feed_forward=build_part(FEED_FORWARDS, "feed-forward", block_spec.feed_forward,
-                                        **common))
-            self.blocks.append(block)
+            arrangement = ARRANGEMENTS[block_spec.arrangement]
+            parts = {}
+            for name, role in arrangement.roles.items():
+                if role not in ROLES:
+                    raise KeyError(f"arrangement {block_spec.arrangement!r} gives part {name!r} the "
+                                   f"unknown role {role!r}; known: {', '.join(sorted(ROLES))}")
+                parts[name] = build_part(ROLES[role], f"{role} ({name})", block_spec.part(name), **common)
+                if role == "mixer":
+                    parts[name].set_position(self.position)
+            unknown = [name for name, _ in block_spec.parts if name not in arrangement.roles]
+            if unknown:
+                raise KeyError(f"arrangement {block_spec.arrangement!r} has no part named "
+                               f"{', '.join(unknown)}; it has: {', '.join(arrangement.roles)}")
+            self.blocks.append(arrangement(width=spec.width, dtype=dtype, parts=parts))
         self.final_norm = build_part(NORMS, "norm", spec.final_norm, **common)
-        self.embedding_table = None
-        self.head_weight = None
-        self.head_packed = None
+        # Queries of a prompt portion are handed to the mixers in tiles of this many; the
+        # mixers say which size their kernels take (all that say so must agree).
+        tiles = {block.mixer.query_tile for block in self.blocks
+                 if getattr(block.mixer, "query_tile", None)}
+        if len(tiles) > 1:
+            raise ValueError(f"the mixers ask for different query tiles: {sorted(tiles)}")
+        self.query_tile = tiles.pop() if tiles else None
         # the mixer of the call that writes a cache entry decides what the entry holds
         self._entry_spec = {}
         for call in spec.schedule:
@@ -57,34 +69,29 @@ class DecoderModel:
                     f"{self._entry_spec[call.cache]}, but needs {mine}")
 
     # ------------------------------------------------------------- parameters
-    def parameters(self) -> Dict[str, ParamSpec]:
-        params = {"embedding.table": ParamSpec((self.spec.vocab_size, self.spec.width), TABLE)}
-        for name, spec in self.position.parameters().items():
-            params[f"position.{name}"] = spec
+    def _named_parts(self):
+        """(prefix of the parameter paths, part) of every part that may own parameters."""
+        yield "embedding.", self.embedding
+        yield "position.", self.position
         for index, block in enumerate(self.blocks):
             for part_name, part in block.parts().items():
-                for name, spec in part.parameters().items():
-                    params[f"blocks.{index}.{part_name}.{name}"] = spec
-        for name, spec in self.final_norm.parameters().items():
-            params[f"final_norm.{name}"] = spec
-        if not self.spec.tie_head:
-            params["head.weight"] = ParamSpec((self.spec.vocab_size, self.spec.width), MATRIX)
-        return params
+                yield f"blocks.{index}.{part_name}.", part
+        yield "final_norm.", self.final_norm
+        yield "head.", self.head
+
+    def parameters(self) -> Dict[str, ParamSpec]:
+        return {prefix + name: spec for prefix, part in self._named_parts()
+                for name, spec in part.parameters().items()}
 
     def bind(self, tensors: Dict[str, torch.Tensor]):
-        def take(prefix, part):
-            part.bind({name: tensors[prefix + name] for name in part.parameters()})
-
-        self.embedding_table = tensors["embedding.table"]
-        take("position.", self.position)
-        for index, block in enumerate(self.blocks):
-            for part_name, part in block.parts().items():
-                take(f"blocks.{index}.{part_name}.", part)
-        take("final_norm.", self.final_norm)
-        # the tied head is the embedding table itself, not a copy
-        # (src/model/paged_decoder.py:300-301)
-        self.head_weight = self.embedding_table if self.spec.tie_head else tensors["head.weight"]
-        self.head_packed = kernels.pack_decode_weight(self.head_weight)
+        for prefix, part in self._named_parts():
+            mine = {name: tensors[prefix + name] for name in part.parameters()}
+            if part is self.head:
+                # a tied head is the token table itself, not a copy
+                # (src/model/paged_decoder.py:300-301)
+                part.bind(mine, embedding_table=tensors["embedding.table"])
+            else:
+                part.bind(mine)
         self.parameter_bytes = sum(t.numel() * t.element_size() for t in tensors.values())
         self.parameter_count = sum(t.numel() for t in tensors.values())
 
@@ -124,7 +131,7 @@ class DecoderModel:
     def graph_safe(self) -> bool:
         """Whether a step of this model may be recorded and replayed as a graph: every part
         says so of itself."""
-        parts = [self.position, self.final_norm] + list(self.blocks)
+        parts = [self.embedding, self.position, self.final_norm, self.head] + list(self.blocks)
         return all(getattr(part, "graph_safe", False) for part in parts)
 
     def forward(self, ctx, views, logit_rows, logits_out):
@@ -132,19 +139,18 @@ class DecoderModel:
         step's tokens) into the float tensor ``logits_out``."""
         tokens = ctx.tokens
         h = ctx.workspace.rows("residual", self.spec.width, torch.float32)[:tokens]
-        kernels.embed(self.embedding_table, self.position.embedding_table(), ctx.token_ids,
-                      ctx.positions, h, token_src=ctx.token_src, carried=ctx.carried_tokens)
+        self.embedding.forward(ctx, self.position.embedding_table(), h)
         for call, view in zip(self.spec.schedule, views):
             self.blocks[call.block].forward(h, ctx, view)
         wanted = logit_rows.numel()
         if wanted == 0:
             return logits_out[:0]
         final = ctx.workspace.rows("final", self.spec.width, self.dtype)[:wanted]
-        pending = self.final_norm.pending(h, final, rows=logit_rows)
-        if pending is None:
-            pending = self.final_norm.forward(h, final, rows=logit_rows)
-        # logits = f @ table^T without bias, always float
-        # (src/model/paged_decoder.py:295-301,605)
+        normed = None
+        if getattr(self.head, "accepts_pending_norm", False):
+            normed = self.final_norm.pending(h, final, rows=logit_rows)
+        if normed is None:
+            normed = self.final_norm.forward(h, final, rows=logit_rows)
         out = logits_out[:wanted]
-        kernels.linear(pending, self.head_weight, None, out, packed=self.head_packed)
+        self.head.forward(normed, out)
         return out

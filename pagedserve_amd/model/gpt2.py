@@ -27,8 +27,8 @@ def build_spec(config: GPT2Config) -> ModelSpec:
         if config.scale_attn_by_inverse_layer_idx:
             scale /= layer + 1
         norm = PartSpec.make("layernorm", eps=config.layer_norm_epsilon)
-        blocks.append(BlockSpec(
-            arrangement="pre_norm",
+        blocks.append(BlockSpec.make(
+            "pre_norm",
             norm1=norm,
             mixer=PartSpec.make("attention", heads=config.n_head, kv_heads=config.n_head,
                                 head_dim=config.head_dim, scale=scale, window=0, bias=True),
@@ -47,6 +47,8 @@ def build_spec(config: GPT2Config) -> ModelSpec:
         final_norm=PartSpec.make("layernorm", eps=config.layer_norm_epsilon),
         tie_head=config.tie_word_embeddings,
         eos_token_id=config.eos_token_id,
+        embedding=PartSpec.make("lookup", scale=1.0),
+        head=PartSpec.make("linear", bias=False),
     )
 
 
@@ -135,4 +137,8 @@ GPT2 = register_architecture(Architecture(
     random_tensors=random_tensors,
     ignorable=ignorable,
     model_type="gpt2",
+    # tensors lie under "transformer." in GPT2LMHeadModel checkpoints and bare in GPT2Model ones;
+    # the head of an untied model is never prefixed
+    strip_prefixes=("transformer.",),
+    stored_name=lambda config, name: name if name.startswith("lm_head.") else "transformer." + name,
 ))

@@ -5,7 +5,7 @@ import os
 
 import torch
 
-from ..config.gpt2 import read_config_json
+from ..config.base import read_config_json
 from ..config.registry import resolve_architecture
 from ..weights.loader import load_parameters
 from ..weights.safetensors_io import write_safetensors
@@ -34,7 +34,8 @@ def load_model(folder, dtype="float32", device="cuda"):
     model = DecoderModel(spec, engine_dtype, device)
     tensors = load_parameters(
         folder, model.parameters(), architecture.weight_sources(config, spec), engine_dtype,
-        device, ignorable=lambda name: architecture.ignorable(config, name))
+        device, strip_prefixes=architecture.strip_prefixes,
+        ignorable=lambda name: architecture.ignorable(config, name))
     model.bind(tensors)
     return model, config
 
@@ -57,37 +58,33 @@ def random_model(config, seed=0, dtype="bfloat16", device="cuda"):
     tensors = {}
     for target, param in model.parameters().items():
         source = sources[target]
-        tensor = drawn[source.name]
-        if source.transpose:
-            tensor = tensor.transpose(0, 1)
+        tensor = source.assemble(drawn.__getitem__)
         if tuple(tensor.shape) != tuple(param.shape):
-            raise ValueError(f"random tensor {source.name} has shape {tuple(tensor.shape)}, "
+            raise ValueError(f"random tensor {source.label()} has shape {tuple(tensor.shape)}, "
                              f"parameter {target} needs {tuple(param.shape)}")
         tensors[target] = tensor.to(target_dtype(param.role, engine_dtype)).contiguous().to(device)
     model.bind(tensors)
     return model, config
 
 
-def write_random_model(folder, config, seed=0, store_dtype=torch.float32, prefix="transformer."):
+def write_random_model(folder, config, seed=0, store_dtype=torch.float32, stored_name=None):
     """Write ``config.json`` and ``model.safetensors`` of a random model of ``config``.
 
-    ``config`` is a typed configuration of a registered architecture or a raw dict
-    with that architecture's config.json keys."""
+    ``config`` is a typed configuration of a registered architecture or a raw dict with that
+    architecture's config.json keys (``architectures`` or ``model_type`` among them).  Tensors
+    are named as the architecture's checkpoints name them, or by ``stored_name(name)``."""
     if isinstance(config, dict):
         raw = dict(config)
-        architecture = resolve_architecture(
-            raw if raw.get("architectures") or raw.get("model_type")
-            else {**raw, "architectures": ["GPT2LMHeadModel"]})
+        architecture = resolve_architecture(raw)
         raw.setdefault("architectures", [architecture.name])
         config = architecture.config_class.from_dict(raw)
     else:
         architecture = resolve_architecture({"architectures": [config.architecture]})
+    if stored_name is None:
+        stored_name = lambda name: architecture.stored_name(config, name)  # noqa: E731
     os.makedirs(folder, exist_ok=True)
     tensors = architecture.random_tensors(config, seed)
-    stored = {}
-    for name, tensor in tensors.items():
-        key = name if name.startswith("lm_head.") else prefix + name
-        stored[key] = tensor.to(store_dtype).contiguous()
+    stored = {stored_name(name): tensor.to(store_dtype).contiguous() for name, tensor in tensors.items()}
     write_safetensors(os.path.join(folder, "model.safetensors"), stored,
                       metadata={"format": "pt", "seed": seed})
     with open(os.path.join(folder, "config.json"), "w") as handle:

@@ -21,7 +21,7 @@ _DTYPE_CODE = {torch.float32: F32, torch.bfloat16: BF16}
 
 _SIGNATURES = {
     "ps_embed": [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int,
-                 c_int, c_int, c_int, c_int, c_void_p],
+                 c_int, c_int, c_int, c_float, c_int, c_void_p],
     "ps_norm": [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_float, c_int,
                 c_int, c_void_p],
     "ps_gemm_nt": [c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int,
@@ -126,8 +126,8 @@ def _ptr(tensor):
     return 0 if tensor is None else tensor.data_ptr()
 
 
-def embed(table, pos_table, ids, positions, out, token_src=None, carried=None):
-    """out[t] = table[id(t)] + pos_table[positions[t]] as float (pos_table may be None).
+def embed(table, pos_table, ids, positions, out, token_src=None, carried=None, scale=1.0):
+    """out[t] = scale * table[id(t)] + pos_table[positions[t]] as float (pos_table may be None).
     id(t) is ``ids[t]``, or ``carried[token_src[t]]`` where ``token_src[t] >= 0``: a token
     that an earlier step chose on the device."""
     _check(table, "table", ndim=2)
@@ -156,7 +156,7 @@ def embed(table, pos_table, ids, positions, out, token_src=None, carried=None):
     _call("ps_embed", table.data_ptr(), _ptr(pos_table), ids.data_ptr(), _ptr(token_src),
           _ptr(carried if token_src is not None else None),
           _ptr(positions if pos_table is not None else None), out.data_ptr(), tokens, width,
-          table.shape[0], max_positions, dtype_code(table.dtype), _stream())
+          table.shape[0], max_positions, float(scale), dtype_code(table.dtype), _stream())
     return out
 
 
@@ -462,7 +462,7 @@ def attention_rowwise(q, k_pool, v_pool, out, tok_item, tok_pos, tables, heads, 
 
 def decode_keys_per_block(head_dim: int, waves: int = 4) -> int:
     """Keys that one block of the split-KV kernel visits per iteration."""
-    lanes = head_dim // 8
+    lanes = -(-head_dim // 8)
     lanes_per_key = 2 if lanes <= 2 else 4 if lanes <= 4 else 8 if lanes <= 8 else 16 if lanes <= 16 else 32
     return (64 // lanes_per_key) * (8 if waves == 16 else 4) * waves
 
@@ -485,6 +485,12 @@ def attention_decode(q, k_pool, v_pool, out, tok_item, tok_pos, tables, heads, s
           tables.shape[1], count, heads, kv_heads, head_dim, page_size, pages, float(scale),
           int(window), int(splits), int(waves), dtype_code(q.dtype), _stream())
     return out
+
+
+def decode_supported(head_dim) -> bool:
+    """Whether the split-KV kernel takes this head size (a lane fetches eight consecutive head
+    dimensions of a key in one piece); the row-wise kernel takes every size up to 256."""
+    return head_dim % 8 == 0 and 0 < head_dim <= 256
 
 
 PREFILL_TILE = 64
@@ -601,6 +607,17 @@ class StepGraph:
             lib.ps_graph_destroy.argtypes = [c_void_p]
             lib.ps_graph_destroy(self.handle)
             self.handle = None
+
+
+_COMPUTE_UNITS = None
+
+
+def compute_units() -> int:
+    """Compute units of the current device (asked once)."""
+    global _COMPUTE_UNITS
+    if _COMPUTE_UNITS is None:
+        _COMPUTE_UNITS = max(1, device_info()["compute_units"])
+    return _COMPUTE_UNITS
 
 
 def device_info():

@@ -13,6 +13,7 @@ import ctypes
 import hashlib
 import os
 import shutil
+import stat
 import subprocess
 import sys
 import tempfile
@@ -85,8 +86,28 @@ def _writable(folder) -> bool:
         return False
 
 
+_PRIVATE_DIR = None
+
+
 def _fallback_dir() -> str:
-    return os.path.join(tempfile.gettempdir(), f"pagedserve_amd-{os.getuid()}")
+    """Where the library is built and looked for when the tree cannot be written: a folder
+    under the temporary directory that belongs to this user alone.  The name can be guessed, so
+    a folder of that name that someone else made, or that others may write, is never used (a
+    library planted there would be loaded): a fresh private folder takes its place for this
+    process."""
+    global _PRIVATE_DIR
+    if _PRIVATE_DIR is not None:
+        return _PRIVATE_DIR
+    path = os.path.join(tempfile.gettempdir(), f"pagedserve_amd-{os.getuid()}")
+    try:
+        os.makedirs(path, mode=0o700, exist_ok=True)
+        status = os.lstat(path)
+        mine = (stat.S_ISDIR(status.st_mode) and status.st_uid == os.getuid()
+                and not status.st_mode & 0o022)
+    except OSError:
+        mine = False
+    _PRIVATE_DIR = path if mine else tempfile.mkdtemp(prefix="pagedserve_amd-")
+    return _PRIVATE_DIR
 
 
 def _say(message, verbose):

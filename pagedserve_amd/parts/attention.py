@@ -25,12 +25,15 @@ class Attention(Mixer):
 
     accepts_pending_norm = True
 
+    # the step's index arrays list the queries of a prompt portion in tiles of this size
+    query_tile = kernels.PREFILL_TILE
+
     def __init__(self, width: int, dtype, heads: int, kv_heads: int, head_dim: int, scale: float,
                  window: int = 0, bias: bool = True):
         if heads % kv_heads != 0:
             raise ValueError(f"heads ({heads}) must be a multiple of kv_heads ({kv_heads})")
-        if head_dim % 16 != 0 or head_dim > 256:
-            raise ValueError(f"head_dim {head_dim} must be a multiple of 16 up to 256")
+        if not 0 < head_dim <= 256:
+            raise ValueError(f"head_dim {head_dim} must lie in 1..256")
         self.width = width
         self.dtype = dtype
         self.heads = heads
@@ -89,19 +92,25 @@ class Attention(Mixer):
                                  tables)
         context = ctx.workspace.rows("attn", self.q_cols, self.dtype)[:tokens]
         singles = ctx.single_tokens.numel() if ctx.single_tokens is not None else 0
+        if not kernels.decode_supported(self.head_dim):
+            # a head size that the split-KV kernel does not take: every token, decoded ones
+            # too, goes to the kernel that takes all sizes
+            singles = 0
         if singles:
             # one-token items: keys of a request are cut into ranges so that few requests
             # still fill the chip
             splits, waves = self._splits(singles, ctx.max_kv_len)
             partial = None
             if splits > 1:
-                # _splits keeps singles * heads * splits below 1024 + singles * heads
-                worst = (1024 + ctx.workspace.max_rows * self.heads) * (self.head_dim + 2)
+                # _splits keeps singles * heads * splits below 4 * units + singles * heads
+                worst = ((4 * kernels.compute_units() + ctx.workspace.max_rows * self.heads)
+                         * (self.head_dim + 2))
                 partial = ctx.workspace.flat("attn_partial", worst, torch.float32)
             kernels.attention_decode(q, cache.k_pool, cache.v_pool, context, ctx.tok_item,
                                      ctx.positions, tables, self.heads, self.scale, splits,
                                      partial=partial, window=self.window, waves=waves,
                                      tok_list=None if singles == tokens else ctx.single_tokens)
+        whole = singles == 0
         if singles < tokens and kernels.prefill_supported(self.dtype, self.head_dim, tables.shape[1]):
             kernels.attention_prefill(q, cache.k_pool, cache.v_pool, context, ctx.tile_item,
                                       ctx.tile_q0, ctx.cu_tokens, ctx.kv_lens, tables,
@@ -110,7 +119,7 @@ class Attention(Mixer):
         elif singles < tokens:
             kernels.attention_rowwise(q, cache.k_pool, cache.v_pool, context, ctx.tok_item,
                                       ctx.positions, tables, self.heads, self.scale, self.window,
-                                      tok_list=None if singles == 0 else ctx.portion_tokens)
+                                      tok_list=None if whole else ctx.portion_tokens)
         kernels.linear(context, self.out_weight, self.out_bias, residual, epilogue="residual",
                        packed=self.out_packed)
 
@@ -124,12 +133,13 @@ class Attention(Mixer):
         of the longest request can feed."""
         visible = max_kv_len if self.window <= 0 else min(max_kv_len, self.window)
         pairs = count * self.heads
-        if pairs >= 384:
+        units = kernels.compute_units()
+        if pairs >= units + units // 2:
             return 1, 4
-        if pairs >= 64 and visible > kernels.decode_keys_per_block(self.head_dim, 4):
+        if pairs >= units // 4 and visible > kernels.decode_keys_per_block(self.head_dim, 4):
             # contexts of several thousand keys: two or three such blocks per request, as
             # long as every block still has a compute unit of its own
-            return max(1, min(256 // pairs, visible // 1024)), 16
+            return max(1, min(units // pairs, visible // 1024)), 16
         most = max(1, -(-visible // kernels.decode_keys_per_block(self.head_dim, 4)))
-        wanted = max(1, -(-1024 // pairs))
+        wanted = max(1, -(-4 * units // pairs))
         return min(most, wanted, 64), 4

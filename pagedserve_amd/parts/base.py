@@ -15,6 +15,8 @@ tensors.  It never sees the model's configuration.
   ``CacheView`` of this call of the layer: pools of a paged key/value entry, or the
   state tensor ``[max_slots, ...]`` of a mixer that declared a ``StateSpec``.
 * ``FeedForward.forward(x, residual, ctx)``: same contract without a cache.
+* ``Embedding.forward(ctx, position_table, out)`` fills the float stream from token ids;
+  ``Head.forward(x, logits)`` turns the (normed) wanted rows into float logits.
 * ``PositionEncoding``: ``embedding_table()`` is added to the token embedding when it
   is not ``None``; ``apply_to_qk(q, k, ctx)`` may transform queries and keys in place
   before they are cached (the default does nothing).
@@ -95,6 +97,28 @@ class PositionEncoding(Part):
 
     def apply_to_qk(self, q, k, ctx):
         return None
+
+
+class Embedding(Part):
+    """``forward(ctx, position_table, out)`` fills the float stream ``out[T, d]`` from the
+    step's token ids; ``table`` is the parameter that a tied head shares."""
+
+    def forward(self, ctx, position_table, out):
+        raise NotImplementedError
+
+
+class Head(Part):
+    """``forward(x, logits)`` writes float logits of the rows ``x`` (normed rows, or a pending
+    norm if ``accepts_pending_norm``).  ``bind`` also receives the token table, which a tied
+    head uses as its matrix."""
+
+    accepts_pending_norm = True
+
+    def bind(self, tensors, embedding_table=None):
+        super().bind(tensors)
+
+    def forward(self, x, logits):
+        raise NotImplementedError
 
 
 class Mixer(Part):

@@ -1,4 +1,10 @@
-"""Arrangements of parts in a block."""
+"""Arrangements of parts in a block.
+
+An arrangement says which named parts it is made of and what each is (``roles``: name ->
+``"norm"``, ``"mixer"`` or ``"feed_forward"``, the registry its kind is looked up in), and in
+which order they run; ``mixer`` is the part whose ``cache_spec`` decides what the block's cache
+entry holds.  The model builds the parts that the block's spec names and hands them
+over as a dict; an arrangement with another number of parts declares other roles."""
 
 from .registry import register_arrangement
 
@@ -8,13 +14,16 @@ class PreNormBlock:
     """``h += mixer(norm1(h))`` then ``h += feed_forward(norm2(h))``
     (src/model/paged_decoder.py:181-189,210-228)."""
 
-    def __init__(self, width, dtype, norm1, mixer, norm2, feed_forward):
+    roles = {"norm1": "norm", "mixer": "mixer", "norm2": "norm", "feed_forward": "feed_forward"}
+
+    def __init__(self, width, dtype, parts):
         self.width = width
         self.dtype = dtype
-        self.norm1 = norm1
-        self.mixer = mixer
-        self.norm2 = norm2
-        self.feed_forward = feed_forward
+        self._parts = dict(parts)
+        self.norm1 = parts["norm1"]
+        self.mixer = parts["mixer"]
+        self.norm2 = parts["norm2"]
+        self.feed_forward = parts["feed_forward"]
 
     @property
     def graph_safe(self):
@@ -22,8 +31,7 @@ class PreNormBlock:
         return all(getattr(part, "graph_safe", False) for part in self.parts().values())
 
     def parts(self):
-        return {"norm1": self.norm1, "mixer": self.mixer, "norm2": self.norm2,
-                "feed_forward": self.feed_forward}
+        return dict(self._parts)
 
     def _normed(self, norm, part, h, ctx):
         """Input of ``part``: the norm as a pending object if the part takes one, else rows."""

@@ -8,6 +8,11 @@ MIXERS: Dict[str, Callable] = {}
 FEED_FORWARDS: Dict[str, Callable] = {}
 POSITIONS: Dict[str, Callable] = {}
 ARRANGEMENTS: Dict[str, Callable] = {}
+EMBEDDINGS: Dict[str, Callable] = {}
+HEADS: Dict[str, Callable] = {}
+
+# role of a block's named part -> the registry its kind is looked up in
+ROLES = {"norm": NORMS, "mixer": MIXERS, "feed_forward": FEED_FORWARDS}
 
 
 def _register(table, what):
@@ -26,6 +31,8 @@ register_mixer = _register(MIXERS, "mixer")
 register_feed_forward = _register(FEED_FORWARDS, "feed-forward")
 register_position = _register(POSITIONS, "position encoding")
 register_arrangement = _register(ARRANGEMENTS, "block arrangement")
+register_embedding = _register(EMBEDDINGS, "embedding")
+register_head = _register(HEADS, "output head")
 
 
 def build_part(table, what, spec, **common):

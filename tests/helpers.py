@@ -24,7 +24,26 @@ TINY_B = {
     "n_positions": 256, "layer_norm_epsilon": 1e-6, "activation_function": "gelu",
     "scale_attn_by_inverse_layer_idx": True, "tie_word_embeddings": True, "eos_token_id": None,
 }
-TINY = {"A": (TINY_A, 8, 0, "transformer."), "B": (TINY_B, 16, 1, "")}
+# The sizes of the reference's own GPT-2 test (testing/test_gpt2.py:13-27: vocabulary 41, width
+# 16, two heads of 8, inner width 32, tanh GELU) with more positions, so that the traces fit,
+# and a head of its own instead of the tied one.
+TINY_C = {
+    "architectures": ["GPT2LMHeadModel"], "model_type": "gpt2",
+    "n_layer": 2, "n_embd": 16, "n_head": 2, "n_inner": 32, "vocab_size": 41,
+    "n_positions": 96, "layer_norm_epsilon": 1e-5, "activation_function": "gelu_new",
+    "scale_attn_by_inverse_layer_idx": False, "tie_word_embeddings": False, "eos_token_id": 1,
+}
+# A head size (20) that is no multiple of 8, widths that are no multiple of 8 either (every
+# product takes the plain kernel), a page size that is no power of two.
+TINY_D = {
+    "architectures": ["GPT2LMHeadModel"], "model_type": "gpt2",
+    "n_layer": 2, "n_embd": 60, "n_head": 3, "n_inner": 100, "vocab_size": 333,
+    "n_positions": 160, "layer_norm_epsilon": 3e-6, "activation_function": "gelu",
+    "scale_attn_by_inverse_layer_idx": True, "tie_word_embeddings": True, "eos_token_id": None,
+}
+# configuration, page size, seed of the weights, prefix of the tensor names
+TINY = {"A": (TINY_A, 8, 0, "transformer."), "B": (TINY_B, 16, 1, ""),
+        "C": (TINY_C, 4, 2, "transformer."), "D": (TINY_D, 12, 3, "")}
 
 
 def lively_tensors(config, seed):
@@ -191,8 +210,10 @@ def live_token_budget(steps, round_to=64):
     return peak
 
 
-def replay_in_process(engine, steps):
-    """Run a trace through an Engine; returns {(request, position): float64 logits row}."""
+def replay_in_process(engine, steps, page_holders=None):
+    """Run a trace through an Engine; returns {(request, position): float64 logits row}.
+    ``page_holders`` (a dict) collects, per physical page of cache group 0, the requests that
+    held it at some time."""
     from pagedserve_amd.engine import StepEntry
 
     rows = {}
@@ -201,6 +222,11 @@ def replay_in_process(engine, steps):
         values = output.logits.double().cpu()
         for index, key in enumerate(output.rows):
             rows[key] = values[index]
+        if page_holders is not None:
+            for rid, record in engine.cache.requests.items():
+                for page in record.tables[0]:
+                    if page >= 0:
+                        page_holders.setdefault(page, set()).add(rid)
         for rid in step["end"]:
             engine.finish(rid)
     return rows
@@ -222,4 +248,4 @@ def max_error(rows, reference):
 
 # |engine - plain| <= TOLERANCE[dtype] * max|plain logits|.  Measured on MI355X: about 2e-6 in
 # float32 and 2e-3 in bfloat16 at every size from the tiny models to GPT-2 small.
-TOLERANCE = {"float32": 2e-5, "bfloat16": 1e-2}
+TOLERANCE = {"float32": 2e-5, "bfloat16": 4e-3}

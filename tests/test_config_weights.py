@@ -69,8 +69,12 @@ def test_spec_is_layer_by_layer_data():
 
 def test_run_order_rules():
     norm = PartSpec.make("layernorm", eps=1e-5)
-    block = BlockSpec("pre_norm", norm, PartSpec.make("attention", heads=1, kv_heads=1, head_dim=16, scale=1.0),
-                      norm, PartSpec.make("dense", inner=8, activation="gelu_erf"))
+    block = BlockSpec.make("pre_norm", norm1=norm,
+                           mixer=PartSpec.make("attention", heads=1, kv_heads=1, head_dim=16, scale=1.0),
+                           norm2=norm, feed_forward=PartSpec.make("dense", inner=8, activation="gelu_erf"))
+    assert block.mixer.kind == "attention" and block.with_part("mixer", norm).mixer is norm
+    with pytest.raises(KeyError, match="no part 'gate'"):
+        block.part("gate")
 
     def spec(schedule):
         return ModelSpec("toy", 10, 16, 8, PartSpec.make("none"), (block,), tuple(schedule), norm, True)
@@ -134,7 +138,7 @@ def test_loader_places_tensors_and_keeps_precisions(tmp_path):
     assert torch.equal(mixer.qkv_bias, tensors["h.1.attn.c_attn.bias"])
     assert torch.equal(model.blocks[2].norm2.gamma, tensors["h.2.ln_2.weight"])
     # the tied head is the embedding table itself (src/model/paged_decoder.py:300-301)
-    assert model.head_weight is model.embedding_table
+    assert model.head.weight is model.embedding.table
     assert torch.equal(model.position.table, tensors["wpe.weight"].to(torch.bfloat16))
     model32, _ = _load_cpu(folder, "float32")
     assert torch.equal(model32.blocks[0].feed_forward.down_weight, tensors["h.0.mlp.c_proj.weight"].t())

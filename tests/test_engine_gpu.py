@@ -17,7 +17,8 @@ ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 
 # prompt + decoded lengths of the two tiny workloads (5, 17, 31 -> 16 tokens; 1, 9, 40, 64, 100 -> 24),
 # as given token sequences, plus one long request each
-LENGTHS = {"A": [5 + 16, 17 + 16, 31 + 16, 90], "B": [1 + 24, 9 + 24, 40 + 24, 64 + 24, 100 + 24, 200]}
+LENGTHS = {"A": [5 + 16, 17 + 16, 31 + 16, 90, 12, 60, 29], "B": [1 + 24, 9 + 24, 40 + 24, 64 + 24, 100 + 24, 200],
+           "C": [5 + 16, 17 + 16, 31 + 16, 90, 12, 60], "D": [25, 33, 64, 88, 124, 150]}
 
 
 def _requests(which, config):
@@ -37,7 +38,7 @@ def _engine(folder, dtype, page_size, pages, max_step_tokens=512):
 @pytest.fixture(scope="module")
 def folders(tmp_path_factory):
     base = tmp_path_factory.mktemp("models")
-    return {which: helpers.tiny_folder(base, which) for which in ("A", "B")}
+    return {which: helpers.tiny_folder(base, which) for which in helpers.TINY}
 
 
 @pytest.fixture(scope="module")
@@ -60,18 +61,26 @@ CUTS = {
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
-@pytest.mark.parametrize("which", ["A", "B"])
+@pytest.mark.parametrize("which", list(helpers.TINY))
 @pytest.mark.parametrize("cut", list(CUTS))
 def test_cuts_match_plain(folders, references, which, dtype, cut):
+    """A: heads of 16; B: heads of 48, inverse-layer scaling, erf GELU; C: the sizes of the
+    reference's own test (heads of 8) with a head that is not tied; D: heads of 20, widths that
+    are no multiple of 8, pages of 12 tokens."""
     folder, config, page_size = folders[which]
     requests = _requests(which, config)
     steps = CUTS[cut](requests)
-    budget = helpers.live_token_budget(steps)
-    # exactly the pages that the live requests need at their peak: pages are used again
-    engine = _engine(folder, dtype, page_size, pages=-(-budget // page_size))
-    rows = helpers.replay_in_process(engine, steps)
+    # exactly the pages that the live requests hold at their peak, each request's tokens
+    # rounded up to whole pages: pages are used again
+    budget = helpers.live_token_budget(steps, round_to=page_size)
+    engine = _engine(folder, dtype, page_size, pages=budget // page_size)
+    holders = {}
+    rows = helpers.replay_in_process(engine, steps, page_holders=holders)
     engine.cache.check_invariants()
     assert not engine.cache.requests
+    assert engine.cache.pools[0].peak_allocated == budget // page_size
+    # some physical page went from one request to another
+    assert any(len(owners) > 1 for owners in holders.values())
     assert len(rows) == sum(len(tokens) for tokens in requests.values())
     error, scale, where = helpers.max_error(rows, references[(which, dtype == "bfloat16")])
     print(f"cut {cut} {which} {dtype}: error/scale {error / scale:.2e}")
@@ -247,3 +256,28 @@ def test_many_live_requests_match_plain(tmp_path, dtype):
     error, scale, where = helpers.max_error(rows, reference)
     assert error <= helpers.TOLERANCE[dtype] * scale, (dtype, error, scale, where)
     engine.cache.check_invariants()
+
+
+@pytest.mark.parametrize("num_layers,dtype", [(2, "float32"), (6, "float32"), (2, "bfloat16")])
+def test_reference_test_configuration(tmp_path, num_layers, dtype):
+    """The configuration and the steps of the reference's own GPT-2 test
+    (testing/test_gpt2.py:13-68): vocabulary 41, 16 positions, width 16, two heads of 8, inner
+    width 32, 2 and 6 layers, pages of 4; the prompt (4, 8, 15, 16) whole, then token 23
+    decoded.  The reference compares with the library's model, in 32-bit; here the plain
+    implementation stands in its place.  (bfloat16 at two layers only: six layers of width 16
+    add up to 4.3e-3 of the largest logit in bfloat16 roundings, measured, where wider models
+    stay near 2e-3; the tolerance is not widened for it.)"""
+    config = {"architectures": ["GPT2LMHeadModel"], "model_type": "gpt2", "vocab_size": 41,
+              "n_positions": 16, "n_embd": 16, "n_layer": num_layers, "n_head": 2, "n_inner": 32,
+              "activation_function": "gelu_new", "bos_token_id": 0, "eos_token_id": 1}
+    folder = str(tmp_path / "reference_config")
+    helpers.write_folder(folder, config, helpers.lively_tensors(config, 7))
+    prompt, following = [4, 8, 15, 16], 23
+    expected = helpers.plain_logits(folder, prompt + [following], bfloat16=dtype == "bfloat16")
+    engine = _engine(folder, dtype, 4, pages=2, max_step_tokens=16)
+    steps = [{"step": 0, "entries": [{"id": "request", "tokens": prompt, "want": [0, 1, 2, 3]}], "end": []},
+             {"step": 1, "entries": [{"id": "request", "tokens": [following], "want": [0]}], "end": ["request"]}]
+    rows = helpers.replay_in_process(engine, steps)
+    error, scale, where = helpers.max_error(rows, {"request": expected})
+    assert len(rows) == 5
+    assert error <= helpers.TOLERANCE[dtype] * scale, (error, scale, where)

@@ -37,6 +37,8 @@ def test_embed(dtype, tokens, width, vocab, positions):
     torch.testing.assert_close(out, expected, atol=0, rtol=0)
     kernels.embed(table, None, ids, pos, out)
     torch.testing.assert_close(out, F.embedding(ids.long(), table.float()), atol=0, rtol=0)
+    kernels.embed(table, pos_table, ids, pos, out, scale=8.0)
+    torch.testing.assert_close(out, expected + 7.0 * F.embedding(ids.long(), table.float()), atol=1e-5, rtol=1e-6)
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
@@ -203,8 +205,33 @@ def _gather(pool, table, length, page_size):
     return pool[pages].permute(1, 0, 2, 3).reshape(pool.shape[1], -1, pool.shape[3])[:, :length]
 
 
+def _attention_expected(q, k_pool, v_pool, tables, tok_item, tok_pos, heads, scale, window=0):
+    """float64 attention of every token over the keys 0..position (the last ``window``) of its
+    request, gathered page by page through the table: softmax(q K^T scale) V, nothing shared
+    with any kernel."""
+    kv_heads, page_size, head_dim = k_pool.shape[1], k_pool.shape[2], k_pool.shape[3]
+    group = heads // kv_heads
+    k_cpu, v_cpu, t_cpu = k_pool.double().cpu(), v_pool.double().cpu(), tables.cpu()
+    q_cpu = q.double().cpu()
+    out = torch.empty_like(q_cpu)
+    for t, (item, pos) in enumerate(zip(torch.as_tensor(tok_item).tolist(), torch.as_tensor(tok_pos).tolist())):
+        first = max(0, pos - window + 1) if window > 0 else 0
+        keys = _gather(k_cpu, t_cpu[item], pos + 1, page_size)[:, first:].repeat_interleave(group, 0)
+        values = _gather(v_cpu, t_cpu[item], pos + 1, page_size)[:, first:].repeat_interleave(group, 0)
+        scores = torch.einsum("hd,hkd->hk", q_cpu[t].reshape(heads, head_dim), keys) * scale
+        out[t] = torch.einsum("hk,hkd->hd", torch.softmax(scores, -1), values).reshape(-1)
+    return out.cuda()
+
+
+# head sizes: multiples of 16, of 8 only (8, 24, 40), and of neither (20, 7, 100); page sizes
+# that are no power of two (12, 5)
+ROWWISE_GEOMETRIES = [(1, 1, 32, 16), (4, 4, 16, 8), (6, 2, 48, 16), (3, 3, 128, 4), (12, 12, 64, 16),
+                      (2, 2, 8, 4), (4, 2, 20, 12), (3, 1, 7, 5), (2, 2, 100, 16), (5, 5, 80, 12),
+                      (2, 1, 256, 16), (6, 2, 24, 12)]
+
+
 @pytest.mark.parametrize("dtype", DTYPES)
-@pytest.mark.parametrize("heads,kv_heads,head_dim,page_size", [(1, 1, 32, 16), (4, 4, 16, 8), (6, 2, 48, 16), (3, 3, 128, 4), (12, 12, 64, 16)])
+@pytest.mark.parametrize("heads,kv_heads,head_dim,page_size", ROWWISE_GEOMETRIES)
 def test_attention_rowwise_decode_contexts(dtype, heads, kv_heads, head_dim, page_size):
     """Single-token queries over fragmented tables; contexts around page edges as in
     testing/test_triton_correctness_matrix.py:9 (1, 15, 16, 17, 31, 32, 33, 128, 512)."""
@@ -228,6 +255,33 @@ def test_attention_rowwise_decode_contexts(dtype, heads, kv_heads, head_dim, pag
         expected = F.scaled_dot_product_attention(query, keys, values).reshape(-1)
         atol, rtol = (3e-5, 3e-5) if dtype == torch.float32 else (2e-2, 2e-2)
         torch.testing.assert_close(out[index].double(), expected, atol=atol, rtol=rtol)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("heads,kv_heads,head_dim,page_size", [(6, 2, 48, 12), (4, 4, 20, 8), (2, 1, 256, 16)])
+@pytest.mark.parametrize("window", [0, 7, 40])
+def test_attention_rowwise_portions_grouped_heads_and_windows(dtype, heads, kv_heads, head_dim, page_size, window):
+    """Portions of several requests in one launch (fresh, continued, a single token), grouped
+    key/value heads with a window, a page size that is no power of two, head sizes 20 and
+    256: against float64 attention over the gathered pages."""
+    from pagedserve_amd.ops import kernels
+
+    items = [(0, 9), (30, 23), (17, 1), (100, 37)]
+    totals = [past + new for past, new in items]
+    k_pool, v_pool, tables = _paged_fixture(dtype, totals, kv_heads, head_dim, page_size, 123)
+    tok_item, tok_pos = [], []
+    for index, (past, new) in enumerate(items):
+        tok_item += [index] * new
+        tok_pos += list(range(past, past + new))
+    q = _rand((len(tok_item), heads * head_dim), dtype, 124)
+    out = torch.full_like(q, float("nan"))
+    scale = head_dim ** -0.5
+    kernels.attention_rowwise(q, k_pool, v_pool, out, torch.tensor(tok_item, dtype=torch.int32, device="cuda"),
+                              torch.tensor(tok_pos, dtype=torch.int32, device="cuda"), tables, heads, scale,
+                              window=window)
+    expected = _attention_expected(q, k_pool, v_pool, tables, tok_item, tok_pos, heads, scale, window)
+    atol, rtol = (3e-5, 3e-5) if dtype == torch.float32 else (2e-2, 2e-2)
+    torch.testing.assert_close(out.double(), expected, atol=atol, rtol=rtol)
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
@@ -263,8 +317,9 @@ def test_attention_rowwise_portion_and_window(dtype, window):
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
-@pytest.mark.parametrize("heads,kv_heads,head_dim,page_size", [(1, 1, 32, 16), (4, 4, 16, 8), (6, 2, 48, 16), (3, 3, 128, 4), (12, 12, 64, 16), (2, 1, 256, 16), (5, 5, 80, 12)])
-@pytest.mark.parametrize("splits", [1, 2, 5, 16])
+@pytest.mark.parametrize("heads,kv_heads,head_dim,page_size", [(1, 1, 32, 16), (4, 4, 16, 8), (6, 2, 48, 16), (3, 3, 128, 4), (12, 12, 64, 16), (2, 1, 256, 16), (5, 5, 80, 12),
+                                                                (2, 2, 8, 4), (6, 2, 24, 12), (3, 3, 40, 16), (4, 1, 200, 5)])
+@pytest.mark.parametrize("splits", [1, 2, 5, 16, 40])
 def test_attention_decode_split_kv(dtype, heads, kv_heads, head_dim, page_size, splits):
     """The split-KV kernel over fragmented tables at the contexts of
     testing/test_triton_correctness_matrix.py:9, for any number of splits (also more than the
@@ -281,21 +336,20 @@ def test_attention_decode_split_kv(dtype, heads, kv_heads, head_dim, page_size, 
     partial = torch.full((count * heads * splits * (head_dim + 2),), float("nan"), device="cuda")
     atol, rtol = (3e-5, 3e-5) if dtype == torch.float32 else (2e-2, 2e-2)
     for window in (0, 20):
-        expected = torch.empty_like(q)
-        kernels.attention_rowwise(q, k_pool, v_pool, expected, tok_item, tok_pos, tables, heads, scale, window=window)
+        expected = _attention_expected(q, k_pool, v_pool, tables, tok_item, tok_pos, heads, scale, window)
         out = torch.full_like(q, float("nan"))
         kernels.attention_decode(q, k_pool, v_pool, out, tok_item, tok_pos, tables, heads, scale, splits,
                                  partial=partial, window=window)
-        torch.testing.assert_close(out.double(), expected.double(), atol=atol, rtol=rtol)
+        torch.testing.assert_close(out.double(), expected, atol=atol, rtol=rtol)
     # a list of tokens: only those rows are written
     chosen = torch.tensor([7, 2, 9], dtype=torch.int32, device="cuda")
     out = torch.full_like(q, 7.0)
     kernels.attention_decode(q, k_pool, v_pool, out, tok_item, tok_pos, tables, heads, scale, splits,
                              partial=partial, tok_list=chosen)
-    kernels.attention_rowwise(q, k_pool, v_pool, expected, tok_item, tok_pos, tables, heads, scale)
+    expected = _attention_expected(q, k_pool, v_pool, tables, tok_item, tok_pos, heads, scale)
     for row in range(count):
         if row in (7, 2, 9):
-            torch.testing.assert_close(out[row].double(), expected[row].double(), atol=atol, rtol=rtol)
+            torch.testing.assert_close(out[row].double(), expected[row], atol=atol, rtol=rtol)
         else:
             assert float((out[row].float() - 7.0).abs().max()) == 0.0
 
@@ -415,12 +469,17 @@ def test_sample_temperature_inverse_cdf():
 def test_kernels_refuse_bad_sizes():
     from pagedserve_amd.ops import kernels
 
-    q = torch.zeros((1, 40), device="cuda")
-    pool = torch.zeros((2, 1, 4, 40), device="cuda")
+    q = torch.zeros((1, 20), device="cuda")
+    pool = torch.zeros((2, 1, 4, 20), device="cuda")
     idx = torch.zeros(1, dtype=torch.int32, device="cuda")
     tables = torch.zeros((1, 2), dtype=torch.int32, device="cuda")
-    with pytest.raises(kernels.KernelError, match="multiple of 16"):
-        kernels.attention_rowwise(q, pool, pool.clone(), q.clone(), idx, idx, tables, 1, 1.0)
+    with pytest.raises(kernels.KernelError, match="multiple of 8"):
+        kernels.attention_decode(q, pool, pool.clone(), q.clone(), idx, idx, tables, 1, 1.0, 1)
+    assert not kernels.decode_supported(20) and kernels.decode_supported(24)
+    wide = torch.zeros((1, 264), device="cuda")
+    wide_pool = torch.zeros((2, 1, 4, 264), device="cuda")
+    with pytest.raises(kernels.KernelError, match="1..256"):
+        kernels.attention_rowwise(wide, wide_pool, wide_pool.clone(), wide.clone(), idx, idx, tables, 1, 1.0)
     with pytest.raises(kernels.KernelError, match="GPU"):
         kernels.norm(torch.zeros(2, 4), torch.ones(4), None, 1e-5, torch.zeros(2, 4))
     with pytest.raises(kernels.KernelError):
@@ -433,7 +492,7 @@ def test_kernels_refuse_bad_sizes():
                                                                 (24, 8, 64, 16), (20, 20, 48, 8), (18, 18, 112, 16)])
 @pytest.mark.parametrize("window", [0, 37])
 def test_attention_prefill_tiles(heads, kv_heads, head_dim, page_size, window):
-    """The tiled kernel against the row-wise one: fresh prompts and later portions of many
+    """The tiled kernel against float64 attention over the gathered pages: fresh prompts and later portions of many
     lengths in one launch (1 < count, portions that start inside a page, more than one tile,
     a tile's last rows empty), fragmented tables, NaN behind every request's last key."""
     from pagedserve_amd.ops import kernels
@@ -463,13 +522,12 @@ def test_attention_prefill_tiles(heads, kv_heads, head_dim, page_size, window):
         return torch.tensor(values, dtype=torch.int32, device="cuda")
 
     scale = head_dim ** -0.5
-    expected = torch.empty_like(q)
-    kernels.attention_rowwise(q, k_pool, v_pool, expected, dev(tok_item), dev(tok_pos), tables, heads, scale, window=window)
+    expected = _attention_expected(q, k_pool, v_pool, tables, tok_item, tok_pos, heads, scale, window)
     out = torch.full_like(q, float("nan"))
     kernels.attention_prefill(q, k_pool, v_pool, out, dev(tile_item), dev(tile_q0), dev(cu), dev(totals),
                               tables, heads, scale, window=window)
     assert torch.isfinite(out.float()).all()
-    torch.testing.assert_close(out.double(), expected.double(), atol=2e-2, rtol=2e-2)
+    torch.testing.assert_close(out.double(), expected, atol=2e-2, rtol=2e-2)
 
 
 def test_attention_prefill_far_key_and_causality():
@@ -587,19 +645,18 @@ def test_attention_decode_sixteen_waves(dtype):
     q = _rand((len(contexts), heads * head_dim), dtype, 92)
     tok_item = torch.arange(len(contexts), dtype=torch.int32, device="cuda")
     tok_pos = torch.tensor([c - 1 for c in contexts], dtype=torch.int32, device="cuda")
-    expected = torch.empty_like(q)
-    kernels.attention_rowwise(q, k_pool, v_pool, expected, tok_item, tok_pos, tables, heads, 0.125)
+    expected = _attention_expected(q, k_pool, v_pool, tables, tok_item, tok_pos, heads, 0.125)
     out = torch.full_like(q, float("nan"))
     kernels.attention_decode(q, k_pool, v_pool, out, tok_item, tok_pos, tables, heads, 0.125, 1, waves=16)
     atol, rtol = (3e-5, 3e-5) if dtype == torch.float32 else (2e-2, 2e-2)
-    torch.testing.assert_close(out.double(), expected.double(), atol=atol, rtol=rtol)
+    torch.testing.assert_close(out.double(), expected, atol=atol, rtol=rtol)
     # two and three ranges per request, merged by the reduce kernel
     for splits in (2, 3):
         partial = torch.full((len(contexts) * heads * splits * (head_dim + 2),), float("nan"), device="cuda")
         out = torch.full_like(q, float("nan"))
         kernels.attention_decode(q, k_pool, v_pool, out, tok_item, tok_pos, tables, heads, 0.125, splits,
                                  partial=partial, waves=16)
-        torch.testing.assert_close(out.double(), expected.double(), atol=atol, rtol=rtol)
+        torch.testing.assert_close(out.double(), expected, atol=atol, rtol=rtol)
 
 
 PACKED_SHAPES = [(1, 50, 64), (8, 768, 3072), (8, 2304, 768), (16, 3072, 768), (17, 768, 768), (5, 1000, 320),

@@ -169,7 +169,8 @@ def _custom_model(tmp_path, schedule, dtype="float32"):
     typed = GPT2Config.from_dict(config)
     spec = dataclasses.replace(arch.build_spec(typed), schedule=tuple(schedule))
     model = DecoderModel(spec, torch.float32 if dtype == "float32" else torch.bfloat16, "cuda")
-    tensors = load_parameters(folder, model.parameters(), arch.weight_sources(typed, spec), model.dtype, "cuda")
+    tensors = load_parameters(folder, model.parameters(), arch.weight_sources(typed, spec), model.dtype, "cuda",
+                              strip_prefixes=arch.strip_prefixes)
     model.bind(tensors)
     engine = Engine(model, num_pages=24, page_size=page_size, max_requests=4, max_step_tokens=64)
     return engine, folder, config
@@ -255,13 +256,14 @@ def test_toy_mixer_with_state_of_its_own(tmp_path):
     arch = resolve_architecture(config)
     typed = GPT2Config.from_dict(config)
     base = arch.build_spec(typed)
-    toy_block = dataclasses.replace(base.blocks[1], mixer=PartSpec.make("toy_running_mean", gain=0.5))
+    toy_block = base.blocks[1].with_part("mixer", PartSpec.make("toy_running_mean", gain=0.5))
     spec = dataclasses.replace(base, blocks=(base.blocks[0], toy_block))
     model = DecoderModel(spec, torch.float32, "cuda")
     sources = arch.weight_sources(typed, base)
     sources = {k: v for k, v in sources.items() if not k.startswith("blocks.1.mixer.")}
     sources["blocks.1.mixer.mix.weight"] = WeightSource("h.1.attn.c_proj.weight", transpose=True)
     tensors = load_parameters(folder, model.parameters(), sources, torch.float32, "cuda",
+                              strip_prefixes=arch.strip_prefixes,
                               ignorable=lambda name: name.startswith("h.1.attn."))
     model.bind(tensors)
     groups, states = model.cache_requirements()
@@ -351,7 +353,7 @@ def test_toy_feed_forward_with_routing(tmp_path):
     typed = GPT2Config.from_dict(config)
     base = arch.build_spec(typed)
     inner = config["n_inner"] // experts
-    routed = dataclasses.replace(base.blocks[1], feed_forward=PartSpec.make("toy_routed", experts=experts, inner=inner))
+    routed = base.blocks[1].with_part("feed_forward", PartSpec.make("toy_routed", experts=experts, inner=inner))
     spec = dataclasses.replace(base, blocks=(base.blocks[0], routed))
     model = DecoderModel(spec, torch.float32, "cuda")
     sources = {k: v for k, v in arch.weight_sources(typed, base).items()
@@ -360,6 +362,7 @@ def test_toy_feed_forward_with_routing(tmp_path):
     sources["blocks.1.feed_forward.up.weight"] = WeightSource("h.1.mlp.c_fc.weight", transpose=True)
     sources["blocks.1.feed_forward.down.weight"] = WeightSource("h.1.mlp.c_proj.weight", transpose=True)
     loaded = load_parameters(folder, model.parameters(), sources, torch.float32, "cuda",
+                             strip_prefixes=arch.strip_prefixes,
                              ignorable=lambda name: name.startswith("h.1.mlp.c_") and name.endswith(".bias"))
     model.bind(loaded)
     engine = Engine(model, num_pages=16, page_size=page_size, max_requests=3, max_step_tokens=64)
@@ -454,6 +457,7 @@ def test_toy_position_encoding_that_rotates_queries_and_keys(tmp_path):
     model = DecoderModel(spec, torch.float32, "cuda")
     sources = {k: v for k, v in arch.weight_sources(typed, base).items() if not k.startswith("position.")}
     loaded = load_parameters(folder, model.parameters(), sources, torch.float32, "cuda",
+                             strip_prefixes=arch.strip_prefixes,
                              ignorable=lambda name: name == "wpe.weight")
     model.bind(loaded)
     engine = Engine(model, num_pages=16, page_size=page_size, max_requests=3, max_step_tokens=64)
@@ -509,11 +513,12 @@ def test_a_windowed_layer_has_pages_of_its_own_and_gives_them_back(tmp_path, dty
     base = arch.build_spec(typed)
     mixer = base.blocks[1].mixer
     from pagedserve_amd.config import PartSpec
-    windowed = dataclasses.replace(base.blocks[1], mixer=PartSpec.make(mixer.kind, **{**mixer.as_dict(), "window": window}))
+    windowed = base.blocks[1].with_part("mixer", PartSpec.make(mixer.kind, **{**mixer.as_dict(), "window": window}))
     spec = dataclasses.replace(base, blocks=(base.blocks[0], windowed))
     torch_dtype = torch.float32 if dtype == "float32" else torch.bfloat16
     model = DecoderModel(spec, torch_dtype, "cuda")
-    model.bind(load_parameters(folder, model.parameters(), arch.weight_sources(typed, spec), torch_dtype, "cuda"))
+    model.bind(load_parameters(folder, model.parameters(), arch.weight_sources(typed, spec), torch_dtype, "cuda",
+                               strip_prefixes=arch.strip_prefixes))
     groups, _ = model.cache_requirements()
     assert sorted(g.window for g in groups) == [0, window]
     # so few pages that the windowed group must reuse what it gave back: two requests of up to

@@ -145,11 +145,26 @@ def test_causality_and_position_table(which):
 
 
 def test_inverse_layer_scaling():
+    """config.json's ``scale_attn_by_inverse_layer_idx`` divides the scores of layer i (from
+    0) by i + 1: the key's documented meaning; the reference never reads it, so nothing in the
+    reference pins it.  What can be pinned: the scale is one multiplication of the scores, so
+    the option equals a model without it whose query weights of layer i are divided by i + 1."""
     config = dict(helpers.TINY_B)
-    assert P.attention_scale(config, 0) == pytest.approx(48 ** -0.5)
-    assert P.attention_scale(config, 2) == pytest.approx(48 ** -0.5 / 3)
     weights = _weights(config, 9)
     ids = helpers.random_tokens(12, config["vocab_size"], 10)
+    folded = dict(weights)
+    d = config["n_embd"]
+    for layer in range(config["n_layer"]):
+        w = weights[f"h.{layer}.attn.c_attn.weight"].clone()
+        bias = weights[f"h.{layer}.attn.c_attn.bias"].clone()
+        w[:, :d] /= layer + 1
+        bias[:d] /= layer + 1
+        folded[f"h.{layer}.attn.c_attn.weight"], folded[f"h.{layer}.attn.c_attn.bias"] = w, bias
+    torch.testing.assert_close(P.forward_logits(config, weights, ids),
+                               P.forward_logits(dict(config, scale_attn_by_inverse_layer_idx=False), folded, ids),
+                               atol=1e-10, rtol=1e-10)
+    assert P.attention_scale(config, 0) == pytest.approx(48 ** -0.5)
+    assert P.attention_scale(config, 2) == pytest.approx(48 ** -0.5 / 3)
     one_layer = dict(config, n_layer=1)
     off = dict(one_layer, scale_attn_by_inverse_layer_idx=False)
     # layer 0 is divided by 1: the option changes nothing in a one-layer model ...
@@ -160,20 +175,44 @@ def test_inverse_layer_scaling():
 
 
 def test_norms_stand_before_the_sublayers():
-    """Pre-norm: scaling the residual stream's input by 1 + tiny noise must change the result
-    through the un-normed skip path; with post-norm it would not.  Checked on one block by
-    the identity h_out - h_in = attn(LN1(h_in)) + mlp(LN2(h_in + attn))."""
-    config = dict(helpers.TINY_A, n_layer=1)
-    weights = _weights(config, 11)
+    """Pre-norm: a norm only feeds its sub-layer, the stream itself is never normed.  LayerNorm
+    forgets a positive factor, so with the feed-forward's output projection zeroed
+    block(3 h) - block(h) = 2 h (the attention term is the same for both), and likewise with
+    the attention's output projection zeroed.  A block that norms after the sum, or norms the
+    stream in place, gives a bounded difference instead."""
+    config = dict(helpers.TINY_A, n_layer=1, layer_norm_epsilon=1e-12)
     g = torch.Generator().manual_seed(12)
     h = torch.randn(7, config["n_embd"], generator=g, dtype=torch.float64)
-    out = P.block(h, weights, config, 0)
-    eps = config["layer_norm_epsilon"]
-    a = P.attention_sublayer(P.layer_norm(h, weights["h.0.ln_1.weight"], weights["h.0.ln_1.bias"], eps),
-                             weights, "h.0.", config["n_head"], P.attention_scale(config, 0))
-    m = P.mlp_sublayer(P.layer_norm(h + a, weights["h.0.ln_2.weight"], weights["h.0.ln_2.bias"], eps),
-                       weights, "h.0.", config["activation_function"])
-    torch.testing.assert_close(out, h + a + m)
+    for silenced in ("mlp.c_proj", "attn.c_proj"):
+        weights = _weights(config, 11)
+        for kind in ("weight", "bias"):
+            weights[f"h.0.{silenced}.{kind}"] = torch.zeros_like(weights[f"h.0.{silenced}.{kind}"])
+        difference = P.block(3.0 * h, weights, config, 0) - P.block(h, weights, config, 0)
+        torch.testing.assert_close(difference, 2.0 * h, atol=1e-8, rtol=0)
+        # the sub-layer that is left does contribute
+        assert float((P.block(h, weights, config, 0) - h).abs().max()) > 1e-2
+
+
+def test_second_norm_reads_the_stream_after_attention():
+    """With the attention's output matrix zeroed its sub-layer adds its output bias b to every
+    row, so the block is h + b + MLP(LN2(h + b)), written here with library routines.  A block
+    whose second norm reads h, or whose feed-forward result replaces the stream, fails."""
+    config = dict(helpers.TINY_B, n_layer=1)
+    weights = _weights(config, 21)
+    weights["h.0.attn.c_proj.weight"] = torch.zeros_like(weights["h.0.attn.c_proj.weight"])
+    b = weights["h.0.attn.c_proj.bias"] * 20.0
+    weights["h.0.attn.c_proj.bias"] = b
+    g = torch.Generator().manual_seed(22)
+    h = torch.randn(5, config["n_embd"], generator=g, dtype=torch.float64)
+    stream = h + b
+    normed = F.layer_norm(stream, (config["n_embd"],), weights["h.0.ln_2.weight"], weights["h.0.ln_2.bias"],
+                          config["layer_norm_epsilon"])
+    hidden = F.gelu(torch.addmm(weights["h.0.mlp.c_fc.bias"], normed, weights["h.0.mlp.c_fc.weight"]))
+    expected = stream + torch.addmm(weights["h.0.mlp.c_proj.bias"], hidden, weights["h.0.mlp.c_proj.weight"])
+    torch.testing.assert_close(P.block(h, weights, config, 0), expected, atol=1e-10, rtol=1e-10)
+    wrong = F.layer_norm(h, (config["n_embd"],), weights["h.0.ln_2.weight"], weights["h.0.ln_2.bias"],
+                         config["layer_norm_epsilon"])
+    assert float((wrong - normed).abs().max()) > 1e-2
 
 
 def test_untied_head_and_greedy():

@@ -363,3 +363,50 @@ def test_running_ahead_decisions(run_ahead):
             assert len(step) <= 4
     else:
         assert scheduler.steps_run_ahead == 0 and engine.most_outstanding == 1
+
+
+@pytest.mark.parametrize("strategy", [ORCA_STRATEGY, SARATHI_STRATEGY])
+def test_decoding_requests_beyond_the_limit_take_turns(strategy):
+    """Six decoding requests, four per iteration: each is served in two of every three
+    iterations, none waits for another to finish (the reference always takes the lowest ids,
+    src/scheduler/orca_scheduler.py:165-166)."""
+    engine = FakeEngine(max_requests=8)
+    scheduler, _ = make(strategy, engine=engine, max_batch_size=6, prefill_chunk_size=8,
+                        max_prefill_requests=6)
+    ids = [scheduler.add_token_request([i + 1, i + 2], max_new_tokens=13) for i in range(6)]
+    while scheduler.waiting:
+        scheduler.step()
+    scheduler.max_batch_size = 4
+    served = {rid: 0 for rid in ids}
+    for _ in range(9):
+        step_ids = list(scheduler.step())
+        assert len(step_ids) == 4
+        for rid in step_ids:
+            served[rid] += 1
+        # entries stay in arrival order
+        assert [rid for rid, _, _ in engine.steps[-1]] == sorted(step_ids)
+    assert set(served.values()) == {6}
+    scheduler.run_until_complete()
+    for i, rid in enumerate(ids):
+        assert scheduler.finished[rid].generated_token_ids == expected_tokens([i + 1, i + 2], 13)
+
+
+def test_no_end_token_can_be_said():
+    """``eos_token_id=None`` means that no token ends a request, whatever the tokenizer's end
+    token is; leaving the argument out takes the tokenizer's."""
+    class EndSampler:
+        def sample(self, logits, params, keys, indices, seeds):
+            return [VOCAB - 1 for _ in indices]
+
+    tokenizer = SimpleNamespace(eos_token_id=VOCAB - 1, encode=lambda text: [1], decode=lambda ids: "")
+    scheduler = ContinuousBatchScheduler(FakeEngine(), EndSampler(), tokenizer=tokenizer,
+                                         eos_token_id=None, max_batch_size=8)
+    rid = scheduler.add_token_request([1, 2], max_new_tokens=4)
+    scheduler.run_until_complete()
+    assert scheduler.finished[rid].generated_token_ids == [VOCAB - 1] * 4
+    assert scheduler.finished[rid].finish_reason == "length"
+    scheduler = ContinuousBatchScheduler(FakeEngine(), EndSampler(), tokenizer=tokenizer, max_batch_size=8)
+    rid = scheduler.add_token_request([1, 2], max_new_tokens=4)
+    scheduler.run_until_complete()
+    assert scheduler.finished[rid].finish_reason == "stop"
+    assert scheduler.finished[rid].generated_token_ids == [VOCAB - 1]
