@@ -7,8 +7,20 @@ function over a batch of single tokens, token selection on the GPU and the copy 
 chosen tokens to the host.  The default run decodes a batch of 8 requests whose contexts
 end at the model's context length, with random weights and uniform-random prompt ids.
 One JSON line is printed: decoded tokens a second (``value``), the 2,048-token prefill
-step (``prefill``), the decode step against the HBM roofline (``roofline``) and decode at
-batch 1 and 64 (``points``).
+step (``prefill``), the decode step against the HBM roofline (``roofline``), decode at
+batch 1 and 64 with contexts that end at the context length, and the benchmark
+configuration's own decode points: prompts of 128 and 512 tokens with 128 output tokens at
+batch 1, 8 and 64 (``points``, tokens a second; ``points_roofline``, each point's fraction of
+the HBM roofline).
+
+    python bench.py --workload medium      GPT-2 medium shape: a Poisson stream of 256
+                                           requests (prompts 32-896, outputs 16-128),
+                                           continuous batching with prompt portions of 512
+    python bench.py --workload xl          GPT-2 XL shape: 64 requests of 768 + 256 tokens,
+                                           temperature 0.8, seed 7
+
+print one JSON line each about their own run (tokens a second, time to first token, time per
+output token, graphs recorded and dropped).
 """
 
 import argparse
@@ -27,6 +39,8 @@ SMALL = {
     "layer_norm_epsilon": 1e-5, "activation_function": "gelu_new", "tie_word_embeddings": True,
     "eos_token_id": None,
 }
+MEDIUM = dict(SMALL, n_layer=24, n_embd=1024, n_head=16, n_inner=4096)
+XL = dict(SMALL, n_layer=48, n_embd=1600, n_head=25, n_inner=6400)
 PAGE_SIZE = 16
 PREFILL_TOKENS = 2048
 
@@ -37,12 +51,12 @@ def _random_prompt(generator, length, vocab):
     return torch.randint(0, vocab, (length,), generator=generator).tolist()
 
 
-def _build(dtype, max_requests, max_step_tokens, layers=None):
+def _build(dtype, max_requests, max_step_tokens, layers=None, shape=SMALL):
     from pagedserve_amd.engine import Engine
     from pagedserve_amd.model import random_model
     from pagedserve_amd.sampling.sampler import Sampler
 
-    raw = dict(SMALL)
+    raw = dict(shape)
     if layers is not None:
         raw["n_layer"] = layers
     model, config = random_model(raw, seed=0, dtype=dtype, device="cuda")
@@ -87,6 +101,40 @@ def decode_run(engine, sampler, config, batch, context_end, steps, warmup, seed=
     torch.cuda.synchronize()
     elapsed = time.perf_counter() - started
     mean_context = context_end - 1 - (steps - 1) / 2.0 - ahead / 2.0
+    while scheduler.has_work():
+        scheduler.step()
+    return elapsed, mean_context
+
+
+def decode_point(engine, sampler, config, batch, prompt_len, output_tokens, warmup=8, seed=0):
+    """Seconds for ``output_tokens`` decode steps of ``batch`` requests with prompts of
+    ``prompt_len`` tokens (the steps after the prompts are in and ``warmup`` further steps
+    have run), and the mean context length during them."""
+    import torch
+
+    from pagedserve_amd.engine import ContinuousBatchScheduler
+    from pagedserve_amd.sampling import SamplingParams
+
+    generator = torch.Generator().manual_seed(seed)
+    ahead = -(-batch * prompt_len // engine.max_step_tokens)
+    new_tokens = output_tokens + warmup + 1 + ahead
+    scheduler = ContinuousBatchScheduler(engine, sampler, max_batch_size=batch,
+                                         scheduling_strategy="orca", eos_token_id=None)
+    params = SamplingParams(max_new_tokens=new_tokens, ignore_eos=True)
+    for _ in range(batch):
+        scheduler.add_token_request(_random_prompt(generator, prompt_len, config.vocab_size),
+                                    new_tokens, sampling=params)
+    while scheduler.waiting:
+        scheduler.step()
+    for _ in range(warmup):
+        scheduler.step()
+    torch.cuda.synchronize()
+    started = time.perf_counter()
+    for _ in range(output_tokens):
+        scheduler.step()
+    torch.cuda.synchronize()
+    elapsed = time.perf_counter() - started
+    mean_context = prompt_len + warmup + ahead / 2.0 + (output_tokens + 1) / 2.0
     while scheduler.has_work():
         scheduler.step()
     return elapsed, mean_context
@@ -138,6 +186,123 @@ def decode_bytes(config, element_size, batch, mean_context):
     return matrices * element_size + vectors * 4 + cache
 
 
+def medium_workload(args):
+    """GPT-2 medium shape: a Poisson stream of 256 requests with uniform-random prompt lengths
+    32-896 and output lengths 16-128, continuous batching with prompt portions of 512."""
+    import random
+
+    import torch
+
+    from pagedserve_amd.engine import ContinuousBatchScheduler
+    from pagedserve_amd.engine.workload import TraceRequest, arrival_offsets, run_arrival_trace
+    from pagedserve_amd.sampling import SamplingParams
+
+    engine, sampler, config = _build(args.dtype, max_requests=64, max_step_tokens=PREFILL_TOKENS,
+                                     layers=args.layers, shape=MEDIUM)
+    scheduler = ContinuousBatchScheduler(engine, sampler, max_batch_size=64, eos_token_id=None,
+                                         scheduling_strategy="sarathi", prefill_chunk_size=512)
+    lengths = random.Random(0)
+    generator = torch.Generator().manual_seed(0)
+    requests = []
+    for _ in range(args.requests):
+        prompt, output = lengths.randint(32, 896), lengths.randint(16, 128)
+        requests.append(TraceRequest(_random_prompt(generator, prompt, config.vocab_size), output,
+                                     SamplingParams(max_new_tokens=output, ignore_eos=True)))
+    # the kernels' code is loaded by a few requests that are not part of the measurement
+    for request in requests[:2]:
+        scheduler.add_token_request(list(request.prompt_token_ids)[:80], 4,
+                                    sampling=SamplingParams(max_new_tokens=4, ignore_eos=True))
+    scheduler.run_until_complete()
+    offsets = arrival_offsets(args.request_rate, len(requests), "poisson", seed=1234)
+    summary = run_arrival_trace(scheduler, requests, offsets, synchronize=torch.cuda.synchronize)
+    engine.cache.check_invariants()
+    graphs = engine.graph_summary()
+
+    def ms(group):
+        return {key: (None if value is None else round(value * 1e3, 3)) for key, value in group.items()}
+
+    return {
+        "metric": "output tok/s of a Poisson stream of 256 requests (GPT-2 medium shape, prompt portions of 512)",
+        "value": round(summary["output_tokens_per_second"], 1), "unit": "tokens/s", "n_gpus": 1,
+        "higher_is_better": True, "dtype": "bf16" if args.dtype == "bfloat16" else "fp32",
+        "data": "synthetic (random weights, uniform-random prompt ids and lengths, seeded arrivals)",
+        "wall_s": round(summary["wall_seconds"], 3), "requests": summary["requests"],
+        "prompt_tokens": summary["prompt_tokens"], "output_tokens": summary["output_tokens"],
+        "total_tok_s": round(summary["total_tokens_per_second"], 1), "iterations": summary["iterations"],
+        "steps_run_ahead": scheduler.steps_run_ahead,
+        "ttft_ms": ms(summary["ttft_seconds"]), "tpot_ms": ms(summary["tpot_seconds"]),
+        "e2e_ms": ms(summary["e2e_seconds"]),
+        "graphs": {"kept": graphs["captured_graphs"], "captures": graphs["captures"],
+                   "evicted": graphs["evicted"], "capture_ms": round(graphs["capture_seconds"] * 1e3, 1),
+                   "replays": graphs["graph_replays"], "layouts_remembered": graphs["layouts_remembered"]},
+        "config": {"model": "gpt2-medium-shape", "n_layer": config.n_layer, "n_layer_of_config": MEDIUM["n_layer"],
+                   "n_embd": config.n_embd, "n_head": config.n_head, "n_inner": config.n_inner,
+                   "vocab_size": config.vocab_size, "n_positions": config.n_positions,
+                   "request_rate": args.request_rate, "arrivals": "poisson seed 1234", "strategy": "sarathi",
+                   "prefill_chunk_size": 512, "max_batch_size": 64, "page_size": PAGE_SIZE},
+    }
+
+
+def xl_workload(args):
+    """GPT-2 XL shape: 64 concurrent requests of 768 prompt + 256 output tokens, temperature
+    0.8, seed 7."""
+    import torch
+
+    from pagedserve_amd.engine import ContinuousBatchScheduler
+    from pagedserve_amd.sampling import SamplingParams
+
+    engine, sampler, config = _build(args.dtype, max_requests=64, max_step_tokens=PREFILL_TOKENS,
+                                     layers=args.layers, shape=XL)
+    scheduler = ContinuousBatchScheduler(engine, sampler, max_batch_size=64, eos_token_id=None)
+    generator = torch.Generator().manual_seed(0)
+    for _ in range(2):
+        scheduler.add_token_request(_random_prompt(generator, 80, config.vocab_size), 4,
+                                    sampling=SamplingParams(max_new_tokens=4, temperature=0.8, seed=7, ignore_eos=True))
+    scheduler.run_until_complete()
+    prompt_len, output_len, batch = 768, 256, 64
+    for _ in range(batch):
+        scheduler.add_token_request(
+            _random_prompt(generator, prompt_len, config.vocab_size), output_len,
+            sampling=SamplingParams(max_new_tokens=output_len, temperature=0.8, seed=7, ignore_eos=True))
+    torch.cuda.synchronize()
+    started = time.perf_counter()
+    while scheduler.waiting:
+        scheduler.step()
+    torch.cuda.synchronize()
+    prefilled = time.perf_counter() - started
+    steps = 0
+    while scheduler.has_work():
+        scheduler.step()
+        steps += 1
+    torch.cuda.synchronize()
+    wall = time.perf_counter() - started
+    engine.cache.check_invariants()
+    decode_tokens = batch * (output_len - 1)
+    element = 2 if args.dtype == "bfloat16" else 4
+    step_seconds = (wall - prefilled) / steps
+    moved = decode_bytes(config, element, batch, prompt_len + output_len / 2.0)
+    graphs = engine.graph_summary()
+    return {
+        "metric": "decode tok/s of 64 requests x (768 prompt + 256 output), temperature 0.8 seed 7 (GPT-2 XL shape)",
+        "value": round(decode_tokens / (wall - prefilled), 1), "unit": "tokens/s", "n_gpus": 1,
+        "higher_is_better": True, "dtype": "bf16" if args.dtype == "bfloat16" else "fp32",
+        "data": "synthetic (random weights, uniform-random prompt ids)",
+        "wall_s": round(wall, 3), "prefill_s": round(prefilled, 3),
+        "prefill_tok_s": round(batch * prompt_len / prefilled, 1), "decode_steps": steps,
+        "ms_per_step": round(step_seconds * 1e3, 4),
+        "roofline": {"bound": "hbm", "achieved": round(moved / step_seconds / 1e9, 1), "peak": HBM_GBPS,
+                     "unit": "GB/s", "frac": round(moved / step_seconds / 1e9 / HBM_GBPS, 4)},
+        "steps_run_ahead": scheduler.steps_run_ahead,
+        "graphs": {"kept": graphs["captured_graphs"], "captures": graphs["captures"],
+                   "evicted": graphs["evicted"], "capture_ms": round(graphs["capture_seconds"] * 1e3, 1)},
+        "config": {"model": "gpt2-xl-shape", "n_layer": config.n_layer, "n_layer_of_config": XL["n_layer"],
+                   "n_embd": config.n_embd, "n_head": config.n_head, "n_inner": config.n_inner,
+                   "vocab_size": config.vocab_size, "n_positions": config.n_positions, "global_batch": batch,
+                   "prompt_len": prompt_len, "output_len": output_len, "temperature": 0.8, "seed": 7,
+                   "page_size": PAGE_SIZE},
+    }
+
+
 def main(argv=None):
     parser = argparse.ArgumentParser()
     parser.add_argument("--gpus", type=int, default=1)
@@ -149,6 +314,12 @@ def main(argv=None):
     parser.add_argument("--no-points", action="store_true", help="skip batch 1 / 64 and prefill")
     parser.add_argument("--prefill-only", action="store_true",
                         help="only the 2,048-token prefill step, --steps times (for profiles)")
+    parser.add_argument("--workload", choices=("small", "medium", "xl"), default="small",
+                        help="small: the decode / prefill record (default); medium: the Poisson "
+                             "stream at GPT-2 medium shape; xl: 64 x (768 + 256) at GPT-2 XL shape")
+    parser.add_argument("--requests", type=int, default=256, help="requests of --workload medium")
+    parser.add_argument("--request-rate", type=float, default=400.0,
+                        help="mean arrivals a second of --workload medium")
     args = parser.parse_args(argv)
     if args.gpus != 1:
         print(f"bench.py measures one GPU; --gpus {args.gpus} is not supported by this engine")
@@ -157,6 +328,10 @@ def main(argv=None):
     import torch
 
     torch.cuda.init()
+    if args.workload != "small":
+        record = medium_workload(args) if args.workload == "medium" else xl_workload(args)
+        print(json.dumps(record), flush=True)
+        return 0
     short = "bf16" if args.dtype == "bfloat16" else "fp32"
     element = 2 if args.dtype == "bfloat16" else 4
     engine, sampler, config = _build(args.dtype, max_requests=64, max_step_tokens=PREFILL_TOKENS,
@@ -206,7 +381,19 @@ def main(argv=None):
             t, _ = decode_run(engine, sampler, config, batch, context, steps, min(args.warmup, 8),
                               seed=batch)
             points[f"decode_b{batch}"] = round(batch * steps / t, 1)
+        # the benchmark configuration's decode points: prompts of 128 and 512 tokens, 128
+        # output tokens, at batch 1, 8 and 64
+        fractions = {}
+        for prompt_len in (128, 512):
+            for batch in (1, 8, 64):
+                t, mean_context = decode_point(engine, sampler, config, batch, prompt_len, 128,
+                                               seed=prompt_len + batch)
+                name = f"p{prompt_len}_b{batch}"
+                points[name] = round(batch * 128 / t, 1)
+                fractions[name] = round(decode_bytes(config, element, batch, mean_context)
+                                        / (t / 128) / 1e9 / HBM_GBPS, 4)
         record["points"] = points
+        record["points_roofline"] = fractions
     print(json.dumps(record), flush=True)
     return 0
 

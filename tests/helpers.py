@@ -113,6 +113,16 @@ def plain_logits(folder, token_ids, bfloat16=False):
     return plain_gpt2.forward_logits(config, weights, token_ids)
 
 
+def plain_logits_of_many(folder, requests, bfloat16=False, device="cpu"):
+    """{request: float64 logits} of the plain implementation with the weights read once; on
+    ``device`` the same torch formulas run in float64 (large models take minutes on the CPU)."""
+    config, weights = plain_gpt2.read_model_folder(folder, torch.float64)
+    if bfloat16:
+        weights = plain_gpt2.round_weights_to_bfloat16(weights)
+    weights = {name: tensor.to(device) for name, tensor in weights.items()}
+    return {rid: plain_gpt2.forward_logits(config, weights, tokens).cpu() for rid, tokens in requests.items()}
+
+
 def random_tokens(count, vocab, seed):
     g = torch.Generator().manual_seed(seed)
     return torch.randint(0, vocab, (count,), generator=g).tolist()

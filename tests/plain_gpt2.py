@@ -111,8 +111,8 @@ def causal_attention(q, k, v, scale, window=0):
     """
     tokens = q.shape[1]
     scores = q @ k.transpose(-1, -2) * scale
-    query_pos = torch.arange(tokens).unsqueeze(1)
-    key_pos = torch.arange(tokens).unsqueeze(0)
+    query_pos = torch.arange(tokens, device=q.device).unsqueeze(1)
+    key_pos = torch.arange(tokens, device=q.device).unsqueeze(0)
     hidden = key_pos > query_pos
     if window > 0:
         hidden = hidden | (query_pos - key_pos >= window)
@@ -175,8 +175,9 @@ def lm_head(h, weights, config):
 def forward_logits(config, weights, token_ids, first_position=0):
     """Logits [T, V] at every position of one whole sequence
     (src/model/paged_decoder.py:316-331)."""
-    ids = torch.as_tensor(token_ids, dtype=torch.long)
-    positions = torch.arange(first_position, first_position + ids.numel())
+    device = weights["wte.weight"].device
+    ids = torch.as_tensor(token_ids, dtype=torch.long, device=device)
+    positions = torch.arange(first_position, first_position + ids.numel(), device=device)
     h = embed(weights["wte.weight"], weights["wpe.weight"], ids, positions)
     for layer_index in range(config["n_layer"]):
         h = block(h, weights, config, layer_index)

@@ -410,3 +410,56 @@ def test_no_end_token_can_be_said():
     scheduler.run_until_complete()
     assert scheduler.finished[rid].finish_reason == "stop"
     assert scheduler.finished[rid].generated_token_ids == [VOCAB - 1]
+
+
+def test_arrival_trace_runner_times_requests_by_its_clock():
+    """Requests are submitted when their time has come (not before), every token gets the time
+    at which its iteration ended, and TTFT / TPOT follow comparison_benchmark.py:444-472."""
+    from pagedserve_amd.engine.workload import (TraceRequest, arrival_offsets, percentile,
+                                                 run_arrival_trace)
+
+    offsets = arrival_offsets(4.0, 5, "poisson", seed=3)
+    assert offsets[0] == 0.0 and offsets == sorted(offsets) and len(offsets) == 5
+    assert offsets == arrival_offsets(4.0, 5, "poisson", seed=3) != arrival_offsets(4.0, 5, "poisson", seed=4)
+    assert arrival_offsets(2.0, 3, "fixed") == [0.0, 0.5, 1.0]
+    assert arrival_offsets(float("inf"), 3) == [0.0, 0.0, 0.0]
+    assert percentile([1, 2, 3, 4], 50) == 2.5 and percentile([5], 99) == 5
+
+    class Clock:
+        now = 0.0
+
+        def __call__(self):
+            return self.now
+
+    clock = Clock()
+    scheduler, engine = make(max_batch_size=8)
+    plain_step = scheduler.step
+
+    def timed_step():
+        clock.now += 0.25          # every iteration takes a quarter of a second
+        return plain_step()
+
+    scheduler.step = timed_step
+
+    def idle(seconds):
+        clock.now += max(seconds, 1e-3)
+
+    requests = [TraceRequest([1, 2, 3], 3), TraceRequest([4, 5], 2), TraceRequest([6], 4)]
+    offsets = [0.0, 0.6, 5.0]
+    summary = run_arrival_trace(scheduler, requests, offsets, clock=clock, idle=idle)
+    records = summary["records"]
+    assert summary["completed"] == 3 and summary["output_tokens"] == 9 and summary["prompt_tokens"] == 6
+    # the first request: tokens at 0.25, 0.5, 0.75
+    assert records[0].token_times == pytest.approx([0.25, 0.5, 0.75])
+    assert records[0].metrics()["ttft"] == pytest.approx(0.25) and records[0].metrics()["tpot"] == pytest.approx(0.25)
+    # the second arrives at 0.6, is seen at 0.75, its first token comes at 1.0
+    assert records[1].submitted_at == pytest.approx(0.75)
+    assert records[1].metrics()["ttft"] == pytest.approx(1.0 - 0.6)
+    assert records[1].metrics()["queue_delay"] == pytest.approx(0.15)
+    # the third waits for its time while nothing runs
+    assert 5.0 <= records[2].submitted_at < 5.01 and len(records[2].token_times) == 4
+    assert summary["wall_seconds"] == pytest.approx(records[2].token_times[-1])
+    assert summary["ttft_seconds"]["max"] == pytest.approx(0.4)
+    for index, request in enumerate(requests):
+        assert scheduler.finished[records[index].request_id].generated_token_ids == \
+            expected_tokens(list(request.prompt_token_ids), request.max_new_tokens)
