@@ -528,6 +528,10 @@ __global__ __launch_bounds__(64 * SK_WAVES) void gemm_nt_skinny_norm_kernel(
 
 // --------------------------------------------------------------------------------- host
 bool ps_gemm_nt_bf16_tiled_supported(const void* a, const void* w, int m, int k, int lda);
+bool ps_gemm_nt_bf16_wide_supported(const void* a, const void* w_packed, int m, int n, int k, int lda);
+int ps_gemm_nt_bf16_wide(const void* a, const void* w_packed, const float* bias, void* c, int m,
+                         int n, int k, int lda, int ldc, int c_dtype, int epilogue,
+                         const KvScatter& scatter, int rows_per_block, hipStream_t s);
 int ps_gemm_nt_bf16_tiled(const void* a, const void* w, const float* bias, void* c, int m, int n,
                           int k, int lda, int ldc, int c_dtype, int epilogue,
                           const KvScatter& scatter, hipStream_t s);
@@ -731,6 +735,8 @@ int ps_gemm_nt_mfma(const void* a, const void* w, const float* bias, void* c, in
                  m, n, k);
     return 1;
   }
+  if (dtype == PS_BF16 && ps_gemm_nt_bf16_wide_supported(a, wp, m, n, k, lda))
+    return ps_gemm_nt_bf16_wide(a, wp, bias, c, m, n, k, lda, ldc, c_dtype, epilogue, scatter, 0, s);
   if (dtype == PS_BF16 && ps_gemm_nt_bf16_tiled_supported(a, w, m, k, lda))
     return ps_gemm_nt_bf16_tiled(a, w, bias, c, m, n, k, lda, ldc, c_dtype, epilogue, scatter, s);
   if (dtype == PS_F32 && c_dtype == PS_F32)

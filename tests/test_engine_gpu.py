@@ -281,3 +281,43 @@ def test_reference_test_configuration(tmp_path, num_layers, dtype):
     error, scale, where = helpers.max_error(rows, {"request": expected})
     assert len(rows) == 5
     assert error <= helpers.TOLERANCE[dtype] * scale, (error, scale, where)
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_more_layouts_than_recorded_graphs_are_kept(folders, references, dtype):
+    """More step layouts than the engine keeps graphs for, each coming back often enough to be
+    recorded, while decode steps replayed from a graph run between them: recorded layouts are
+    dropped (their graphs destroyed only once nothing launched before can still be running) and
+    every logit still matches the plain implementation."""
+    from pagedserve_amd.engine import Engine, StepEntry
+    from pagedserve_amd.model import load_model
+
+    folder, config, page_size = folders["B"]
+    requests = _requests("B", config)
+    model, _ = load_model(folder, dtype=dtype)
+    engine = Engine(model, num_pages=40, page_size=page_size, max_requests=4, max_step_tokens=128)
+    engine.max_graphs = 3
+    rows = {}
+
+    def run(entries):
+        out = engine.step(entries)
+        values = out.logits.double().cpu()
+        for index, key in enumerate(out.rows):
+            rows[key] = values[index]
+
+    run([StepEntry("r5", requests["r5"][:60], list(range(60)))])
+    decoded = 60
+    for size in (2, 3, 4, 5, 6, 7):            # six layouts of a prompt portion, each four times
+        for repeat in range(4):
+            name = f"r{repeat % 4}"
+            run([StepEntry(name, requests[name][:size], list(range(size)))])
+            engine.finish(name)
+            run([StepEntry("r5", [requests["r5"][decoded]], [0])])     # a replayed decode step
+            decoded += 1
+    summary = engine.graph_summary()
+    assert summary["captures"] >= 7 and summary["evicted"] >= 4 and summary["captured_graphs"] <= 3, summary
+    assert not summary["capture_failures"], summary
+    error, scale, where = helpers.max_error(rows, references[("B", dtype == "bfloat16")])
+    assert error <= helpers.TOLERANCE[dtype] * scale, (error, scale, where)
+    torch.cuda.synchronize()
+    engine.cache.check_invariants()

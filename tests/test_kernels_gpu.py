@@ -758,3 +758,80 @@ def test_linear_chain_with_packed_activations(m, inner, width):
         (F.layer_norm(h.double(), (width,), gamma.double(), beta.double(), 1e-5).to(dtype).double()
          @ up.double().t() + up_bias.double()), approximate="tanh").to(dtype).double() @ down.double().t() + down_bias.double()
     assert (fast.double() - reference).abs().max().item() <= 2e-2 * reference.abs().max().item()
+
+
+def _wide_entry():
+    import ctypes
+
+    from pagedserve_amd.ops import library
+
+    lib = library.load_library()
+    fn = lib.ps_gemm_nt_wide
+    fn.argtypes = [ctypes.c_void_p] * 4 + [ctypes.c_int] * 8 + [ctypes.c_void_p]
+    fn.restype = ctypes.c_int
+    return lib, fn
+
+
+@pytest.mark.parametrize("m,n,k", [(256, 512, 1024), (300, 1000, 320), (333, 770, 64), (512, 3072, 1024), (97, 257, 128),
+                                   (2048, 768, 3072), (700, 1600, 1600), (130, 2304, 704)])
+@pytest.mark.parametrize("rows_per_block", [32, 64, 128])
+@pytest.mark.parametrize("epilogue", ["none", "gelu_tanh", "residual"])
+def test_gemm_wide_block_shapes(m, n, k, rows_per_block, epilogue):
+    """The product whose weights come out of the packed copy straight into registers, at each
+    of its block shapes: one k tile and many (the ring of three and its last tiles), rows and
+    columns that end inside a block, a column count that ends inside a 16-row tile of the copy."""
+    from pagedserve_amd.ops import kernels
+
+    if epilogue == "gelu_tanh" and rows_per_block != 64 and m > 400:
+        pytest.skip("one block shape is enough for the activation at the larger sizes")
+    lib, fn = _wide_entry()
+    a = _rand((m, k), torch.bfloat16, 310, 1.0)
+    w = _rand((n, k), torch.bfloat16, 311, 1.0 / math.sqrt(k))
+    bias = _rand((n,), torch.float32, 312)
+    packed = kernels.pack_decode_weight(w)
+    product = a.double() @ w.double().t() + bias.double()
+    if epilogue == "residual":
+        out = _rand((m, n), torch.float32, 313)
+        expected = out.double() + product
+    else:
+        out = torch.full((m, n), float("nan"), dtype=torch.bfloat16, device="cuda")
+        expected = F.gelu(product, approximate="tanh") if epilogue == "gelu_tanh" else product
+    status = fn(a.data_ptr(), packed.data_ptr(), bias.data_ptr(), out.data_ptr(), m, n, k, a.stride(0),
+                out.stride(0), 0 if out.dtype == torch.float32 else 1, kernels.EPILOGUES[epilogue],
+                rows_per_block, torch.cuda.current_stream().cuda_stream)
+    assert status == 0, lib.ps_last_error().decode()
+    atol, rtol = (1e-4, 1e-5) if epilogue == "residual" else (4e-2, 2e-2)
+    torch.testing.assert_close(out.double(), expected, atol=atol, rtol=rtol)
+
+
+def test_linear_takes_the_wide_product_for_long_k():
+    """Through ``kernels.linear``: many rows, a long k and the packed copy select the wide
+    product (same result as without the copy, which takes the kernel with both operands in
+    LDS), also with the key/value scatter behind it."""
+    from pagedserve_amd.ops import kernels
+
+    m, k = 600, 1024
+    heads, kv_heads, head_dim, page_size = 8, 4, 64, 16
+    q_cols, kv_cols = heads * head_dim, kv_heads * head_dim
+    n = q_cols + 2 * kv_cols
+    lens = [350, 280]
+    k_pool, v_pool, tables = _paged_fixture(torch.bfloat16, lens, kv_heads, head_dim, page_size, 320)
+    tok_item = torch.tensor([0] * 330 + [1] * 270, dtype=torch.int32, device="cuda")
+    tok_pos = torch.tensor(list(range(20, 350)) + list(range(10, 280)), dtype=torch.int32, device="cuda")
+    x = _rand((m, k), torch.bfloat16, 321)
+    w = _rand((n, k), torch.bfloat16, 322, 1.0 / math.sqrt(k))
+    bias = _rand((n,), torch.float32, 323)
+    packed = kernels.pack_decode_weight(w)
+    plain = torch.empty((m, n), dtype=torch.bfloat16, device="cuda")
+    kernels.linear(x, w, bias, plain)
+    k_ref, v_ref = k_pool.clone(), v_pool.clone()
+    kernels.kv_write(plain[:, q_cols:q_cols + kv_cols], plain[:, q_cols + kv_cols:], k_ref, v_ref, tok_item, tok_pos, tables)
+    out = torch.empty_like(plain)
+    kernels.linear(x, w, bias, out, packed=packed,
+                   scatter=(k_pool, v_pool, tok_item, tok_pos, tables, q_cols, kv_cols))
+    expected = x.double() @ w.double().t() + bias.double()
+    torch.testing.assert_close(out.double(), expected, atol=4e-2, rtol=2e-2)
+    # the two kernels add the k tiles in the same order: the same bits
+    assert torch.equal(out, plain)
+    assert torch.equal(k_pool.view(torch.int16), k_ref.view(torch.int16))
+    assert torch.equal(v_pool.view(torch.int16), v_ref.view(torch.int16))
