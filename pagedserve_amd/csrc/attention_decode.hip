@@ -28,6 +28,7 @@ struct Raw8;
 template <>
 struct Raw8<float> {
   float4 a, b;
+  template <bool NT>
   __device__ inline void load(const float* p) {
     a = *reinterpret_cast<const float4*>(p);
     b = *reinterpret_cast<const float4*>(p + 4);
@@ -41,7 +42,20 @@ struct Raw8<float> {
 template <>
 struct Raw8<bf16_t> {
   uint4 raw;
-  __device__ inline void load(const bf16_t* p) { raw = *reinterpret_cast<const uint4*>(p); }
+  // NT: a load that leaves no line behind in the caches.  Keys and values are read once per
+  // step; with more blocks than compute units, where memory bandwidth is the limit, such loads
+  // measured 13 % faster (5.7 against 5.0 TB/s at 64 requests); with fewer blocks, where the
+  // latency of a block's one round of loads is the limit, slightly slower.
+  template <bool NT>
+  __device__ inline void load(const bf16_t* p) {
+    if constexpr (NT) {
+      typedef __attribute__((ext_vector_type(4))) uint32_t vec_t;
+      const vec_t v = __builtin_nontemporal_load(reinterpret_cast<const vec_t*>(p));
+      raw = make_uint4(v.x, v.y, v.z, v.w);
+    } else {
+      raw = *reinterpret_cast<const uint4*>(p);
+    }
+  }
   __device__ inline void widen(float* out) const {
     const uint32_t w[4] = {raw.x, raw.y, raw.z, raw.w};
 #pragma unroll
@@ -83,7 +97,7 @@ __device__ inline float groups_sum(float v) {
   return xor_sum<32>(v);
 }
 
-template <typename T, int LPK, int AD_WAVES, int AD_UNROLL>
+template <typename T, int LPK, int AD_WAVES, int AD_UNROLL, bool NT>
 __global__ __launch_bounds__(64 * AD_WAVES) void attention_decode_kernel(
     const T* __restrict__ q, int64_t q_stride, const T* __restrict__ k_pool,
     const T* __restrict__ v_pool, T* __restrict__ out, int64_t out_stride,
@@ -148,8 +162,8 @@ __global__ __launch_bounds__(64 * AD_WAVES) void attention_decode_kernel(
       const int64_t offset =
           (((int64_t)safe_page * kv_heads + kv_head) * page_size + within[u]) * head_dim +
           (has_dims ? dim0 : 0);
-      kr[u].load(k_pool + offset);
-      vr[u].load(v_pool + offset);
+      kr[u].template load<NT>(k_pool + offset);
+      vr[u].template load<NT>(v_pool + offset);
     }
     float s[AD_UNROLL];
     float m_new = m;
@@ -283,13 +297,23 @@ static int launch_decode(const void* q, int64_t q_stride, const void* k_pool, co
     while ((1 << page_shift) < page_size) ++page_shift;
   }
   dim3 grid(count, heads, splits);
-#define PS_LAUNCH_ADW(LPK, WAVES)                                                                \
-  hipLaunchKernelGGL((attention_decode_kernel<T, LPK, WAVES, (WAVES == 16 && sizeof(T) == 2 ? 8 : 4)>), grid, \
+#define PS_LAUNCH_ADN(LPK, WAVES, NT)                                                            \
+  hipLaunchKernelGGL((attention_decode_kernel<T, LPK, WAVES, (WAVES == 16 && sizeof(T) == 2 ? 8 : 4), NT>), grid, \
                      dim3(64 * WAVES), 0, s,                                                     \
                      (const T*)q, q_stride, (const T*)k_pool, (const T*)v_pool, (T*)out,         \
                      out_stride, partial, tok_list, tok_item, tok_pos, tables, table_width,      \
                      heads, kv_heads, head_dim, page_size, page_shift, num_pages,                \
                      scale * 1.4426950408889634f, window, splits)
+  // more blocks than compute units: the step is bound by memory bandwidth, not by one round trip
+  const bool streaming = sizeof(T) == 2 && (int64_t)count * heads * splits > ps_compute_units();
+#define PS_LAUNCH_ADW(LPK, WAVES)          \
+  do {                                     \
+    if (streaming) {                       \
+      PS_LAUNCH_ADN(LPK, WAVES, true);     \
+    } else {                               \
+      PS_LAUNCH_ADN(LPK, WAVES, false);    \
+    }                                      \
+  } while (0)
 #define PS_LAUNCH_AD(LPK)            \
   do {                               \
     if (waves == 16) {               \
@@ -306,6 +330,7 @@ static int launch_decode(const void* q, int64_t q_stride, const void* k_pool, co
   else PS_LAUNCH_AD(32);
 #undef PS_LAUNCH_AD
 #undef PS_LAUNCH_ADW
+#undef PS_LAUNCH_ADN
   PS_CHECK_LAUNCH("ps_attention_decode");
   if (splits > 1) {
     hipLaunchKernelGGL(attention_reduce_kernel<T>, dim3(count, heads), dim3(64), 0, s, partial,

@@ -224,3 +224,6 @@ void ps_set_error(const char* fmt, ...);
       return 2;                                                            \
     }                                                                      \
   } while (0)
+
+// Compute units of the current device (asked once per device; elementwise.hip).
+int ps_compute_units();

@@ -36,6 +36,19 @@ extern "C" int ps_device_info(int* compute_units, int* lds_bytes, char* arch, in
   return 0;
 }
 
+// Compute units of the current device, asked once per device: launch shapes follow it.
+int ps_compute_units() {
+  static int cached[64];
+  int device = 0;
+  if (hipGetDevice(&device) != hipSuccess || device < 0 || device >= 64) return 256;
+  if (cached[device] == 0) {
+    hipDeviceProp_t prop;
+    if (hipGetDeviceProperties(&prop, device) != hipSuccess || prop.multiProcessorCount <= 0) return 256;
+    cached[device] = prop.multiProcessorCount;
+  }
+  return cached[device];
+}
+
 // ---------------------------------------------------------------- embedding
 // h0[t] = scale * wte[id[t]] + wpe[pos[t]]  (reference: src/model/paged_decoder.py:306-314,
 // where the scale is 1).

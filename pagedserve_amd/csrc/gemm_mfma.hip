@@ -562,7 +562,7 @@ static int launch_tiled(const void* a, const void* w, const float* bias, void* c
   constexpr int bk = TG_ROW_BYTES / (int)sizeof(T);
   int k_splits = 1;
   if (epilogue == PS_EPI_RESIDUAL) {
-    const int wanted = (768 + tiles_m * tiles_n - 1) / (tiles_m * tiles_n);
+    const int wanted = (3 * ps_compute_units() + tiles_m * tiles_n - 1) / (tiles_m * tiles_n);
     const int possible = k / (8 * bk) > 0 ? k / (8 * bk) : 1;
     k_splits = wanted < possible ? wanted : possible;
   }
@@ -597,7 +597,7 @@ static void launch_skinny_mb(const void* a, const void* w, const float* bias, vo
   // number of column blocks is a multiple of 8).
   const int row_blocks = (m + 15) / 16;
   const int grid_xy = ((n + 15) / 16) * k_splits;
-  int z = 256 / grid_xy;
+  int z = ps_compute_units() / grid_xy;
   z = z < 1 ? 1 : (z > row_blocks ? row_blocks : z);
   const int per = (row_blocks + z - 1) / z;
   dim3 grid((n + 15) / 16, k_splits, (row_blocks + per - 1) / per);

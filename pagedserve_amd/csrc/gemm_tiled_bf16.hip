@@ -202,8 +202,8 @@ static int launch_variant(const void* a, const void* w, const float* bias, void*
   // place (residual epilogue) k is split over blocks.  Float atomics are slow, so this pays
   // only while the output is small.
   int k_splits = 1;
-  if (epilogue == PS_EPI_RESIDUAL && tiles_m * tiles_n <= 64 && k >= 2048) {
-    k_splits = 256 / (tiles_m * tiles_n);
+  if (epilogue == PS_EPI_RESIDUAL && tiles_m * tiles_n <= ps_compute_units() / 4 && k >= 2048) {
+    k_splits = ps_compute_units() / (tiles_m * tiles_n);
     if (k_splits > k / 256) k_splits = k / 256;
   }
   int k_chunk = (k / TB_BK + k_splits - 1) / k_splits * TB_BK;
@@ -225,7 +225,7 @@ static int launch_variant(const void* a, const void* w, const float* bias, void*
   return 0;
 }
 
-// Tile shapes by the number of blocks they give: the chip has 256 compute units, and a product
+// Tile shapes by the number of blocks they give against the chip's compute units: a product
 // of this size is over in a few microseconds, so filling them counts for more than the reuse
 // inside a large tile.
 template <typename TOut>
@@ -234,9 +234,10 @@ static int launch_tiled_bf16(const void* a, const void* w, const float* bias, vo
                              const KvScatter& scatter, hipStream_t s) {
   const int64_t tiles_128 = (int64_t)((m + 127) / 128) * ((n + 127) / 128);
   const int64_t tiles_128_64 = (int64_t)((m + 127) / 128) * ((n + 63) / 64);
-  if (m > 64 && tiles_128 >= 768)
+  const int units = ps_compute_units();
+  if (m > 64 && tiles_128 >= 3 * units)
     return launch_variant<2, 2, 2, TOut>(a, w, bias, c, m, n, k, lda, ldc, epilogue, scatter, s);
-  if (m > 64 && tiles_128_64 >= 384)
+  if (m > 64 && tiles_128_64 >= units + units / 2)
     return launch_variant<2, 1, 2, TOut>(a, w, bias, c, m, n, k, lda, ldc, epilogue, scatter, s);
   // 64 x 64 tiles.  What a compute unit has in flight decides how long a k tile takes to
   // arrive from memory.  Many blocks fill a unit by their number and keep two stages, which
@@ -247,9 +248,9 @@ static int launch_tiled_bf16(const void* a, const void* w, const float* bias, vo
   // that takes most of the LDS keeps the next launch's blocks out until it has ended.
   const int64_t tiles_64 = (int64_t)((m + 63) / 64) * ((n + 63) / 64);
   const int k_tiles = k / TB_BK;
-  if (m <= 64 && tiles_64 <= 256 && k > 1024)
+  if (m <= 64 && tiles_64 <= units && k > 1024)
     return launch_variant<1, 1, 8, TOut>(a, w, bias, c, m, n, k, lda, ldc, epilogue, scatter, s);
-  if ((tiles_64 <= 512 && k_tiles > 2) || k >= 2048)
+  if ((tiles_64 <= 2 * units && k_tiles > 2) || k >= 2048)
     return launch_variant<1, 1, 4, TOut>(a, w, bias, c, m, n, k, lda, ldc, epilogue, scatter, s);
   return launch_variant<1, 1, 2, TOut>(a, w, bias, c, m, n, k, lda, ldc, epilogue, scatter, s);
 }

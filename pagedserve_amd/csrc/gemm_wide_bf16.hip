@@ -279,7 +279,7 @@ int ps_gemm_nt_bf16_wide(const void* a, const void* w_packed, const float* bias,
     // them for most of the chip, blocks of 32 rows below that; blocks of 128 rows only draw
     // level at shapes of thousands of rows and columns
     const int64_t columns = (n + GW_BN - 1) / GW_BN;
-    rows_per_block = columns * ((m + 63) / 64) >= 160 ? 64 : 32;
+    rows_per_block = columns * ((m + 63) / 64) >= ps_compute_units() * 5 / 8 ? 64 : 32;
   }
 #define PS_WIDE(WM, ST)                                                                                \
   (c_dtype == PS_F32                                                                                   \
