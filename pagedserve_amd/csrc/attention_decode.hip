@@ -11,7 +11,9 @@
 // triton_paged_attention.py:219-223) over the keys it visits and the states are merged once
 // at the end: across lane groups by shuffles, across the four waves through LDS.  With one
 // split the block writes the output; otherwise it writes (acc, m, l) and
-// attention_reduce_kernel merges the splits.
+// attention_reduce_kernel merges the splits.  Without an output tensor (out == nullptr) the
+// records (acc, m, l) are all that is written, whatever the number of splits: the kernel in
+// attention_merge_linear.hip merges them inside the output projection.
 #include <math.h>
 
 #include <mutex>
@@ -240,7 +242,7 @@ __global__ __launch_bounds__(64 * AD_WAVES) void attention_decode_kernel(
     block_l += s_ml[w][1] * c;
     if (d < head_dim) value += s_acc[w][d] * c;
   }
-  if (splits == 1) {
+  if (splits == 1 && out != nullptr) {
     if (d < head_dim)
       out[(int64_t)t * out_stride + (int64_t)head * head_dim + d] = from_float<T>(value / block_l);
   } else {
@@ -332,7 +334,7 @@ static int launch_decode(const void* q, int64_t q_stride, const void* k_pool, co
 #undef PS_LAUNCH_ADW
 #undef PS_LAUNCH_ADN
   PS_CHECK_LAUNCH("ps_attention_decode");
-  if (splits > 1) {
+  if (splits > 1 && out != nullptr) {
     hipLaunchKernelGGL(attention_reduce_kernel<T>, dim3(count, heads), dim3(64), 0, s, partial,
                        (T*)out, out_stride, tok_list, heads, head_dim, splits);
     PS_CHECK_LAUNCH("ps_attention_decode(reduce)");
@@ -404,6 +406,7 @@ extern "C" int ps_attention_decode_static(const void* q, int64_t q_stride, const
   if (check_decode_sizes("ps_attention_decode_static", count, heads, kv_heads, head_dim, page_size,
                          num_pages, table_width, window, splits, waves, dtype))
     return 1;
+  PS_REQUIRE(out != nullptr, "ps_attention_decode_static: no output tensor");
   float* partial = nullptr;
   if (splits > 1) {
     const int64_t need = (int64_t)count * heads * splits * (head_dim + 2);
@@ -430,6 +433,32 @@ extern "C" int ps_attention_decode_static(const void* q, int64_t q_stride, const
                                head_dim, page_size, num_pages, scale, window, splits, waves, s);
 }
 
+// The partial records only (see pagedserve_hip.h).
+extern "C" int ps_attention_decode_partial(const void* q, int64_t q_stride, const void* k_pool,
+                                           const void* v_pool, float* partial,
+                                           int64_t partial_floats, const int* tok_list,
+                                           const int* tok_item, const int* tok_pos,
+                                           const int* tables, int table_width, int count,
+                                           int heads, int kv_heads, int head_dim, int page_size,
+                                           int num_pages, float scale, int window, int splits,
+                                           int waves, int dtype, void* stream) {
+  if (check_decode_sizes("ps_attention_decode_partial", count, heads, kv_heads, head_dim,
+                         page_size, num_pages, table_width, window, splits, waves, dtype))
+    return 1;
+  const int64_t need = (int64_t)count * heads * splits * (head_dim + 2);
+  PS_REQUIRE(partial != nullptr && partial_floats >= need,
+             "ps_attention_decode_partial: the records need %lld floats", (long long)need);
+  if (count == 0) return 0;
+  hipStream_t s = (hipStream_t)stream;
+  if (dtype == PS_F32)
+    return launch_decode<float>(q, q_stride, k_pool, v_pool, nullptr, 0, partial, tok_list,
+                                tok_item, tok_pos, tables, table_width, count, heads, kv_heads,
+                                head_dim, page_size, num_pages, scale, window, splits, waves, s);
+  return launch_decode<bf16_t>(q, q_stride, k_pool, v_pool, nullptr, 0, partial, tok_list,
+                               tok_item, tok_pos, tables, table_width, count, heads, kv_heads,
+                               head_dim, page_size, num_pages, scale, window, splits, waves, s);
+}
+
 extern "C" int ps_attention_decode(const void* q, int64_t q_stride, const void* k_pool,
                                    const void* v_pool, void* out, int64_t out_stride,
                                    float* partial, int64_t partial_floats, const int* tok_list,
@@ -440,6 +469,7 @@ extern "C" int ps_attention_decode(const void* q, int64_t q_stride, const void* 
   if (check_decode_sizes("ps_attention_decode", count, heads, kv_heads, head_dim, page_size,
                          num_pages, table_width, window, splits, waves, dtype))
     return 1;
+  PS_REQUIRE(out != nullptr, "ps_attention_decode: no output tensor");
   if (splits > 1) {
     const int64_t need = (int64_t)count * heads * splits * (head_dim + 2);
     PS_REQUIRE(partial != nullptr && partial_floats >= need,

@@ -1,0 +1,187 @@
+// The merge of decode attention's key ranges inside the output projection, for steps of up
+// to 16 single-token items (bfloat16, head sizes that are multiples of 64):
+//
+//   residual[t, :] += concat_h(softmax-merged context of head h of token t) W^T + bias
+//
+// attention_decode_kernel leaves, per (token, head, range), the unnormalised sum of values
+// `acc`, the maximum `m` (in units of log 2) and the sum `l` of its range.  Merging them is
+// out = sum_s acc_s 2^(m_s - M) / sum_s l_s 2^(m_s - M).  A kernel of its own for that costs a
+// launch and a trip to memory per layer, as much as the attention of a small batch itself;
+// doing it in front of an output projection whose every block needs every head costs the same
+// again, since each block then pulls every record through its one compute unit (measured both
+// ways: blocks of 16 columns with the heads spread over their waves are slower than the merge
+// kernel they replace).  Here the projection is split over the heads instead: block (c, h) is
+// one wave that merges head h of all rows (each lane the 16 values of its own row that it
+// needs as matrix-core operand, so no lane talks to another, and the loads of all ranges are
+// in flight together), multiplies them with the piece of W that belongs to its columns and to
+// head h (out of the packed copy of W, pagedserve_hip.h), and adds the result into the float
+// residual rows with atomic adds; the blocks of head 0 add the bias.  The sum over heads is
+// therefore made by the adds, in an order that differs from run to run within float rounding,
+// as for every product here whose k range is split over blocks.
+#include "gemm_bf16_common.h"
+
+typedef __attribute__((__vector_size__(4 * sizeof(float)))) float f32x4_t;
+
+template <int STEPS, int TILES>   // head_dim / 64; tiles of 16 columns per block
+__global__ __launch_bounds__(64) void attention_merge_linear_kernel(
+    const float* __restrict__ partial, const int* __restrict__ tok_list, int count, int heads,
+    int splits, const bf16_t* __restrict__ wp, const float* __restrict__ bias,
+    float* __restrict__ residual, int64_t ld_res, int n) {
+  constexpr int HEAD_DIM = STEPS * 64;
+  constexpr int STRIDE = HEAD_DIM + 2;
+  const int lane = threadIdx.x;
+  const int row = lane & 15;           // activation row (token of the step)
+  const int group = lane >> 4;         // which 16 of every 64 head dimensions
+  const int head = blockIdx.y;
+  const bool has_row = row < count;
+  const int safe_row = has_row ? row : 0;
+  const float* records = partial + ((int64_t)safe_row * heads + head) * splits * STRIDE;
+
+  // the pieces of W: tiles of 16 columns, k steps head * STEPS ..., element
+  // ((tile * k_steps + step) * 2 + h) * 512 + lane * 8 of the packed copy; asked for first,
+  // they travel while the records are merged
+  const int k_steps = heads * STEPS;
+  const int tiles_n = (n + 15) / 16;
+  uint4 w_raw[TILES][STEPS][2];
+#pragma unroll
+  for (int c = 0; c < TILES; ++c) {
+    int tile = blockIdx.x * TILES + c;
+    if (tile >= tiles_n) tile = tiles_n - 1;     // beyond n: never stored
+    const bf16_t* w_tile = wp + ((int64_t)tile * k_steps + (int64_t)head * STEPS) * 1024 + lane * 8;
+#pragma unroll
+    for (int st = 0; st < STEPS; ++st)
+#pragma unroll
+      for (int h = 0; h < 2; ++h)
+        w_raw[c][st][h] = *reinterpret_cast<const uint4*>(w_tile + (st * 2 + h) * 512);
+  }
+
+  // Merge as the ranges come (a running maximum, earlier sums rescaled when it moves), so that
+  // no load waits for a result.
+  float total_m = -INFINITY;
+  float total_l = 0.f;
+  float value[STEPS][2][8];
+#pragma unroll
+  for (int st = 0; st < STEPS; ++st)
+#pragma unroll
+    for (int h = 0; h < 2; ++h)
+#pragma unroll
+      for (int e = 0; e < 8; ++e) value[st][h][e] = 0.f;
+#pragma unroll 4
+  for (int s = 0; s < splits; ++s) {
+    const float* record = records + s * STRIDE;
+    const float m_s = record[HEAD_DIM];
+    const float l_s = record[HEAD_DIM + 1];
+    float2 piece[STEPS][2][4];
+#pragma unroll
+    for (int st = 0; st < STEPS; ++st)
+#pragma unroll
+      for (int h = 0; h < 2; ++h)
+#pragma unroll
+        for (int q = 0; q < 4; ++q)
+          // the k values that lane group `group` holds in product h of step st (the order of
+          // the packed copy): 64 st + 16 group + 8 h ...; records start at multiples of 8 bytes
+          piece[st][h][q] = *reinterpret_cast<const float2*>(record + st * 64 + group * 16 + h * 8 + 2 * q);
+    const float new_m = fmaxf(total_m, m_s);
+    // an empty range has m = -inf and sums of zero: it changes nothing
+    const float keep = (total_m == -INFINITY) ? 0.f : __builtin_amdgcn_exp2f(total_m - new_m);
+    const float weight = (m_s == -INFINITY) ? 0.f : __builtin_amdgcn_exp2f(m_s - new_m);
+    total_l = total_l * keep + l_s * weight;
+#pragma unroll
+    for (int st = 0; st < STEPS; ++st)
+#pragma unroll
+      for (int h = 0; h < 2; ++h)
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+          value[st][h][2 * q] = fmaf(piece[st][h][q].x, weight, value[st][h][2 * q] * keep);
+          value[st][h][2 * q + 1] = fmaf(piece[st][h][q].y, weight, value[st][h][2 * q + 1] * keep);
+        }
+    total_m = new_m;
+  }
+  const float inverse = (has_row && total_l > 0.f) ? 1.f / total_l : 0.f;
+
+  f32x4_t acc[TILES];
+#pragma unroll
+  for (int c = 0; c < TILES; ++c) acc[c] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+  for (int st = 0; st < STEPS; ++st)
+#pragma unroll
+    for (int h = 0; h < 2; ++h) {
+      uint4 x_raw;
+      x_raw.x = pack2_bf16(value[st][h][0] * inverse, value[st][h][1] * inverse);
+      x_raw.y = pack2_bf16(value[st][h][2] * inverse, value[st][h][3] * inverse);
+      x_raw.z = pack2_bf16(value[st][h][4] * inverse, value[st][h][5] * inverse);
+      x_raw.w = pack2_bf16(value[st][h][6] * inverse, value[st][h][7] * inverse);
+#pragma unroll
+      for (int c = 0; c < TILES; ++c)
+        acc[c] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(*reinterpret_cast<const bf16x8*>(&w_raw[c][st][h]),
+                                                         *reinterpret_cast<const bf16x8*>(&x_raw), acc[c], 0, 0, 0);
+    }
+  // element i of lane l: column (l / 16) * 4 + i of the tile, row l % 16
+  if (!has_row) return;
+  const int t = tok_list ? tok_list[row] : row;
+#pragma unroll
+  for (int c = 0; c < TILES; ++c)
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int col = (blockIdx.x * TILES + c) * 16 + group * 4 + i;
+      if (col >= n) continue;
+      float v = acc[c][i];
+      if (head == 0 && bias != nullptr) v += bias[col];
+      unsafeAtomicAdd(residual + (int64_t)t * ld_res + col, v);
+    }
+}
+
+bool ps_attention_merge_linear_supported(int count, int head_dim, int dtype) {
+  return dtype == PS_BF16 && count >= 1 && count <= 16 && head_dim % 64 == 0 && head_dim <= 256;
+}
+
+// tiles_per_block: 16-column tiles that one wave computes (1 or 2; 0 lets the sizes decide)
+extern "C" int ps_attention_merge_linear(const float* partial, int64_t partial_floats,
+                                         const int* tok_list, int count, int heads, int head_dim,
+                                         int splits, const void* w_packed, const float* bias,
+                                         float* residual, int64_t ld_res, int n,
+                                         int tiles_per_block, void* stream) {
+  PS_REQUIRE(count >= 0 && heads > 0 && heads <= 65535 && splits >= 1 && splits <= 64 && n > 0 &&
+                 ld_res >= n,
+             "ps_attention_merge_linear: bad sizes (count %d, heads %d, splits %d, n %d)", count,
+             heads, splits, n);
+  PS_REQUIRE(ps_attention_merge_linear_supported(count > 0 ? count : 1, head_dim, PS_BF16),
+             "ps_attention_merge_linear: up to 16 rows and head sizes of 64, 128, 192 or 256, not "
+             "%d rows of head size %d", count, head_dim);
+  PS_REQUIRE(partial != nullptr && partial_floats >= (int64_t)count * heads * splits * (head_dim + 2),
+             "ps_attention_merge_linear: the records need %lld floats",
+             (long long)count * heads * splits * (head_dim + 2));
+  PS_REQUIRE(w_packed != nullptr && residual != nullptr &&
+                 (reinterpret_cast<uintptr_t>(w_packed) & 15u) == 0 &&
+                 (reinterpret_cast<uintptr_t>(partial) & 7u) == 0,
+             "ps_attention_merge_linear: null or unaligned operand");
+  PS_REQUIRE(tiles_per_block >= 0 && tiles_per_block <= 2,
+             "ps_attention_merge_linear: one or two tiles per block, not %d", tiles_per_block);
+  if (count == 0) return 0;
+  if (tiles_per_block == 0) tiles_per_block = 1;
+  const int tiles_n = (n + 15) / 16;
+  dim3 grid((tiles_n + tiles_per_block - 1) / tiles_per_block, heads);
+  hipStream_t s = (hipStream_t)stream;
+#define PS_LAUNCH_AML(STEPS, TILES)                                                               \
+  hipLaunchKernelGGL((attention_merge_linear_kernel<STEPS, TILES>), grid, dim3(64), 0, s, partial, \
+                     tok_list, count, heads, splits, (const bf16_t*)w_packed, bias, residual,     \
+                     ld_res, n)
+#define PS_LAUNCH_AMLT(STEPS)         \
+  do {                                \
+    if (tiles_per_block == 2) {       \
+      PS_LAUNCH_AML(STEPS, 2);        \
+    } else {                          \
+      PS_LAUNCH_AML(STEPS, 1);        \
+    }                                 \
+  } while (0)
+  switch (head_dim / 64) {
+    case 1: PS_LAUNCH_AMLT(1); break;
+    case 2: PS_LAUNCH_AMLT(2); break;
+    case 3: PS_LAUNCH_AMLT(3); break;
+    default: PS_LAUNCH_AMLT(4); break;
+  }
+#undef PS_LAUNCH_AMLT
+#undef PS_LAUNCH_AML
+  PS_CHECK_LAUNCH("ps_attention_merge_linear");
+  return 0;
+}

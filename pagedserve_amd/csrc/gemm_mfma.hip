@@ -544,7 +544,9 @@ bool ps_gemm_nt_mfma_supported(const void* a, const void* w, int k, int lda, int
 }
 
 // Whether norm + product run as one launch.
-// Every block normalises the rows again, so the fusion only pays while there are few blocks.
+// Every block normalises the rows again, so the fusion only pays while there are few blocks
+// (for the output head of 50,257 columns it measured 1 % slower per decode step than the
+// norm kernel in front of the two-tile skinny product).
 bool ps_norm_gemm_fusable(const void* w, const NormPrologue& norm, int m, int n, int k, int dtype) {
   return dtype == PS_BF16 && m <= 16 && n <= 8192 && k <= SN_MAX_K && k % 8 == 0 &&
          norm.ldh % 4 == 0 && aligned16(w) && aligned16(norm.h) && aligned16(norm.gamma) &&

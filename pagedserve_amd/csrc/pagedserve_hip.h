@@ -116,6 +116,28 @@ int ps_attention_decode(const void* q, int64_t q_stride, const void* k_pool, con
                         int head_dim, int page_size, int num_pages, float scale, int window,
                         int splits, int waves, int dtype, void* stream);
 
+// Only the records of ps_attention_decode: (unnormalised sum of values [head_dim], maximum in
+// units of log 2, sum) per (token, head, range) at partial[((n * heads + head) * splits + s) *
+// (head_dim + 2)], also with one range; nothing is merged and no output rows are written.
+int ps_attention_decode_partial(const void* q, int64_t q_stride, const void* k_pool,
+                                const void* v_pool, float* partial, int64_t partial_floats,
+                                const int* tok_list, const int* tok_item, const int* tok_pos,
+                                const int* tables, int table_width, int count, int heads,
+                                int kv_heads, int head_dim, int page_size, int num_pages,
+                                float scale, int window, int splits, int waves, int dtype,
+                                void* stream);
+
+// The merge of those records inside the output projection, for up to 16 tokens and head sizes
+// that are multiples of 64 (bfloat16 weights in their packed copy, n output columns,
+// k = heads * head_dim):  residual[t(r), :] += merged context of row r  W^T + bias, where
+// t(r) = tok_list ? tok_list[r] : r.  One wave per (tiles_per_block tiles of 16 columns, head);
+// the heads' contributions are added with float atomics.  tiles_per_block: 1, 2, or 0 for the
+// library's choice.
+int ps_attention_merge_linear(const float* partial, int64_t partial_floats, const int* tok_list,
+                              int count, int heads, int head_dim, int splits,
+                              const void* w_packed, const float* bias, float* residual,
+                              int64_t ld_res, int n, int tiles_per_block, void* stream);
+
 // ps_attention_decode for callers that cannot allocate device memory: code under HIP graph
 // capture, tight serving loops, harnesses that forbid hipMalloc.  It has no counterpart in the
 // reference.  The partial results of the key ranges go into a device array that is part of the

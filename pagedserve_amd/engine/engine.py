@@ -160,6 +160,17 @@ class Engine:
                                        device=self.device)[:, :vocab]
         return self._logits
 
+    def _context_class(self, longest: int) -> int:
+        """Launch shapes inside a graph must not depend on a step's lengths, but a step whose
+        longest context is 200 keys should not be cut into the ranges of one of 1,000: the
+        longest cached length of a step falls into a class (256, 1,024, 4,096, ... keys, the
+        last one the model's positions), the class is part of a graph's key, and the parts see
+        the class's bound as ``ctx.max_kv_len``."""
+        bound = 256
+        while bound < longest and bound < self.spec.max_positions:
+            bound *= 4
+        return min(bound, self.spec.max_positions)
+
     # ------------------------------------------------------------------- step
     def _validate(self, entries):
         if not entries:
@@ -432,7 +443,9 @@ class Engine:
         mode = 2 if isinstance(greedy, list) else int(bool(greedy))   # how tokens are chosen
         if self.use_graphs and self._graphs:
             # every entry brings one token and wants its logits: the lean path
-            plan = self._graphs.get((items, items, items, items, 0, mode))
+            requests = self.cache.requests
+            longest = 1 + max(requests[entry.request_id].length for entry in entries)
+            plan = self._graphs.get((items, items, items, items, 0, mode, self._context_class(longest)))
             if (plan is not None and plan.logits.data_ptr() == self._logit_buffer(items).data_ptr()
                     and all(len(e.tokens) == 1 and len(e.want) == 1 for e in entries)):
                 return self._replay(plan, entries, greedy)
@@ -440,13 +453,14 @@ class Engine:
         wanted = len(row_keys)
         logits = self._logit_buffer(wanted)
         singles = ctx.single_tokens.numel()
-        graph_key = (ctx.tokens, items, wanted, singles, ctx.tile_item.numel(), mode)
+        kv_class = self._context_class(ctx.max_kv_len)
+        graph_key = (ctx.tokens, items, wanted, singles, ctx.tile_item.numel(), mode, kv_class)
         if not self.use_graphs or graph_key in self._graph_failures:
             out, tokens = self._forward(ctx, rows, logits, wanted, greedy)
             return StepOutput(logits=out, rows=row_keys, tokens=tokens)
         # launch shapes inside a graph must not depend on this step's lengths
         exact_kv_len = ctx.max_kv_len
-        ctx.max_kv_len = self.spec.max_positions
+        ctx.max_kv_len = kv_class
         plan = self._graphs.get(graph_key)
         if plan is not None and plan.logits.data_ptr() == logits.data_ptr():
             # recorded: the indices are on their way already (``_pack`` copied them)

@@ -35,6 +35,11 @@ _SIGNATURES = {
                             c_int64, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int,
                             c_int, c_int, c_int, c_int, c_float, c_int, c_int, c_int, c_int,
                             c_void_p],
+    "ps_attention_decode_partial": [c_void_p, c_int64, c_void_p, c_void_p, c_void_p, c_int64, c_void_p,
+                                    c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int,
+                                    c_int, c_int, c_float, c_int, c_int, c_int, c_int, c_void_p],
+    "ps_attention_merge_linear": [c_void_p, c_int64, c_void_p, c_int, c_int, c_int, c_int, c_void_p,
+                                  c_void_p, c_void_p, c_int64, c_int, c_int, c_void_p],
     "ps_attention_prefill": [c_void_p, c_int64, c_void_p, c_void_p, c_void_p, c_int64, c_void_p,
                              c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int,
                              c_int, c_int, c_int, c_float, c_int, c_int, c_int, c_void_p],
@@ -491,6 +496,67 @@ def decode_supported(head_dim) -> bool:
     """Whether the split-KV kernel takes this head size (a lane fetches eight consecutive head
     dimensions of a key in one piece); the row-wise kernel takes every size up to 256."""
     return head_dim % 8 == 0 and 0 < head_dim <= 256
+
+
+def merge_linear_supported(dtype, tokens, head_dim, packed) -> bool:
+    """Whether ``attention_decode_partial`` + ``attention_merge_linear`` take a step: bfloat16,
+    up to 16 single-token items, a head size that is a multiple of 64, and the packed copy of the
+    output projection's matrix."""
+    return (dtype == torch.bfloat16 and packed is not None and 1 <= tokens <= 16
+            and head_dim % 64 == 0 and head_dim <= 256)
+
+
+def attention_decode_partial(q, k_pool, v_pool, partial, tok_item, tok_pos, tables, heads, scale, splits,
+                             window=0, tok_list=None, waves=4):
+    """The per-range records of decode attention only (``partial``: float scratch of
+    ``count * heads * splits * (head_dim + 2)`` values); ``attention_merge_linear`` merges them."""
+    _check(q, "q", ndim=2)
+    pages, kv_heads, page_size, head_dim = _check_pools(k_pool, v_pool, q.dtype)
+    q_stride = _rows(q, "q")
+    tokens = q.shape[0]
+    if q.shape[1] != heads * head_dim:
+        raise KernelError("attention: q rows must hold heads x head_dim values")
+    _check_step_index(tok_item, tok_pos, tables, tokens)
+    count = tokens
+    if tok_list is not None:
+        _check(tok_list, "tok_list", torch.int32, 1)
+        if not tok_list.is_contiguous():
+            raise KernelError("attention: tok_list must be contiguous")
+        count = tok_list.numel()
+    _check(partial, "partial", torch.float32)
+    if not partial.is_contiguous():
+        raise KernelError("attention_decode_partial: scratch must be contiguous")
+    _call("ps_attention_decode_partial", q.data_ptr(), q_stride, k_pool.data_ptr(), v_pool.data_ptr(),
+          partial.data_ptr(), partial.numel(), _ptr(tok_list), tok_item.data_ptr(), tok_pos.data_ptr(),
+          tables.data_ptr(), tables.shape[1], count, heads, kv_heads, head_dim, page_size, pages,
+          float(scale), int(window), int(splits), int(waves), dtype_code(q.dtype), _stream())
+    return count
+
+
+def attention_merge_linear(partial, count, heads, head_dim, splits, w, packed, bias, residual, tok_list=None,
+                           tiles_per_block=0):
+    """residual[t] += (merged attention output of row r) w^T + bias for the ``count`` rows whose
+    records ``attention_decode_partial`` left in ``partial``; ``packed`` is ``pack_decode_weight(w)``."""
+    _check(partial, "partial", torch.float32)
+    _check(residual, "residual", torch.float32, 2)
+    _check(w, "w", torch.bfloat16, 2)
+    n, k = w.shape
+    if k != heads * head_dim or residual.shape[1] != n:
+        raise KernelError(f"attention_merge_linear: w {tuple(w.shape)} does not fit {heads} heads of "
+                          f"{head_dim} and rows of {residual.shape[1]}")
+    if packed is None or packed.dtype != torch.bfloat16 or not packed.is_contiguous() \
+            or packed.numel() != -(-n // 16) * 16 * k:
+        raise KernelError("attention_merge_linear: the packed copy does not belong to w")
+    if bias is not None:
+        _check(bias, "bias", torch.float32, 1)
+        if bias.numel() != n:
+            raise KernelError("attention_merge_linear: bias does not match n")
+    if tok_list is None and residual.shape[0] < count:
+        raise KernelError("attention_merge_linear: fewer residual rows than records")
+    _call("ps_attention_merge_linear", partial.data_ptr(), partial.numel(), _ptr(tok_list), int(count),
+          int(heads), int(head_dim), int(splits), packed.data_ptr(), _ptr(bias), residual.data_ptr(),
+          _rows(residual, "residual"), n, int(tiles_per_block), _stream())
+    return residual
 
 
 PREFILL_TILE = 64

@@ -100,7 +100,8 @@ def test_running_ahead_gives_the_same_tokens_and_stops_at_the_end_token(folders)
 
 def test_running_ahead_with_temperature_draws_the_same_tokens(folders):
     """Drawn tokens (seeded) are the same whether the host's sampler picks them from the
-    logits after each step, the step picks them on the device, or steps run ahead."""
+    logits after each step, the step picks them on the device, or steps run ahead, under
+    Orca's whole prompts as under Sarathi's portions beside decoded tokens."""
     from pagedserve_amd.engine import ContinuousBatchScheduler, Engine
     from pagedserve_amd.model import load_model
     from pagedserve_amd.sampling import Sampler, SamplingParams
@@ -111,11 +112,14 @@ def test_running_ahead_with_temperature_draws_the_same_tokens(folders):
     temperatures = [6.0, 0.0, 12.0]
     model, _ = load_model(folder, dtype="float32")
     results = []
-    for on_device, run_ahead in ((False, False), (True, False), (True, True)):
+    for on_device, run_ahead, strategy in ((False, False, "orca"), (True, False, "orca"), (True, True, "orca"),
+                                          (True, True, "sarathi"), (False, False, "sarathi")):
         engine = Engine(model, num_pages=32, page_size=page_size, max_requests=4, max_step_tokens=64)
         engine.supports_draws = on_device
         scheduler = ContinuousBatchScheduler(engine, Sampler(engine.device, 4), max_batch_size=4,
-                                             eos_token_id=None, run_ahead=run_ahead)
+                                             eos_token_id=None, run_ahead=run_ahead,
+                                             scheduling_strategy=strategy, prefill_chunk_size=5,
+                                             max_prefill_requests=2)
         ids = [scheduler.add_token_request(prompt, budget, sampling=SamplingParams(
                    max_new_tokens=budget, temperature=temperature, seed=11 + i))
                for i, (prompt, budget, temperature) in enumerate(zip(prompts, budgets, temperatures))]
@@ -125,7 +129,7 @@ def test_running_ahead_with_temperature_draws_the_same_tokens(folders):
         if run_ahead:
             assert scheduler.steps_run_ahead > 10
         engine.cache.check_invariants()
-    assert results[0] == results[1] == results[2]
+    assert all(result == results[0] for result in results)
     # the draws are no argmax in disguise
     raw, weights = plain_gpt2.read_model_folder(folder)
     assert results[0][0] != plain_gpt2.greedy_generate(raw, weights, prompts[0], budgets[0])

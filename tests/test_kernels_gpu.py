@@ -835,3 +835,46 @@ def test_linear_takes_the_wide_product_for_long_k():
     assert torch.equal(out, plain)
     assert torch.equal(k_pool.view(torch.int16), k_ref.view(torch.int16))
     assert torch.equal(v_pool.view(torch.int16), v_ref.view(torch.int16))
+
+
+@pytest.mark.parametrize("heads,kv_heads,head_dim,page_size", [(12, 12, 64, 16), (4, 2, 128, 12), (2, 1, 256, 16), (3, 3, 192, 8)])
+@pytest.mark.parametrize("count", [1, 8, 16])
+@pytest.mark.parametrize("splits", [1, 3, 8])
+def test_attention_records_merged_inside_the_output_projection(heads, kv_heads, head_dim, page_size, count, splits):
+    """Decode attention that leaves only its per-range records, and the output projection that
+    merges them head by head: residual + softmax(q K^T) V W^T + bias in float64 over the
+    gathered pages; contexts around page edges, ranges without keys, a width that ends inside
+    a tile of 16 columns, rows beyond the count untouched."""
+    from pagedserve_amd.ops import kernels
+
+    dtype = torch.bfloat16
+    contexts = [1, 15, 16, 17, 31, 33, 128, 512, 700, 64, 2, 300, 90, 257, 1000, 48][:count]
+    k_pool, v_pool, tables = _paged_fixture(dtype, contexts, kv_heads, head_dim, page_size, 401)
+    q = _rand((count, heads * head_dim), dtype, 402)
+    width = 200 if heads * head_dim > 200 else 40
+    w = _rand((width, heads * head_dim), dtype, 403, 1.0 / math.sqrt(heads * head_dim))
+    bias = _rand((width,), torch.float32, 404)
+    packed = kernels.pack_decode_weight(w)
+    tok_item = torch.arange(count, dtype=torch.int32, device="cuda")
+    tok_pos = torch.tensor([c - 1 for c in contexts], dtype=torch.int32, device="cuda")
+    scale = head_dim ** -0.5
+    start = _rand((count + 2, width), torch.float32, 405)
+    residual = start.clone()
+    partial = torch.full((count * heads * splits * (head_dim + 2) + 8,), float("nan"), device="cuda")
+    assert kernels.merge_linear_supported(dtype, count, head_dim, packed)
+    kernels.attention_decode_partial(q, k_pool, v_pool, partial, tok_item, tok_pos, tables, heads, scale, splits)
+    kernels.attention_merge_linear(partial, count, heads, head_dim, splits, w, packed, bias, residual)
+    context = _attention_expected(q, k_pool, v_pool, tables, tok_item, tok_pos, heads, scale)
+    expected = start[:count].double() + context.to(dtype).double() @ w.double().t() + bias.double()
+    torch.testing.assert_close(residual[:count].double(), expected, atol=2e-2, rtol=2e-2)
+    assert torch.equal(residual[count:], start[count:])
+    # rows named by a list land at the listed tokens
+    chosen = torch.tensor(list(range(count))[::-1], dtype=torch.int32, device="cuda")
+    residual = start.clone()
+    kernels.attention_decode_partial(q, k_pool, v_pool, partial, tok_item, tok_pos, tables, heads, scale, splits,
+                                     tok_list=chosen)
+    kernels.attention_merge_linear(partial, count, heads, head_dim, splits, w, packed, bias, residual, tok_list=chosen)
+    torch.testing.assert_close(residual[:count].double(), expected, atol=2e-2, rtol=2e-2)
+    assert not kernels.merge_linear_supported(dtype, 17, head_dim, packed)
+    assert not kernels.merge_linear_supported(dtype, count, 48, packed)
+    assert not kernels.merge_linear_supported(torch.float32, count, head_dim, packed)
