@@ -233,10 +233,11 @@ __global__ __launch_bounds__(256) void gemm_nt_bf16_wide_kernel(
 // (the copy's tiles), rows of A can be loaded in pieces of 16 bytes, there are enough rows
 // and columns for its tiles to fill a good part of the chip, and k is long: at k below 1,024
 // (GPT-2 small's products into the layer) the kernel with both operands in LDS is as fast or
-// faster, measured at 2,048 rows.
+// faster, measured at 2,048 rows, and at k = 1,024 with a few hundred rows likewise.
 bool ps_gemm_nt_bf16_wide_supported(const void* a, const void* w_packed, int m, int n, int k,
                                     int lda) {
-  return w_packed != nullptr && m >= 256 && n >= 512 && k >= 1024 && k % TB_BK == 0 && lda % 8 == 0 &&
+  return w_packed != nullptr && m >= 256 && n >= 512 && (k >= 1536 || (k >= 1024 && m >= 1024)) &&
+         k % TB_BK == 0 && lda % 8 == 0 &&
          (reinterpret_cast<uintptr_t>(a) & 15u) == 0 &&
          (reinterpret_cast<uintptr_t>(w_packed) & 15u) == 0;
 }

@@ -810,7 +810,7 @@ def test_linear_takes_the_wide_product_for_long_k():
     LDS), also with the key/value scatter behind it."""
     from pagedserve_amd.ops import kernels
 
-    m, k = 600, 1024
+    m, k = 600, 1536
     heads, kv_heads, head_dim, page_size = 8, 4, 64, 16
     q_cols, kv_cols = heads * head_dim, kv_heads * head_dim
     n = q_cols + 2 * kv_cols
