@@ -230,15 +230,18 @@ __global__ __launch_bounds__(256) void gemm_nt_bf16_wide_kernel(
 
 // --------------------------------------------------------------------------------- host
 // Whether this kernel takes the product: the packed copy of W is there, k is a multiple of 64
-// (the copy's tiles), rows of A can be loaded in pieces of 16 bytes, there are enough rows
-// and columns for its tiles to fill a good part of the chip, and k is long: at k below 1,024
-// (GPT-2 small's products into the layer) the kernel with both operands in LDS is as fast or
-// faster, measured at 2,048 rows, and at k = 1,024 with a few hundred rows likewise.
+// (the copy's tiles), rows of A can be loaded in pieces of 16 bytes, k is long and blocks of
+// 64 rows x 256 columns fill most of the chip.  Measured with weights that no cache holds (a
+// different copy at every launch, as in a step through many layers), at 2,048 rows: 4096 x 1024
+// 28.5 us against 42.4 for the kernel with both operands in LDS, 4800 x 1600 47.4 against 58.1,
+// 1600 x 6400 68.0 against 92.5; but 768 x 3072 (three blocks side by side) 29.9 against 27.1,
+// and at k = 768 the two are level.  (With the same weights at every launch, out of the L2,
+// this kernel looks better than it is.)
 bool ps_gemm_nt_bf16_wide_supported(const void* a, const void* w_packed, int m, int n, int k,
                                     int lda) {
-  return w_packed != nullptr && m >= 256 && n >= 512 && (k >= 1536 || (k >= 1024 && m >= 1024)) &&
-         k % TB_BK == 0 && lda % 8 == 0 &&
-         (reinterpret_cast<uintptr_t>(a) & 15u) == 0 &&
+  const int64_t blocks = (int64_t)((n + GW_BN - 1) / GW_BN) * ((m + 63) / 64);
+  return w_packed != nullptr && k >= 1024 && blocks >= ps_compute_units() * 5 / 8 &&
+         k % TB_BK == 0 && lda % 8 == 0 && (reinterpret_cast<uintptr_t>(a) & 15u) == 0 &&
          (reinterpret_cast<uintptr_t>(w_packed) & 15u) == 0;
 }
 
@@ -275,13 +278,9 @@ static int launch_wide(const void* a, const void* wp, const float* bias, void* c
 int ps_gemm_nt_bf16_wide(const void* a, const void* w_packed, const float* bias, void* c, int m,
                          int n, int k, int lda, int ldc, int c_dtype, int epilogue,
                          const KvScatter& scatter, int rows_per_block, hipStream_t s) {
-  if (rows_per_block == 0) {
-    // measured at 2,048 rows: blocks of 64 rows are the fastest as soon as there are enough of
-    // them for most of the chip, blocks of 32 rows below that; blocks of 128 rows only draw
-    // level at shapes of thousands of rows and columns
-    const int64_t columns = (n + GW_BN - 1) / GW_BN;
-    rows_per_block = columns * ((m + 63) / 64) >= ps_compute_units() * 5 / 8 ? 64 : 32;
-  }
+  // blocks of 64 rows measured fastest wherever this kernel is ahead at all; blocks of 128
+  // rows draw level at shapes of thousands of rows and columns, blocks of 32 rows never do
+  if (rows_per_block == 0) rows_per_block = 64;
 #define PS_WIDE(WM, ST)                                                                                \
   (c_dtype == PS_F32                                                                                   \
        ? launch_wide<WM, ST, float>(a, w_packed, bias, c, m, n, k, lda, ldc, epilogue, scatter, s)      \
@@ -291,6 +290,7 @@ int ps_gemm_nt_bf16_wide(const void* a, const void* w_packed, const float* bias,
   if (rows_per_block == 128) return PS_WIDE(4, 3);
   if (rows_per_block == 64) return PS_WIDE(2, 3);
   if (rows_per_block == 32) return PS_WIDE(1, 3);
+
 #undef PS_WIDE
   ps_set_error("ps_linear: the wide product has blocks of 128, 64 or 32 rows, not %d", rows_per_block);
   return 1;

@@ -810,14 +810,14 @@ def test_linear_takes_the_wide_product_for_long_k():
     LDS), also with the key/value scatter behind it."""
     from pagedserve_amd.ops import kernels
 
-    m, k = 600, 1536
-    heads, kv_heads, head_dim, page_size = 8, 4, 64, 16
+    m, k = 1300, 1024
+    heads, kv_heads, head_dim, page_size = 32, 16, 64, 16
     q_cols, kv_cols = heads * head_dim, kv_heads * head_dim
-    n = q_cols + 2 * kv_cols
-    lens = [350, 280]
+    n = q_cols + 2 * kv_cols          # 4,096 columns: 16 x 21 blocks of 64 rows x 256 columns
+    lens = [700, 650]
     k_pool, v_pool, tables = _paged_fixture(torch.bfloat16, lens, kv_heads, head_dim, page_size, 320)
-    tok_item = torch.tensor([0] * 330 + [1] * 270, dtype=torch.int32, device="cuda")
-    tok_pos = torch.tensor(list(range(20, 350)) + list(range(10, 280)), dtype=torch.int32, device="cuda")
+    tok_item = torch.tensor([0] * 680 + [1] * 620, dtype=torch.int32, device="cuda")
+    tok_pos = torch.tensor(list(range(20, 700)) + list(range(30, 650)), dtype=torch.int32, device="cuda")
     x = _rand((m, k), torch.bfloat16, 321)
     w = _rand((n, k), torch.bfloat16, 322, 1.0 / math.sqrt(k))
     bias = _rand((n,), torch.float32, 323)
