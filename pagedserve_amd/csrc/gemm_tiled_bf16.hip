@@ -239,6 +239,10 @@ static int launch_tiled_bf16(const void* a, const void* w, const float* bias, vo
     return launch_variant<2, 2, 2, TOut>(a, w, bias, c, m, n, k, lda, ldc, epilogue, scatter, s);
   if (m > 64 && tiles_128_64 >= units + units / 2)
     return launch_variant<2, 1, 2, TOut>(a, w, bias, c, m, n, k, lda, ldc, epilogue, scatter, s);
+  // a long k with a block per compute unit: four stages of 128 x 64 (2048 x 1024 x 4096 with
+  // weights from memory: 34.7 us against 37.8 for 64 x 64 tiles)
+  if (m > 64 && k >= 2048 && tiles_128_64 >= units)
+    return launch_variant<2, 1, 4, TOut>(a, w, bias, c, m, n, k, lda, ldc, epilogue, scatter, s);
   // 64 x 64 tiles.  What a compute unit has in flight decides how long a k tile takes to
   // arrive from memory.  Many blocks fill a unit by their number and keep two stages, which
   // lets five of them in; up to two blocks per unit get four stages each; a single row of
