@@ -422,10 +422,12 @@ extern "C" int ps_attention_prefill(const void* q, int64_t q_stride, const void*
   }
   hipStream_t s = (hipStream_t)stream;
   dim3 grid(heads, tiles);
-  // With few blocks each takes a compute unit for itself, and four waves along the keys
+  // With few blocks (up to three for two compute units: 2 x 1,024 tokens of 12 heads measured
+  // 1 % of the step ahead) each takes a compute unit for itself, and four waves along the keys
   // shorten the longest block (if the caller knows of no long context, that does not pay);
   // with many, smaller blocks that share a unit balance better.
-  const bool wide = (int64_t)tiles * heads <= 256 && (max_kv_len <= 0 || max_kv_len >= 512);
+  const bool wide = (int64_t)tiles * heads <= ps_compute_units() * 3 / 2 &&
+                    (max_kv_len <= 0 || max_kv_len >= 512);
 #define PS_LAUNCH_AP(NDB)                                                                       \
   do {                                                                                          \
     if (wide)                                                                                   \

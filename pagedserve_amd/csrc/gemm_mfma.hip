@@ -592,7 +592,7 @@ template <typename TOut, int EPI>
 static void launch_skinny_mb(const void* a, const void* w, const float* bias, void* c, int m,
                              int n, int k, int lda, int ldc, int k_chunk, int k_splits,
                              const KvScatter& scatter, const bf16_t* wp, int layouts,
-                             hipStream_t s) {
+                             bool two_tiles, hipStream_t s) {
   // Rows go 16 to an accumulator, up to four accumulators to a block.  Where the columns and
   // the k ranges give few blocks, the rows are spread over more of them (every one reads the
   // same weights, which the L2 absorbs; blocks that differ only in z run on one XCD when the
@@ -616,7 +616,14 @@ static void launch_skinny_mb(const void* a, const void* w, const float* bias, vo
     if (three) PS_LAUNCH_SKU(MB, 1, 3);                                                        \
     else PS_LAUNCH_SKU(MB, 1, SK_UNROLL);                                                      \
   } while (0)
-  if (per <= 1 && k_splits == 1 && n >= 16 * 1024) {
+  if (two_tiles && per >= 2) {
+    // very many blocks (wide models): two tiles of columns per block halve what the blocks
+    // fetch of the rows of A, which at 17 to 64 rows is most of their traffic
+    grid.x = (n + 31) / 32;
+    if (per == 2) PS_LAUNCH_SKU(2, 2, 2);
+    else if (per == 3) PS_LAUNCH_SKU(3, 2, 2);
+    else PS_LAUNCH_SKU(4, 2, 2);
+  } else if (per <= 1 && k_splits == 1 && n >= 16 * 1024) {
     // the output head: two tiles of columns per block
     grid.x = (n + 31) / 32;
     if (three) PS_LAUNCH_SKU(1, 2, 3);
@@ -646,10 +653,19 @@ static int launch_skinny(const void* a, const void* w, const float* bias, void* 
   int k_chunk = (k + k_splits - 1) / k_splits;
   k_chunk = (k_chunk + 255) / 256 * 256;
   k_splits = (k + k_chunk - 1) / k_chunk;
+  // More rows than 16 and half as many blocks again as compute units: two column tiles per
+  // block and ranges of 640 k (64 x 1600 x 6400 with weights from memory: 13.6 us against
+  // 17.7; at 1024 x 4096 and below the single tile stays ahead).
+  const bool two_tiles = epilogue == PS_EPI_RESIDUAL && m > 16 && k_splits > 1 &&
+                         (int64_t)((n + 15) / 16) * k_splits >= ps_compute_units() * 3 / 2;
+  if (two_tiles) {
+    k_chunk = 640;
+    k_splits = (k + k_chunk - 1) / k_chunk;
+  }
 #define PS_SKINNY_CASE(EPI)                                                                      \
   case EPI:                                                                                      \
     launch_skinny_mb<TOut, EPI>(a, w, bias, c, m, n, k, lda, ldc, k_chunk, k_splits, scatter, wp, \
-                                layouts, s);                                                     \
+                                layouts, two_tiles, s);                                          \
     break
   switch (epilogue) {
     PS_SKINNY_CASE(PS_EPI_NONE);

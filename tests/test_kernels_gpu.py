@@ -109,6 +109,9 @@ GEMM_SHAPES = [(1, 50, 64), (5, 1000, 96), (64, 2304, 768), (130, 70, 320), (33,
                # 17 to 64 rows: rows spread over blocks where the columns give few of them, and
                # the eight-stage tiles for a k beyond one round of the skinny kernel's loads
                (64, 768, 768), (40, 400, 1600), (50, 4800, 1600), (33, 330, 2112), (64, 1600, 6400),
+               # so many blocks that two column tiles go to a block (residual epilogue), with a
+               # ragged last tile and a last k range of one step
+               (33, 1290, 5184), (20, 1600, 6400),
                # few rows and very many columns: two tiles of columns per block, ragged end
                (9, 16411, 320), (16, 20000, 768)]
 
@@ -660,7 +663,8 @@ def test_attention_decode_sixteen_waves(dtype):
 
 
 PACKED_SHAPES = [(1, 50, 64), (8, 768, 3072), (8, 2304, 768), (16, 3072, 768), (17, 768, 768), (5, 1000, 320),
-                 (64, 2304, 768), (48, 100, 3072), (9, 16411, 320), (16, 330, 1600), (40, 400, 1600), (300, 1000, 320)]
+                 (64, 2304, 768), (48, 100, 3072), (9, 16411, 320), (16, 330, 1600), (40, 400, 1600), (300, 1000, 320),
+                 (40, 1600, 6400), (33, 1290, 5184)]
 
 
 @pytest.mark.parametrize("m,n,k", PACKED_SHAPES)
@@ -716,7 +720,7 @@ def test_linear_with_packed_weights(m, n, k, epilogue):
 
 
 @pytest.mark.parametrize("m", [17, 32, 47, 64])
-@pytest.mark.parametrize("inner,width", [(3072, 768), (320, 128), (1600, 1600)])
+@pytest.mark.parametrize("inner,width", [(3072, 768), (320, 128), (1600, 1600), (6400, 1600)])
 def test_linear_chain_with_packed_activations(m, inner, width):
     """Norm, product, activation, product as a decode step of 17 to 64 rows runs them: the
     normed rows and the hidden rows may travel in the lanes' operand order.  The result equals
