@@ -9,7 +9,8 @@ int ps_gemm_nt_simple(const void* a, const void* w, const float* bias, void* c, 
                       hipStream_t s);
 int ps_gemm_nt_mfma(const void* a, const void* w, const float* bias, void* c, int m, int n, int k,
                     int lda, int ldc, int dtype, int c_dtype, int epilogue,
-                    const KvScatter& scatter, const void* w_packed, int layouts, hipStream_t s);
+                    const KvScatter& scatter, const void* w_packed, int layouts,
+                    const TopChoice& top, hipStream_t s);
 bool ps_gemm_nt_mfma_skinny(const void* a, const void* w, int m, int n, int k, int lda, int dtype,
                             int epilogue);
 int ps_norm_layout(const float* x, const int* rows, const float* gamma, const float* beta,
@@ -74,6 +75,13 @@ extern "C" int ps_linear(const PsLinearArgs* p, void* stream) {
       while ((1 << scatter.page_shift) < p->page_size) ++scatter.page_shift;
     }
   }
+  if (p->top_tokens != nullptr) {
+    PS_REQUIRE(p->top_keys != nullptr && p->top_ticket != nullptr && p->top_done != nullptr,
+               "ps_linear: choosing tokens needs keys, a ticket and a place for the answer");
+    PS_REQUIRE(p->epilogue == PS_EPI_NONE && p->c_dtype == PS_F32 && scatter.k_pool == nullptr,
+               "ps_linear: tokens are chosen from a plain float output");
+    *p->top_done = 0;
+  }
   if (m == 0) return 0;
   hipStream_t s = (hipStream_t)stream;
 
@@ -119,9 +127,16 @@ extern "C" int ps_linear(const PsLinearArgs* p, void* stream) {
       layouts |= 2;
       *p->c_layout = 1;
     }
+    TopChoice top = {};
+    if (p->top_tokens != nullptr && ps_gemm_nt_mfma_skinny(a, p->w, m, n, k, lda, p->dtype, p->epilogue)) {
+      top.keys = reinterpret_cast<unsigned long long*>(p->top_keys);
+      top.ticket = p->top_ticket;
+      top.tokens = p->top_tokens;
+      *p->top_done = 1;
+    }
     return ps_gemm_nt_mfma(a, p->w, p->bias, p->c, m, n, k, lda, p->ldc, p->dtype, p->c_dtype,
                            p->epilogue, scatter, p->dtype == PS_BF16 ? p->w_packed : nullptr,
-                           layouts, s);
+                           layouts, top, s);
   }
   PS_REQUIRE(layouts == 0, "ps_linear: packed input rows need operands that the matrix-core kernels take");
   int status = ps_gemm_nt_simple(a, p->w, p->bias, p->c, m, n, k, lda, p->ldc, p->dtype,

@@ -276,11 +276,91 @@ __device__ inline void skinny_epilogue(float (*partial)[MB][4][64], const float*
   }
 }
 
+// Each row's largest value and its column among the block's NT tiles, from the partial tiles
+// that the epilogue has just summed (the same sum in the same order, so the value is the one
+// stored), raised into the row's keys; the last block to finish turns keys into tokens.
+template <int MB, int NT>
+__device__ inline void skinny_top_choice(float (*partial)[SK_WAVES][MB][4][64], const float* bias,
+                                         int m, int n, int n0, int row0, const TopChoice& top) {
+  __shared__ int s_last;
+  const int col_in = threadIdx.x & 15;
+  const int row_in = threadIdx.x >> 4;
+  const int i = col_in & 3;
+  const int lane = (col_in >> 2) * 16 + row_in;
+  const int block = blockIdx.x + gridDim.x * (blockIdx.y + gridDim.y * blockIdx.z);
+#pragma unroll
+  for (int b = 0; b < MB; ++b) {
+    const int row = row0 + b * 16 + row_in;
+    unsigned long long best = 0;
+#pragma unroll
+    for (int j = 0; j < NT; ++j) {
+      const int col = n0 + j * 16 + col_in;
+      if (col < n && row < m) {
+        const float v = partial[j][0][b][i][lane] + partial[j][1][b][i][lane] +
+                        partial[j][2][b][i][lane] + partial[j][3][b][i][lane] +
+                        (bias != nullptr ? bias[col] : 0.f);
+        const unsigned long long key = top_choice_key(v, col);
+        best = key > best ? key : best;
+      }
+    }
+    // the 16 threads of a row are 16 consecutive lanes of one wave
+#pragma unroll
+    for (int off = 8; off >= 1; off >>= 1) {
+      const unsigned long long other = __shfl_xor(best, off, 64);
+      best = other > best ? other : best;
+    }
+    // (reading the key first, to skip an atomic that would change nothing, costs a trip to
+    // memory of its own and measured 3 us slower at 1,571 blocks)
+    if (col_in == 0 && row < m)
+      __hip_atomic_fetch_max(top_choice_slot(top, row, block & (PS_TOP_SLOTS - 1)), best,
+                             __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  }
+  // the block's maxima have been performed before its ticket is drawn
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    // Atomics on one address are performed one after the other, some ten nanoseconds each:
+    // a block draws from one of PS_TOP_SLOTS counters, and only the last of each draws from
+    // the common one.
+    const int blocks = gridDim.x * gridDim.y * gridDim.z;
+    const int group = block & (PS_TOP_SLOTS - 1);
+    const int in_group = (blocks - group + PS_TOP_SLOTS - 1) / PS_TOP_SLOTS;
+    const int groups = blocks < PS_TOP_SLOTS ? blocks : PS_TOP_SLOTS;
+    int last = __hip_atomic_fetch_add(top_choice_ticket(top, 1 + group), 1, __ATOMIC_RELAXED,
+                                      __HIP_MEMORY_SCOPE_AGENT) == in_group - 1;
+    if (last)
+      last = __hip_atomic_fetch_add(top_choice_ticket(top, 0), 1, __ATOMIC_RELAXED,
+                                    __HIP_MEMORY_SCOPE_AGENT) == groups - 1;
+    s_last = last;
+  }
+  __syncthreads();
+  if (!s_last) return;
+  // 16 threads per row, one key each
+  for (int base = 0; base < m; base += 64 * SK_WAVES / PS_TOP_SLOTS) {
+    const int row = base + (int)threadIdx.x / PS_TOP_SLOTS;
+    unsigned long long best = 0;
+    if (row < m) {
+      unsigned long long* slot = top_choice_slot(top, row, threadIdx.x & (PS_TOP_SLOTS - 1));
+      best = __hip_atomic_load(slot, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      __hip_atomic_store(slot, 0ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
+#pragma unroll
+    for (int off = 8; off >= 1; off >>= 1) {
+      const unsigned long long other = __shfl_xor(best, off, 64);
+      best = other > best ? other : best;
+    }
+    if (row < m && (threadIdx.x & (PS_TOP_SLOTS - 1)) == 0)
+      top.tokens[row] = (int)(0xFFFFFFFFu - (unsigned int)(best & 0xFFFFFFFFull));
+  }
+  if (threadIdx.x <= PS_TOP_SLOTS)
+    __hip_atomic_store(top_choice_ticket(top, threadIdx.x), 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+
 template <typename TOut, int EPI, int MB, int NT, int UNROLL>
 __global__ __launch_bounds__(64 * SK_WAVES) void gemm_nt_skinny_kernel(
     const bf16_t* __restrict__ a, const bf16_t* __restrict__ w, const float* __restrict__ bias,
     TOut* __restrict__ c, int m, int n, int k, int lda, int ldc, int k_chunk, int k_splits,
-    KvScatter scatter, const bf16_t* __restrict__ wp, int layouts) {
+    KvScatter scatter, const bf16_t* __restrict__ wp, int layouts, TopChoice top) {
   // layouts: bit 0, the rows of A lie in the packed order (packed_offset); bit 1, C is to be
   // written in it.
   // NT tiles of 16 columns per block share the loads of the rows of A: with very many
@@ -389,6 +469,8 @@ __global__ __launch_bounds__(64 * SK_WAVES) void gemm_nt_skinny_kernel(
   for (int j = 0; j < NT; ++j)
     skinny_epilogue<TOut, EPI, MB>(partial[j], bias, c, m, n, ldc, n0 + j * 16, row0, split,
                                    k_splits, scatter, layouts & 2);
+  if (EPI == PS_EPI_NONE && sizeof(TOut) == 4 && top.keys != nullptr)
+    skinny_top_choice<MB, NT>(partial, bias, m, n, n0, row0, top);
 }
 
 // ---------------------------------------------------------------- skinny with fused norm
@@ -592,7 +674,7 @@ template <typename TOut, int EPI>
 static void launch_skinny_mb(const void* a, const void* w, const float* bias, void* c, int m,
                              int n, int k, int lda, int ldc, int k_chunk, int k_splits,
                              const KvScatter& scatter, const bf16_t* wp, int layouts,
-                             bool two_tiles, hipStream_t s) {
+                             bool two_tiles, const TopChoice& top, hipStream_t s) {
   // Rows go 16 to an accumulator, up to four accumulators to a block.  Where the columns and
   // the k ranges give few blocks, the rows are spread over more of them (every one reads the
   // same weights, which the L2 absorbs; blocks that differ only in z run on one XCD when the
@@ -610,7 +692,7 @@ static void launch_skinny_mb(const void* a, const void* w, const float* bias, vo
 #define PS_LAUNCH_SKU(MB, NT, UNROLL)                                                          \
   hipLaunchKernelGGL((gemm_nt_skinny_kernel<TOut, EPI, MB, NT, UNROLL>), grid, block, 0, s,    \
                      (const bf16_t*)a, (const bf16_t*)w, bias, (TOut*)c, m, n, k, lda, ldc,    \
-                     k_chunk, k_splits, scatter, wp, layouts)
+                     k_chunk, k_splits, scatter, wp, layouts, top)
 #define PS_LAUNCH_SK(MB)                                                                       \
   do {                                                                                         \
     if (three) PS_LAUNCH_SKU(MB, 1, 3);                                                        \
@@ -632,7 +714,7 @@ static void launch_skinny_mb(const void* a, const void* w, const float* bias, vo
     // up to 16 rows leave registers for twice the loads: a k of up to 2048 in one round
     hipLaunchKernelGGL((gemm_nt_skinny_kernel<TOut, EPI, 1, 1, 2 * SK_UNROLL>), grid, block, 0, s,
                        (const bf16_t*)a, (const bf16_t*)w, bias, (TOut*)c, m, n, k, lda, ldc,
-                       k_chunk, k_splits, scatter, wp, layouts);
+                       k_chunk, k_splits, scatter, wp, layouts, top);
   } else if (per <= 1) PS_LAUNCH_SK(1);
   else if (per == 2) PS_LAUNCH_SK(2);
   else if (per == 3) PS_LAUNCH_SK(3);
@@ -644,7 +726,7 @@ static void launch_skinny_mb(const void* a, const void* w, const float* bias, vo
 template <typename TOut>
 static int launch_skinny(const void* a, const void* w, const float* bias, void* c, int m, int n,
                          int k, int lda, int ldc, int epilogue, const KvScatter& scatter,
-                         const bf16_t* wp, int layouts, hipStream_t s) {
+                         const bf16_t* wp, int layouts, const TopChoice& top, hipStream_t s) {
   if (k % 64 != 0) wp = nullptr;   // the packed copy exists for whole steps of 64 only
   // A block covers 1024 k with one round of loads.  Longer k is split over blocks where the
   // partial sums can be added in place (residual epilogue), else the block loops.
@@ -665,7 +747,7 @@ static int launch_skinny(const void* a, const void* w, const float* bias, void* 
 #define PS_SKINNY_CASE(EPI)                                                                      \
   case EPI:                                                                                      \
     launch_skinny_mb<TOut, EPI>(a, w, bias, c, m, n, k, lda, ldc, k_chunk, k_splits, scatter, wp, \
-                                layouts, two_tiles, s);                                          \
+                                layouts, two_tiles, top, s);                                     \
     break
   switch (epilogue) {
     PS_SKINNY_CASE(PS_EPI_NONE);
@@ -741,12 +823,15 @@ bool ps_gemm_nt_mfma_skinny(const void* a, const void* w, int m, int n, int k, i
 
 int ps_gemm_nt_mfma(const void* a, const void* w, const float* bias, void* c, int m, int n, int k,
                     int lda, int ldc, int dtype, int c_dtype, int epilogue,
-                    const KvScatter& scatter, const void* w_packed, int layouts, hipStream_t s) {
+                    const KvScatter& scatter, const void* w_packed, int layouts,
+                    const TopChoice& top, hipStream_t s) {
   const bf16_t* wp = (const bf16_t*)w_packed;
   if (ps_gemm_nt_mfma_skinny(a, w, m, n, k, lda, dtype, epilogue)) {
     if (c_dtype == PS_F32)
-      return launch_skinny<float>(a, w, bias, c, m, n, k, lda, ldc, epilogue, scatter, wp, layouts, s);
-    return launch_skinny<bf16_t>(a, w, bias, c, m, n, k, lda, ldc, epilogue, scatter, wp, layouts, s);
+      return launch_skinny<float>(a, w, bias, c, m, n, k, lda, ldc, epilogue, scatter, wp, layouts,
+                                  top, s);
+    return launch_skinny<bf16_t>(a, w, bias, c, m, n, k, lda, ldc, epilogue, scatter, wp, layouts,
+                                 top, s);
   }
   if (layouts != 0) {
     ps_set_error("ps_linear: packed activations go with the skinny product only (m %d, n %d, k %d)",

@@ -13,6 +13,37 @@ struct KvScatter {
   int table_width, q_cols, kv_cols, head_dim, kv_heads, page_size, page_shift, num_pages;
 };
 
+// The product of the output head may also choose each row's token (the column of its largest
+// value, the lowest one on ties) instead of leaving that to a kernel of its own.  Blocks
+// raise 64-bit keys (value in an order that integers keep, then the column counted from
+// above) with atomic maxima, spread over PS_TOP_SLOTS keys per row, 256 bytes apart, so that
+// few blocks meet at one address and the keys lie on many memory channels (atomics on one
+// address, and on one channel, are performed one after the other: 1,571 blocks drawing from
+// one ticket added 27 us to the kernel, 12,568 maxima within one kilobyte 10 us).  The block
+// that draws the last ticket reads the keys, writes the tokens, and leaves keys and tickets
+// at zero for the next launch.  Launches that share keys must not overlap.
+#define PS_TOP_SLOTS 16
+#define PS_TOP_STRIDE 32      // 64-bit words from one key to the next, and 2 ints from ticket to ticket: 256 bytes,
+                              // so that keys and tickets spread over the memory channels
+struct TopChoice {
+  unsigned long long* keys;   // null: no choice; else [rows * PS_TOP_SLOTS] keys, zero between launches
+  int* ticket;                // 1 + PS_TOP_SLOTS counters, zero between launches
+  int* tokens;                // [rows]
+};
+__device__ inline unsigned long long* top_choice_slot(const TopChoice& top, int row, int slot) {
+  return top.keys + ((int64_t)row * PS_TOP_SLOTS + slot) * PS_TOP_STRIDE;
+}
+__device__ inline int* top_choice_ticket(const TopChoice& top, int index) {
+  return top.ticket + index * 2 * PS_TOP_STRIDE;
+}
+
+__device__ inline unsigned long long top_choice_key(float v, int col) {
+  if (v == 0.f) v = 0.f;   // one zero
+  const unsigned int bits = __float_as_uint(v);
+  const unsigned int ordered = (bits & 0x80000000u) ? ~bits : (bits | 0x80000000u);
+  return ((unsigned long long)ordered << 32) | (unsigned long long)(0xFFFFFFFFu - (unsigned int)col);
+}
+
 // Activations of a decode step (17 to 64 rows) may lie in the order in which the lanes of the
 // skinny product hold their operand, like the packed weight copies: rows in blocks of 16, the
 // 16 x 64 tile of row block t and columns 64 s .. 64 s + 63 at element (t * (cols / 64) + s) *

@@ -83,6 +83,17 @@ typedef struct PsLinearArgs {
   int c_rows;             // rows that c has room for (the packed order rounds m up to 16)
   int norm_out_rows;      // rows that norm_out has room for
   int* c_layout;          // null, or where ps_linear says how it wrote c: 0 rows, 1 packed
+  // Null, or: the caller also wants tokens[r] = the column of the largest value of row r of c
+  // (the lowest such column on ties), as ps_sample gives it without a temperature.  Float
+  // output and the plain epilogue only.  The kernels for few bfloat16 rows do it in their
+  // epilogue and *top_done becomes 1; otherwise it becomes 0, nothing is written to tokens,
+  // and the caller runs ps_sample.  top_keys: m * 16 * 32 64-bit words, top_ticket: 17 * 64 ints; both
+  // zero before the first call and left at zero by every call, and not shared by launches
+  // that may overlap.
+  int* top_tokens;
+  void* top_keys;
+  int* top_ticket;
+  int* top_done;
 } PsLinearArgs;
 
 int ps_linear(const PsLinearArgs* args, void* stream);

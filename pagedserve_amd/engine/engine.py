@@ -110,6 +110,10 @@ class Engine:
                              for _ in range(2)]
         self._tokens_ready = [torch.cuda.Event(), torch.cuda.Event()]
         self._tokens_turn = 0
+        from ..ops import kernels
+
+        self._top_choice = kernels.TopChoice(min(self._tokens.numel(), 64), self.device)
+        self.tokens_chosen_by_head = 0   # greedy steps (launched or recorded) without a sampling launch
         self._carried_rows = 0    # rows of the last step whose chosen tokens a step may carry on
         # The engine's work runs on a stream of its own (default priority): a capture cannot
         # record from the default stream.
@@ -405,16 +409,21 @@ class Engine:
         return ctx, view("rows"), row_keys
 
     def _forward(self, ctx, rows, logits, wanted, greedy):
-        out = self.model.forward(ctx, self.views, rows, logits)
-        tokens = None
-        if greedy and wanted:
-            from ..ops import kernels
+        from ..ops import kernels
 
-            if isinstance(greedy, list):
-                inv_temperature, uniform = self._draw_views
-                tokens = kernels.sample(out, inv_temperature, uniform, self._tokens[:wanted])
-            else:
-                tokens = kernels.sample(out, None, None, self._tokens[:wanted])
+        if not (greedy and wanted):
+            return self.model.forward(ctx, self.views, rows, logits), None
+        tokens = self._tokens[:wanted]
+        if isinstance(greedy, list):
+            out = self.model.forward(ctx, self.views, rows, logits)
+            inv_temperature, uniform = self._draw_views
+            return out, kernels.sample(out, inv_temperature, uniform, tokens)
+        # the most likely token: chosen by the head's own kernel where it can
+        out = self.model.forward(ctx, self.views, rows, logits, choose=(self._top_choice, tokens))
+        if self.model.tokens_chosen:
+            self.tokens_chosen_by_head += 1
+        else:
+            kernels.sample(out, None, None, tokens)
         return out, tokens
 
     def _run(self, entries, greedy=False) -> StepOutput:

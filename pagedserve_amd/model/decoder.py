@@ -134,9 +134,12 @@ class DecoderModel:
         parts = [self.embedding, self.position, self.final_norm, self.head] + list(self.blocks)
         return all(getattr(part, "graph_safe", False) for part in parts)
 
-    def forward(self, ctx, views, logit_rows, logits_out):
+    def forward(self, ctx, views, logit_rows, logits_out, choose=None):
         """Run the step's tokens; write logits of ``logit_rows`` (int32 indices into the
-        step's tokens) into the float tensor ``logits_out``."""
+        step's tokens) into the float tensor ``logits_out``.  ``choose = (kernels.TopChoice,
+        tokens)``: a head that can also writes each row's most likely token into ``tokens``;
+        ``self.tokens_chosen`` says whether it did."""
+        self.tokens_chosen = False
         tokens = ctx.tokens
         h = ctx.workspace.rows("residual", self.spec.width, torch.float32)[:tokens]
         self.embedding.forward(ctx, self.position.embedding_table(), h)
@@ -152,5 +155,8 @@ class DecoderModel:
         if normed is None:
             normed = self.final_norm.forward(h, final, rows=logit_rows)
         out = logits_out[:wanted]
-        self.head.forward(normed, out)
+        if choose is not None and getattr(self.head, "chooses_tokens", False):
+            self.tokens_chosen = bool(self.head.forward(normed, out, choose=choose))
+        else:
+            self.head.forward(normed, out)
         return out

@@ -231,6 +231,8 @@ class _LinearArgs(ctypes.Structure):
         ("w_packed", c_void_p),
         ("a_packed", c_int), ("c_packed_request", c_int), ("c_rows", c_int),
         ("norm_out_rows", c_int), ("c_layout", ctypes.POINTER(c_int)),
+        ("top_tokens", c_void_p), ("top_keys", c_void_p), ("top_ticket", c_void_p),
+        ("top_done", ctypes.POINTER(c_int)),
     ]
 
 
@@ -282,8 +284,23 @@ def _row_capacity(tensor, columns: int) -> int:
     return int(elements // columns)
 
 
+TOP_SLOTS = 16   # keys per row of a TopChoice (csrc/linear.h: PS_TOP_SLOTS)
+
+
+class TopChoice:
+    """What a product needs to choose each row's token in its own epilogue: 16 keys per row
+    and 17 tickets, zero between launches (the kernel leaves them so).  One per stream: launches
+    that share it must not overlap."""
+
+    def __init__(self, rows: int, device):
+        self.rows = int(rows)
+        # 256 bytes from key to key and from ticket to ticket (csrc/linear.h: PS_TOP_STRIDE)
+        self.keys = torch.zeros(self.rows * TOP_SLOTS * 32, dtype=torch.int64, device=device)
+        self.ticket = torch.zeros((1 + TOP_SLOTS) * 64, dtype=torch.int32, device=device)
+
+
 def linear(x, w, bias, out, epilogue="none", scatter=None, packed=None, a_packed=False,
-           packed_out=False):
+           packed_out=False, choose=None):
     """out = epilogue(x w^T + bias) where ``x`` is a tensor or a ``PendingNorm``.
 
     ``scatter = (k_pool, v_pool, tok_item, tok_pos, tables, q_cols, kv_cols)`` also stores the
@@ -294,7 +311,12 @@ def linear(x, w, bias, out, epilogue="none", scatter=None, packed=None, a_packed
     second one's lanes hold them (``csrc/linear.h: packed_offset``).  ``packed_out=True`` allows
     that for ``out`` (whose storage must have room for the rows rounded up to 16) and makes the
     call return ``(out, written_packed)``; the buffer then goes to the next call with
-    ``a_packed=written_packed`` and means nothing to anyone else."""
+    ``a_packed=written_packed`` and means nothing to anyone else.
+
+    ``choose = (TopChoice, tokens)`` asks for ``tokens[r]`` = the column of the largest value of
+    row ``r`` of a float ``out`` (the lowest on ties), as ``sample`` gives it without a
+    temperature; the call then returns ``(out, chosen)``, and where ``chosen`` is False the
+    kernel that ran could not do it and ``tokens`` is untouched."""
     _check(w, "w", ndim=2)
     _check(out, "out", ndim=2)
     n, k = w.shape
@@ -378,6 +400,19 @@ def linear(x, w, bias, out, epilogue="none", scatter=None, packed=None, a_packed
         args.c_packed_request = 1
         args.c_rows = _row_capacity(out, n)
         args.c_layout = ctypes.pointer(layout)
+    done = c_int(0)
+    if choose is not None:
+        top, tokens = choose
+        _check(tokens, "tokens", torch.int32, 1)
+        if out.dtype != torch.float32 or epilogue != "none" or scatter is not None or packed_out:
+            raise KernelError("linear: tokens are chosen from a plain float output")
+        if tokens.numel() < m or not tokens.is_contiguous():
+            raise KernelError(f"linear: {m} rows need as many tokens")
+        if top.rows >= m:            # (more rows than there are keys for: the caller samples)
+            args.top_tokens = tokens.data_ptr()
+            args.top_keys = top.keys.data_ptr()
+            args.top_ticket = top.ticket.data_ptr()
+            args.top_done = ctypes.pointer(done)
     lib = load_library()
     fn = _BOUND.get("ps_linear")
     if fn is None:
@@ -395,6 +430,8 @@ def linear(x, w, bias, out, epilogue="none", scatter=None, packed=None, a_packed
         raise KernelError(f"ps_linear failed ({status}): {lib.ps_last_error().decode('utf-8', 'replace')}")
     if packed_out:
         return out, bool(layout.value)
+    if choose is not None:
+        return out, bool(done.value)
     return out
 
 

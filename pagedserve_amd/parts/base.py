@@ -113,6 +113,10 @@ class Head(Part):
     head uses as its matrix."""
 
     accepts_pending_norm = True
+    # True: ``forward`` takes ``choose=(kernels.TopChoice, tokens)`` and returns whether it
+    # also wrote each row's most likely token into ``tokens`` (greedy decoding without a
+    # sampling launch); the caller samples from the logits where it did not.
+    chooses_tokens = False
 
     def bind(self, tensors, embedding_table=None):
         super().bind(tensors)

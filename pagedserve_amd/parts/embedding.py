@@ -62,6 +62,12 @@ class LinearHead(Head):
         self.bias_vector = tensors.get("bias")
         self.packed = kernels.pack_decode_weight(self.weight)
 
-    def forward(self, x, logits):
-        kernels.linear(x, self.weight, self.bias_vector, logits, packed=self.packed)
-        return logits
+    chooses_tokens = True
+
+    def forward(self, x, logits, choose=None):
+        if choose is None:
+            kernels.linear(x, self.weight, self.bias_vector, logits, packed=self.packed)
+            return False
+        _, chosen = kernels.linear(x, self.weight, self.bias_vector, logits, packed=self.packed,
+                                   choose=choose)
+        return chosen

@@ -321,3 +321,32 @@ def test_more_layouts_than_recorded_graphs_are_kept(folders, references, dtype):
     assert error <= helpers.TOLERANCE[dtype] * scale, (error, scale, where)
     torch.cuda.synchronize()
     engine.cache.check_invariants()
+
+
+@pytest.mark.parametrize("live", [3, 20])
+def test_greedy_tokens_are_the_argmax_of_the_logits(folders, live):
+    """Greedy steps in bfloat16, replayed from a graph: the tokens that the step chooses are the
+    columns of the largest logits of the same step.  With 20 requests decoding the head's own
+    kernel chooses them (no sampling launch); with 3 the norm is fused into the head's product
+    and the sampling kernel does."""
+    from pagedserve_amd.engine import Engine, StepEntry
+    from pagedserve_amd.model import load_model
+
+    folder, config, page_size = folders["A"]
+    model, _ = load_model(folder, dtype="bfloat16")
+    engine = Engine(model, num_pages=24 * live, page_size=page_size, max_requests=live, max_step_tokens=64)
+    prompts = {f"g{i}": helpers.random_tokens(3 + i % 5, config["vocab_size"], 700 + i) for i in range(live)}
+    for name, prompt in prompts.items():
+        engine.step([StepEntry(name, prompt, [])])
+    last = {name: [prompt[-1]] for name, prompt in prompts.items()}
+    for step in range(8):
+        entries = [StepEntry(name, last[name], [0]) for name in prompts]
+        out = engine.step(entries, greedy=True)
+        tokens = out.token_list()
+        assert tokens == out.logits.argmax(dim=1).tolist(), step
+        for name, token in zip(prompts, tokens):
+            last[name] = [token]
+    assert (engine.tokens_chosen_by_head > 0) == (live > 16)
+    assert engine.graph_summary()["graph_replays"] >= 4
+    torch.cuda.synchronize()
+    assert int(engine._top_choice.keys.abs().sum()) == 0 and int(engine._top_choice.ticket.abs().sum()) == 0

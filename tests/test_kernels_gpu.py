@@ -882,3 +882,62 @@ def test_attention_records_merged_inside_the_output_projection(heads, kv_heads, 
     assert not kernels.merge_linear_supported(dtype, 17, head_dim, packed)
     assert not kernels.merge_linear_supported(dtype, count, 48, packed)
     assert not kernels.merge_linear_supported(torch.float32, count, head_dim, packed)
+
+
+@pytest.mark.parametrize("m,n,k", [(1, 50257, 768), (8, 50257, 768), (16, 1000, 320), (20, 20011, 768), (32, 16411, 320),
+                                   (5, 257, 64), (3, 41, 128), (9, 1000, 1600)])
+@pytest.mark.parametrize("with_bias", [False, True])
+def test_head_product_chooses_the_tokens(m, n, k, with_bias):
+    """The product of few bfloat16 rows also writes each row's column of the largest value,
+    the lowest such column on a tie, as the sampling kernel does from the stored logits; three
+    calls in a row with other inputs use the same keys, which every call leaves at zero."""
+    from pagedserve_amd.ops import kernels
+
+    dtype = torch.bfloat16
+    w = _rand((n, k), dtype, 400, 1.0 / math.sqrt(k))
+    bias = _rand((n,), torch.float32, 401) if with_bias else None
+    packed = kernels.pack_decode_weight(w)
+    top = kernels.TopChoice(m, "cuda")
+    for call in range(3):
+        a = _rand((m, k), dtype, 402 + call, 1.0)
+        if call == 2:
+            # a tie for the largest value of every row: the column that wins gets a twin, once
+            # before and once behind it
+            plain = torch.empty((m, n), dtype=torch.float32, device="cuda")
+            kernels.linear(a, w, bias, plain, packed=packed)
+            w = w.clone()
+            for row in range(m):
+                winner = int(plain[row].argmax())
+                twin = (winner + 1 + 2 * row) % n if row % 2 else (winner - 1 - 2 * row) % n
+                w[twin] = w[winner]
+                if bias is not None:
+                    bias[twin] = bias[winner]
+            packed = kernels.pack_decode_weight(w)
+        out = torch.full((m, n), float("nan"), dtype=torch.float32, device="cuda")
+        tokens = torch.full((m + 3,), -7, dtype=torch.int32, device="cuda")
+        _, chosen = kernels.linear(a, w, bias, out, packed=packed, choose=(top, tokens))
+        assert chosen
+        expected = torch.empty(m, dtype=torch.int32, device="cuda")
+        kernels.sample(out, None, None, expected)
+        assert torch.equal(tokens[:m], expected), (call, tokens[:m], expected)
+        assert torch.equal(expected.long(), out.argmax(dim=1))
+        assert (tokens[m:] == -7).all()
+        assert int(top.keys.abs().sum()) == 0 and int(top.ticket.abs().sum()) == 0
+
+
+def test_head_product_leaves_the_choice_where_it_cannot_make_it():
+    """More rows than the kernels for few rows take, and the 32-bit path: the call says that it
+    chose nothing, and the tokens stay as they were."""
+    from pagedserve_amd.ops import kernels
+
+    for dtype, m, n, k in ((torch.bfloat16, 40, 20011, 128), (torch.float32, 4, 300, 64)):
+        a = _rand((m, k), dtype, 410, 1.0)
+        w = _rand((n, k), dtype, 411, 1.0 / math.sqrt(k))
+        out = torch.empty((m, n), dtype=torch.float32, device="cuda")
+        tokens = torch.full((m,), -7, dtype=torch.int32, device="cuda")
+        top = kernels.TopChoice(m, "cuda")
+        _, chosen = kernels.linear(a, w, None, out, choose=(top, tokens))
+        assert not chosen and (tokens == -7).all()
+        torch.testing.assert_close(out.double(), a.double() @ w.double().t(), atol=2e-2, rtol=2e-2)
+    with pytest.raises(kernels.KernelError, match="plain float output"):
+        kernels.linear(a, w, None, out, epilogue="gelu_tanh", choose=(top, tokens))
