@@ -812,7 +812,7 @@ int ps_norm_gemm_fused(const NormPrologue& norm, const void* w, const float* bia
 // when the weights come from memory and not from a cache; the tiled kernel walks k tile by
 // tile and wins only where there are tiles enough to fill the chip (the output head).
 // A k beyond one round of the skinny kernel's loads makes it loop; there the tiled kernel
-// with its deep ring of stages is ahead, except where partial sums of a split k can be
+// with its ring of stages is ahead, except where partial sums of a split k can be
 // added in place (residual epilogue), which keeps every block at one round.
 bool ps_gemm_nt_mfma_skinny(const void* a, const void* w, int m, int n, int k, int lda, int dtype,
                             int epilogue) {

@@ -107,7 +107,7 @@ GEMM_SHAPES = [(1, 50, 64), (5, 1000, 96), (64, 2304, 768), (130, 70, 320), (33,
                # and with ragged rows of eight columns
                (1100, 2800, 128), (1027, 2801, 192), (3500, 3530, 64),
                # 17 to 64 rows: rows spread over blocks where the columns give few of them, and
-               # the eight-stage tiles for a k beyond one round of the skinny kernel's loads
+               # the tiled kernel for a k beyond one round of the skinny kernel's loads
                (64, 768, 768), (40, 400, 1600), (50, 4800, 1600), (33, 330, 2112), (64, 1600, 6400),
                # so many blocks that two column tiles go to a block (residual epilogue), with a
                # ragged last tile and a last k range of one step
