@@ -237,6 +237,10 @@ static int launch_tiled_bf16(const void* a, const void* w, const float* bias, vo
   const int units = ps_compute_units();
   if (m > 64 && tiles_128 >= 3 * units)
     return launch_variant<2, 2, 2, TOut>(a, w, bias, c, m, n, k, lda, ldc, epilogue, scatter, s);
+  // 128 x 64: three stages while two blocks per unit hold them all (1100 x 3072 x 1024 with
+  // weights from memory: 16.1 against 17.7 us), two stages, which let a third block in, beyond
+  if (m > 64 && tiles_128_64 >= units + units / 2 && tiles_128_64 <= 2 * units)
+    return launch_variant<2, 1, 3, TOut>(a, w, bias, c, m, n, k, lda, ldc, epilogue, scatter, s);
   if (m > 64 && tiles_128_64 >= units + units / 2)
     return launch_variant<2, 1, 2, TOut>(a, w, bias, c, m, n, k, lda, ldc, epilogue, scatter, s);
   // a long k with a block per compute unit: four stages of 128 x 64 (2048 x 1024 x 4096 with
@@ -254,6 +258,9 @@ static int launch_tiled_bf16(const void* a, const void* w, const float* bias, vo
   const int k_tiles = k / TB_BK;
   if ((tiles_64 <= 2 * units && k_tiles > 2) || k >= 2048)
     return launch_variant<1, 1, 4, TOut>(a, w, bias, c, m, n, k, lda, ldc, epilogue, scatter, s);
+  // up to three blocks per unit: three stages each (544 x 4096 x 1024: 15.9 against 18.2 us)
+  if (tiles_64 <= 3 * units && k_tiles > 2)
+    return launch_variant<1, 1, 3, TOut>(a, w, bias, c, m, n, k, lda, ldc, epilogue, scatter, s);
   return launch_variant<1, 1, 2, TOut>(a, w, bias, c, m, n, k, lda, ldc, epilogue, scatter, s);
 }
 
