@@ -69,6 +69,7 @@ extern "C" int ps_linear(const PsLinearArgs* p, void* stream) {
     scatter.kv_heads = p->kv_heads;
     scatter.page_size = p->page_size;
     scatter.num_pages = p->num_pages;
+    scatter.cache_only = p->scatter_only;
     scatter.page_shift = -1;
     if ((p->page_size & (p->page_size - 1)) == 0) {
       scatter.page_shift = 0;

@@ -143,7 +143,8 @@ __device__ inline void store_wave_tile(f32x16 (&acc)[WM][WN], float* region, int
         continue;
       }
       if (full) {
-        store8(out, v);
+        // (eight key or value columns that go to their page and that nobody reads from c)
+        if (!(scatters && pool != nullptr && scatter.cache_only)) store8(out, v);
       } else {
         for (int q = 0; q < 8; ++q)
           if (col0 + q < n) out[q] = from_float<TOut>(v[q]);

@@ -11,6 +11,7 @@ struct KvScatter {
   const int* tok_pos;
   const int* tables;
   int table_width, q_cols, kv_cols, head_dim, kv_heads, page_size, page_shift, num_pages;
+  int cache_only;        // the key and value columns need not be written to the output as well
 };
 
 // The product of the output head may also choose each row's token (the column of its largest

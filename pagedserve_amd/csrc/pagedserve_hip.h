@@ -94,6 +94,10 @@ typedef struct PsLinearArgs {
   void* top_keys;
   int* top_ticket;
   int* top_done;
+  // With a scatter: nobody reads the key and value columns of c (attention takes them from
+  // the pages), so a kernel may leave them unwritten; they are unspecified afterwards.  The
+  // tiled kernel for many rows does, which takes 40 % off what a prompt's QKV product writes.
+  int scatter_only;
 } PsLinearArgs;
 
 int ps_linear(const PsLinearArgs* args, void* stream);

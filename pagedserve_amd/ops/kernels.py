@@ -233,6 +233,7 @@ class _LinearArgs(ctypes.Structure):
         ("norm_out_rows", c_int), ("c_layout", ctypes.POINTER(c_int)),
         ("top_tokens", c_void_p), ("top_keys", c_void_p), ("top_ticket", c_void_p),
         ("top_done", ctypes.POINTER(c_int)),
+        ("scatter_only", c_int),
     ]
 
 
@@ -300,12 +301,14 @@ class TopChoice:
 
 
 def linear(x, w, bias, out, epilogue="none", scatter=None, packed=None, a_packed=False,
-           packed_out=False, choose=None):
+           packed_out=False, choose=None, scatter_only=False):
     """out = epilogue(x w^T + bias) where ``x`` is a tensor or a ``PendingNorm``.
 
     ``scatter = (k_pool, v_pool, tok_item, tok_pos, tables, q_cols, kv_cols)`` also stores the
     key and value columns of a ``[q | k | v]`` output into their cache pages.  ``packed`` is
     ``pack_decode_weight(w)`` or None; the kernels for few rows read it instead of ``w``.
+    ``scatter_only=True`` says that nobody reads the key and value columns of ``out``: a kernel
+    may then leave them unwritten (unspecified afterwards), which the one for many rows does.
 
     Between two products of 17 to 64 rows the activations may travel in the order in which the
     second one's lanes hold them (``csrc/linear.h: packed_offset``).  ``packed_out=True`` allows
@@ -395,6 +398,7 @@ def linear(x, w, bias, out, epilogue="none", scatter=None, packed=None, a_packed
         args.q_cols, args.kv_cols = int(q_cols), int(kv_cols)
         args.head_dim, args.kv_heads = head_dim, kv_heads
         args.page_size, args.num_pages = page_size, pages
+        args.scatter_only = 1 if scatter_only else 0
     layout = c_int(0)
     if packed_out:
         args.c_packed_request = 1

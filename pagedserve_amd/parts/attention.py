@@ -82,7 +82,8 @@ class Attention(Mixer):
             # keys and values go to their pages from the product's own epilogue
             kernels.linear(x, self.qkv_weight, self.qkv_bias, qkv,
                            scatter=(cache.k_pool, cache.v_pool, ctx.tok_item, ctx.positions, tables,
-                                    self.q_cols, self.kv_cols), packed=self.qkv_packed)
+                                    self.q_cols, self.kv_cols), packed=self.qkv_packed,
+                           scatter_only=True)
         else:
             kernels.linear(x, self.qkv_weight, self.qkv_bias, qkv, packed=self.qkv_packed)
             if rotates:

@@ -636,6 +636,18 @@ def test_linear_scatters_keys_and_values(dtype, m, k, geometry):
                        k_ref.view(torch.int16 if dtype == torch.bfloat16 else torch.int32))
     assert torch.equal(v_pool.view(torch.int16 if dtype == torch.bfloat16 else torch.int32),
                        v_ref.view(torch.int16 if dtype == torch.bfloat16 else torch.int32))
+    # a caller that reads keys and values from the pages alone: the query columns and the
+    # pages are the same, the other columns may stay as they were
+    k_pool.zero_()
+    v_pool.zero_()
+    k_ref.zero_()
+    v_ref.zero_()
+    kernels.kv_write(plain[:, q_cols:q_cols + kv_cols], plain[:, q_cols + kv_cols:], k_ref, v_ref, tok_item, tok_pos, tables)
+    out = torch.zeros_like(plain)
+    kernels.linear(x, w, bias, out, scatter=(k_pool, v_pool, tok_item, tok_pos, tables, q_cols, kv_cols),
+                   scatter_only=True)
+    torch.testing.assert_close(out[:, :q_cols], plain[:, :q_cols], atol=0, rtol=0)
+    assert torch.equal(k_pool, k_ref) and torch.equal(v_pool, v_ref)
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
