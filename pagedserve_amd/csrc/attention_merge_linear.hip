@@ -12,8 +12,8 @@
 // ways: blocks of 16 columns with the heads spread over their waves are slower than the merge
 // kernel they replace).  Here the projection is split over the heads instead: block (c, h) is
 // one wave that merges head h of all rows (each lane the 16 values of its own row that it
-// needs as matrix-core operand, so no lane talks to another, and the loads of all ranges are
-// in flight together), multiplies them with the piece of W that belongs to its columns and to
+// needs as matrix-core operand; with fewer than 9 rows the lanes of the free operand columns
+// take a share of the ranges each and exchange their sums), multiplies them with the piece of W that belongs to its columns and to
 // head h (out of the packed copy of W, pagedserve_hip.h), and adds the result into the float
 // residual rows with atomic adds; the blocks of head 0 add the bias.  The sum over heads is
 // therefore made by the adds, in an order that differs from run to run within float rounding,
@@ -22,19 +22,30 @@
 
 typedef __attribute__((__vector_size__(4 * sizeof(float)))) float f32x4_t;
 
-template <int STEPS, int TILES>   // head_dim / 64; tiles of 16 columns per block
+template <int STEPS, int PARTS>   // head_dim / 64; lanes that share the ranges of a row
 __global__ __launch_bounds__(64) void attention_merge_linear_kernel(
     const float* __restrict__ partial, const int* __restrict__ tok_list, int count, int heads,
     int splits, const bf16_t* __restrict__ wp, const float* __restrict__ bias,
     float* __restrict__ residual, int64_t ld_res, int n) {
+  constexpr int TILES = 1;             // tiles of 16 columns per block (two measured slower)
+  constexpr int rows_pow2 = 16 / PARTS;
+  constexpr int parts = PARTS;
   constexpr int HEAD_DIM = STEPS * 64;
   constexpr int STRIDE = HEAD_DIM + 2;
   const int lane = threadIdx.x;
-  const int row = lane & 15;           // activation row (token of the step)
+  const int column = lane & 15;        // column of the matrix-core operand: a row of the step
   const int group = lane >> 4;         // which 16 of every 64 head dimensions
   const int head = blockIdx.y;
-  const bool has_row = row < count;
-  const int safe_row = has_row ? row : 0;
+  // Fewer rows than 16 leave operand columns free: they take a share of the ranges of the rows
+  // that are there (row = column mod rows_pow2, the smallest power of two that holds the
+  // rows; the column's other bits pick every parts-th range), and the shares are merged by
+  // lane exchanges afterwards.  One row with 64 ranges then costs four records per lane
+  // instead of 64.
+  const int row = column & (rows_pow2 - 1);
+  const int part = column / rows_pow2;
+  const bool has_row = column < count;       // this lane's results are stored
+  const bool merges = row < count;
+  const int safe_row = merges ? row : 0;
   const float* records = partial + ((int64_t)safe_row * heads + head) * splits * STRIDE;
 
   // the pieces of W: tiles of 16 columns, k steps head * STEPS ..., element
@@ -67,7 +78,7 @@ __global__ __launch_bounds__(64) void attention_merge_linear_kernel(
 #pragma unroll
       for (int e = 0; e < 8; ++e) value[st][h][e] = 0.f;
 #pragma unroll 4
-  for (int s = 0; s < splits; ++s) {
+  for (int s = part; s < splits; s += parts) {
     const float* record = records + s * STRIDE;
     const float m_s = record[HEAD_DIM];
     const float l_s = record[HEAD_DIM + 1];
@@ -97,7 +108,25 @@ __global__ __launch_bounds__(64) void attention_merge_linear_kernel(
         }
     total_m = new_m;
   }
-  const float inverse = (has_row && total_l > 0.f) ? 1.f / total_l : 0.f;
+  // the shares of a row: lanes whose column differs in the bits above the row's
+#pragma unroll
+  for (int offset = rows_pow2; offset < 16; offset <<= 1) {
+    const float other_m = __shfl_xor(total_m, offset, 64);
+    const float other_l = __shfl_xor(total_l, offset, 64);
+    const float new_m = fmaxf(total_m, other_m);
+    const float keep = (total_m == -INFINITY) ? 0.f : __builtin_amdgcn_exp2f(total_m - new_m);
+    const float weight = (other_m == -INFINITY) ? 0.f : __builtin_amdgcn_exp2f(other_m - new_m);
+    total_l = total_l * keep + other_l * weight;
+#pragma unroll
+    for (int st = 0; st < STEPS; ++st)
+#pragma unroll
+      for (int h = 0; h < 2; ++h)
+#pragma unroll
+        for (int e = 0; e < 8; ++e)
+          value[st][h][e] = fmaf(__shfl_xor(value[st][h][e], offset, 64), weight, value[st][h][e] * keep);
+    total_m = new_m;
+  }
+  const float inverse = (merges && total_l > 0.f) ? 1.f / total_l : 0.f;
 
   f32x4_t acc[TILES];
 #pragma unroll
@@ -118,7 +147,7 @@ __global__ __launch_bounds__(64) void attention_merge_linear_kernel(
     }
   // element i of lane l: column (l / 16) * 4 + i of the tile, row l % 16
   if (!has_row) return;
-  const int t = tok_list ? tok_list[row] : row;
+  const int t = tok_list ? tok_list[column] : column;
 #pragma unroll
   for (int c = 0; c < TILES; ++c)
 #pragma unroll
@@ -135,7 +164,7 @@ bool ps_attention_merge_linear_supported(int count, int head_dim, int dtype) {
   return dtype == PS_BF16 && count >= 1 && count <= 16 && head_dim % 64 == 0 && head_dim <= 256;
 }
 
-// tiles_per_block: 16-column tiles that one wave computes (1 or 2; 0 lets the sizes decide)
+// tiles_per_block: 16-column tiles that one wave computes (0 or 1: one; two measured slower)
 extern "C" int ps_attention_merge_linear(const float* partial, int64_t partial_floats,
                                          const int* tok_list, int count, int heads, int head_dim,
                                          int splits, const void* w_packed, const float* bias,
@@ -155,32 +184,38 @@ extern "C" int ps_attention_merge_linear(const float* partial, int64_t partial_f
                  (reinterpret_cast<uintptr_t>(w_packed) & 15u) == 0 &&
                  (reinterpret_cast<uintptr_t>(partial) & 7u) == 0,
              "ps_attention_merge_linear: null or unaligned operand");
-  PS_REQUIRE(tiles_per_block >= 0 && tiles_per_block <= 2,
-             "ps_attention_merge_linear: one or two tiles per block, not %d", tiles_per_block);
+  PS_REQUIRE(tiles_per_block >= 0 && tiles_per_block <= 1,
+             "ps_attention_merge_linear: one tile of 16 columns per block, not %d", tiles_per_block);
   if (count == 0) return 0;
   if (tiles_per_block == 0) tiles_per_block = 1;
   const int tiles_n = (n + 15) / 16;
   dim3 grid((tiles_n + tiles_per_block - 1) / tiles_per_block, heads);
   hipStream_t s = (hipStream_t)stream;
-#define PS_LAUNCH_AML(STEPS, TILES)                                                               \
-  hipLaunchKernelGGL((attention_merge_linear_kernel<STEPS, TILES>), grid, dim3(64), 0, s, partial, \
+  // shares of the ranges for the free operand columns where there are many ranges (up to 8
+  // ranges a lane has them all in flight at once, and shares measured no faster)
+  int rows_pow2 = 1;
+  while (rows_pow2 < count) rows_pow2 <<= 1;
+  if (splits <= 8) rows_pow2 = 16;
+  const int parts = 16 / rows_pow2;
+#define PS_LAUNCH_AML(STEPS, PARTS)                                                               \
+  hipLaunchKernelGGL((attention_merge_linear_kernel<STEPS, PARTS>), grid, dim3(64), 0, s, partial, \
                      tok_list, count, heads, splits, (const bf16_t*)w_packed, bias, residual,     \
                      ld_res, n)
-#define PS_LAUNCH_AMLT(STEPS)         \
-  do {                                \
-    if (tiles_per_block == 2) {       \
-      PS_LAUNCH_AML(STEPS, 2);        \
-    } else {                          \
-      PS_LAUNCH_AML(STEPS, 1);        \
-    }                                 \
+#define PS_LAUNCH_AMLP(STEPS)                     \
+  do {                                            \
+    if (parts == 1) PS_LAUNCH_AML(STEPS, 1);      \
+    else if (parts == 2) PS_LAUNCH_AML(STEPS, 2); \
+    else if (parts == 4) PS_LAUNCH_AML(STEPS, 4); \
+    else if (parts == 8) PS_LAUNCH_AML(STEPS, 8); \
+    else PS_LAUNCH_AML(STEPS, 16);                \
   } while (0)
   switch (head_dim / 64) {
-    case 1: PS_LAUNCH_AMLT(1); break;
-    case 2: PS_LAUNCH_AMLT(2); break;
-    case 3: PS_LAUNCH_AMLT(3); break;
-    default: PS_LAUNCH_AMLT(4); break;
+    case 1: PS_LAUNCH_AMLP(1); break;
+    case 2: PS_LAUNCH_AMLP(2); break;
+    case 3: PS_LAUNCH_AMLP(3); break;
+    default: PS_LAUNCH_AMLP(4); break;
   }
-#undef PS_LAUNCH_AMLT
+#undef PS_LAUNCH_AMLP
 #undef PS_LAUNCH_AML
   PS_CHECK_LAUNCH("ps_attention_merge_linear");
   return 0;

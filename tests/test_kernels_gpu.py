@@ -854,8 +854,8 @@ def test_linear_takes_the_wide_product_for_long_k():
 
 
 @pytest.mark.parametrize("heads,kv_heads,head_dim,page_size", [(12, 12, 64, 16), (4, 2, 128, 12), (2, 1, 256, 16), (3, 3, 192, 8)])
-@pytest.mark.parametrize("count", [1, 8, 16])
-@pytest.mark.parametrize("splits", [1, 3, 8])
+@pytest.mark.parametrize("count", [1, 2, 3, 5, 8, 16])
+@pytest.mark.parametrize("splits", [1, 3, 8, 20, 64])
 def test_attention_records_merged_inside_the_output_projection(heads, kv_heads, head_dim, page_size, count, splits):
     """Decode attention that leaves only its per-range records, and the output projection that
     merges them head by head: residual + softmax(q K^T) V W^T + bias in float64 over the
