@@ -162,6 +162,73 @@ def test_long_decoding(folders, dtype):
         engine.step([StepEntry("r", [1], [0])])          # the position table is exhausted
 
 
+LONG = {
+    "architectures": ["GPT2LMHeadModel"], "model_type": "gpt2",
+    "n_layer": 2, "n_embd": 128, "n_head": 2, "n_inner": 192, "vocab_size": 97,
+    "n_positions": 3072, "layer_norm_epsilon": 1e-5, "activation_function": "gelu_new",
+    "scale_attn_by_inverse_layer_idx": False, "tie_word_embeddings": True, "eos_token_id": None,
+}
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_decoding_over_long_contexts(tmp_path, dtype, monkeypatch):
+    """Contexts of 2,900 and 1,500 tokens (heads of 64): prompts in portions, then tokens
+    decoded one by one, first for one request, then for both together.  With so many keys per
+    request the decode kernel cuts them into more than twenty ranges, which in bfloat16 the
+    output projection merges with the ranges of a row shared among its lanes."""
+    from pagedserve_amd.engine import Engine, StepEntry
+    from pagedserve_amd.model import load_model
+    from pagedserve_amd.ops import kernels
+
+    merged = []
+    merge = kernels.attention_merge_linear
+
+    def recording(partial, count, heads, head_dim, splits, *args, **kwargs):
+        merged.append((count, splits))
+        return merge(partial, count, heads, head_dim, splits, *args, **kwargs)
+
+    monkeypatch.setattr(kernels, "attention_merge_linear", recording)
+    folder = helpers.write_folder(os.path.join(str(tmp_path), "long"), LONG, helpers.lively_tensors(LONG, 9))
+    lengths = {"far": 2900, "near": 1500}
+    decoded = 24
+    tokens = {name: helpers.random_tokens(n + decoded, LONG["vocab_size"], 520 + i)
+              for i, (name, n) in enumerate(lengths.items())}
+    reference = {name: helpers.plain_logits(folder, tokens[name], bfloat16=dtype == "bfloat16") for name in tokens}
+    model, _ = load_model(folder, dtype=dtype)
+    engine = Engine(model, num_pages=(2900 + 1500 + 2 * decoded) // 16 + 4, page_size=16, max_requests=2,
+                    max_step_tokens=1024)
+    worst = 0.0
+
+    def check(out, places):
+        nonlocal worst
+        values = out.logits.double().cpu()
+        for row, (name, position) in enumerate(places):
+            worst = max(worst, float((values[row] - reference[name][position]).abs().max()))
+
+    for name, length in lengths.items():
+        for begin in range(0, length, 1024):
+            part = tokens[name][begin:min(begin + 1024, length)]
+            last = begin + len(part) == length
+            out = engine.step([StepEntry(name, part, [len(part) - 1] if last else [])])
+            if last:
+                check(out, [(name, length - 1)])
+    held = dict(lengths)
+    for step in range(decoded):
+        names = ["far"] if step < 8 else ["far", "near"]
+        out = engine.step([StepEntry(name, [tokens[name][held[name]]], [0]) for name in names])
+        check(out, [(name, held[name]) for name in names])
+        for name in names:
+            held[name] += 1
+    scale = max(float(reference[name].abs().max()) for name in reference)
+    assert worst <= helpers.TOLERANCE[dtype] * scale, (worst, scale)
+    engine.cache.check_invariants()
+    if dtype == "bfloat16":
+        # (launches that were recorded into graphs are counted once)
+        assert {count for count, _ in merged} == {1, 2} and min(splits for _, splits in merged) > 8, merged
+    else:
+        assert not merged
+
+
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 def test_first_tokens_of_a_sequence(folders, dtype):
     """Positions 0, 1, 2 in every arrangement: alone, one by one, and beside another request."""
