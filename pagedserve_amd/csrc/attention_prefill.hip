@@ -27,7 +27,7 @@
 //     delivers from the row-major tile: within 16 lanes, lane r points at 4 dimensions of key
 //     r / 4 and receives dimension r of four keys.
 //
-// head_dim is any multiple of 16 up to 128; other sizes, and block tables wider than
+// head_dim is any multiple of 16 up to 256; other sizes, and block tables wider than
 // AP_TABLE_MAX pages, run on the row-wise kernel.
 #include <math.h>
 
@@ -72,6 +72,7 @@ __global__ __launch_bounds__(128 * KS) void attention_prefill_kernel(
   // 12 heads: 1.5 us less per launch).
   constexpr int FIT = (KS >= 4 ? 65536 : 98304) / STAGE_BYTES;
   constexpr int STAGES = FIT >= 4 ? 4 : (FIT >= 2 ? FIT : 2);
+  static_assert(NDB <= 8 || STAGES == 2, "head sizes beyond 128 rely on a ring of two stages");
   constexpr int INSTRUCTIONS = KS * NDB;         // load instructions per operand and stage
   // every wave issues the same number of loads (the counter of loads in flight is per wave):
   // where they do not divide evenly the last ones are issued twice
@@ -249,19 +250,43 @@ __global__ __launch_bounds__(128 * KS) void attention_prefill_kernel(
     u32x4 kr[NDB];
     u32x2 vr[2][NDB32][2];
     if (active) {
+      if constexpr (NDB <= 8) {
 #pragma unroll
-      for (int step = 0; step < NDB; ++step)
-        asm volatile("ds_read_b128 %0, %1" : "=v"(kr[step]) : "v"(stage_base + k_off[step]) : "memory");
+        for (int step = 0; step < NDB; ++step)
+          asm volatile("ds_read_b128 %0, %1" : "=v"(kr[step]) : "v"(stage_base + k_off[step]) : "memory");
 #pragma unroll
-      for (int run = 0; run < 2; ++run)
+        for (int run = 0; run < 2; ++run)
 #pragma unroll
-        for (int db = 0; db < NDB32; ++db)
+          for (int db = 0; db < NDB32; ++db)
 #pragma unroll
-          for (int second = 0; second < 2; ++second)
-            asm volatile("ds_read_b64_tr_b16 %0, %1"
-                         : "=v"(vr[run][db][second])
-                         : "v"(stage_base + v_off[run][db][second])
-                         : "memory");
+            for (int second = 0; second < 2; ++second)
+              asm volatile("ds_read_b64_tr_b16 %0, %1"
+                           : "=v"(vr[run][db][second])
+                           : "v"(stage_base + v_off[run][db][second])
+                           : "memory");
+      } else {
+        // Head sizes beyond 128 need more registers than a wave's 256 vector registers: the
+        // compiler then moves values to the accumulation registers where it sees fit, also a
+        // register that an assembly read above has not yet filled.  Here the reads are the
+        // compiler's own (it waits for them itself, and for every load in flight before them,
+        // which costs nothing with a ring of two stages: none is in flight at this point).
+        typedef short ap_i16x4 __attribute__((ext_vector_type(4)));
+#pragma unroll
+        for (int step = 0; step < NDB; ++step)
+          kr[step] = *reinterpret_cast<const __attribute__((address_space(3))) u32x4*>(
+              (uintptr_t)(stage_base + k_off[step]));
+#pragma unroll
+        for (int run = 0; run < 2; ++run)
+#pragma unroll
+          for (int db = 0; db < NDB32; ++db)
+#pragma unroll
+            for (int second = 0; second < 2; ++second) {
+              const ap_i16x4 raw = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
+                  reinterpret_cast<__attribute__((address_space(3))) ap_i16x4*>(
+                      (uintptr_t)(stage_base + v_off[run][db][second])));
+              vr[run][db][second] = *reinterpret_cast<const u32x2*>(&raw);
+            }
+      }
     }
     // Everything read by assembly is waited for before the compiler's own code goes on (it
     // does not know that those registers are still on their way).
@@ -408,8 +433,8 @@ extern "C" int ps_attention_prefill(const void* q, int64_t q_stride, const void*
   PS_REQUIRE(dtype == PS_BF16, "ps_attention_prefill: bfloat16 only (dtype %d)", dtype);
   PS_REQUIRE(heads % kv_heads == 0,
              "ps_attention_prefill: heads (%d) must be a multiple of kv_heads (%d)", heads, kv_heads);
-  PS_REQUIRE(head_dim > 0 && head_dim % 16 == 0 && head_dim <= 128,
-             "ps_attention_prefill: head_dim %d must be a multiple of 16 up to 128", head_dim);
+  PS_REQUIRE(head_dim > 0 && head_dim % 16 == 0 && head_dim <= 256,
+             "ps_attention_prefill: head_dim %d must be a multiple of 16 up to 256", head_dim);
   PS_REQUIRE(window >= 0 && tiles <= 65535, "ps_attention_prefill: bad window or too many tiles (%d)", tiles);
   PS_REQUIRE(scale > 0.f, "ps_attention_prefill: the score scale must be positive, got %g", scale);
   PS_REQUIRE(table_width <= AP_TABLE_MAX,
@@ -455,7 +480,23 @@ extern "C" int ps_attention_prefill(const void* q, int64_t q_stride, const void*
     case 5: PS_LAUNCH_AP(5); break;
     case 6: PS_LAUNCH_AP(6); break;
     case 7: PS_LAUNCH_AP(7); break;
-    default: PS_LAUNCH_AP(8); break;
+    case 8: PS_LAUNCH_AP(8); break;
+    // head sizes beyond 128: blocks of four waves only, each wave with the whole register
+    // file of its SIMD (accumulators and operands of 256 dimensions take 450 registers)
+#define PS_LAUNCH_AP_LARGE(NDB)                                                                 \
+  hipLaunchKernelGGL((attention_prefill_kernel<NDB, 2>), grid, dim3(256), 0, s,                 \
+                     (const bf16_t*)q, q_stride, (const bf16_t*)k_pool, (const bf16_t*)v_pool,  \
+                     (bf16_t*)out, out_stride, tile_item, tile_q0, cu_tokens, kv_lens, tables,  \
+                     table_width, heads, kv_heads, page_size, page_shift, num_pages, scale, window)
+    case 9: PS_LAUNCH_AP_LARGE(9); break;
+    case 10: PS_LAUNCH_AP_LARGE(10); break;
+    case 11: PS_LAUNCH_AP_LARGE(11); break;
+    case 12: PS_LAUNCH_AP_LARGE(12); break;
+    case 13: PS_LAUNCH_AP_LARGE(13); break;
+    case 14: PS_LAUNCH_AP_LARGE(14); break;
+    case 15: PS_LAUNCH_AP_LARGE(15); break;
+    default: PS_LAUNCH_AP_LARGE(16); break;
+#undef PS_LAUNCH_AP_LARGE
   }
 #undef PS_LAUNCH_AP
   PS_CHECK_LAUNCH("ps_attention_prefill");

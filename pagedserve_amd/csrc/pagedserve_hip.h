@@ -172,7 +172,7 @@ int ps_attention_decode_static(const void* q, int64_t q_stride, const void* k_po
                                void* stream);
 
 // Tiled attention on the matrix cores for items that bring several tokens (bfloat16, head_dim a
-// multiple of 16 up to 128).  Tile i covers queries tile_q0[i] .. tile_q0[i] + 63 of item
+// multiple of 16 up to 256).  Tile i covers queries tile_q0[i] .. tile_q0[i] + 63 of item
 // tile_item[i]; cu_tokens and kv_lens describe the step's items.  Blocks start in the order of
 // the list (all heads of tile 0, then of tile 1, ...): list the tiles that see the most keys first.
 // max_kv_len: no query sees more keys than that (0: unknown); it only steers the launch shape.

@@ -609,7 +609,7 @@ PREFILL_TABLE_MAX = 2048
 def prefill_supported(dtype, head_dim, table_width=0) -> bool:
     """Whether the tiled matrix-core kernel takes this storage type, head size and width of
     the block tables (it keeps a tile's table entries in LDS)."""
-    return (dtype == torch.bfloat16 and head_dim % 16 == 0 and head_dim <= 128
+    return (dtype == torch.bfloat16 and head_dim % 16 == 0 and head_dim <= 256
             and table_width <= PREFILL_TABLE_MAX)
 
 

@@ -492,7 +492,9 @@ def test_kernels_refuse_bad_sizes():
 
 @pytest.mark.parametrize("heads,kv_heads,head_dim,page_size", [(1, 1, 32, 16), (4, 4, 16, 8), (6, 2, 48, 16), (2, 2, 128, 4), (12, 12, 64, 16), (3, 1, 80, 12),
                                                                 # more than 256 blocks: the kernel's other arrangement of waves
-                                                                (24, 8, 64, 16), (20, 20, 48, 8), (18, 18, 112, 16)])
+                                                                (24, 8, 64, 16), (20, 20, 48, 8), (18, 18, 112, 16),
+                                                                # head sizes beyond 128: blocks of four waves only
+                                                                (2, 1, 256, 16), (3, 3, 192, 8), (2, 2, 144, 12), (12, 4, 160, 16), (1, 1, 208, 16)])
 @pytest.mark.parametrize("window", [0, 37])
 def test_attention_prefill_tiles(heads, kv_heads, head_dim, page_size, window):
     """The tiled kernel against float64 attention over the gathered pages: fresh prompts and later portions of many
