@@ -5,8 +5,10 @@ Options keep the reference's names and meanings where it has them (``--strategy`
 ``--kv-cache-memory-utilization``, ``--kv-cache-safety-mb``, ``--dtype``); ``--model`` is a
 model folder (or ``reference`` for a small random model) instead of a fixed list of names,
 and ``--disable-hip-graphs`` takes the place of ``--disable-cuda-graphs`` (also accepted).
-There is one attention implementation and no quantized cache, so the reference's
-``--decode-attention-backend`` and ``--kv-cache-dtype`` have nothing to choose.
+There is one attention implementation and no quantized cache: the reference's
+``--decode-attention-backend`` is accepted with its values (``torch``, ``triton``) so that its
+command lines keep working, and every value runs the HIP kernels; ``--kv-cache-dtype`` takes
+``model`` only and refuses ``int8`` with a message.
 """
 
 import argparse
@@ -18,6 +20,8 @@ from pagedserve_amd.engine.scheduler import ORCA_STRATEGY, SUPPORTED_SCHEDULING_
 from pagedserve_amd.sampling.params import SamplingParams
 
 SUPPORTED_DTYPES = ("float32", "bfloat16")
+SUPPORTED_DECODE_ATTENTION_BACKENDS = ("hip", "torch", "triton")   # main.py:27 of the reference, plus ours
+SUPPORTED_KV_CACHE_DTYPES = ("model", "int8")                      # main.py:28
 
 
 def parse_args(argv=None):
@@ -41,6 +45,12 @@ def parse_args(argv=None):
     parser.add_argument("--num-kv-pages", type=int, help="explicit number of KV pages")
     parser.add_argument("--block-size", type=int, default=16, help="tokens per KV page")
     parser.add_argument("--dtype", choices=SUPPORTED_DTYPES, default="float32", help="execution dtype")
+    parser.add_argument("--decode-attention-backend", choices=SUPPORTED_DECODE_ATTENTION_BACKENDS,
+                        default="hip",
+                        help="accepted for the reference's command lines; every value runs the "
+                             "HIP kernels")
+    parser.add_argument("--kv-cache-dtype", choices=SUPPORTED_KV_CACHE_DTYPES, default="model",
+                        help="KV storage dtype: the model's (quantized caches are not built)")
     parser.add_argument("--disable-hip-graphs", "--disable-cuda-graphs", dest="disable_hip_graphs",
                         action="store_true", help="disable HIP-graph replay of decode steps")
     parser.add_argument("--random-weights", action="store_true",
@@ -53,7 +63,13 @@ def parse_args(argv=None):
     parser.add_argument("--temperature", type=float, default=0.0, help="0 = greedy")
     parser.add_argument("--sample-seed", type=int, help="seed of temperature sampling")
     parser.add_argument("--ignore-eos", action="store_true")
-    return parser.parse_args(argv)
+    args = parser.parse_args(argv)
+    if args.kv_cache_dtype != "model":
+        parser.error("--kv-cache-dtype int8: quantized caches are not built; the cache has the model's dtype")
+    if args.decode_attention_backend != "hip":
+        print(f"note: --decode-attention-backend {args.decode_attention_backend} runs the HIP kernels, "
+              "the only implementation here", file=sys.stderr)
+    return args
 
 
 def main(argv=None):

@@ -463,3 +463,27 @@ def test_arrival_trace_runner_times_requests_by_its_clock():
     for index, request in enumerate(requests):
         assert scheduler.finished[records[index].request_id].generated_token_ids == \
             expected_tokens(list(request.prompt_token_ids), request.max_new_tokens)
+
+
+def test_command_line_takes_the_reference_options(capsys):
+    """Option names of the reference's main.py:257-342; its two backend options are accepted as
+    far as they mean something here."""
+    import os
+    import sys
+
+    sys.path.insert(0, os.path.dirname(os.path.dirname(os.path.abspath(__file__))))
+    import main
+
+    args = main.parse_args(["--model", "reference", "--strategy", "sarathi", "--prefill-chunk-size", "32",
+                            "--max-batch-size", "4", "--kv-cache-memory-mb", "64",
+                            "--kv-cache-memory-utilization", "0.5", "--kv-cache-safety-mb", "128",
+                            "--dtype", "bfloat16", "--decode-attention-backend", "triton",
+                            "--kv-cache-dtype", "model", "--disable-cuda-graphs"])
+    assert args.strategy == "sarathi" and args.prefill_chunk_size == 32 and args.max_batch_size == 4
+    assert args.kv_cache_memory_mb == 64 and args.disable_hip_graphs and args.dtype == "bfloat16"
+    assert "HIP kernels" in capsys.readouterr().err
+    with pytest.raises(SystemExit):
+        main.parse_args(["--kv-cache-dtype", "int8"])
+    assert "quantized caches are not built" in capsys.readouterr().err
+    with pytest.raises(SystemExit):
+        main.parse_args(["--decode-attention-backend", "flash"])
