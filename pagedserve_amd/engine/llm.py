@@ -46,9 +46,25 @@ def build_scheduler(model=REFERENCE_MODEL, scheduling_strategy=ORCA_STRATEGY, pr
                     kv_cache_safety_mb=DEFAULT_KV_SAFETY_MB, execution_dtype="float32",
                     enable_hip_graphs=True, block_size=16, num_kv_pages=None,
                     max_num_batched_tokens=None, max_prefill_requests=None, random_weights=False,
-                    seed=0, eos_token_id="config"):
+                    seed=0, eos_token_id="config", model_name=None, enable_cuda_graphs=None,
+                    decode_attention_backend="hip", kv_cache_dtype="model"):
     """Load ``model`` (a folder, or ``"reference"`` for a small random model) and return a
-    ``ContinuousBatchScheduler`` ready for ``add_request`` / ``run_until_complete``."""
+    ``ContinuousBatchScheduler`` ready for ``add_request`` / ``run_until_complete``.
+
+    The reference's names for the same things are taken as well (main.py:136-150):
+    ``model_name`` for ``model``, ``enable_cuda_graphs`` for ``enable_hip_graphs``; its
+    ``decode_attention_backend`` values all run the HIP kernels, and ``kv_cache_dtype`` can
+    only be ``"model"`` (quantized caches are not built)."""
+    if model_name is not None:
+        model = model_name
+    if enable_cuda_graphs is not None:
+        enable_hip_graphs = bool(enable_cuda_graphs)
+    if decode_attention_backend not in ("hip", "torch", "triton"):
+        raise ValueError(f"Unknown decode attention backend '{decode_attention_backend}'. "
+                         "Choose one of: hip, torch, triton (all run the HIP kernels)")
+    if kv_cache_dtype != "model":
+        raise ValueError(f"KV cache dtype '{kv_cache_dtype}': quantized caches are not built; "
+                         "the cache has the model's dtype ('model')")
     if not torch.cuda.is_available():
         raise RuntimeError("pagedserve_amd needs a GPU (MI355X); there is no CPU path")
     dtype = resolve_dtype(execution_dtype)

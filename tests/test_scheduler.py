@@ -487,3 +487,15 @@ def test_command_line_takes_the_reference_options(capsys):
     assert "quantized caches are not built" in capsys.readouterr().err
     with pytest.raises(SystemExit):
         main.parse_args(["--decode-attention-backend", "flash"])
+
+
+def test_python_entry_takes_the_reference_keyword_names():
+    """build_scheduler(model_name=..., enable_cuda_graphs=..., decode_attention_backend=...,
+    kv_cache_dtype=...) of the reference's main.py:136-150; what cannot be had is refused
+    before anything is loaded."""
+    from pagedserve_amd.engine.llm import build_scheduler
+
+    with pytest.raises(ValueError, match="quantized caches are not built"):
+        build_scheduler(model_name="reference", kv_cache_dtype="int8")
+    with pytest.raises(ValueError, match="Unknown decode attention backend"):
+        build_scheduler(model_name="reference", decode_attention_backend="flash")
