@@ -124,16 +124,32 @@ __global__ __launch_bounds__(256) void gemm_nt_bf16_tiled_kernel(
   // across tiles: before the last step of a tile the wave waits for the next tile's loads
   // and meets the other waves, with three steps' products already queued in the matrix core,
   // then fetches the next tile's first operands.
-  bf16x8 fa[2][WM], fw[2][WN];
-  auto fetch = [&](int kt, int s, bf16x8* da, bf16x8* dw) {
-    const unsigned char* stage = lds + (kt % STAGES) * STAGE_BYTES;
-    const int slot = ((2 * s + (lane >> 5)) ^ key) << 4;
+  //
+  // The reads are written as assembly with counted waits.  Left to itself the compiler waits
+  // for every LDS read in flight (lgkmcnt(0)) before each product, the ones it has just issued
+  // for the next step included, so that every step paid a whole trip to LDS and a k tile of a
+  // lone block took 800 cycles, of which the matrix instructions are 128.  LDS reads come back
+  // in the order of issue: waiting until READS are left in flight leaves exactly the next
+  // step's.
+  typedef unsigned int tb_u32x4 __attribute__((ext_vector_type(4)));
+  constexpr int READS = WM + WN;    // LDS reads of one k step
+  tb_u32x4 fa[2][WM], fw[2][WN];
+  const uint32_t lds_base = (uint32_t)(uintptr_t)(lds_ptr_t)lds;
+  auto fetch = [&](int kt, int s, tb_u32x4* da, tb_u32x4* dw) {
+    const uint32_t stage = lds_base + (uint32_t)((kt % STAGES) * STAGE_BYTES);
+    const uint32_t slot = (uint32_t)(((2 * s + (lane >> 5)) ^ key) << 4);
 #pragma unroll
     for (int i = 0; i < WM; ++i)
-      da[i] = *reinterpret_cast<const bf16x8*>(stage + a_row + i * 32 * TB_ROW + slot);
+      asm volatile("ds_read_b128 %0, %1"
+                   : "=v"(da[i])
+                   : "v"(stage + (uint32_t)(a_row + i * 32 * TB_ROW) + slot)
+                   : "memory");
 #pragma unroll
     for (int j = 0; j < WN; ++j)
-      dw[j] = *reinterpret_cast<const bf16x8*>(stage + w_row + j * 32 * TB_ROW + slot);
+      asm volatile("ds_read_b128 %0, %1"
+                   : "=v"(dw[j])
+                   : "v"(stage + (uint32_t)(w_row + j * 32 * TB_ROW) + slot)
+                   : "memory");
   };
   constexpr int STEPS = TB_BK / 16;
   static_assert(STEPS % 2 == 0, "the operand buffers alternate per step");
@@ -154,6 +170,7 @@ __global__ __launch_bounds__(256) void gemm_nt_bf16_tiled_kernel(
     for (int s = 0; s < STEPS; ++s) {
       if (s + 1 < STEPS) {
         fetch(kt, s + 1, fa[(s + 1) & 1], fw[(s + 1) & 1]);
+        asm volatile("s_waitcnt lgkmcnt(%0)" ::"n"(READS) : "memory");   // step s has arrived
       } else if (kt + 1 < k_tiles) {
         // own reads of this tile are complete before the others may overwrite its stage
         asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
@@ -161,13 +178,22 @@ __global__ __launch_bounds__(256) void gemm_nt_bf16_tiled_kernel(
         const int last = k_tiles - 1 < kt + STAGES - 1 ? k_tiles - 1 : kt + STAGES - 1;
         wait_ahead_and_sync<LOADS, STAGES - 2>(last - (kt + 1));
         fetch(kt + 1, 0, fa[0], fw[0]);
+      } else {
+        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
       }
+      // the registers are used only behind the wait (the compiler does not know that the
+      // assembly above left them on their way)
+#pragma unroll
+      for (int i = 0; i < WM; ++i) asm volatile("" : "+v"(fa[s & 1][i]));
+#pragma unroll
+      for (int j = 0; j < WN; ++j) asm volatile("" : "+v"(fw[s & 1][j]));
 #pragma unroll
       for (int i = 0; i < WM; ++i)
 #pragma unroll
         for (int j = 0; j < WN; ++j)
-          acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa[s & 1][i], fw[s & 1][j],
-                                                              acc[i][j], 0, 0, 0);
+          acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(
+              *reinterpret_cast<const bf16x8*>(&fa[s & 1][i]),
+              *reinterpret_cast<const bf16x8*>(&fw[s & 1][j]), acc[i][j], 0, 0, 0);
     }
   }
 
