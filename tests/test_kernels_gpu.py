@@ -492,12 +492,16 @@ def test_kernels_refuse_bad_sizes():
 
 @pytest.mark.parametrize("heads,kv_heads,head_dim,page_size", [(1, 1, 32, 16), (4, 4, 16, 8), (6, 2, 48, 16), (2, 2, 128, 4), (12, 12, 64, 16), (3, 1, 80, 12),
                                                                 # more than 256 blocks: the kernel's other arrangement of waves
-                                                                (24, 8, 64, 16), (20, 20, 48, 8), (18, 18, 112, 16),
+                                                                (24, 8, 64, 16), (20, 20, 48, 8), (18, 18, 112, 16), (26, 13, 128, 16), (26, 26, 96, 8),
+                                                                (26, 26, 16, 8), (26, 13, 32, 16), (28, 7, 80, 16), (2, 2, 96, 8), (3, 1, 112, 16),
                                                                 # head sizes beyond 128: blocks of four waves only
                                                                 (2, 1, 256, 16), (3, 3, 192, 8), (2, 2, 144, 12), (12, 4, 160, 16), (1, 1, 208, 16)])
 @pytest.mark.parametrize("window", [0, 37])
 def test_attention_prefill_tiles(heads, kv_heads, head_dim, page_size, window):
-    """The tiled kernel against float64 attention over the gathered pages: fresh prompts and later portions of many
+    """The tiled kernel against float64 attention over the gathered pages (every head size in
+    steps of 16 up to 128 in both arrangements of waves, larger ones in the one they have: the
+    kernel reads LDS by assembly into registers that the compiler must leave alone until the
+    wait, which a run of every variant checks): fresh prompts and later portions of many
     lengths in one launch (1 < count, portions that start inside a page, more than one tile,
     a tile's last rows empty), fragmented tables, NaN behind every request's last key."""
     from pagedserve_amd.ops import kernels
