@@ -274,7 +274,9 @@ static int launch_wide(const void* a, const void* wp, const float* bias, void* c
   return 0;
 }
 
-// rows_per_block: 128, 64 or 32; 0 lets the number of tiles decide
+// rows_per_block: 64 or 32; 0 means 64.  (Blocks of 128 rows measured no faster and need
+// more than a wave's 256 vector registers: the compiler then parks values in accumulation
+// registers, also weight fragments that the assembly loads have not yet delivered.)
 int ps_gemm_nt_bf16_wide(const void* a, const void* w_packed, const float* bias, void* c, int m,
                          int n, int k, int lda, int ldc, int c_dtype, int epilogue,
                          const KvScatter& scatter, int rows_per_block, hipStream_t s) {
@@ -287,12 +289,11 @@ int ps_gemm_nt_bf16_wide(const void* a, const void* w_packed, const float* bias,
        : launch_wide<WM, ST, bf16_t>(a, w_packed, bias, c, m, n, k, lda, ldc, epilogue, scatter, s))
   // (rings of four and five sets measured no faster than three at any shape: the products do
   // not wait for memory)
-  if (rows_per_block == 128) return PS_WIDE(4, 3);
   if (rows_per_block == 64) return PS_WIDE(2, 3);
   if (rows_per_block == 32) return PS_WIDE(1, 3);
 
 #undef PS_WIDE
-  ps_set_error("ps_linear: the wide product has blocks of 128, 64 or 32 rows, not %d", rows_per_block);
+  ps_set_error("ps_linear: the wide product has blocks of 64 or 32 rows, not %d", rows_per_block);
   return 1;
 }
 
