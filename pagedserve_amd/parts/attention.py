@@ -143,14 +143,15 @@ class Attention(Mixer):
 
     def _merged_splits(self, count: int, max_kv_len: int) -> int:
         """Ranges per request for the path that merges them inside the output projection, or 0
-        where the other path is as fast or faster (measured at 12 heads of 64: from about ten
-        requests on, and where the contexts feed fewer than three ranges): about three blocks of
+        where the other path is as fast or faster (more (token, head) pairs than three quarters
+        of the compute units: 16 requests of 12 heads still gain 2 %; and where the contexts
+        feed fewer than three ranges): about three blocks of
         four waves per compute unit, never more ranges than the keys of the longest request
         can feed."""
         visible = max_kv_len if self.window <= 0 else min(max_kv_len, self.window)
         pairs = count * self.heads
         most = -(-visible // kernels.decode_keys_per_block(self.head_dim, 4))
-        if pairs > kernels.compute_units() // 2 or most < 3:
+        if pairs > kernels.compute_units() * 3 // 4 or most < 3:
             return 0
         wanted = max(1, -(-3 * kernels.compute_units() // pairs))
         return min(most, wanted, 64)
