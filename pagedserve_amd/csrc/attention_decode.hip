@@ -123,8 +123,20 @@ __global__ __launch_bounds__(64 * AD_WAVES) void attention_decode_kernel(
   const int dim0 = (lane % LPK) * 8;
   const bool has_dims = dim0 < head_dim;
 
+  // tok_item == null: token t is item t (a step of single tokens only).  The row of the
+  // block table is then known without a load, and when it is short its entries are asked for
+  // at once, beside the position, instead of behind it: one trip to memory less on the way to
+  // the first keys (lane l holds entries l and l + 64; the lanes hand them to each other).
+  const bool direct = tok_item == nullptr;
+  const bool prefetched = direct && table_width <= 128;
+  int held0 = 0, held1 = 0;
+  if (prefetched) {
+    const int* row = tables + (int64_t)t * table_width;
+    held0 = row[lane < table_width ? lane : table_width - 1];
+    if (table_width > 64) held1 = row[lane + 64 < table_width ? lane + 64 : table_width - 1];
+  }
   const int pos = tok_pos[t];
-  const int* table = tables + (int64_t)tok_item[t] * table_width;
+  const int* table = tables + (int64_t)(direct ? t : tok_item[t]) * table_width;
   const int first_key = (window > 0 && pos - window + 1 > 0) ? pos - window + 1 : 0;
   const int end_key = pos + 1;
   int chunk = (end_key - first_key + splits - 1) / splits;
@@ -154,7 +166,17 @@ __global__ __launch_bounds__(64 * AD_WAVES) void attention_decode_kernel(
       const int safe_key = key < range_end ? key : range_end - 1;
       const int logical = page_shift >= 0 ? (safe_key >> page_shift) : safe_key / page_size;
       within[u] = safe_key - logical * page_size;
-      page[u] = table[logical < table_width ? logical : table_width - 1];
+      const int entry = logical < table_width ? logical : table_width - 1;
+      if (prefetched) {
+        const int low = __shfl(held0, entry & 63, 64);
+        page[u] = low;
+        if (table_width > 64) {
+          const int high = __shfl(held1, entry & 63, 64);
+          page[u] = entry < 64 ? low : high;
+        }
+      } else {
+        page[u] = table[entry];
+      }
       valid[u] = key < range_end && logical < table_width;
     }
 #pragma unroll

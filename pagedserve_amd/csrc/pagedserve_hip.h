@@ -123,7 +123,9 @@ int ps_attention_rowwise(const void* q, int64_t q_stride, const void* k_pool, co
 // The same result for single queries, with each token's keys cut into `splits` ranges that
 // run as separate blocks of `waves` (4 or 16) waves; `partial` is scratch of
 // count * heads * splits * (head_dim + 2) floats (unused when splits == 1).  head_dim is a
-// multiple of 8 up to 256.
+// multiple of 8 up to 256.  tok_item may be null (here and in the two variants below): token t
+// is then item t, row t of `tables`, as in a step of single tokens, and the kernel asks for its
+// block table beside the position instead of behind the item index.
 int ps_attention_decode(const void* q, int64_t q_stride, const void* k_pool, const void* v_pool,
                         void* out, int64_t out_stride, float* partial, int64_t partial_floats,
                         const int* tok_list, const int* tok_item, const int* tok_pos,

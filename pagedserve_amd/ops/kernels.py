@@ -447,13 +447,22 @@ def _check_pools(k_pool, v_pool, dtype):
     return k_pool.shape  # pages, kv_heads, page_size, head_dim
 
 
-def _check_step_index(tok_item, tok_pos, tables, tokens):
-    _check(tok_item, "tok_item", torch.int32, 1)
+def _check_step_index(tok_item, tok_pos, tables, tokens, direct_items=False):
+    """``direct_items``: the caller's kernel takes ``tok_item=None`` for "token t is item t"."""
     _check(tok_pos, "tok_pos", torch.int32, 1)
     _check(tables, "tables", torch.int32, 2)
-    if tok_item.numel() < tokens or tok_pos.numel() < tokens:
-        raise KernelError("one item index and one position per token are needed")
-    if not (tok_item.is_contiguous() and tok_pos.is_contiguous() and tables.is_contiguous()):
+    if tok_item is None:
+        if not direct_items:
+            raise KernelError("this kernel needs the item index of every token")
+        if tables.shape[0] < tokens:
+            raise KernelError("without item indices the block table needs a row per token")
+    else:
+        _check(tok_item, "tok_item", torch.int32, 1)
+        if tok_item.numel() < tokens or not tok_item.is_contiguous():
+            raise KernelError("one item index per token is needed, contiguous")
+    if tok_pos.numel() < tokens:
+        raise KernelError("one position per token is needed")
+    if not (tok_pos.is_contiguous() and tables.is_contiguous()):
         raise KernelError("step index tensors must be contiguous")
 
 
@@ -474,7 +483,8 @@ def kv_write(k, v, k_pool, v_pool, tok_item, tok_pos, tables):
           kv_heads, head_dim, page_size, pages, dtype_code(k.dtype), _stream())
 
 
-def _attention_args(q, k_pool, v_pool, out, tok_item, tok_pos, tables, heads, tok_list):
+def _attention_args(q, k_pool, v_pool, out, tok_item, tok_pos, tables, heads, tok_list,
+                    direct_items=False):
     _check(q, "q", ndim=2)
     _check(out, "out", q.dtype, 2)
     pages, kv_heads, page_size, head_dim = _check_pools(k_pool, v_pool, q.dtype)
@@ -483,7 +493,7 @@ def _attention_args(q, k_pool, v_pool, out, tok_item, tok_pos, tables, heads, to
     tokens = q.shape[0]
     if q.shape[1] != heads * head_dim or out.shape[1] != heads * head_dim or out.shape[0] != tokens:
         raise KernelError("attention: q/out rows must hold heads x head_dim values")
-    _check_step_index(tok_item, tok_pos, tables, tokens)
+    _check_step_index(tok_item, tok_pos, tables, tokens, direct_items)
     count = tokens
     if tok_list is not None:
         _check(tok_list, "tok_list", torch.int32, 1)
@@ -516,9 +526,11 @@ def decode_keys_per_block(head_dim: int, waves: int = 4) -> int:
 def attention_decode(q, k_pool, v_pool, out, tok_item, tok_pos, tables, heads, scale, splits,
                      partial=None, window=0, tok_list=None, waves=4):
     """The same result as ``attention_rowwise`` by the split-KV kernel; ``partial`` is float
-    scratch of ``count * heads * splits * (head_dim + 2)`` values when ``splits > 1``."""
+    scratch of ``count * heads * splits * (head_dim + 2)`` values when ``splits > 1``.
+    ``tok_item=None`` says that token t is item t (row t of ``tables``), as in a step of single
+    tokens: the kernel then fetches its block table one trip to memory earlier."""
     pages, kv_heads, page_size, head_dim, q_stride, out_stride, count = _attention_args(
-        q, k_pool, v_pool, out, tok_item, tok_pos, tables, heads, tok_list)
+        q, k_pool, v_pool, out, tok_item, tok_pos, tables, heads, tok_list, direct_items=True)
     floats = 0
     if splits > 1:
         _check(partial, "partial", torch.float32)
@@ -527,7 +539,7 @@ def attention_decode(q, k_pool, v_pool, out, tok_item, tok_pos, tables, heads, s
         floats = partial.numel()
     _call("ps_attention_decode", q.data_ptr(), q_stride, k_pool.data_ptr(), v_pool.data_ptr(),
           out.data_ptr(), out_stride, _ptr(partial if splits > 1 else None), floats,
-          _ptr(tok_list), tok_item.data_ptr(), tok_pos.data_ptr(), tables.data_ptr(),
+          _ptr(tok_list), _ptr(tok_item), tok_pos.data_ptr(), tables.data_ptr(),
           tables.shape[1], count, heads, kv_heads, head_dim, page_size, pages, float(scale),
           int(window), int(splits), int(waves), dtype_code(q.dtype), _stream())
     return out
@@ -550,14 +562,15 @@ def merge_linear_supported(dtype, tokens, head_dim, packed) -> bool:
 def attention_decode_partial(q, k_pool, v_pool, partial, tok_item, tok_pos, tables, heads, scale, splits,
                              window=0, tok_list=None, waves=4):
     """The per-range records of decode attention only (``partial``: float scratch of
-    ``count * heads * splits * (head_dim + 2)`` values); ``attention_merge_linear`` merges them."""
+    ``count * heads * splits * (head_dim + 2)`` values); ``attention_merge_linear`` merges them.
+    ``tok_item=None``: token t is item t, as for ``attention_decode``."""
     _check(q, "q", ndim=2)
     pages, kv_heads, page_size, head_dim = _check_pools(k_pool, v_pool, q.dtype)
     q_stride = _rows(q, "q")
     tokens = q.shape[0]
     if q.shape[1] != heads * head_dim:
         raise KernelError("attention: q rows must hold heads x head_dim values")
-    _check_step_index(tok_item, tok_pos, tables, tokens)
+    _check_step_index(tok_item, tok_pos, tables, tokens, direct_items=True)
     count = tokens
     if tok_list is not None:
         _check(tok_list, "tok_list", torch.int32, 1)
@@ -568,7 +581,7 @@ def attention_decode_partial(q, k_pool, v_pool, partial, tok_item, tok_pos, tabl
     if not partial.is_contiguous():
         raise KernelError("attention_decode_partial: scratch must be contiguous")
     _call("ps_attention_decode_partial", q.data_ptr(), q_stride, k_pool.data_ptr(), v_pool.data_ptr(),
-          partial.data_ptr(), partial.numel(), _ptr(tok_list), tok_item.data_ptr(), tok_pos.data_ptr(),
+          partial.data_ptr(), partial.numel(), _ptr(tok_list), _ptr(tok_item), tok_pos.data_ptr(),
           tables.data_ptr(), tables.shape[1], count, heads, kv_heads, head_dim, page_size, pages,
           float(scale), int(window), int(splits), int(waves), dtype_code(q.dtype), _stream())
     return count

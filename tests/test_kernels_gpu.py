@@ -344,6 +344,13 @@ def test_attention_decode_split_kv(dtype, heads, kv_heads, head_dim, page_size, 
         kernels.attention_decode(q, k_pool, v_pool, out, tok_item, tok_pos, tables, heads, scale, splits,
                                  partial=partial, window=window)
         torch.testing.assert_close(out.double(), expected, atol=atol, rtol=rtol)
+        # no item index: token t is item t (tables of 66 to 258 entries: short ones are held
+        # in registers, over 64 in two, long ones are read as before); the same sums in the
+        # same order, so not a bit differs
+        direct = torch.full_like(q, float("nan"))
+        kernels.attention_decode(q, k_pool, v_pool, direct, None, tok_pos, tables, heads, scale, splits,
+                                 partial=partial, window=window)
+        assert torch.equal(direct, out)
     # a list of tokens: only those rows are written
     chosen = torch.tensor([7, 2, 9], dtype=torch.int32, device="cuda")
     out = torch.full_like(q, 7.0)
@@ -355,6 +362,13 @@ def test_attention_decode_split_kv(dtype, heads, kv_heads, head_dim, page_size, 
             torch.testing.assert_close(out[row].double(), expected[row], atol=atol, rtol=rtol)
         else:
             assert float((out[row].float() - 7.0).abs().max()) == 0.0
+    direct = torch.full_like(q, 7.0)
+    kernels.attention_decode(q, k_pool, v_pool, direct, None, tok_pos, tables, heads, scale, splits,
+                             partial=partial, tok_list=chosen)
+    assert torch.equal(direct, out)
+    with pytest.raises(kernels.KernelError, match="row per token"):
+        kernels.attention_decode(q, k_pool, v_pool, direct, None, tok_pos, tables[:3], heads, scale, splits,
+                                 partial=partial)
 
 
 def test_attention_far_key_stands_out():
@@ -377,13 +391,15 @@ def test_attention_far_key_stands_out():
         tok_item = torch.arange(2, dtype=torch.int32, device="cuda")
         tok_pos = torch.full((2,), context - 1, dtype=torch.int32, device="cuda")
         partial = torch.empty(2 * heads * 7 * (head_dim + 2), device="cuda")
-        for kernel in ("rowwise", "decode1", "decode7"):
+        # "direct": without the item index, tables of 46 entries held in one register a lane
+        for kernel in ("rowwise", "decode1", "decode7", "direct1", "direct7"):
             out = torch.empty_like(q)
             if kernel == "rowwise":
                 kernels.attention_rowwise(q, k_pool, v_pool, out, tok_item, tok_pos, tables, heads, head_dim ** -0.5)
             else:
-                kernels.attention_decode(q, k_pool, v_pool, out, tok_item, tok_pos, tables, heads,
-                                         head_dim ** -0.5, int(kernel[6:]), partial=partial)
+                kernels.attention_decode(q, k_pool, v_pool, out,
+                                         tok_item if kernel.startswith("decode") else None, tok_pos,
+                                         tables, heads, head_dim ** -0.5, int(kernel[6:]), partial=partial)
             for item, head, key in targets:
                 page = int(tables[item, key // page_size])
                 expected = v_pool[page, head, key % page_size].float()
