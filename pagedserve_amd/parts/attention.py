@@ -162,18 +162,24 @@ class Attention(Mixer):
         return min(most, wanted, 64)
 
     def _splits(self, count: int, max_kv_len: int):
-        """(ranges per request, waves per block).  Many (token, head) pairs fill the chip with
-        one block of 4 waves each; with fewer pairs and long contexts one block of 16 waves
-        takes a whole request's keys, so that no second launch is needed to merge ranges
-        (1024 keys and more per block: what one compute unit can pull is the limit then, and
-        ranges go to further units); few
-        pairs are cut into ranges so that the chip is filled, never into more than the keys
-        of the longest request can feed."""
+        """(ranges per request, waves per block).  Many (token, head) pairs (from one and a
+        half per compute unit) fill the chip with one block of 4 waves each.  Up to one pair per
+        unit and long contexts: one block of 16 waves takes a whole request's keys, so that no
+        second launch is needed to merge ranges (1024 keys and more per block: what one compute
+        unit can pull is the limit then, and ranges go to further units).  Between the two,
+        blocks of 16 waves would come two to some units and one to the others, and the kernel
+        would last as long as the units with two (24 requests of 12 heads at 1,000 keys: 22.3
+        us, with 4 waves and one range 24.6): there, and with few pairs, the keys are cut into
+        ranges until about four blocks of 4 waves come to a unit (19.0 us with the launch that
+        merges them; from 32 requests on that launch costs more than the ranges gain), never
+        into more than the keys of the longest request can feed."""
         visible = max_kv_len if self.window <= 0 else min(max_kv_len, self.window)
         pairs = count * self.heads
         units = kernels.compute_units()
         if pairs >= units + units // 2:
             return 1, 4
+        if pairs > units:
+            return max(1, min(-(-4 * units // pairs), visible // 256)), 4
         if pairs >= units // 4 and visible > kernels.decode_keys_per_block(self.head_dim, 4):
             # contexts of several thousand keys: two or three such blocks per request, as
             # long as every block still has a compute unit of its own

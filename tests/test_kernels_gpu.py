@@ -366,6 +366,7 @@ def test_attention_decode_split_kv(dtype, heads, kv_heads, head_dim, page_size, 
     kernels.attention_decode(q, k_pool, v_pool, direct, None, tok_pos, tables, heads, scale, splits,
                              partial=partial, tok_list=chosen)
     assert torch.equal(direct, out)
+
     with pytest.raises(kernels.KernelError, match="row per token"):
         kernels.attention_decode(q, k_pool, v_pool, direct, None, tok_pos, tables[:3], heads, scale, splits,
                                  partial=partial)
@@ -584,12 +585,14 @@ def test_attention_prefill_far_key_and_causality():
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
-@pytest.mark.parametrize("m,n,k", [(1, 48, 64), (8, 2304, 768), (16, 100, 1024), (13, 257, 96), (17, 192, 768), (5, 64, 1600), (200, 320, 96)])
+@pytest.mark.parametrize("m,n,k", [(1, 48, 64), (8, 2304, 768), (16, 100, 1024), (13, 257, 96), (17, 192, 768), (5, 64, 1600), (200, 320, 96),
+                                   (40, 2304, 768), (64, 3072, 768), (33, 100, 1024), (50, 8000, 64), (64, 16400, 64)])
 @pytest.mark.parametrize("epilogue", ["none", "gelu_tanh", "residual"])
 @pytest.mark.parametrize("rms", [False, True])
 def test_linear_with_pending_norm(dtype, m, n, k, epilogue, rms):
-    """Norm + product as one call: fused for bfloat16 with up to 16 rows and k <= 1024, two
-    launches otherwise; with and without a row gather."""
+    """Norm + product as one call: fused for bfloat16 with up to 16 rows, k <= 1024 and up to
+    8,192 columns, two launches otherwise (17 to 64 rows: the normed rows travel in the lanes'
+    operand order); with and without a row gather."""
     from pagedserve_amd.ops import kernels
 
     h = _rand((m + 3, k), torch.float32, 70, 2.0) + 0.5
@@ -672,6 +675,41 @@ def test_linear_scatters_keys_and_values(dtype, m, k, geometry):
     assert torch.equal(k_pool, k_ref) and torch.equal(v_pool, v_ref)
 
 
+@pytest.mark.parametrize("m", [8, 24, 64])
+def test_norm_product_scatters_keys_and_values(m):
+    """Norm, [q | k | v] product and the store into the pages as one call (one launch up to 16
+    rows): the output is that of the norm and the product one after the other (up to the
+    rounding of the normed rows), and the pages hold exactly the key and value columns of it."""
+    from pagedserve_amd.ops import kernels
+
+    dtype = torch.bfloat16
+    heads, kv_heads, head_dim, page_size, k = 6, 3, 32, 8, 192
+    q_cols, kv_cols = heads * head_dim, kv_heads * head_dim
+    n = q_cols + 2 * kv_cols
+    lens = [5 + index for index in range(m)]
+    k_pool, v_pool, tables = _paged_fixture(dtype, lens, kv_heads, head_dim, page_size, 301)
+    tok_item = torch.arange(m, dtype=torch.int32, device="cuda")
+    tok_pos = torch.tensor([length - 1 for length in lens], dtype=torch.int32, device="cuda")
+    h = _rand((m, k), torch.float32, 302, 2.0)
+    gamma = 1.0 + _rand((k,), torch.float32, 303, 0.2)
+    beta = _rand((k,), torch.float32, 304, 0.2)
+    w = _rand((n, k), dtype, 305, 1.0 / math.sqrt(k))
+    bias = _rand((n,), torch.float32, 306)
+    packed = kernels.pack_decode_weight(w)
+    normed = kernels.norm(h, gamma, beta, 1e-5, torch.empty((m, k), dtype=dtype, device="cuda"))
+    plain = torch.empty((m, n), dtype=dtype, device="cuda")
+    kernels.linear(normed, w, bias, plain, packed=packed)
+    k_ref, v_ref = k_pool.clone(), v_pool.clone()
+    out = torch.empty_like(plain)
+    scratch = torch.empty((m, k), dtype=dtype, device="cuda")
+    kernels.linear(kernels.PendingNorm(h, gamma, beta, 1e-5, False, scratch), w, bias, out, packed=packed,
+                   scatter=(k_pool, v_pool, tok_item, tok_pos, tables, q_cols, kv_cols))
+    torch.testing.assert_close(out.float(), plain.float(), atol=4e-2, rtol=2e-2)
+    kernels.kv_write(out[:, q_cols:q_cols + kv_cols], out[:, q_cols + kv_cols:], k_ref, v_ref, tok_item, tok_pos, tables)
+    view = torch.int16
+    assert torch.equal(k_pool.view(view), k_ref.view(view)) and torch.equal(v_pool.view(view), v_ref.view(view))
+
+
 @pytest.mark.parametrize("dtype", DTYPES)
 def test_attention_decode_sixteen_waves(dtype):
     from pagedserve_amd.ops import kernels
@@ -694,6 +732,7 @@ def test_attention_decode_sixteen_waves(dtype):
         kernels.attention_decode(q, k_pool, v_pool, out, tok_item, tok_pos, tables, heads, 0.125, splits,
                                  partial=partial, waves=16)
         torch.testing.assert_close(out.double(), expected, atol=atol, rtol=rtol)
+
 
 
 PACKED_SHAPES = [(1, 50, 64), (8, 768, 3072), (8, 2304, 768), (16, 3072, 768), (17, 768, 768), (5, 1000, 320),
