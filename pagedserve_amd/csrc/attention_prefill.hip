@@ -238,6 +238,9 @@ __global__ __launch_bounds__(128 * KS) void attention_prefill_kernel(
     if (ahead <= 0) ap_wait_loads_and_sync<0>();
     else if (ahead == 1) ap_wait_loads_and_sync<LOADS>();
     else ap_wait_loads_and_sync<2 * LOADS>();
+    // the stage that the tile before this one lay in is free since the barrier: the tile that
+    // is STAGES - 1 ahead is asked for at once
+    if (t + STAGES - 1 < tiles) issue(t + STAGES - 1, k0 + (STAGES - 1) * AP_KEYS);
     // this wave's run of 32 keys; it is skipped where no query of the wave can see it
     const int kw = k0 + wave_k * 32;
     const bool active = wave_active && kw <= wave_last && kw < key_end &&
@@ -302,8 +305,6 @@ __global__ __launch_bounds__(128 * KS) void attention_prefill_kernel(
                                                   qf[step], s, 0, 0, 0);
       }
     }
-    // the tile that is STAGES - 1 ahead is asked for while the matrix cores work on S
-    if (t + STAGES - 1 < tiles) issue(t + STAGES - 1, k0 + (STAGES - 1) * AP_KEYS);
     if (!active) continue;
     // the whole run is visible to every query of the wave: no mask
     const bool masked = kw + 31 > wave_first || kw + 32 > key_end ||
