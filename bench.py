@@ -48,7 +48,8 @@ PREFILL_TOKENS = 2048
 def _random_prompt(generator, length, vocab):
     import torch
 
-    return torch.randint(0, vocab, (length,), generator=generator).tolist()
+    # (an int64 array, as the scheduler hands long prompt portions to the step function)
+    return torch.randint(0, vocab, (length,), generator=generator).numpy()
 
 
 def _build(dtype, max_requests, max_step_tokens, layers=None, shape=SMALL):
@@ -210,7 +211,7 @@ def medium_workload(args):
                                      SamplingParams(max_new_tokens=output, ignore_eos=True)))
     # the kernels' code is loaded by a few requests that are not part of the measurement
     for request in requests[:2]:
-        scheduler.add_token_request(list(request.prompt_token_ids)[:80], 4,
+        scheduler.add_token_request(request.prompt_token_ids[:80], 4,
                                     sampling=SamplingParams(max_new_tokens=4, ignore_eos=True))
     scheduler.run_until_complete()
     offsets = arrival_offsets(args.request_rate, len(requests), "poisson", seed=1234)

@@ -124,6 +124,7 @@ class Engine:
         self.max_layouts_remembered = 512
         self._graphs = {}        # key -> StepGraph
         self._graph_seen = {}     # layout -> steps that ran without a graph (buffers exist now)
+        self._layouts = {}        # (tokens, items, wanted, singles, tiles) -> offsets, size, device views
         self._graph_failures = {}
         self._graph_retired = []  # (event, graph): dropped, destroyed once the event has happened
         self.graphs_captured = 0
@@ -284,20 +285,35 @@ class Engine:
         tiles = sum(-(-count // tile) for count in counts if count > 1) if tile else 0
         groups = len(cache.groups)
         width = self.table_width
-        offsets = {}
-        cursor = 0
-        for name, size in (("token_ids", tokens), ("token_src", tokens), ("positions", tokens),
-                           ("tok_item", tokens),
-                           ("cu_tokens", items + 1), ("kv_lens", items), ("slots", items),
-                           ("rows", wanted), ("inv_temperature", wanted), ("uniform", wanted),
-                           ("single_tokens", singles),
-                           ("portion_tokens", tokens - singles), ("tile_item", tiles),
-                           ("tile_q0", tiles)):
-            offsets[name] = (cursor, size)
-            cursor += size
-        for group in range(groups):
-            offsets[f"tables{group}"] = (cursor, items * width)
-            cursor += items * width
+        # where each index array lies, and the device views of them, are the same for every
+        # step of a layout: they are made once
+        layout_key = (tokens, items, wanted, singles, tiles)
+        layout = self._layouts.get(layout_key)
+        if layout is None:
+            offsets = {}
+            cursor = 0
+            for name, size in (("token_ids", tokens), ("token_src", tokens), ("positions", tokens),
+                               ("tok_item", tokens),
+                               ("cu_tokens", items + 1), ("kv_lens", items), ("slots", items),
+                               ("rows", wanted), ("inv_temperature", wanted), ("uniform", wanted),
+                               ("single_tokens", singles),
+                               ("portion_tokens", tokens - singles), ("tile_item", tiles),
+                               ("tile_q0", tiles)):
+                offsets[name] = (cursor, size)
+                cursor += size
+            for group in range(groups):
+                offsets[f"tables{group}"] = (cursor, items * width)
+                cursor += items * width
+            views = {name: self._meta_device[begin:begin + size]
+                     for name, (begin, size) in offsets.items()}
+            for group in range(groups):
+                views[f"tables{group}"] = views[f"tables{group}"].view(items, width)
+            for name in ("inv_temperature", "uniform"):
+                views[name] = views[name].view(torch.float32)
+            if len(self._layouts) >= 512:
+                self._layouts.clear()
+            layout = self._layouts[layout_key] = (offsets, cursor, views)
+        offsets, cursor, views = layout
         turn = self._meta_turn
         self._meta_turn ^= 1
         if self._meta_pending[turn]:
@@ -359,10 +375,11 @@ class Engine:
                     portion_tokens[portion_cursor:portion_cursor + count] = np.arange(
                         flat, flat + count, dtype=np.int32)
                     portion_cursor += count
-                    for q0 in range(0, count, tile) if tile else ():
-                        tile_item[tile_cursor] = index
-                        tile_q0[tile_cursor] = q0
-                        tile_cursor += 1
+                    if tile:
+                        here = -(-count // tile)
+                        tile_item[tile_cursor:tile_cursor + here] = index
+                        tile_q0[tile_cursor:tile_cursor + here] = np.arange(0, count, tile, dtype=np.int32)
+                        tile_cursor += here
                 for place in entry.want:
                     rows[row_cursor] = flat + int(place)
                     row_keys.append((entry.request_id, start + int(place)))
@@ -389,24 +406,19 @@ class Engine:
         self._meta_pending[turn] = True
         self._last_layout = (offsets, cursor)
 
-        def view(name):
-            begin, size = offsets[name]
-            return device[begin:begin + size]
-
         ctx = StepContext(
             tokens=tokens, dtype=self.dtype, device=self.device, items=step_items,
-            token_ids=view("token_ids"), positions=view("positions"), tok_item=view("tok_item"),
-            cu_tokens=view("cu_tokens"), kv_lens=view("kv_lens"), slots=view("slots"),
-            tables=[view(f"tables{group}").view(items, width) for group in range(groups)],
+            token_ids=views["token_ids"], positions=views["positions"], tok_item=views["tok_item"],
+            cu_tokens=views["cu_tokens"], kv_lens=views["kv_lens"], slots=views["slots"],
+            tables=[views[f"tables{group}"] for group in range(groups)],
             page_size=self.page_size, workspace=self.workspace,
             decode_only=singles == items, max_kv_len=max_kv,
-            single_tokens=view("single_tokens"), portion_tokens=view("portion_tokens"),
+            single_tokens=views["single_tokens"], portion_tokens=views["portion_tokens"],
             max_positions=self.spec.max_positions,
-            tile_item=view("tile_item"), tile_q0=view("tile_q0"),
-            token_src=view("token_src"), carried_tokens=self._tokens)
-        self._draw_views = (view("inv_temperature").view(torch.float32),
-                            view("uniform").view(torch.float32))
-        return ctx, view("rows"), row_keys
+            tile_item=views["tile_item"], tile_q0=views["tile_q0"],
+            token_src=views["token_src"], carried_tokens=self._tokens)
+        self._draw_views = (views["inv_temperature"], views["uniform"])
+        return ctx, views["rows"], row_keys
 
     def _forward(self, ctx, rows, logits, wanted, greedy):
         from ..ops import kernels

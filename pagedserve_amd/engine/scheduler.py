@@ -40,6 +40,8 @@ either way.
 from dataclasses import dataclass, field
 from typing import Dict, List, Optional
 
+import numpy as np
+
 from ..sampling.params import SamplingParams, fresh_seed, uniform_for
 from .engine import StepEntry
 
@@ -66,6 +68,7 @@ class RequestState:
     prefill_cursor: int = 0                     # prompt tokens that are cached
     finish_reason: Optional[str] = None
     last_served: int = -1                       # ticket of its last turn; tickets grow with time
+    prompt_array: Optional[object] = field(default=None, repr=False)   # the prompt as an int64 array
 
     @property
     def is_prefilling(self) -> bool:
@@ -329,8 +332,15 @@ class ContinuousBatchScheduler:
                 # only the portion that ends the prompt produces a token
                 # (src/scheduler/orca_scheduler.py:191)
                 want = [size - 1] if size == request.prompt_left else []
-                entries.append(StepEntry(request.request_id,
-                                         request.prompt_token_ids[start:start + size], want))
+                if size > 16:
+                    # long portions travel as slices of one array, made once: the step function
+                    # checks and packs arrays without a loop over their tokens
+                    if request.prompt_array is None:
+                        request.prompt_array = np.asarray(request.prompt_token_ids, dtype=np.int64)
+                    tokens = request.prompt_array[start:start + size]
+                else:
+                    tokens = request.prompt_token_ids[start:start + size]
+                entries.append(StepEntry(request.request_id, tokens, want))
             else:
                 entries.append(StepEntry(request.request_id, [request.pending_token_id], [0]))
         return entries
