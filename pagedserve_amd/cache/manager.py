@@ -111,6 +111,8 @@ class RequestCache:
     length: int = 0
     # per group: logical page index -> physical page, -1 once a window has passed it
     tables: List[List[int]] = field(default_factory=list)
+    # positions that the pages held in every group have room for (``grow`` keeps it)
+    capacity: int = 0
 
 
 RELEASED = -1
@@ -133,6 +135,7 @@ class CacheManager:
                 seen.add(entry)
         self.page_size = page_size
         self.max_slots = max_slots
+        self._windowed = any(group.window > 0 for group in self.groups)
         self.dtype = dtype
         self.device = torch.device(device)
         self.max_positions = max_positions
@@ -202,8 +205,16 @@ class CacheManager:
         slot = self.free_slots.pop()
         for tensor in self.state_tensors.values():
             tensor[slot].zero_()
-        self.requests[request_id] = RequestCache(slot=slot, tables=[[] for _ in self.groups])
+        record = RequestCache(slot=slot, tables=[[] for _ in self.groups])
+        record.capacity = self._capacity(record)
+        self.requests[request_id] = record
         return slot
+
+    def _capacity(self, record) -> int:
+        """Positions that the record's pages have room for in every group (no group: no limit)."""
+        if not record.tables:
+            return 1 << 62
+        return min(len(table) for table in record.tables) * self.page_size
 
     def length(self, request_id: Hashable) -> int:
         return self.requests[request_id].length
@@ -236,6 +247,8 @@ class CacheManager:
         if self.max_positions is not None and new_length > self.max_positions:
             raise ValueError(
                 f"request {request_id!r} would reach {new_length} positions, the model has {self.max_positions}")
+        if new_length <= record.capacity:
+            return      # (most decode steps: the last page still has room)
         missing = self.pages_missing(request_id, new_length)
         if not any(missing):
             return
@@ -251,16 +264,18 @@ class CacheManager:
             table.extend(pages)
             if self.table_arrays is not None:
                 self.table_arrays[group_index][record.slot, first:first + count] = pages
+        record.capacity = self._capacity(record)
 
     def commit(self, request_id: Hashable, new_length: int):
         """The step that wrote positions ``< new_length`` succeeded."""
         record = self.requests[request_id]
         if new_length < record.length:
             raise ValueError("a request's cache cannot shrink")
-        for group_index, table in enumerate(record.tables):
-            if len(table) * self.page_size < new_length:
-                raise RuntimeError("commit beyond the pages that were taken")
+        if new_length > record.capacity:
+            raise RuntimeError("commit beyond the pages that were taken")
         record.length = new_length
+        if not self._windowed:
+            return
         for group_index, group in enumerate(self.groups):
             if group.window <= 0:
                 continue
@@ -346,6 +361,10 @@ class CacheManager:
             if len(held) + len(free) != pool.num_pages:
                 raise AssertionError(
                     f"group {group_index}: {pool.num_pages - len(held) - len(free)} pages lost")
+        for request_id, record in self.requests.items():
+            if record.capacity != self._capacity(record) or record.length > record.capacity:
+                raise AssertionError(f"request {request_id!r}: room for {record.capacity} positions "
+                                     f"noted, {self._capacity(record)} held, {record.length} used")
         slots = [record.slot for record in self.requests.values()]
         if len(set(slots)) != len(slots) or set(slots) & set(self.free_slots):
             raise AssertionError("a slot is held twice")

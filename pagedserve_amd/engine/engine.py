@@ -184,12 +184,23 @@ class Engine:
         total = 0
         new = 0
         vocab = self.spec.vocab_size
+        requests = self.cache.requests
+        max_positions = self.spec.max_positions
         for entry in entries:
             if entry.request_id in seen:
                 # src/model/iteration.py:61-63
                 raise StepError(f"request {entry.request_id!r} appears twice in one step")
             seen.add(entry.request_id)
             count = len(entry.tokens)
+            if count == 1 and entry.want == [0]:
+                # a decoded token with its logits wanted: the short way through the checks below
+                record = requests.get(entry.request_id)
+                carry = entry.carry
+                if (record is not None and 0 <= entry.tokens[0] < vocab
+                        and record.length < max_positions
+                        and (carry is None or 0 <= carry < self._carried_rows)):
+                    total += 1
+                    continue
             if count == 0:
                 raise StepError(f"request {entry.request_id!r} brings no tokens")
             if count > 16:
@@ -247,7 +258,9 @@ class Engine:
                     cache.admit(entry.request_id)
                     admitted.append(entry.request_id)
                     record = cache.requests[entry.request_id]
-                cache.grow(entry.request_id, record.length + len(entry.tokens))
+                needed = record.length + len(entry.tokens)
+                if needed > record.capacity:
+                    cache.grow(entry.request_id, needed)
             caller = torch.cuda.current_stream(self.device)
             if caller.cuda_stream == self.stream.cuda_stream:
                 with kernels.on_stream(self.stream):

@@ -34,6 +34,31 @@ def test_pages_follow_the_length():
     manager.check_invariants()
 
 
+def test_room_in_the_last_page_is_noted_and_not_exceeded():
+    """The positions that a request's pages have room for are kept beside its length: growing
+    inside them takes nothing, committing beyond them is an error, and a pool that runs out
+    leaves them as they were."""
+    manager = _manager(pages=3, page_size=4)
+    manager.admit("r")
+    assert manager.requests["r"].capacity == 0
+    manager.grow("r", 5)
+    assert manager.requests["r"].capacity == 8 and manager.pools[0].num_free == 1
+    manager.grow("r", 8)
+    assert manager.pools[0].num_free == 1
+    with pytest.raises(RuntimeError, match="beyond the pages"):
+        manager.commit("r", 9)
+    manager.commit("r", 8)
+    manager.admit("s")
+    manager.grow("s", 4)
+    with pytest.raises(CacheFull):
+        manager.grow("r", 9)
+    assert manager.requests["r"].capacity == 8
+    manager.check_invariants()
+    manager.requests["r"].capacity = 12         # a wrong note is found
+    with pytest.raises(AssertionError, match="room for 12"):
+        manager.check_invariants()
+
+
 def test_prompt_of_four_with_pages_of_four():
     # prompt 4, page 4 -> 2 pages after one decoded token (testing/test_project.py:709-710)
     manager = _manager(page_size=4)
