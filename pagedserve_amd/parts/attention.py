@@ -125,11 +125,15 @@ class Attention(Mixer):
                          * (self.head_dim + 2))
                 partial = ctx.workspace.flat("attn_partial", worst, torch.float32)
             # in a step of single tokens only, token t is item t: without the index the kernel
-            # asks for its block table a trip to memory earlier (64 requests: 1.6 % of the step;
-            # the path above, of few blocks with one or two pages each, measured 0.6 % slower
-            # with it and keeps the index)
+            # asks for its block table a trip to memory earlier (64 requests of 12 heads: 1.6 %
+            # of the step).  The path above, of few blocks with one or two pages each, measured
+            # 0.6 % slower with it, and so did a grid of more than four blocks per compute unit,
+            # which waits for bytes and not for a trip (64 requests of 25 heads: 1 us a launch):
+            # both keep the index.
+            direct = (singles == tokens
+                      and singles * self.heads * splits <= 4 * kernels.compute_units())
             kernels.attention_decode(q, cache.k_pool, cache.v_pool, context,
-                                     None if singles == tokens else ctx.tok_item,
+                                     None if direct else ctx.tok_item,
                                      ctx.positions, tables, self.heads, self.scale, splits,
                                      partial=partial, window=self.window, waves=waves,
                                      tok_list=None if singles == tokens else ctx.single_tokens)
