@@ -104,3 +104,54 @@ def test_long_contexts_decode_in_ranges(tmp_path, dtype):
     error, scale, where = helpers.max_error(rows, reference)
     assert error <= helpers.TOLERANCE[dtype] * scale, (dtype, error, scale, where)
     engine.cache.check_invariants()
+
+
+@pytest.mark.parametrize("seed", [1, 2, 3])
+def test_random_configurations_in_32_bit(tmp_path, seed):
+    """Eight configurations drawn at random for each seed (1 to 25 heads of 4 to 256 dimensions,
+    inner widths and vocabularies that are multiples of nothing, 1 to 3 layers, pages of 1 to 64
+    tokens, both activations, tied and untied heads), each replayed as a mixed trace with
+    portions of random sizes and pages that are used again, against the plain implementation
+    in 32-bit, where the tolerance leaves no room for a wrong key, page, column or norm.  Every
+    kernel meets sizes here that no fixed configuration of the other tests has."""
+    import os
+    import random
+
+    from pagedserve_amd.engine import Engine
+    from pagedserve_amd.model import load_model
+
+    rng = random.Random(seed)
+    for trial in range(8):
+        heads = rng.choice([1, 2, 3, 4, 5, 6, 7, 8, 12, 16, 25])
+        head_dim = rng.choice([4, 8, 12, 16, 20, 24, 32, 40, 48, 64, 72, 80, 96, 112, 128, 144, 192, 256]
+                              if heads <= 4 else [4, 8, 16, 20, 24, 32, 48, 64, 80])
+        width = heads * head_dim
+        positions = rng.choice([96, 160, 256, 300])
+        config = {
+            "architectures": ["GPT2LMHeadModel"], "model_type": "gpt2", "n_layer": rng.choice([1, 1, 2, 3]),
+            "n_embd": width, "n_head": heads,
+            "n_inner": rng.choice([width, 2 * width, 4 * width, width + 8, 3 * width + 4, 100, 64, 320, 1000]),
+            "vocab_size": rng.choice([5, 17, 41, 100, 257, 1000, 2049, 5000]), "n_positions": positions,
+            "layer_norm_epsilon": rng.choice([1e-5, 1e-6, 3e-4]),
+            "activation_function": rng.choice(["gelu_new", "gelu"]),
+            "scale_attn_by_inverse_layer_idx": rng.choice([False, True]),
+            "tie_word_embeddings": rng.choice([True, True, False]), "eos_token_id": None,
+        }
+        page = rng.choice([1, 2, 3, 4, 5, 8, 12, 16, 32, 64])
+        folder = helpers.write_folder(os.path.join(str(tmp_path), f"m{trial}"), config,
+                                      helpers.lively_tensors(config, 7000 + 100 * seed + trial))
+        requests = {f"r{i}": helpers.random_tokens(rng.randint(3, min(90, positions - 2)), config["vocab_size"],
+                                                   1000 * seed + 10 * trial + i)
+                    for i in range(rng.randint(3, 9))}
+        reference = {name: helpers.plain_logits(folder, tokens) for name, tokens in requests.items()}
+        model, _ = load_model(folder, dtype="float32")
+        max_live = rng.randint(1, 6)
+        steps = helpers.trace_mixed(requests, max_live=max_live, portion=tuple(rng.randint(1, 40) for _ in range(4)),
+                                    decode_tail=rng.randint(1, 10), seed=trial)
+        pages = -(-helpers.live_token_budget(steps, round_to=page) // page) + max_live + 1
+        engine = Engine(model, num_pages=pages, page_size=page, max_requests=max_live, max_step_tokens=512)
+        rows = helpers.replay_in_process(engine, steps)
+        error, scale, where = helpers.max_error(rows, reference)
+        assert error <= helpers.TOLERANCE["float32"] * scale, (config, page, error, scale, where)
+        engine.cache.check_invariants()
+        torch.cuda.synchronize()
