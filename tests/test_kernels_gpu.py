@@ -446,7 +446,7 @@ def test_kv_write_places_tokens(dtype):
 def test_sample_argmax_and_ties():
     from pagedserve_amd.ops import kernels
 
-    for vocab in (7, 257, 1000, 50257):
+    for vocab in (7, 257, 1000, 16385, 50257, 53249, 65537):
         logits = _rand((5, vocab), torch.float32, vocab)
         logits[2, vocab // 2] = 50.0
         logits[3, 1] = 60.0
@@ -457,26 +457,36 @@ def test_sample_argmax_and_ties():
         assert out[3].item() == 1
 
 
-def test_sample_temperature_inverse_cdf():
+@pytest.mark.parametrize("vocab,rows", [(1000, 64), (5, 16), (16384, 12), (16385, 12), (50257, 24), (53249, 8),
+                                        (65536, 8), (70001, 8)])
+def test_sample_temperature_inverse_cdf(vocab, rows):
+    """The token drawn is the one whose share of the cumulative distribution (in id order) holds
+    the row's uniform number; rows of up to 16,384, 53,248 and 65,536 ids take the kernels that
+    keep the row in registers (16, 52 and 64 ids a lane), longer ones the kernel that reads the
+    row three times.  Uniform numbers at and near 0 and 1 are among them."""
     from pagedserve_amd.ops import kernels
 
-    vocab = 1000
-    logits = _rand((64, vocab), torch.float32, 77, 2.0)
+    logits = _rand((rows, vocab), torch.float32, 77, 2.0)
     g = torch.Generator().manual_seed(78)
-    uniform = torch.rand(64, generator=g).cuda()
+    uniform = torch.rand(rows, generator=g)
+    uniform[1], uniform[2], uniform[3] = 0.0, 0.999999, 1e-7
+    uniform = uniform.cuda()
     temperature = 0.8
-    inv_t = torch.full((64,), 1.0 / temperature, device="cuda")
+    inv_t = torch.full((rows,), 1.0 / temperature, device="cuda")
     inv_t[0] = 0.0   # greedy row inside a sampling batch
-    out = torch.empty(64, dtype=torch.int32, device="cuda")
+    out = torch.empty(rows, dtype=torch.int32, device="cuda")
     kernels.sample(logits, inv_t, uniform, out)
     probs = torch.softmax(logits.double() / temperature, dim=-1)
     cdf = probs.cumsum(-1)
     assert out[0].item() == int(torch.argmax(logits[0]))
-    for row in range(1, 64):
+    for row in range(1, rows):
         token = out[row].item()
+        assert 0 <= token < vocab
         upper = float(cdf[row, token])
         lower = float(cdf[row, token - 1]) if token > 0 else 0.0
         assert lower - 1e-5 <= float(uniform[row]) <= upper + 1e-5, (row, token)
+    if vocab != 1000:
+        return
     # frequencies follow the probabilities on a small vocabulary
     small = torch.tensor([[0.0, 1.0, 2.0, -1.0, 0.5]], device="cuda").repeat(4000, 1)
     u = torch.rand(4000, generator=g).cuda()
