@@ -105,9 +105,7 @@ class Attention(Mixer):
             # a decode step of few tokens over long contexts: the key ranges are merged inside
             # the output projection, which is split over the heads: no launch for the merge
             splits = merged_splits
-            worst = ((4 * kernels.compute_units() + ctx.workspace.max_rows * self.heads)
-                     * (self.head_dim + 2))
-            partial = ctx.workspace.flat("attn_partial", worst, torch.float32)
+            partial = self._range_records(ctx)
             kernels.attention_decode_partial(q, cache.k_pool, cache.v_pool, partial, ctx.tok_item,
                                              ctx.positions, tables, self.heads, self.scale, splits,
                                              window=self.window, waves=4)
@@ -120,10 +118,7 @@ class Attention(Mixer):
             splits, waves = self._splits(singles, ctx.max_kv_len)
             partial = None
             if splits > 1:
-                # _splits keeps singles * heads * splits below 4 * units + singles * heads
-                worst = ((4 * kernels.compute_units() + ctx.workspace.max_rows * self.heads)
-                         * (self.head_dim + 2))
-                partial = ctx.workspace.flat("attn_partial", worst, torch.float32)
+                partial = self._range_records(ctx)
             # in a step of single tokens only, token t is item t: without the index the kernel
             # asks for its block table a trip to memory earlier (64 requests of 12 heads: 1.6 %
             # of the step).  The path above, of few blocks with one or two pages each, measured
@@ -150,6 +145,14 @@ class Attention(Mixer):
         kernels.linear(context, self.out_weight, self.out_bias, residual, epilogue="residual",
                        packed=self.out_packed)
 
+    def _range_records(self, ctx):
+        """Scratch for one record per (token, head, key range): always asked for at its largest
+        (both rules below keep tokens x heads x ranges under six blocks per compute unit beside
+        one per pair), so that it never moves under the launches that recorded steps hold."""
+        worst = ((6 * kernels.compute_units() + ctx.workspace.max_rows * self.heads)
+                 * (self.head_dim + 2))
+        return ctx.workspace.flat("attn_partial", worst, torch.float32)
+
     def _merged_splits(self, count: int, max_kv_len: int) -> int:
         """Ranges per request for the path that merges them inside the output projection, or 0
         where the other path is as fast or faster (more (token, head) pairs than three quarters
@@ -167,7 +170,8 @@ class Attention(Mixer):
 
     def _splits(self, count: int, max_kv_len: int):
         """(ranges per request, waves per block).  Many (token, head) pairs (from one and a
-        half per compute unit) fill the chip with one block of 4 waves each.  Up to one pair per
+        half per compute unit) fill the chip with one block of 4 waves each (cut into ranges
+        at contexts of 2,048 keys and more while fewer than four pairs come to a unit).  Up to one pair per
         unit and long contexts: one block of 16 waves takes a whole request's keys, so that no
         second launch is needed to merge ranges (1024 keys and more per block: what one compute
         unit can pull is the limit then, and ranges go to further units).  Between the two,
@@ -180,8 +184,14 @@ class Attention(Mixer):
         visible = max_kv_len if self.window <= 0 else min(max_kv_len, self.window)
         pairs = count * self.heads
         units = kernels.compute_units()
-        if pairs >= units + units // 2:
+        if pairs >= 4 * units:
             return 1, 4
+        if pairs >= units + units // 2:
+            # One block of 4 waves per pair fills the chip at short contexts.  At long ones a
+            # handful of blocks per unit, each walking thousands of keys, leaves units idle
+            # towards the end: ranges until six blocks come to a unit (32 requests of 12 heads
+            # at 8,192 keys: 126 instead of 172 us), none under 2,048 keys.
+            return max(1, min(-(-6 * units // pairs), visible // 1024)), 4
         if pairs > units:
             return max(1, min(-(-4 * units // pairs), visible // 256)), 4
         if pairs >= units // 4 and visible > kernels.decode_keys_per_block(self.head_dim, 4):
