@@ -171,7 +171,8 @@ class Attention(Mixer):
     def _splits(self, count: int, max_kv_len: int):
         """(ranges per request, waves per block).  Many (token, head) pairs (from one and a
         half per compute unit) fill the chip with one block of 4 waves each (cut into ranges
-        at contexts of 2,048 keys and more while fewer than four pairs come to a unit).  Up to one pair per
+        at contexts of 2,048 keys and more while fewer than three and a half pairs come to a
+        unit).  Up to one pair per
         unit and long contexts: one block of 16 waves takes a whole request's keys, so that no
         second launch is needed to merge ranges (1024 keys and more per block: what one compute
         unit can pull is the limit then, and ranges go to further units).  Between the two,
@@ -184,7 +185,7 @@ class Attention(Mixer):
         visible = max_kv_len if self.window <= 0 else min(max_kv_len, self.window)
         pairs = count * self.heads
         units = kernels.compute_units()
-        if pairs >= 4 * units:
+        if 2 * pairs >= 7 * units:
             return 1, 4
         if pairs >= units + units // 2:
             # One block of 4 waves per pair fills the chip at short contexts.  At long ones a
@@ -193,7 +194,14 @@ class Attention(Mixer):
             # at 8,192 keys: 126 instead of 172 us), none under 2,048 keys.
             return max(1, min(-(-6 * units // pairs), visible // 1024)), 4
         if pairs > units:
-            return max(1, min(-(-4 * units // pairs), visible // 256)), 4
+            # (four blocks to a unit, six over thousands of keys)
+            blocks = (6 if visible >= 4096 else 4) * units
+            return max(1, min(-(-blocks // pairs), visible // 256)), 4
+        if 4 * pairs >= 3 * units and visible >= 4096:
+            # nearly a pair per unit over thousands of keys: six blocks of 4 waves to a unit are
+            # ahead of one block of 16 waves per pair (17 requests of 12 heads at 4,096 keys:
+            # 41.4 against 44.2 us, at 16,384 keys 141 against 155)
+            return min(-(-6 * units // pairs), 64), 4
         if pairs >= units // 4 and visible > kernels.decode_keys_per_block(self.head_dim, 4):
             # contexts of several thousand keys: two or three such blocks per request, as
             # long as every block still has a compute unit of its own
