@@ -169,19 +169,26 @@ class Attention(Mixer):
         return min(most, wanted, 64)
 
     def _splits(self, count: int, max_kv_len: int):
-        """(ranges per request, waves per block).  Many (token, head) pairs (from one and a
-        half per compute unit) fill the chip with one block of 4 waves each (cut into ranges
-        at contexts of 2,048 keys and more while fewer than three and a half pairs come to a
-        unit).  Up to one pair per
-        unit and long contexts: one block of 16 waves takes a whole request's keys, so that no
-        second launch is needed to merge ranges (1024 keys and more per block: what one compute
-        unit can pull is the limit then, and ranges go to further units).  Between the two,
-        blocks of 16 waves would come two to some units and one to the others, and the kernel
-        would last as long as the units with two (24 requests of 12 heads at 1,000 keys: 22.3
-        us, with 4 waves and one range 24.6): there, and with few pairs, the keys are cut into
-        ranges until about four blocks of 4 waves come to a unit (19.0 us with the launch that
-        merges them; from 32 requests on that launch costs more than the ranges gain), never
-        into more than the keys of the longest request can feed."""
+        """(ranges per request, waves per block) of the decode kernel, by the number of (token,
+        head) pairs per compute unit and the keys that a query sees:
+
+        * from three and a half pairs per unit: one block of 4 waves per pair fills the chip;
+        * from one and a half: the same at short contexts; from 2,048 keys on a handful of long
+          blocks per unit would leave units idle towards the end, so the keys are cut into
+          ranges until six blocks come to a unit;
+        * between one and one and a half: blocks of 16 waves would come two to some units and
+          one to the others, and the kernel would last as long as the units with two (24
+          requests of 12 heads at 1,000 keys: 22.3 us): ranges of 4-wave blocks, four blocks to a
+          unit (19.0 us with the launch that merges them), six over thousands of keys;
+        * up to one pair per unit: one block of 16 waves takes a whole request's keys and no
+          second launch is needed (two or three such blocks per request while each still has
+          a unit of its own); just under a pair per unit and from 4,096 keys on, ranges of
+          4-wave blocks are ahead again;
+        * few pairs: ranges of 4-wave blocks until four blocks come to a unit.
+
+        Never more ranges than the keys of the longest request can feed, and never more than
+        six blocks per unit beside one per pair (the scratch for the records is sized for
+        that)."""
         visible = max_kv_len if self.window <= 0 else min(max_kv_len, self.window)
         pairs = count * self.heads
         units = kernels.compute_units()
