@@ -1,0 +1,50 @@
+"""The rule that picks the decode attention's launch shape, on the CPU: whatever the sizes, the
+ranges fit the scratch that the part asks for, and the documented cases come out as documented."""
+
+import pytest
+
+from pagedserve_amd.ops import kernels
+from pagedserve_amd.parts.attention import Attention
+
+
+def _part(heads, head_dim=64, window=0):
+    part = Attention.__new__(Attention)
+    part.heads, part.head_dim, part.window = heads, head_dim, window
+    return part
+
+
+@pytest.mark.parametrize("units", [256, 304, 64])
+def test_ranges_fit_the_scratch_and_the_kernel(monkeypatch, units):
+    monkeypatch.setattr(kernels, "compute_units", lambda: units)
+    for heads in (1, 2, 3, 12, 16, 25, 40, 96):
+        for head_dim in (8, 64, 128, 256):
+            for window in (0, 300):
+                part = _part(heads, head_dim, window)
+                for count in list(range(1, 70)) + [100, 128, 256, 300]:
+                    for context in (1, 17, 100, 256, 300, 1000, 1024, 2048, 4096, 8192, 16384, 1 << 20):
+                        splits, waves = part._splits(count, context)
+                        assert 1 <= splits <= 64 and waves in (4, 16)
+                        # what Attention._range_records holds: six blocks per unit beside one per pair
+                        assert count * heads * splits <= 6 * units + count * heads
+                        merged = part._merged_splits(count, context)
+                        assert 0 <= merged <= 64
+                        assert count * heads * merged <= 6 * units + count * heads
+
+
+def test_documented_cases(monkeypatch):
+    monkeypatch.setattr(kernels, "compute_units", lambda: 256)
+    part = _part(12)
+    assert part._splits(64, 1024) == (1, 4)          # three pairs per unit at 1,024 keys
+    assert part._splits(100, 8192) == (1, 4)         # more than three and a half pairs per unit
+    assert part._splits(32, 8192) == (4, 4)          # one and a half pairs per unit, long contexts
+    assert part._splits(32, 1024) == (1, 4)
+    assert part._splits(24, 1024) == (4, 4)          # between one and one and a half
+    assert part._splits(24, 300) == (1, 4)
+    assert part._splits(20, 1024) == (1, 16)         # up to one pair per unit
+    assert part._splits(17, 16384) == (8, 4)         # ... over thousands of keys
+    assert part._splits(8, 16384) == (2, 16)
+    assert part._splits(1, 16384) == (64, 4)         # few pairs: ranges until four blocks per unit
+    assert part._merged_splits(8, 1024) == 8 and part._merged_splits(1, 16384) == 64
+    assert part._merged_splits(17, 1024) == 0 and part._merged_splits(8, 200) == 0
+    # a window bounds the keys that a query sees
+    assert _part(12, window=256)._splits(32, 8192) == (1, 4)
