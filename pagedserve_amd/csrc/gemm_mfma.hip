@@ -504,7 +504,7 @@ __global__ __launch_bounds__(64 * SK_WAVES) void gemm_nt_skinny_norm_kernel(
   //    owns columns 4 * lane + 256 * i (one 16-byte load each); all loads of the four rows and
   //    of the scale and shift leave together.
   {
-    constexpr int V4 = SN_MAX_K / 256;
+    constexpr int V4 = UNROLL * SK_WAVES / 4;   // 256 columns each: what the rounds of k cover
     const float4 zero4 = {0.f, 0.f, 0.f, 0.f};
     float4 g[V4], bt[V4], v[NR][V4];
     bool in_row[V4];
@@ -515,17 +515,24 @@ __global__ __launch_bounds__(64 * SK_WAVES) void gemm_nt_skinny_norm_kernel(
       const int t = token < m ? token : m - 1;
       src[j] = norm.h + (int64_t)(norm.rows ? norm.rows[t] : t) * norm.ldh;
     }
+    int safe[V4];
 #pragma unroll
     for (int i = 0; i < V4; ++i) {
       const int col = 4 * lane + 256 * i;
       in_row[i] = col < k;
-      const int safe = in_row[i] ? col : 0;
-      g[i] = *reinterpret_cast<const float4*>(norm.gamma + safe);
-      bt[i] = (!norm.rms && norm.beta != nullptr)
-                  ? *reinterpret_cast<const float4*>(norm.beta + safe)
-                  : zero4;
+      safe[i] = in_row[i] ? col : 0;
+    }
+    // row by row, the scale and shift behind them: the sums of a row start when the row is there
 #pragma unroll
-      for (int j = 0; j < NR; ++j) v[j][i] = *reinterpret_cast<const float4*>(src[j] + safe);
+    for (int j = 0; j < NR; ++j)
+#pragma unroll
+      for (int i = 0; i < V4; ++i) v[j][i] = *reinterpret_cast<const float4*>(src[j] + safe[i]);
+#pragma unroll
+    for (int i = 0; i < V4; ++i) {
+      g[i] = *reinterpret_cast<const float4*>(norm.gamma + safe[i]);
+      bt[i] = (!norm.rms && norm.beta != nullptr)
+                  ? *reinterpret_cast<const float4*>(norm.beta + safe[i])
+                  : zero4;
     }
     // 2. this wave's weights.  A wave's loads come back in the order in which they left, so
     //    these leave after the loads of the rows (which come from the L2 and are there first)
@@ -542,41 +549,52 @@ __global__ __launch_bounds__(64 * SK_WAVES) void gemm_nt_skinny_norm_kernel(
       wf[u][0] = *reinterpret_cast<const uint4*>(w_ptr + p0);
       wf[u][1] = *reinterpret_cast<const uint4*>(w_ptr + p1);
     }
-    // rows beyond m (the same for the whole wave) are not worked on
+    // The rows of a wave go through every stage together (the sums of all, the means of all,
+    // ...), so that the lane exchanges and the square root of one row run behind those of
+    // the others instead of one after the other.  A wave whose last rows lie beyond m works
+    // on copies of row m - 1 and writes zeros for them.
+    float sum[NR], sq[NR], mean[NR], inv_std[NR];
+#pragma unroll
+    for (int j = 0; j < NR; ++j) {
+      sum[j] = 0.f;
+#pragma unroll
+      for (int i = 0; i < V4; ++i) {
+        if (!in_row[i]) v[j][i] = zero4;
+        sum[j] += (v[j][i].x + v[j][i].y) + (v[j][i].z + v[j][i].w);
+      }
+    }
+#pragma unroll
+    for (int j = 0; j < NR; ++j) mean[j] = norm.rms ? 0.f : wave_sum(sum[j]) / (float)k;
+#pragma unroll
+    for (int j = 0; j < NR; ++j) {
+      sq[j] = 0.f;
+#pragma unroll
+      for (int i = 0; i < V4; ++i) {
+        if (in_row[i]) {
+          v[j][i].x -= mean[j];
+          v[j][i].y -= mean[j];
+          v[j][i].z -= mean[j];
+          v[j][i].w -= mean[j];
+        }
+        sq[j] += (v[j][i].x * v[j][i].x + v[j][i].y * v[j][i].y) +
+                 (v[j][i].z * v[j][i].z + v[j][i].w * v[j][i].w);
+      }
+    }
+#pragma unroll
+    for (int j = 0; j < NR; ++j) inv_std[j] = 1.0f / sqrtf(wave_sum(sq[j]) / (float)k + norm.eps);
 #pragma unroll
     for (int j = 0; j < NR; ++j) {
       const int token = wave + j * SK_WAVES;
-      const bool live = token < m;
-      float sum = 0.f, sq = 0.f, mean = 0.f, inv_std = 0.f;
-      if (live) {
-#pragma unroll
-        for (int i = 0; i < V4; ++i) {
-          if (!in_row[i]) v[j][i] = zero4;
-          sum += (v[j][i].x + v[j][i].y) + (v[j][i].z + v[j][i].w);
-        }
-        mean = norm.rms ? 0.f : wave_sum(sum) / (float)k;
-#pragma unroll
-        for (int i = 0; i < V4; ++i) {
-          if (in_row[i]) {
-            v[j][i].x -= mean;
-            v[j][i].y -= mean;
-            v[j][i].z -= mean;
-            v[j][i].w -= mean;
-          }
-          sq += (v[j][i].x * v[j][i].x + v[j][i].y * v[j][i].y) +
-                (v[j][i].z * v[j][i].z + v[j][i].w * v[j][i].w);
-        }
-        inv_std = 1.0f / sqrtf(wave_sum(sq) / (float)k + norm.eps);
-      }
+      const bool live = token < m;     // the same for the whole wave
 #pragma unroll
       for (int i = 0; i < V4; ++i) {
         if (!in_row[i]) continue;
         uint2 packed = {0u, 0u};
         if (live) {
-          const float y0 = v[j][i].x * inv_std * g[i].x + bt[i].x;
-          const float y1 = v[j][i].y * inv_std * g[i].y + bt[i].y;
-          const float y2 = v[j][i].z * inv_std * g[i].z + bt[i].z;
-          const float y3 = v[j][i].w * inv_std * g[i].w + bt[i].w;
+          const float y0 = v[j][i].x * inv_std[j] * g[i].x + bt[i].x;
+          const float y1 = v[j][i].y * inv_std[j] * g[i].y + bt[i].y;
+          const float y2 = v[j][i].z * inv_std[j] * g[i].z + bt[i].z;
+          const float y3 = v[j][i].w * inv_std[j] * g[i].w + bt[i].w;
           packed.x = pack2_bf16(y0, y1);
           packed.y = pack2_bf16(y2, y3);
         }
