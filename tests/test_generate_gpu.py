@@ -430,3 +430,47 @@ def test_many_requests_under_page_pressure_match_plain(folders, strategy):
     llm.engine.cache.check_invariants()
     assert not llm.engine.cache.requests
     assert llm.scheduler.iterations > 20       # they did not all fit at once
+
+
+@pytest.mark.parametrize("seed", [1, 2, 3])
+def test_random_schedules_match_plain(tmp_path, seed):
+    """Random sets of requests under random schedules (strategy, portion size, batch limit,
+    token budget, page size, few or many pages, recorded steps or not), greedy, in 32-bit:
+    every output equals the plain implementation's continuation, whatever the schedule, and
+    the cache's books are right afterwards.  The weights are lively and the head is untied, so
+    that the tokens change from place to place."""
+    import random
+
+    from pagedserve_amd.engine.llm import LLM
+    from pagedserve_amd.sampling import SamplingParams
+
+    rng = random.Random(seed)
+    config = {"architectures": ["GPT2LMHeadModel"], "model_type": "gpt2", "n_layer": 2, "n_embd": 64,
+              "n_head": 4, "n_inner": 256, "vocab_size": 512, "n_positions": 160,
+              "layer_norm_epsilon": 1e-5, "activation_function": "gelu_new",
+              "tie_word_embeddings": False, "eos_token_id": None}
+    folder = helpers.write_folder(str(tmp_path / "model"), config, helpers.lively_tensors(config, 900 + seed))
+    raw, weights = plain_gpt2.read_model_folder(folder)
+    for trial in range(8):
+        count = rng.randint(1, 14)
+        prompts = [helpers.random_tokens(rng.randint(1, 70), 512, seed * 10000 + trial * 100 + i)
+                   for i in range(count)]
+        news = [rng.randint(1, 40) for _ in range(count)]
+        strategy = rng.choice(["orca", "sarathi"])
+        chunk = rng.choice([1, 2, 3, 5, 8, 16, 33, 64])
+        batch = rng.randint(1, 8)
+        block = rng.choice([1, 2, 4, 8, 16])
+        need = max(-(-(len(p) + n) // block) for p, n in zip(prompts, news))
+        pages = need + rng.randint(0, 3 * need) + 1
+        budget = rng.choice([None, None, batch + 1, 16, 64])
+        graphs = rng.random() < 0.7
+        case = (f"trial {trial}: {count} requests, {strategy}, portions of {chunk}, {batch} at a time, "
+                f"pages of {block}, {pages} pages, budget {budget}, recorded steps {graphs}")
+        llm = LLM(folder, dtype="float32", num_kv_pages=pages, block_size=block, max_batch_size=batch,
+                  scheduling_strategy=strategy, prefill_chunk_size=chunk, max_num_batched_tokens=budget,
+                  enable_hip_graphs=graphs, eos_token_id=None)
+        outputs = llm.generate(prompts, [SamplingParams(max_new_tokens=n) for n in news])
+        expected = [plain_gpt2.greedy_generate(raw, weights, prompt, n) for prompt, n in zip(prompts, news)]
+        assert [list(o.token_ids) for o in outputs] == expected, case
+        llm.engine.cache.check_invariants()
+        assert not llm.engine.cache.requests, case
