@@ -155,17 +155,21 @@ class Attention(Mixer):
 
     def _merged_splits(self, count: int, max_kv_len: int) -> int:
         """Ranges per request for the path that merges them inside the output projection, or 0
-        where the other path is as fast or faster (more (token, head) pairs than three quarters
-        of the compute units: 16 requests of 12 heads still gain 2 %; and where the contexts
-        feed fewer than three ranges): about three blocks of
-        four waves per compute unit, never more ranges than the keys of the longest request
-        can feed."""
+        where the other path is as fast or faster: more (token, head) pairs than three quarters
+        of the compute units (16 requests of 12 heads still gain 2 %), and, from half a pair
+        per unit on, contexts that feed fewer than three ranges (16 requests over 100 keys:
+        3 % slower).  Fewer pairs take this path at every length, also with a single range:
+        the other path would cut 130 to 250 keys into two ranges and merge them with a launch
+        of its own (1 to 4 requests over 20 to 250 keys: 5 % of the step, 8 requests 2 %).
+        About three blocks of four waves per compute unit, never more ranges than the keys of
+        the longest request can feed."""
         visible = max_kv_len if self.window <= 0 else min(max_kv_len, self.window)
         pairs = count * self.heads
-        most = -(-visible // kernels.decode_keys_per_block(self.head_dim, 4))
-        if pairs > kernels.compute_units() * 3 // 4 or most < 3:
+        units = kernels.compute_units()
+        most = max(1, -(-visible // kernels.decode_keys_per_block(self.head_dim, 4)))
+        if pairs > units * 3 // 4 or (most < 3 and 2 * pairs > units):
             return 0
-        wanted = max(1, -(-3 * kernels.compute_units() // pairs))
+        wanted = max(1, -(-3 * units // pairs))
         return min(most, wanted, 64)
 
     def _splits(self, count: int, max_kv_len: int):

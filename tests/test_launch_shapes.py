@@ -45,6 +45,10 @@ def test_documented_cases(monkeypatch):
     assert part._splits(8, 16384) == (2, 16)
     assert part._splits(1, 16384) == (64, 4)         # few pairs: ranges until four blocks per unit
     assert part._merged_splits(8, 1024) == 8 and part._merged_splits(1, 16384) == 64
-    assert part._merged_splits(17, 1024) == 0 and part._merged_splits(8, 200) == 0
+    assert part._merged_splits(17, 1024) == 0
+    # few pairs merge inside the projection at every length; from half a pair per unit on only
+    # where the keys feed three ranges
+    assert part._merged_splits(8, 200) == 2 and part._merged_splits(1, 20) == 1
+    assert part._merged_splits(16, 200) == 0 and part._merged_splits(16, 1024) == 4
     # a window bounds the keys that a query sees
     assert _part(12, window=256)._splits(32, 8192) == (1, 4)
