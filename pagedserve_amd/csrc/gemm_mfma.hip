@@ -725,11 +725,17 @@ static void launch_skinny_mb(const void* a, const void* w, const float* bias, vo
     if (per == 2) PS_LAUNCH_SKU(2, 2, 2);
     else if (per == 3) PS_LAUNCH_SKU(3, 2, 2);
     else PS_LAUNCH_SKU(4, 2, 2);
-  } else if (per <= 1 && k_splits == 1 && n >= 16 * 1024) {
-    // the output head: two tiles of columns per block
+  } else if (per <= 2 && k_splits == 1 && n >= 16 * 1024) {
+    // the output head: two tiles of columns per block (also at 17 to 32 rows: 50,257 x 768 at
+    // 17 rows takes 27 us with one tile per block)
     grid.x = (n + 31) / 32;
-    if (three) PS_LAUNCH_SKU(1, 2, 3);
-    else PS_LAUNCH_SKU(1, 2, SK_UNROLL);
+    if (per <= 1) {
+      if (three) PS_LAUNCH_SKU(1, 2, 3);
+      else PS_LAUNCH_SKU(1, 2, SK_UNROLL);
+    } else {
+      if (three) PS_LAUNCH_SKU(2, 2, 3);
+      else PS_LAUNCH_SKU(2, 2, SK_UNROLL);
+    }
   } else if (per <= 1 && k_chunk > SK_WAVES * SK_UNROLL * 64) {
     // up to 16 rows leave registers for twice the loads: a k of up to 2048 in one round
     hipLaunchKernelGGL((gemm_nt_skinny_kernel<TOut, EPI, 1, 1, 2 * SK_UNROLL>), grid, block, 0, s,
