@@ -198,7 +198,7 @@ def medium_workload(args):
     import torch
 
     from pagedserve_amd.engine import ContinuousBatchScheduler
-    from pagedserve_amd.engine.workload import TraceRequest, arrival_offsets, run_arrival_trace
+    from pagedserve_amd.engine.workload import TraceRequest, arrival_times, run_arrival_trace
     from pagedserve_amd.sampling import SamplingParams
 
     engine, sampler, config = _build(args.dtype, max_requests=64, max_step_tokens=PREFILL_TOKENS,
@@ -217,7 +217,7 @@ def medium_workload(args):
         scheduler.add_token_request(request.prompt_token_ids[:80], 4,
                                     sampling=SamplingParams(max_new_tokens=4, ignore_eos=True))
     scheduler.run_until_complete()
-    offsets = arrival_offsets(args.request_rate, len(requests), "poisson", seed=1234)
+    offsets = arrival_times(len(requests), args.request_rate, "poisson", seed=1234)
     summary = run_arrival_trace(scheduler, requests, offsets, synchronize=torch.cuda.synchronize)
     engine.cache.check_invariants()
     graphs = engine.graph_summary()

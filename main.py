@@ -5,10 +5,10 @@ Options keep the reference's names and meanings where it has them (``--strategy`
 ``--kv-cache-memory-utilization``, ``--kv-cache-safety-mb``, ``--dtype``); ``--model`` is a
 model folder (or ``reference`` for a small random model) instead of a fixed list of names,
 and ``--disable-hip-graphs`` takes the place of ``--disable-cuda-graphs`` (also accepted).
-There is one attention implementation and no quantized cache: the reference's
-``--decode-attention-backend`` is accepted with its values (``torch``, ``triton``) so that its
-command lines keep working, and every value runs the HIP kernels; ``--kv-cache-dtype`` takes
-``model`` only and refuses ``int8`` with a message.
+There is one attention implementation and no quantized cache: ``--decode-attention-backend``
+takes ``hip`` only (the reference's ``torch`` and ``triton`` do not exist here and are refused
+with a message that says so), and ``--kv-cache-dtype`` takes ``model`` only and refuses
+``int8``.
 """
 
 import argparse
@@ -20,7 +20,7 @@ from pagedserve_amd.engine.scheduler import ORCA_STRATEGY, SUPPORTED_SCHEDULING_
 from pagedserve_amd.sampling.params import SamplingParams
 
 SUPPORTED_DTYPES = ("float32", "bfloat16")
-SUPPORTED_DECODE_ATTENTION_BACKENDS = ("hip", "torch", "triton")   # main.py:27 of the reference, plus ours
+SUPPORTED_DECODE_ATTENTION_BACKENDS = ("hip",)    # the reference's option (main.py:27) with the one value built here
 SUPPORTED_KV_CACHE_DTYPES = ("model", "int8")                      # main.py:28
 
 
@@ -45,10 +45,8 @@ def parse_args(argv=None):
     parser.add_argument("--num-kv-pages", type=int, help="explicit number of KV pages")
     parser.add_argument("--block-size", type=int, default=16, help="tokens per KV page")
     parser.add_argument("--dtype", choices=SUPPORTED_DTYPES, default="float32", help="execution dtype")
-    parser.add_argument("--decode-attention-backend", choices=SUPPORTED_DECODE_ATTENTION_BACKENDS,
-                        default="hip",
-                        help="accepted for the reference's command lines; every value runs the "
-                             "HIP kernels")
+    parser.add_argument("--decode-attention-backend", default="hip",
+                        help="attention implementation: 'hip', the only one built")
     parser.add_argument("--kv-cache-dtype", choices=SUPPORTED_KV_CACHE_DTYPES, default="model",
                         help="KV storage dtype: the model's (quantized caches are not built)")
     parser.add_argument("--disable-hip-graphs", "--disable-cuda-graphs", dest="disable_hip_graphs",
@@ -66,9 +64,9 @@ def parse_args(argv=None):
     args = parser.parse_args(argv)
     if args.kv_cache_dtype != "model":
         parser.error("--kv-cache-dtype int8: quantized caches are not built; the cache has the model's dtype")
-    if args.decode_attention_backend != "hip":
-        print(f"note: --decode-attention-backend {args.decode_attention_backend} runs the HIP kernels, "
-              "the only implementation here", file=sys.stderr)
+    if args.decode_attention_backend not in SUPPORTED_DECODE_ATTENTION_BACKENDS:
+        parser.error(f"--decode-attention-backend {args.decode_attention_backend}: this engine has one "
+                     "attention implementation, 'hip' (hand-written kernels); leave the option out")
     return args
 
 

@@ -32,6 +32,9 @@ class Architecture:
     strip_prefixes: tuple = ()
     # (config, canonical tensor name) -> the name under which the random-weights mode stores it
     stored_name: Callable[[Any, str], str] = lambda config, name: name
+    # named raw configurations of this architecture (config.json keys) that a model name may
+    # stand for instead of a folder: small random models for trying the engine out
+    presets: tuple = ()      # ((name, raw config dict), ...)
 
 
 ARCHITECTURES: Dict[str, Architecture] = {}
@@ -47,6 +50,21 @@ def register_architecture(entry: Architecture) -> Architecture:
 def _load_builtin():
     # Importing the module registers it.
     from ..model import gpt2  # noqa: F401
+
+
+def find_preset(name: str):
+    """The raw configuration that an architecture registered under ``name``, or None."""
+    _load_builtin()
+    for entry in ARCHITECTURES.values():
+        for preset, raw in entry.presets:
+            if preset == name:
+                return dict(raw)
+    return None
+
+
+def preset_names():
+    _load_builtin()
+    return sorted(preset for entry in ARCHITECTURES.values() for preset, _ in entry.presets)
 
 
 def resolve_architecture(raw_config: dict) -> Architecture:

@@ -421,6 +421,10 @@ __global__ __launch_bounds__(128 * KS) void attention_prefill_kernel(
   }
 }
 
+// What the host has to know of this file's constants to list a step's tiles.
+extern "C" int ps_attention_prefill_query_tile(void) { return AP_QUERIES; }
+extern "C" int ps_attention_prefill_table_max(void) { return AP_TABLE_MAX; }
+
 extern "C" int ps_attention_prefill(const void* q, int64_t q_stride, const void* k_pool,
                                     const void* v_pool, void* out, int64_t out_stride,
                                     const int* tile_item, const int* tile_q0, int tiles,

@@ -185,6 +185,11 @@ int ps_attention_prefill(const void* q, int64_t q_stride, const void* k_pool, co
                          int num_pages, float scale, int window, int max_kv_len, int dtype,
                          void* stream);
 
+// The two constants of that kernel that a caller builds its index arrays by: queries per tile,
+// and the widest block table (entries per item) that it takes.
+int ps_attention_prefill_query_tile(void);
+int ps_attention_prefill_table_max(void);
+
 // tokens[r] = argmax (inv_temperature[r] == 0) or a draw from softmax(logits * inv_temperature[r])
 // by inverse CDF at uniform[r] in [0, 1).
 int ps_sample(const float* logits, int64_t ld, const float* inv_temperature, const float* uniform,

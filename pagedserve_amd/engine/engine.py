@@ -91,10 +91,10 @@ class Engine:
         self.views = model.cache_views(self.cache)
         self.workspace = Workspace(max_step_tokens, self.device)
         self.table_width = -(-self.spec.max_positions // page_size)
-        # queries of an item with several tokens are listed in tiles of the size that the
-        # model's mixers ask for (None: no mixer wants tiles)
-        self.query_tile = getattr(model, "query_tile", None)
-        capacity = (9 * max_step_tokens + 5 * max_requests + 1
+        # queries of an item with several tokens are listed in tiles, once for every tile size
+        # that a mixer of the model asks for (none: no mixer wants tiles)
+        self.query_tiles = tuple(getattr(model, "query_tiles", ()))
+        capacity = ((7 + 2 * max(1, len(self.query_tiles))) * max_step_tokens + 5 * max_requests + 1
                     + len(groups) * max_requests * self.table_width + 16)
         self._meta_device = torch.empty(capacity, dtype=torch.int32, device=self.device)
         self._meta_host = [torch.empty(capacity, dtype=torch.int32, pin_memory=True) for _ in range(2)]
@@ -120,12 +120,13 @@ class Engine:
         self.stream = torch.cuda.Stream(device=self.device)
         # a part that looks at host values of a step cannot be replayed
         self.use_graphs = use_graphs and getattr(model, "graph_safe", False)
-        self.max_graphs = 48     # recorded layouts kept; the least recently made goes first
+        self.max_graphs = 48     # recorded layouts kept; the least recently replayed goes first
         self.max_layouts_remembered = 512
         self._graphs = {}        # key -> StepGraph
         self._graph_seen = {}     # layout -> steps that ran without a graph (buffers exist now)
         self._layouts = {}        # (tokens, items, wanted, singles, tiles) -> offsets, size, device views
         self._graph_failures = {}
+        self._workspace_moved = 0
         self._graph_retired = []  # (event, graph): dropped, destroyed once the event has happened
         self.graphs_captured = 0
         self.graphs_evicted = 0
@@ -278,9 +279,11 @@ class Engine:
                 caller.wait_stream(self.stream)
         except Exception:
             # requests that this step admitted leave no trace
-            # (src/scheduler/orca_scheduler.py:243-247)
+            # (src/scheduler/orca_scheduler.py:243-247), and no later step may carry on rows
+            # of a step before this one
             for request_id in admitted:
                 cache.release(request_id)
+            self._carried_rows = 0
             raise
         for entry in entries:
             cache.commit(entry.request_id, cache.requests[entry.request_id].length + len(entry.tokens))
@@ -299,8 +302,8 @@ class Engine:
         wanted = sum(wants)
         singles = counts.count(1)
         # items with several tokens are cut into tiles of queries for the mixers' tiled kernels
-        tile = self.query_tile
-        tiles = sum(-(-count // tile) for count in counts if count > 1) if tile else 0
+        tile_sizes = self.query_tiles
+        tiles = tuple(sum(-(-count // tile) for count in counts if count > 1) for tile in tile_sizes)
         groups = len(cache.groups)
         width = self.table_width
         # where each index array lies, and the device views of them, are the same for every
@@ -315,10 +318,13 @@ class Engine:
                                ("cu_tokens", items + 1), ("kv_lens", items), ("slots", items),
                                ("rows", wanted), ("inv_temperature", wanted), ("uniform", wanted),
                                ("single_tokens", singles),
-                               ("portion_tokens", tokens - singles), ("tile_item", tiles),
-                               ("tile_q0", tiles)):
+                               ("portion_tokens", tokens - singles)):
                 offsets[name] = (cursor, size)
                 cursor += size
+            for tile, count in zip(tile_sizes, tiles):
+                for name in (f"tile_item{tile}", f"tile_q0{tile}"):
+                    offsets[name] = (cursor, count)
+                    cursor += count
             for group in range(groups):
                 offsets[f"tables{group}"] = (cursor, items * width)
                 cursor += items * width
@@ -375,8 +381,10 @@ class Engine:
             tok_item, cu, kv_lens = section("tok_item"), section("cu_tokens"), section("kv_lens")
             rows = section("rows")
             single_tokens, portion_tokens = section("single_tokens"), section("portion_tokens")
-            tile_item, tile_q0 = section("tile_item"), section("tile_q0")
-            flat = row_cursor = single_cursor = portion_cursor = max_kv = tile_cursor = 0
+            tile_lists = [(tile, section(f"tile_item{tile}"), section(f"tile_q0{tile}"))
+                          for tile in tile_sizes]
+            tile_cursors = [0] * len(tile_sizes)
+            flat = row_cursor = single_cursor = portion_cursor = max_kv = 0
             for index, (entry, record, start, count) in enumerate(zip(entries, records, starts, counts)):
                 token_ids[flat:flat + count] = entry.tokens
                 if entry.carry is not None:
@@ -393,11 +401,12 @@ class Engine:
                     portion_tokens[portion_cursor:portion_cursor + count] = np.arange(
                         flat, flat + count, dtype=np.int32)
                     portion_cursor += count
-                    if tile:
+                    for which, (tile, tile_item, tile_q0) in enumerate(tile_lists):
                         here = -(-count // tile)
-                        tile_item[tile_cursor:tile_cursor + here] = index
-                        tile_q0[tile_cursor:tile_cursor + here] = np.arange(0, count, tile, dtype=np.int32)
-                        tile_cursor += here
+                        at = tile_cursors[which]
+                        tile_item[at:at + here] = index
+                        tile_q0[at:at + here] = np.arange(0, count, tile, dtype=np.int32)
+                        tile_cursors[which] = at + here
                 for place in entry.want:
                     rows[row_cursor] = flat + int(place)
                     row_keys.append((entry.request_id, start + int(place)))
@@ -405,13 +414,14 @@ class Engine:
                 step_items.append(StepItem(entry.request_id, record.slot, start, count, flat))
                 flat += count
             cu[items] = flat
-            if tile_cursor > 1:
-                # tiles that see the most keys first: the kernel's blocks start in this order,
-                # and the longest should not be the last to start
-                keys = np.asarray(starts, dtype=np.int64)[tile_item] + tile_q0
-                order = np.argsort(-keys, kind="stable")
-                tile_item[:] = tile_item[order]
-                tile_q0[:] = tile_q0[order]
+            for (tile, tile_item, tile_q0), filled in zip(tile_lists, tile_cursors):
+                if filled > 1:
+                    # tiles that see the most keys first: the kernel's blocks start in this
+                    # order, and the longest should not be the last to start
+                    keys = np.asarray(starts, dtype=np.int64)[tile_item] + tile_q0
+                    order = np.argsort(-keys, kind="stable")
+                    tile_item[:] = tile_item[order]
+                    tile_q0[:] = tile_q0[order]
         if isinstance(select, list):
             section("inv_temperature").view(np.float32)[:] = [a for a, _ in select]
             section("uniform").view(np.float32)[:] = [b for _, b in select]
@@ -433,7 +443,8 @@ class Engine:
             decode_only=singles == items, max_kv_len=max_kv,
             single_tokens=views["single_tokens"], portion_tokens=views["portion_tokens"],
             max_positions=self.spec.max_positions,
-            tile_item=views["tile_item"], tile_q0=views["tile_q0"],
+            query_tiles={tile: (views[f"tile_item{tile}"], views[f"tile_q0{tile}"])
+                         for tile in tile_sizes},
             token_src=views["token_src"], carried_tokens=self._tokens)
         self._draw_views = (views["inv_temperature"], views["uniform"])
         return ctx, views["rows"], row_keys
@@ -480,20 +491,30 @@ class Engine:
         later ones copy their indices and replay it."""
         items = len(entries)
         mode = 2 if isinstance(greedy, list) else int(bool(greedy))   # how tokens are chosen
+        if self._graphs and self.workspace.moved != self._workspace_moved:
+            # a scratch buffer was replaced by a larger one: recorded launches hold the old address
+            for plan in self._graphs.values():
+                self._retire_graph(plan)
+            self._graphs.clear()
+            self._graph_seen.clear()
+        self._workspace_moved = self.workspace.moved
         if self.use_graphs and self._graphs:
             # every entry brings one token and wants its logits: the lean path
             requests = self.cache.requests
             longest = 1 + max(requests[entry.request_id].length for entry in entries)
-            plan = self._graphs.get((items, items, items, items, 0, mode, self._context_class(longest)))
+            key = (items, items, items, items, 0, mode, self._context_class(longest))
+            plan = self._graphs.get(key)
             if (plan is not None and plan.logits.data_ptr() == self._logit_buffer(items).data_ptr()
                     and all(len(e.tokens) == 1 and len(e.want) == 1 for e in entries)):
+                self._used(key, plan)
                 return self._replay(plan, entries, greedy)
         ctx, rows, row_keys = self._pack(entries, greedy)
         wanted = len(row_keys)
         logits = self._logit_buffer(wanted)
         singles = ctx.single_tokens.numel()
         kv_class = self._context_class(ctx.max_kv_len)
-        graph_key = (ctx.tokens, items, wanted, singles, ctx.tile_item.numel(), mode, kv_class)
+        tiles = sum(lists[0].numel() for lists in ctx.query_tiles.values())
+        graph_key = (ctx.tokens, items, wanted, singles, tiles, mode, kv_class)
         if not self.use_graphs or graph_key in self._graph_failures:
             out, tokens = self._forward(ctx, rows, logits, wanted, greedy)
             return StepOutput(logits=out, rows=row_keys, tokens=tokens)
@@ -503,6 +524,7 @@ class Engine:
         plan = self._graphs.get(graph_key)
         if plan is not None and plan.logits.data_ptr() == logits.data_ptr():
             # recorded: the indices are on their way already (``_pack`` copied them)
+            self._used(graph_key, plan)
             plan.graph.launch()
             return StepOutput(logits=plan.logits[:wanted], rows=row_keys, tokens=plan.tokens)
         # The first step of a layout runs directly, so that every buffer exists before a
@@ -554,6 +576,13 @@ class Engine:
         self.capture_seconds += time.perf_counter() - capture_started
         graph.launch()
         return StepOutput(logits=out, rows=row_keys, tokens=tokens)
+
+    def _used(self, key, plan):
+        """A replayed layout moves to the end of the line: the one dropped when the ring is full
+        is the one that has not been replayed for longest, not the one recorded first."""
+        if len(self._graphs) > 1:
+            del self._graphs[key]
+            self._graphs[key] = plan
 
     def _retire_graph(self, plan):
         """A recorded layout is dropped.  Its last launch may still be running (the engine never

@@ -6,16 +6,15 @@ and a safety margin, main.py:48-73), and wires cache, engine, sampler and schedu
 model is named by its folder (``config.json`` + ``model.safetensors``), not by a fixed list.
 """
 
-import json
-import os
-import tempfile
 from dataclasses import dataclass
 from typing import List, Optional, Sequence, Union
 
 import torch
 
 from ..cache.manager import kv_cache_budget
-from ..model.loading import load_model, resolve_dtype, write_random_model
+from ..config.base import read_config_json
+from ..config.registry import find_preset
+from ..model.loading import load_model, random_model, resolve_dtype
 from ..sampling.params import SamplingParams
 from .engine import Engine
 from .scheduler import ORCA_STRATEGY, ContinuousBatchScheduler
@@ -24,14 +23,7 @@ from .tokenizer import load_tokenizer
 MIB = 1024 * 1024
 DEFAULT_KV_MEMORY_UTILIZATION = 0.90   # main.py:30
 DEFAULT_KV_SAFETY_MB = 3072            # main.py:31
-REFERENCE_MODEL = "reference"
-
-# Sizes of the reference's built-in random model (main.py:104-115), as GPT-2 keys.
-REFERENCE_MODEL_CONFIG = {
-    "architectures": ["GPT2LMHeadModel"], "model_type": "gpt2", "vocab_size": 257,
-    "n_embd": 64, "n_layer": 2, "n_head": 4, "n_inner": 256, "n_positions": 128,
-    "activation_function": "gelu", "layer_norm_epsilon": 1e-5, "eos_token_id": 256,
-}
+REFERENCE_MODEL = "reference"   # a preset that the architecture's registry entry names
 
 
 def _bytes_per_page(model, page_size, dtype):
@@ -48,20 +40,21 @@ def build_scheduler(model=REFERENCE_MODEL, scheduling_strategy=ORCA_STRATEGY, pr
                     max_num_batched_tokens=None, max_prefill_requests=None, random_weights=False,
                     seed=0, eos_token_id="config", model_name=None, enable_cuda_graphs=None,
                     decode_attention_backend="hip", kv_cache_dtype="model"):
-    """Load ``model`` (a folder, or ``"reference"`` for a small random model) and return a
-    ``ContinuousBatchScheduler`` ready for ``add_request`` / ``run_until_complete``.
+    """Load ``model`` (a folder, or a preset's name such as ``"reference"`` for a small random
+    model) and return a ``ContinuousBatchScheduler`` ready for ``add_request`` /
+    ``run_until_complete``.
 
     The reference's names for the same things are taken as well (main.py:136-150):
-    ``model_name`` for ``model``, ``enable_cuda_graphs`` for ``enable_hip_graphs``; its
-    ``decode_attention_backend`` values all run the HIP kernels, and ``kv_cache_dtype`` can
-    only be ``"model"`` (quantized caches are not built)."""
+    ``model_name`` for ``model``, ``enable_cuda_graphs`` for ``enable_hip_graphs``.  Of its
+    ``decode_attention_backend`` only ``"hip"`` exists here and of ``kv_cache_dtype`` only
+    ``"model"`` (quantized caches are not built); other values are errors."""
     if model_name is not None:
         model = model_name
     if enable_cuda_graphs is not None:
         enable_hip_graphs = bool(enable_cuda_graphs)
-    if decode_attention_backend not in ("hip", "torch", "triton"):
-        raise ValueError(f"Unknown decode attention backend '{decode_attention_backend}'. "
-                         "Choose one of: hip, torch, triton (all run the HIP kernels)")
+    if decode_attention_backend != "hip":
+        raise ValueError(f"Unknown decode attention backend '{decode_attention_backend}': "
+                         "the one implementation here is 'hip'")
     if kv_cache_dtype != "model":
         raise ValueError(f"KV cache dtype '{kv_cache_dtype}': quantized caches are not built; "
                          "the cache has the model's dtype ('model')")
@@ -69,20 +62,15 @@ def build_scheduler(model=REFERENCE_MODEL, scheduling_strategy=ORCA_STRATEGY, pr
         raise RuntimeError("pagedserve_amd needs a GPU (MI355X); there is no CPU path")
     dtype = resolve_dtype(execution_dtype)
     device = torch.device("cuda")
-    scratch = None
-    if model == REFERENCE_MODEL:
-        scratch = tempfile.mkdtemp(prefix="pagedserve_reference_")
-        write_random_model(scratch, dict(REFERENCE_MODEL_CONFIG), seed=seed)
-        folder = scratch
+    preset = find_preset(model) if isinstance(model, str) else None
+    if preset is not None:
+        # random weights are drawn in memory: the tensors that writing a folder and loading it
+        # would give, without the folder
+        loaded, config = random_model(preset, seed=seed, dtype=dtype, device=device)
     elif random_weights:
-        with open(os.path.join(model, "config.json")) as handle:
-            raw = json.load(handle)
-        scratch = tempfile.mkdtemp(prefix="pagedserve_random_")
-        write_random_model(scratch, raw, seed=seed)
-        folder = scratch
+        loaded, config = random_model(read_config_json(model), seed=seed, dtype=dtype, device=device)
     else:
-        folder = model
-    loaded, config = load_model(folder, dtype=dtype, device=device)
+        loaded, config = load_model(model, dtype=dtype, device=device)
     if max_batch_size is None:
         max_batch_size = 32          # main.py:180-181 (its GPU default)
     if max_batch_size <= 0:
@@ -115,7 +103,7 @@ def build_scheduler(model=REFERENCE_MODEL, scheduling_strategy=ORCA_STRATEGY, pr
     # "config": what config.json says (null there means that no token ends a request); an
     # explicit value, None included, overrides it.  The scheduler never asks the tokenizer.
     eos = config.eos_token_id if eos_token_id == "config" else eos_token_id
-    tokenizer = load_tokenizer(None if model == REFERENCE_MODEL else model, config.vocab_size, eos)
+    tokenizer = load_tokenizer(None if preset is not None else model, config.vocab_size, eos)
     scheduler = ContinuousBatchScheduler(
         engine, Sampler(device, max_batch_size), tokenizer=tokenizer,
         max_batch_size=max_batch_size, eos_token_id=eos,

@@ -368,7 +368,13 @@ class ContinuousBatchScheduler:
             flight = self._take_off()
             if flight is None:
                 return {}
-        self._inflight = self._take_off_ahead(flight)
+        try:
+            self._inflight = self._take_off_ahead(flight)
+        except Exception:
+            # the step ahead failed in a way that the ordinary start would not report: the
+            # iteration that is already running keeps its tokens and lands on the next call
+            self._inflight = flight
+            raise
         return self._land(flight)
 
     def _choose_on_device(self, receivers, ahead):

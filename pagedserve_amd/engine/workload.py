@@ -1,15 +1,16 @@
 """Requests that arrive over time, run through the scheduler, with the times that serving is
 judged by.
 
-The reference's benchmark draws arrival offsets (fixed or Poisson, ``random.expovariate`` from
-a seeded generator, the first at 0: comparison_benchmark.py:356-387), submits each request when
-its time has come, and records when every token of a request appeared; from those times it
-derives time to first token, time per output token and end-to-end time
+The reference's benchmark lets requests arrive at a fixed pace or as a Poisson process
+(comparison_benchmark.py:356-387), submits each request when its time has come, and records
+when every token of a request appeared; from those times it derives time to first token, time
+per output token and end-to-end time with their mean, median, 95th and 99th percentile
 (comparison_benchmark.py:444-472).  This module does the same above
 ``ContinuousBatchScheduler``: one loop that adds what has arrived and runs an iteration.
 The clock is a parameter, so the loop can be tested on the CPU with a clock of its own.
 """
 
+import itertools
 import math
 import random
 import time
@@ -19,24 +20,29 @@ from typing import Callable, List, Optional, Sequence
 from ..sampling.params import SamplingParams
 
 
-def arrival_offsets(request_rate: float, num_requests: int, pattern: str = "poisson", seed: int = 1234):
-    """Seconds after the start at which each request arrives.  ``poisson``: exponential gaps
-    of mean ``1 / request_rate``; ``fixed``: equal gaps; an infinite rate: all at once."""
-    if num_requests <= 0:
+ARRIVAL_PROCESSES = ("poisson", "even", "burst")
+
+
+def arrival_times(count: int, rate: Optional[float] = None, process: str = "poisson", seed: int = 0):
+    """When each of ``count`` requests arrives, in seconds after the start, ascending, the
+    first at 0.  ``burst``: all at once (``rate`` is not looked at; an infinite rate means the
+    same under every process); ``even``: one every ``1 / rate`` seconds; ``poisson``: the gaps
+    are independent draws from the exponential distribution of mean ``1 / rate``, taken from a
+    generator of its own that ``seed`` fixes (the arrival model of comparison_benchmark.py:356-387)."""
+    if process not in ARRIVAL_PROCESSES:
+        raise ValueError(f"unknown arrival process {process!r}; known: {', '.join(ARRIVAL_PROCESSES)}")
+    if count <= 0:
         return []
-    if math.isinf(request_rate):
-        return [0.0] * num_requests
-    if request_rate <= 0:
-        raise ValueError("request_rate must be positive")
-    if pattern == "fixed":
-        return [index / request_rate for index in range(num_requests)]
-    if pattern != "poisson":
-        raise ValueError(f"Unknown arrival pattern: {pattern}")
-    generator = random.Random(seed)
-    offsets = [0.0]
-    for _ in range(1, num_requests):
-        offsets.append(offsets[-1] + generator.expovariate(request_rate))
-    return offsets
+    if process == "burst" or (rate is not None and math.isinf(rate)):
+        return [0.0] * count
+    if rate is None or not rate > 0:
+        raise ValueError("the arrival rate (requests a second) must be positive")
+    if process == "even":
+        gaps = itertools.repeat(1.0 / rate, count - 1)
+    else:
+        draw = random.Random(seed).expovariate
+        gaps = (draw(rate) for _ in range(count - 1))
+    return list(itertools.accumulate(gaps, initial=0.0))
 
 
 @dataclass
@@ -82,9 +88,9 @@ def percentile(values: Sequence[float], q: float) -> float:
 def summarize(values: Sequence[float]) -> dict:
     values = list(values)
     if not values:
-        return {"mean": None, "p50": None, "p99": None, "max": None}
+        return {"mean": None, "p50": None, "p95": None, "p99": None, "max": None}
     return {"mean": sum(values) / len(values), "p50": percentile(values, 50),
-            "p99": percentile(values, 99), "max": max(values)}
+            "p95": percentile(values, 95), "p99": percentile(values, 99), "max": max(values)}
 
 
 def run_arrival_trace(scheduler, requests: Sequence[TraceRequest], offsets: Sequence[float],

@@ -49,13 +49,10 @@ class DecoderModel:
                                f"{', '.join(unknown)}; it has: {', '.join(arrangement.roles)}")
             self.blocks.append(arrangement(width=spec.width, dtype=dtype, parts=parts))
         self.final_norm = build_part(NORMS, "norm", spec.final_norm, **common)
-        # Queries of a prompt portion are handed to the mixers in tiles of this many; the
-        # mixers say which size their kernels take (all that say so must agree).
-        tiles = {block.mixer.query_tile for block in self.blocks
-                 if getattr(block.mixer, "query_tile", None)}
-        if len(tiles) > 1:
-            raise ValueError(f"the mixers ask for different query tiles: {sorted(tiles)}")
-        self.query_tile = tiles.pop() if tiles else None
+        # Queries of a prompt portion are handed to the mixers in tiles; each mixer says which
+        # size its kernel takes, and the step lists the tiles once per size that is asked for.
+        self.query_tiles = tuple(sorted({int(block.mixer.query_tile) for block in self.blocks
+                                         if getattr(block.mixer, "query_tile", None)}))
         # the mixer of the call that writes a cache entry decides what the entry holds
         self._entry_spec = {}
         for call in spec.schedule:
@@ -92,6 +89,7 @@ class DecoderModel:
                 part.bind(mine, embedding_table=tensors["embedding.table"])
             else:
                 part.bind(mine)
+        self.tensors = dict(tensors)     # parameter path -> the tensor that was bound (no copies)
         self.parameter_bytes = sum(t.numel() * t.element_size() for t in tensors.values())
         self.parameter_count = sum(t.numel() for t in tensors.values())
 

@@ -129,6 +129,14 @@ def random_tensors(config: GPT2Config, seed: int):
     return tensors
 
 
+# Sizes of the reference's built-in random model (main.py:104-115), as config.json keys.
+REFERENCE_PRESET = {
+    "architectures": ["GPT2LMHeadModel"], "model_type": "gpt2", "vocab_size": 257,
+    "n_embd": 64, "n_layer": 2, "n_head": 4, "n_inner": 256, "n_positions": 128,
+    "activation_function": "gelu", "layer_norm_epsilon": 1e-5, "eos_token_id": 256,
+}
+
+
 GPT2 = register_architecture(Architecture(
     name="GPT2LMHeadModel",
     config_class=GPT2Config,
@@ -141,4 +149,5 @@ GPT2 = register_architecture(Architecture(
     # the head of an untied model is never prefixed
     strip_prefixes=("transformer.",),
     stored_name=lambda config, name: name if name.startswith("lm_head.") else "transformer." + name,
+    presets=(("reference", REFERENCE_PRESET),),
 ))

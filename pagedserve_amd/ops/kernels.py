@@ -613,10 +613,27 @@ def attention_merge_linear(partial, count, heads, head_dim, splits, w, packed, b
     return residual
 
 
-PREFILL_TILE = 64
+PREFILL_TILE = 64          # queries per block of the tiled prefill kernel
+PREFILL_TABLE_MAX = 2048   # block-table entries of an item that it keeps in LDS
+_PREFILL_CHECKED = False
 
 
-PREFILL_TABLE_MAX = 2048
+def prefill_limits():
+    """(queries per tile, widest block table) as the loaded library was built."""
+    lib = load_library()
+    lib.ps_attention_prefill_query_tile.restype = c_int
+    lib.ps_attention_prefill_table_max.restype = c_int
+    return lib.ps_attention_prefill_query_tile(), lib.ps_attention_prefill_table_max()
+
+
+def _check_prefill_constants():
+    global _PREFILL_CHECKED
+    if not _PREFILL_CHECKED:
+        if prefill_limits() != (PREFILL_TILE, PREFILL_TABLE_MAX):
+            raise KernelError(f"attention_prefill: this module lists queries in tiles of {PREFILL_TILE} "
+                              f"and tables of up to {PREFILL_TABLE_MAX}, the library was built for "
+                              f"{prefill_limits()}; rebuild the library")
+        _PREFILL_CHECKED = True
 
 
 def prefill_supported(dtype, head_dim, table_width=0) -> bool:
@@ -631,6 +648,7 @@ def attention_prefill(q, k_pool, v_pool, out, tile_item, tile_q0, cu_tokens, kv_
     """Attention of items with several tokens, 64 queries per block, on the matrix cores.
     Blocks start in the order of the tile list: the tiles that see the most keys belong first.
     ``max_kv_len`` (no query sees more keys; 0 = unknown) only steers the launch shape."""
+    _check_prefill_constants()
     _check(q, "q", torch.bfloat16, 2)
     _check(out, "out", torch.bfloat16, 2)
     pages, kv_heads, page_size, head_dim = _check_pools(k_pool, v_pool, q.dtype)

@@ -25,7 +25,8 @@ class Attention(Mixer):
 
     accepts_pending_norm = True
 
-    # the step's index arrays list the queries of a prompt portion in tiles of this size
+    # the step's index arrays list the queries of a prompt portion in tiles of this size (the
+    # tiled kernel's; ``kernels.attention_prefill`` checks it against the library's)
     query_tile = kernels.PREFILL_TILE
 
     def __init__(self, width: int, dtype, heads: int, kv_heads: int, head_dim: int, scale: float,
@@ -134,8 +135,9 @@ class Attention(Mixer):
                                      tok_list=None if singles == tokens else ctx.single_tokens)
         whole = singles == 0
         if singles < tokens and kernels.prefill_supported(self.dtype, self.head_dim, tables.shape[1]):
-            kernels.attention_prefill(q, cache.k_pool, cache.v_pool, context, ctx.tile_item,
-                                      ctx.tile_q0, ctx.cu_tokens, ctx.kv_lens, tables,
+            tile_item, tile_q0 = ctx.query_tiles[self.query_tile]
+            kernels.attention_prefill(q, cache.k_pool, cache.v_pool, context, tile_item,
+                                      tile_q0, ctx.cu_tokens, ctx.kv_lens, tables,
                                       self.heads, self.scale, self.window,
                                       max_kv_len=ctx.max_kv_len)
         elif singles < tokens:
@@ -148,10 +150,12 @@ class Attention(Mixer):
     def _range_records(self, ctx):
         """Scratch for one record per (token, head, key range): always asked for at its largest
         (both rules below keep tokens x heads x ranges under six blocks per compute unit beside
-        one per pair), so that it never moves under the launches that recorded steps hold."""
+        one per pair), so that it never moves under the launches that recorded steps hold.
+        Layers of equal heads and head size share one buffer; a layer of other sizes has its
+        own, so that no layer makes another's grow."""
         worst = ((6 * kernels.compute_units() + ctx.workspace.max_rows * self.heads)
                  * (self.head_dim + 2))
-        return ctx.workspace.flat("attn_partial", worst, torch.float32)
+        return ctx.workspace.flat(f"attn_partial_{self.heads}x{self.head_dim}", worst, torch.float32)
 
     def _merged_splits(self, count: int, max_kv_len: int) -> int:
         """Ranges per request for the path that merges them inside the output projection, or 0

@@ -158,6 +158,9 @@ class Workspace:
         self.max_rows = max_rows
         self.device = torch.device(device)
         self._buffers: Dict[tuple, torch.Tensor] = {}
+        # counts the buffers that were replaced by larger ones: whoever holds addresses
+        # (recorded graphs) compares it with the value at the time of recording
+        self.moved = 0
 
     def rows(self, name: str, columns: int, dtype: torch.dtype, max_rows: Optional[int] = None):
         key = (name, columns, dtype, max_rows or self.max_rows)
@@ -173,6 +176,8 @@ class Workspace:
         key = (name, dtype)
         buffer = self._buffers.get(key)
         if buffer is None or buffer.numel() < numel:
+            if buffer is not None:
+                self.moved += 1
             buffer = torch.empty(numel, dtype=dtype, device=self.device)
             self._buffers[key] = buffer
         return buffer
@@ -214,8 +219,10 @@ class StepContext:
     single_tokens: Optional[torch.Tensor] = None   # int32: step indices of one-token items
     portion_tokens: Optional[torch.Tensor] = None  # int32: step indices of all other tokens
     max_positions: int = 0
-    tile_item: Optional[torch.Tensor] = None       # int32: item of each 64-query tile
-    tile_q0: Optional[torch.Tensor] = None         # int32: first query of the tile in its item
+    # For every tile size that a mixer asked for (``Mixer.query_tile``): the queries of the
+    # items with several tokens, cut into tiles of that many.  size -> (int32 item of each tile,
+    # int32 first query of the tile within its item), the tiles that see the most keys first.
+    query_tiles: Optional[Dict[int, tuple]] = None
     token_src: Optional[torch.Tensor] = None       # int32 [T]: >= 0: the token is carried_tokens[src]
     carried_tokens: Optional[torch.Tensor] = None  # int32: tokens that the last step chose
     extra: Optional[dict] = None

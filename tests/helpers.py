@@ -104,12 +104,16 @@ def tiny_folder(tmp_path, which):
     return folder, config, page_size
 
 
-def plain_logits(folder, token_ids, bfloat16=False):
+def plain_logits(folder, token_ids, bfloat16=False, stored_activations=False):
     """float64 logits [T, V] of the plain implementation; with ``bfloat16`` the matrices
-    are first rounded as a bfloat16 engine stores them."""
+    are first rounded as a bfloat16 engine stores them, and with ``stored_activations`` also
+    the activations that such an engine writes to memory between two kernels."""
     config, weights = plain_gpt2.read_model_folder(folder, torch.float64)
     if bfloat16:
         weights = plain_gpt2.round_weights_to_bfloat16(weights)
+    if stored_activations:
+        with plain_gpt2.activations_stored_as(torch.bfloat16):
+            return plain_gpt2.forward_logits(config, weights, token_ids)
     return plain_gpt2.forward_logits(config, weights, token_ids)
 
 

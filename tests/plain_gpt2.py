@@ -46,6 +46,36 @@ def round_weights_to_bfloat16(weights):
     return rounded
 
 
+# None: activations keep the precision of the arithmetic.  torch.bfloat16: the activations that
+# an engine writes to memory between two kernels (normed rows, queries / keys / values, the
+# attention output, the activated hidden rows) are rounded to that type and back, as a bfloat16
+# engine stores them; the residual stream, the statistics and the logits are not (they are
+# 32-bit in such an engine).  The formulas are the same either way.
+ACTIVATION_STORAGE = None
+
+
+class activations_stored_as:
+    """``with activations_stored_as(torch.bfloat16): forward_logits(...)``."""
+
+    def __init__(self, dtype):
+        self.dtype = dtype
+
+    def __enter__(self):
+        global ACTIVATION_STORAGE
+        self.previous, ACTIVATION_STORAGE = ACTIVATION_STORAGE, self.dtype
+
+    def __exit__(self, *exc):
+        global ACTIVATION_STORAGE
+        ACTIVATION_STORAGE = self.previous
+        return False
+
+
+def stored(x):
+    if ACTIVATION_STORAGE is None:
+        return x
+    return x.to(ACTIVATION_STORAGE).to(x.dtype)
+
+
 def embed(wte, wpe, token_ids, positions):
     """h0[t] = wte[id[t]] + wpe[pos[t]]   (src/model/paged_decoder.py:306-314)."""
     return wte[token_ids] + wpe[positions]
@@ -134,19 +164,19 @@ def attention_scale(config, layer_index):
 def attention_sublayer(x, weights, prefix, n_head, scale):
     """Packed QKV projection, thirds, heads, attention, merge, output projection
     (src/model/paged_decoder.py:52-53,75-94)."""
-    qkv = conv1d(x, weights[prefix + "attn.c_attn.weight"], weights[prefix + "attn.c_attn.bias"])
+    qkv = stored(conv1d(x, weights[prefix + "attn.c_attn.weight"], weights[prefix + "attn.c_attn.bias"]))
     width = x.shape[-1]
     q, k, v = qkv[:, :width], qkv[:, width:2 * width], qkv[:, 2 * width:]
     context = causal_attention(split_heads(q, n_head), split_heads(k, n_head),
                                split_heads(v, n_head), scale)
-    return conv1d(merge_heads(context), weights[prefix + "attn.c_proj.weight"],
+    return conv1d(stored(merge_heads(context)), weights[prefix + "attn.c_proj.weight"],
                   weights[prefix + "attn.c_proj.bias"])
 
 
 def mlp_sublayer(x, weights, prefix, activation):
     """fc, activation, projection (src/model/paged_decoder.py:186-188)."""
     hidden = conv1d(x, weights[prefix + "mlp.c_fc.weight"], weights[prefix + "mlp.c_fc.bias"])
-    hidden = ACTIVATIONS[activation](hidden)
+    hidden = stored(ACTIVATIONS[activation](hidden))
     return conv1d(hidden, weights[prefix + "mlp.c_proj.weight"], weights[prefix + "mlp.c_proj.bias"])
 
 
@@ -155,10 +185,10 @@ def block(h, weights, config, layer_index):
     (src/model/paged_decoder.py:181-189)."""
     prefix = f"h.{layer_index}."
     eps = config.get("layer_norm_epsilon", 1e-5)
-    normed = layer_norm(h, weights[prefix + "ln_1.weight"], weights[prefix + "ln_1.bias"], eps)
+    normed = stored(layer_norm(h, weights[prefix + "ln_1.weight"], weights[prefix + "ln_1.bias"], eps))
     h = h + attention_sublayer(normed, weights, prefix, config["n_head"],
                                attention_scale(config, layer_index))
-    normed = layer_norm(h, weights[prefix + "ln_2.weight"], weights[prefix + "ln_2.bias"], eps)
+    normed = stored(layer_norm(h, weights[prefix + "ln_2.weight"], weights[prefix + "ln_2.bias"], eps))
     return h + mlp_sublayer(normed, weights, prefix, config.get("activation_function", "gelu_new"))
 
 
@@ -166,7 +196,7 @@ def lm_head(h, weights, config):
     """Final LayerNorm, then logits = f @ wte^T without bias when the head is tied,
     else f @ lm_head.weight^T (src/model/paged_decoder.py:291-301,330)."""
     eps = config.get("layer_norm_epsilon", 1e-5)
-    final = layer_norm(h, weights["ln_f.weight"], weights["ln_f.bias"], eps)
+    final = stored(layer_norm(h, weights["ln_f.weight"], weights["ln_f.bias"], eps))
     if config.get("tie_word_embeddings", True):
         return final @ weights["wte.weight"].transpose(0, 1)
     return final @ weights["lm_head.weight"].transpose(0, 1)

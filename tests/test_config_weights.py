@@ -212,3 +212,30 @@ def test_random_weights_mode_writes_a_loadable_folder(tmp_path):
     assert not torch.equal(other_weights["wte.weight"], weights["wte.weight"])
     model, _ = _load_cpu(folder, "float32")
     assert isinstance(model, DecoderModel)
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("which", ["A", "B", "C"])
+def test_random_weights_in_memory_are_the_folder_loaders_tensors(tmp_path, which, dtype):
+    """``random_model`` (what the benchmark and ``--random-weights`` use) binds bit for bit the
+    tensors that ``write_random_model`` + ``load_model`` bind: the same draws, the same joined
+    and transposed layouts, the same dtype per role, the tied head the table itself."""
+    from pagedserve_amd.model.loading import random_model
+
+    raw = dict(helpers.TINY[which][0])
+    folder = str(tmp_path / "random")
+    write_random_model(folder, raw, seed=11)
+    from_folder, config_a = load_model(folder, dtype=dtype, device="cpu")
+    in_memory, config_b = random_model(raw, seed=11, dtype=dtype, device="cpu")
+    assert config_a == config_b
+    assert sorted(from_folder.tensors) == sorted(in_memory.tensors) == sorted(from_folder.parameters())
+    for name, tensor in from_folder.tensors.items():
+        other = in_memory.tensors[name]
+        assert tensor.dtype == other.dtype and tensor.shape == other.shape, name
+        assert tensor.is_contiguous() and other.is_contiguous(), name
+        assert torch.equal(tensor, other), name
+    for model in (from_folder, in_memory):
+        tied = model.spec.tie_head
+        assert (model.head.weight is model.embedding.table) == tied
+    other_seed, _ = random_model(raw, seed=12, dtype=dtype, device="cpu")
+    assert not torch.equal(other_seed.tensors["embedding.table"], in_memory.tensors["embedding.table"])

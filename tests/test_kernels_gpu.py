@@ -1024,3 +1024,11 @@ def test_head_product_leaves_the_choice_where_it_cannot_make_it():
         torch.testing.assert_close(out.double(), a.double() @ w.double().t(), atol=2e-2, rtol=2e-2)
     with pytest.raises(kernels.KernelError, match="plain float output"):
         kernels.linear(a, w, None, out, epilogue="gelu_tanh", choose=(top, tokens))
+
+
+def test_the_tile_that_the_step_lists_is_the_kernels_own():
+    """Queries per tile and the widest block table of the tiled prefill kernel are constants of
+    the HIP source; the Python side lists a step's tiles by the same numbers."""
+    from pagedserve_amd.ops import kernels
+
+    assert kernels.prefill_limits() == (kernels.PREFILL_TILE, kernels.PREFILL_TABLE_MAX)

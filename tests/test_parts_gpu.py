@@ -579,3 +579,65 @@ def test_a_windowed_layer_has_pages_of_its_own_and_gives_them_back(tmp_path, dty
         scale = float(expected[rid].abs().max())
         error = max(float((got[rid][p] - expected[rid][p]).abs().max()) for p in got[rid])
         assert len(got[rid]) == len(requests[rid]) and error <= tolerance * scale, (rid, error, scale)
+
+
+def test_mixers_may_ask_for_query_tiles_of_different_sizes(tmp_path):
+    """Layer 1's mixer is a toy that wants the queries of a prompt portion in tiles of 24 and
+    checks what it is handed; layer 0 keeps the attention part with the tiled kernel's 64.  The
+    step lists the tiles once per size, each list starting with the tiles that see most keys."""
+    import dataclasses
+
+    from pagedserve_amd.config import GPT2Config, PartSpec, resolve_architecture
+    from pagedserve_amd.engine import Engine, StepEntry
+    from pagedserve_amd.model import DecoderModel
+    from pagedserve_amd.ops import kernels
+    from pagedserve_amd.parts import MIXERS, Mixer, register_mixer
+
+    seen = []
+    if "toy_tiles" not in MIXERS:
+        @register_mixer("toy_tiles")
+        class Tiles(Mixer):
+            query_tile = 24
+
+            def __init__(self, width, dtype):
+                self.width, self.dtype = width, dtype
+
+            def forward(self, x, residual, ctx, cache):
+                item, q0 = ctx.query_tiles[self.query_tile]
+                MIXERS["toy_tiles"].seen.append((item.tolist(), q0.tolist()))
+
+    MIXERS["toy_tiles"].seen = seen
+    config, page_size, seed, prefix = helpers.TINY["A"]
+    folder = helpers.write_folder(os.path.join(str(tmp_path), "tiles"), config,
+                                  helpers.lively_tensors(config, seed), prefix)
+    arch = resolve_architecture(config)
+    typed = GPT2Config.from_dict(config)
+    base = arch.build_spec(typed)
+    spec = dataclasses.replace(base, blocks=(base.blocks[0],
+                                             base.blocks[1].with_part("mixer", PartSpec.make("toy_tiles"))))
+    model = DecoderModel(spec, torch.bfloat16, "cuda")
+    assert model.query_tiles == (24, kernels.PREFILL_TILE)
+    from pagedserve_amd.weights import load_parameters
+
+    sources = {k: v for k, v in arch.weight_sources(typed, base).items()
+               if not k.startswith("blocks.1.mixer.")}
+    loaded = load_parameters(folder, model.parameters(), sources, torch.bfloat16, "cuda",
+                             strip_prefixes=arch.strip_prefixes,
+                             ignorable=lambda name: name.startswith("h.1.attn."))
+    model.bind(loaded)
+    engine = Engine(model, num_pages=40, page_size=page_size, max_requests=4, max_step_tokens=128)
+    ids = helpers.random_tokens(120, config["vocab_size"], 3)
+    # "a" has 30 keys behind it when its portion of 50 comes; "b" is new and brings 70; "c" one token
+    engine.step([StepEntry("a", ids[:30], [])])
+    seen.clear()
+    out = engine.step([StepEntry("a", ids[30:80], [49]), StepEntry("c", ids[:1], [0]),
+                       StepEntry("b", ids[:70], [69])])
+    assert out.logits.shape[0] == 3 and bool(torch.isfinite(out.logits).all())
+    items, q0 = seen[0]
+    # a: tiles at 0, 24, 48 (keys seen 30 + q0); b: 0, 24, 48 (keys seen q0): most keys first
+    keys = [(30 if item == 0 else 0) + start for item, start in zip(items, q0)]
+    assert sorted(zip(items, q0)) == [(0, 0), (0, 24), (0, 48), (2, 0), (2, 24), (2, 48)]
+    assert keys == sorted(keys, reverse=True)
+    # the other size's list is what the attention part of layer 0 read (64: one tile of a, two of b)
+    assert sorted(zip(*[t.tolist() for t in engine._pack(
+        [StepEntry("a", ids[80:90], [])])[0].query_tiles[64]])) == [(0, 0)]

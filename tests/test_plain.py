@@ -233,3 +233,25 @@ def test_bfloat16_rounding_touches_matrices_only():
     assert torch.equal(rounded["h.0.ln_1.bias"], weights["h.0.ln_1.bias"])
     assert not torch.equal(rounded["wte.weight"], weights["wte.weight"])
     assert torch.equal(rounded["wte.weight"], weights["wte.weight"].to(torch.bfloat16).double())
+
+
+def test_rounded_stores_change_nothing_but_the_stored_activations():
+    """``activations_stored_as(torch.bfloat16)`` rounds what a bfloat16 engine writes to memory
+    between kernels and nothing else: switched off it is the identity; switched on the logits
+    move by bfloat16 roundings (not more than a few parts in a thousand of the largest), and a
+    stored value is a bfloat16 number."""
+    import helpers
+
+    config = dict(helpers.TINY_A)
+    weights = {name: tensor.double() for name, tensor in helpers.lively_tensors(config, 3).items()}
+    ids = helpers.random_tokens(20, config["vocab_size"], 4)
+    exact = P.forward_logits(config, weights, ids)
+    assert P.stored(exact) is exact
+    with P.activations_stored_as(torch.bfloat16):
+        rounded = P.forward_logits(config, weights, ids)
+        value = P.stored(torch.tensor([1.0 + 2.0 ** -10], dtype=torch.float64))
+        assert float(value) == 1.0
+    assert P.ACTIVATION_STORAGE is None
+    assert torch.equal(exact, P.forward_logits(config, weights, ids))
+    change = float((rounded - exact).abs().max() / exact.abs().max())
+    assert 1e-5 < change < 1e-2, change

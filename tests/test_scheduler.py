@@ -415,15 +415,25 @@ def test_no_end_token_can_be_said():
 def test_arrival_trace_runner_times_requests_by_its_clock():
     """Requests are submitted when their time has come (not before), every token gets the time
     at which its iteration ended, and TTFT / TPOT follow comparison_benchmark.py:444-472."""
-    from pagedserve_amd.engine.workload import (TraceRequest, arrival_offsets, percentile,
-                                                 run_arrival_trace)
+    from pagedserve_amd.engine.workload import (TraceRequest, arrival_times, percentile,
+                                                 run_arrival_trace, summarize)
 
-    offsets = arrival_offsets(4.0, 5, "poisson", seed=3)
+    offsets = arrival_times(5, 4.0, "poisson", seed=3)
     assert offsets[0] == 0.0 and offsets == sorted(offsets) and len(offsets) == 5
-    assert offsets == arrival_offsets(4.0, 5, "poisson", seed=3) != arrival_offsets(4.0, 5, "poisson", seed=4)
-    assert arrival_offsets(2.0, 3, "fixed") == [0.0, 0.5, 1.0]
-    assert arrival_offsets(float("inf"), 3) == [0.0, 0.0, 0.0]
+    assert offsets == arrival_times(5, 4.0, "poisson", seed=3) != arrival_times(5, 4.0, "poisson", seed=4)
+    # the mean gap of many draws is 1 / rate
+    many = arrival_times(4001, 50.0, "poisson", seed=1)
+    assert abs(many[-1] / 4000 - 1 / 50.0) < 0.002
+    assert arrival_times(3, 2.0, "even") == [0.0, 0.5, 1.0]
+    assert arrival_times(3, float("inf")) == [0.0, 0.0, 0.0] == arrival_times(3, process="burst")
+    assert arrival_times(0, 1.0) == []
+    with pytest.raises(ValueError):
+        arrival_times(3, 0.0)
+    with pytest.raises(ValueError):
+        arrival_times(3, 1.0, "bursty")
     assert percentile([1, 2, 3, 4], 50) == 2.5 and percentile([5], 99) == 5
+    spread = summarize(range(101))
+    assert (spread["p50"], spread["p95"], spread["p99"], spread["max"]) == (50, 95, 99, 100)
 
     class Clock:
         now = 0.0
@@ -477,11 +487,14 @@ def test_command_line_takes_the_reference_options(capsys):
     args = main.parse_args(["--model", "reference", "--strategy", "sarathi", "--prefill-chunk-size", "32",
                             "--max-batch-size", "4", "--kv-cache-memory-mb", "64",
                             "--kv-cache-memory-utilization", "0.5", "--kv-cache-safety-mb", "128",
-                            "--dtype", "bfloat16", "--decode-attention-backend", "triton",
+                            "--dtype", "bfloat16", "--decode-attention-backend", "hip",
                             "--kv-cache-dtype", "model", "--disable-cuda-graphs"])
     assert args.strategy == "sarathi" and args.prefill_chunk_size == 32 and args.max_batch_size == 4
     assert args.kv_cache_memory_mb == 64 and args.disable_hip_graphs and args.dtype == "bfloat16"
-    assert "HIP kernels" in capsys.readouterr().err
+    # a backend that is not built is an error that names the one that is, not a silent alias
+    with pytest.raises(SystemExit):
+        main.parse_args(["--decode-attention-backend", "triton"])
+    assert "'hip'" in capsys.readouterr().err
     with pytest.raises(SystemExit):
         main.parse_args(["--kv-cache-dtype", "int8"])
     assert "quantized caches are not built" in capsys.readouterr().err
@@ -497,5 +510,6 @@ def test_python_entry_takes_the_reference_keyword_names():
 
     with pytest.raises(ValueError, match="quantized caches are not built"):
         build_scheduler(model_name="reference", kv_cache_dtype="int8")
-    with pytest.raises(ValueError, match="Unknown decode attention backend"):
-        build_scheduler(model_name="reference", decode_attention_backend="flash")
+    for backend in ("flash", "torch", "triton"):
+        with pytest.raises(ValueError, match="Unknown decode attention backend.*'hip'"):
+            build_scheduler(model_name="reference", decode_attention_backend=backend)

@@ -55,9 +55,8 @@ def test_real_sizes_match_plain(shape_models, name, dtype):
     model, _ = load_model(folder, dtype=dtype)
     worst = {}
     cuts = [("whole", helpers.trace_whole), ("mixed", helpers.trace_mixed),
-            ("tail", lambda r: helpers.trace_tail_decoded(r, tail=20))]
-    if name == "small":
-        cuts.append(("portions", helpers.trace_portions))
+            ("tail", lambda r: helpers.trace_tail_decoded(r, tail=20)),
+            ("portions", helpers.trace_portions)]
     for cut, builder in cuts:
         steps = builder(requests)
         pages = helpers.live_token_budget(steps, round_to=16) // 16
