@@ -21,6 +21,14 @@ the HBM roofline).
 
 print one JSON line each about their own run (tokens a second, time to first token, time per
 output token, graphs recorded and dropped).
+
+    python bench.py --kernels [--shape small|medium|xl|all] [--only name,name]
+
+times every kernel of a decode step (1, 8 and 64 requests over 1,024 keys) and of the prefill
+step (2 x 1,024 tokens) alone, on weights that no cache holds (a graph of launches that rotate
+over copies of them, at least 25 launches untimed and 100 timed), and prints a table (to
+standard error) and one JSON line: microseconds, bytes, flops, and both as fractions of the
+published peaks and of two measured ones (a device copy and the library's 4096-cubed product).
 """
 
 import argparse
@@ -307,6 +315,35 @@ def xl_workload(args):
     }
 
 
+SHAPES = {"small": SMALL, "medium": MEDIUM, "xl": XL}
+
+
+def kernel_tables(args):
+    """``--kernels``: the per-kernel tables of ``pagedserve_amd.measure.kernel_table``."""
+    from pagedserve_amd.measure import kernel_table as table
+
+    only = [piece for piece in (args.only or "").split(",") if piece] or None
+    peaks = table.measured_peaks()
+    print(f"measured peaks: copy {peaks['copy_GBps']} GB/s (published HBM {HBM_GBPS:.0f}), 4096-cubed "
+          f"bfloat16 product of the library {peaks['product_4096_TFLOPs']} TFLOP/s (published "
+          f"{PEAK_TFLOPS['bf16']:.0f})", file=sys.stderr, flush=True)
+    names = list(SHAPES) if args.shape == "all" else [args.shape]
+    tables = {}
+    for name in names:
+        raw = SHAPES[name]
+        for rows in [int(piece) for piece in args.rows.split(",")]:
+            key = f"{name}_decode_b{rows}_ctx{raw['n_positions']}"
+            tables[key] = table.decode_table(raw, rows, raw["n_positions"], peaks, PAGE_SIZE, only)
+            print(table.format_table(key, tables[key]), file=sys.stderr, flush=True)
+        if not args.no_prefill:
+            key = f"{name}_prefill_2x{PREFILL_TOKENS // 2}"
+            tables[key] = table.prefill_table(raw, 2, PREFILL_TOKENS // 2, peaks, PAGE_SIZE, only)
+            print(table.format_table(key, tables[key]), file=sys.stderr, flush=True)
+    return {"metric": "microseconds per kernel, weights from memory", "unit": "us", "dtype": "bf16",
+            "published_peak": {"hbm_GBps": HBM_GBPS, "bf16_TFLOPs": PEAK_TFLOPS["bf16"]},
+            "measured_peak": peaks, "tables": tables}
+
+
 def main(argv=None):
     parser = argparse.ArgumentParser()
     parser.add_argument("--gpus", type=int, default=1)
@@ -324,6 +361,13 @@ def main(argv=None):
     parser.add_argument("--requests", type=int, default=256, help="requests of --workload medium")
     parser.add_argument("--request-rate", type=float, default=400.0,
                         help="mean arrivals a second of --workload medium")
+    parser.add_argument("--kernels", action="store_true",
+                        help="time every kernel of the decode and prefill steps alone (see above)")
+    parser.add_argument("--shape", choices=("small", "medium", "xl", "all"), default="small",
+                        help="layer sizes of --kernels")
+    parser.add_argument("--rows", default="1,8,64", help="decode batch sizes of --kernels")
+    parser.add_argument("--only", help="--kernels: only kernels whose name holds one of these (comma-separated)")
+    parser.add_argument("--no-prefill", action="store_true", help="--kernels: decode tables only")
     args = parser.parse_args(argv)
     if args.gpus != 1:
         print(f"bench.py measures one GPU; --gpus {args.gpus} is not supported by this engine")
@@ -332,6 +376,9 @@ def main(argv=None):
     import torch
 
     torch.cuda.init()
+    if args.kernels:
+        print(json.dumps(kernel_tables(args)), flush=True)
+        return 0
     if args.workload != "small":
         record = medium_workload(args) if args.workload == "medium" else xl_workload(args)
         print(json.dumps(record), flush=True)

@@ -14,16 +14,23 @@
 // one wave that merges head h of all rows (each lane the 16 values of its own row that it
 // needs as matrix-core operand; with fewer than 9 rows the lanes of the free operand columns
 // take a share of the ranges each and exchange their sums), multiplies them with the piece of W that belongs to its columns and to
-// head h (out of the packed copy of W, pagedserve_hip.h), and adds the result into the float
-// residual rows with atomic adds; the blocks of head 0 add the bias.  The sum over heads is
+// head h (out of the packed copy of W, pagedserve_hip.h); the waves of a block (up to four
+// heads) sum their results through LDS and the first adds them into the float residual rows
+// with atomic adds; the blocks of the first heads add the bias.  The sum over heads is
 // therefore made by the adds, in an order that differs from run to run within float rounding,
 // as for every product here whose k range is split over blocks.
 #include "gemm_bf16_common.h"
 
 typedef __attribute__((__vector_size__(4 * sizeof(float)))) float f32x4_t;
 
-template <int STEPS, int PARTS>   // head_dim / 64; lanes that share the ranges of a row
-__global__ __launch_bounds__(64) void attention_merge_linear_kernel(
+// STEPS: head_dim / 64; PARTS: lanes that share the ranges of a row; GROUP: heads per block, one
+// wave each, whose results are summed through LDS before they are added to the residual rows.
+// Float atomic adds on a few rows are performed at some 15 per nanosecond on this chip, however
+// many blocks issue them (measured: 24 blocks adding 8 rows of 768 floats each take 10 us, 48
+// take 17): with a wave per head, 12 heads adding into 8 rows of 768 were 74,000 atomic adds and
+// most of this kernel's time.  Four heads to a block leave a quarter of them.
+template <int STEPS, int PARTS, int GROUP>
+__global__ __launch_bounds__(64 * GROUP) void attention_merge_linear_kernel(
     const float* __restrict__ partial, const int* __restrict__ tok_list, int count, int heads,
     int splits, const bf16_t* __restrict__ wp, const float* __restrict__ bias,
     float* __restrict__ residual, int64_t ld_res, int n) {
@@ -32,10 +39,13 @@ __global__ __launch_bounds__(64) void attention_merge_linear_kernel(
   constexpr int parts = PARTS;
   constexpr int HEAD_DIM = STEPS * 64;
   constexpr int STRIDE = HEAD_DIM + 2;
-  const int lane = threadIdx.x;
+  const int lane = threadIdx.x & 63;
+  const int wave = threadIdx.x >> 6;
   const int column = lane & 15;        // column of the matrix-core operand: a row of the step
   const int group = lane >> 4;         // which 16 of every 64 head dimensions
-  const int head = blockIdx.y;
+  // (a wave beyond the last head works on a copy of the last head and adds nothing)
+  const bool real_head = blockIdx.y * GROUP + wave < heads;
+  const int head = real_head ? blockIdx.y * GROUP + wave : heads - 1;
   // Fewer rows than 16 leave operand columns free: they take a share of the ranges of the rows
   // that are there (row = column mod rows_pow2, the smallest power of two that holds the
   // rows; the column's other bits pick every parts-th range), and the shares are merged by
@@ -146,6 +156,20 @@ __global__ __launch_bounds__(64) void attention_merge_linear_kernel(
                                                          *reinterpret_cast<const bf16x8*>(&x_raw), acc[c], 0, 0, 0);
     }
   // element i of lane l: column (l / 16) * 4 + i of the tile, row l % 16
+  if (GROUP > 1) {
+    // the heads of this block are summed by its first wave
+    __shared__ f32x4_t sums[GROUP > 1 ? GROUP - 1 : 1][TILES][64];
+    if (wave > 0)
+#pragma unroll
+      for (int c = 0; c < TILES; ++c)
+        sums[wave - 1][c][lane] = real_head ? acc[c] : f32x4_t{0.f, 0.f, 0.f, 0.f};
+    __syncthreads();
+    if (wave > 0) return;
+#pragma unroll
+    for (int w = 0; w < GROUP - 1; ++w)
+#pragma unroll
+      for (int c = 0; c < TILES; ++c) acc[c] += sums[w][c][lane];
+  }
   if (!has_row) return;
   const int t = tok_list ? tok_list[column] : column;
 #pragma unroll
@@ -155,7 +179,7 @@ __global__ __launch_bounds__(64) void attention_merge_linear_kernel(
       const int col = (blockIdx.x * TILES + c) * 16 + group * 4 + i;
       if (col >= n) continue;
       float v = acc[c][i];
-      if (head == 0 && bias != nullptr) v += bias[col];
+      if (blockIdx.y == 0 && bias != nullptr) v += bias[col];
       unsafeAtomicAdd(residual + (int64_t)t * ld_res + col, v);
     }
 }
@@ -164,7 +188,8 @@ bool ps_attention_merge_linear_supported(int count, int head_dim, int dtype) {
   return dtype == PS_BF16 && count >= 1 && count <= 16 && head_dim % 64 == 0 && head_dim <= 256;
 }
 
-// tiles_per_block: 16-column tiles that one wave computes (0 or 1: one; two measured slower)
+// tiles_per_block: 0, or how many heads a block takes (1, 2 or 4 waves whose results are summed
+// before they are added to the residual rows); 0 leaves the choice to this file.
 extern "C" int ps_attention_merge_linear(const float* partial, int64_t partial_floats,
                                          const int* tok_list, int count, int heads, int head_dim,
                                          int splits, const void* w_packed, const float* bias,
@@ -184,12 +209,24 @@ extern "C" int ps_attention_merge_linear(const float* partial, int64_t partial_f
                  (reinterpret_cast<uintptr_t>(w_packed) & 15u) == 0 &&
                  (reinterpret_cast<uintptr_t>(partial) & 7u) == 0,
              "ps_attention_merge_linear: null or unaligned operand");
-  PS_REQUIRE(tiles_per_block >= 0 && tiles_per_block <= 1,
-             "ps_attention_merge_linear: one tile of 16 columns per block, not %d", tiles_per_block);
+  PS_REQUIRE(tiles_per_block == 0 || tiles_per_block == 1 || tiles_per_block == 2 || tiles_per_block == 4,
+             "ps_attention_merge_linear: 1, 2 or 4 heads per block, not %d", tiles_per_block);
   if (count == 0) return 0;
-  if (tiles_per_block == 0) tiles_per_block = 1;
   const int tiles_n = (n + 15) / 16;
-  dim3 grid((tiles_n + tiles_per_block - 1) / tiles_per_block, heads);
+  // Four heads to a block save three quarters of the atomic adds, but a block then pulls four
+  // waves' records through one compute unit, and fewer blocks than units leave units idle.
+  // Measured (8 rows x 8 ranges, 12 heads of 64: 5.9 us with one head per block, 6.4 with four;
+  // 16 rows x 2 ranges: 5.9 and 4.4; one row x 8 ranges: 5.4 and 4.8; 16 heads and more: four
+  // heads ahead or level throughout): four where the records are few or the blocks still fill
+  // the chip, else one.
+  int group_heads = tiles_per_block;
+  if (group_heads == 0) {
+    const int wanted = heads >= 4 ? 4 : (heads >= 2 ? 2 : 1);
+    const bool light = splits <= 2 || count * splits <= 16;
+    const bool fills = tiles_n * ((heads + wanted - 1) / wanted) >= ps_compute_units();
+    group_heads = (light || fills) ? wanted : 1;
+  }
+  dim3 grid(tiles_n, (heads + group_heads - 1) / group_heads);
   hipStream_t s = (hipStream_t)stream;
   // shares of the ranges for the free operand columns where there are many ranges (up to 8
   // ranges a lane has them all in flight at once, and shares measured no faster)
@@ -197,10 +234,16 @@ extern "C" int ps_attention_merge_linear(const float* partial, int64_t partial_f
   while (rows_pow2 < count) rows_pow2 <<= 1;
   if (splits <= 8) rows_pow2 = 16;
   const int parts = 16 / rows_pow2;
-#define PS_LAUNCH_AML(STEPS, PARTS)                                                               \
-  hipLaunchKernelGGL((attention_merge_linear_kernel<STEPS, PARTS>), grid, dim3(64), 0, s, partial, \
-                     tok_list, count, heads, splits, (const bf16_t*)w_packed, bias, residual,     \
-                     ld_res, n)
+#define PS_LAUNCH_AMLG(STEPS, PARTS, GROUP)                                                     \
+  hipLaunchKernelGGL((attention_merge_linear_kernel<STEPS, PARTS, GROUP>), grid, dim3(64 * GROUP), \
+                     0, s, partial, tok_list, count, heads, splits, (const bf16_t*)w_packed, bias, \
+                     residual, ld_res, n)
+#define PS_LAUNCH_AML(STEPS, PARTS)                        \
+  do {                                                     \
+    if (group_heads == 4) PS_LAUNCH_AMLG(STEPS, PARTS, 4); \
+    else if (group_heads == 2) PS_LAUNCH_AMLG(STEPS, PARTS, 2); \
+    else PS_LAUNCH_AMLG(STEPS, PARTS, 1);                  \
+  } while (0)
 #define PS_LAUNCH_AMLP(STEPS)                     \
   do {                                            \
     if (parts == 1) PS_LAUNCH_AML(STEPS, 1);      \
@@ -217,6 +260,7 @@ extern "C" int ps_attention_merge_linear(const float* partial, int64_t partial_f
   }
 #undef PS_LAUNCH_AMLP
 #undef PS_LAUNCH_AML
+#undef PS_LAUNCH_AMLG
   PS_CHECK_LAUNCH("ps_attention_merge_linear");
   return 0;
 }

@@ -147,9 +147,9 @@ int ps_attention_decode_partial(const void* q, int64_t q_stride, const void* k_p
 // The merge of those records inside the output projection, for up to 16 tokens and head sizes
 // that are multiples of 64 (bfloat16 weights in their packed copy, n output columns,
 // k = heads * head_dim):  residual[t(r), :] += merged context of row r  W^T + bias, where
-// t(r) = tok_list ? tok_list[r] : r.  One wave per (tile of 16 columns, head); the heads'
-// contributions are added with float atomics.  tiles_per_block: 0 or 1 (a wave that takes
-// two tiles measured slower and is not built).
+// t(r) = tok_list ? tok_list[r] : r.  One wave per (tile of 16 columns, head), up to four heads
+// to a block, whose sum is added with float atomics.  tiles_per_block: 0 (the library chooses),
+// or the heads per block: 1, 2 or 4.
 int ps_attention_merge_linear(const float* partial, int64_t partial_floats, const int* tok_list,
                               int count, int heads, int head_dim, int splits,
                               const void* w_packed, const float* bias, float* residual,

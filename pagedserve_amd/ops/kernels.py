@@ -588,9 +588,11 @@ def attention_decode_partial(q, k_pool, v_pool, partial, tok_item, tok_pos, tabl
 
 
 def attention_merge_linear(partial, count, heads, head_dim, splits, w, packed, bias, residual, tok_list=None,
-                           tiles_per_block=0):
+                           heads_per_block=0):
     """residual[t] += (merged attention output of row r) w^T + bias for the ``count`` rows whose
-    records ``attention_decode_partial`` left in ``partial``; ``packed`` is ``pack_decode_weight(w)``."""
+    records ``attention_decode_partial`` left in ``partial``; ``packed`` is ``pack_decode_weight(w)``.
+    ``heads_per_block``: 0 (the library chooses), 1, 2 or 4 heads whose results a block sums
+    before it adds them to the rows."""
     _check(partial, "partial", torch.float32)
     _check(residual, "residual", torch.float32, 2)
     _check(w, "w", torch.bfloat16, 2)
@@ -609,7 +611,7 @@ def attention_merge_linear(partial, count, heads, head_dim, splits, w, packed, b
         raise KernelError("attention_merge_linear: fewer residual rows than records")
     _call("ps_attention_merge_linear", partial.data_ptr(), partial.numel(), _ptr(tok_list), int(count),
           int(heads), int(head_dim), int(splits), packed.data_ptr(), _ptr(bias), residual.data_ptr(),
-          _rows(residual, "residual"), n, int(tiles_per_block), _stream())
+          _rows(residual, "residual"), n, int(heads_per_block), _stream())
     return residual
 
 

@@ -924,14 +924,16 @@ def test_linear_takes_the_wide_product_for_long_k():
     assert torch.equal(v_pool.view(torch.int16), v_ref.view(torch.int16))
 
 
-@pytest.mark.parametrize("heads,kv_heads,head_dim,page_size", [(12, 12, 64, 16), (4, 2, 128, 12), (2, 1, 256, 16), (3, 3, 192, 8)])
+@pytest.mark.parametrize("heads,kv_heads,head_dim,page_size", [(12, 12, 64, 16), (4, 2, 128, 12), (2, 1, 256, 16), (3, 3, 192, 8),
+                                                               (5, 5, 64, 16)])
 @pytest.mark.parametrize("count", [1, 2, 3, 5, 8, 16])
 @pytest.mark.parametrize("splits", [1, 3, 8, 20, 64])
 def test_attention_records_merged_inside_the_output_projection(heads, kv_heads, head_dim, page_size, count, splits):
     """Decode attention that leaves only its per-range records, and the output projection that
     merges them head by head: residual + softmax(q K^T) V W^T + bias in float64 over the
     gathered pages; contexts around page edges, ranges without keys, a width that ends inside
-    a tile of 16 columns, rows beyond the count untouched."""
+    a tile of 16 columns, rows beyond the count untouched; with one, two and four heads to a
+    block (head counts that are no multiple of either), and with the library's own choice."""
     from pagedserve_amd.ops import kernels
 
     dtype = torch.bfloat16
@@ -955,6 +957,14 @@ def test_attention_records_merged_inside_the_output_projection(heads, kv_heads, 
     expected = start[:count].double() + context.to(dtype).double() @ w.double().t() + bias.double()
     torch.testing.assert_close(residual[:count].double(), expected, atol=2e-2, rtol=2e-2)
     assert torch.equal(residual[count:], start[count:])
+    for heads_per_block in (1, 2, 4):
+        grouped = start.clone()
+        kernels.attention_merge_linear(partial, count, heads, head_dim, splits, w, packed, bias, grouped,
+                                       heads_per_block=heads_per_block)
+        torch.testing.assert_close(grouped[:count].double(), expected, atol=2e-2, rtol=2e-2)
+        # the same products, summed in another order
+        torch.testing.assert_close(grouped[:count], residual[:count], atol=1e-4, rtol=1e-4)
+        assert torch.equal(grouped[count:], start[count:])
     # rows named by a list land at the listed tokens
     chosen = torch.tensor(list(range(count))[::-1], dtype=torch.int32, device="cuda")
     residual = start.clone()
