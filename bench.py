@@ -1,34 +1,42 @@
-"""Decode and prefill throughput of the engine on one MI355X, GPT-2 small shape, bfloat16.
+"""Decode and prefill throughput of the engine on one MI355X, bfloat16, random weights.
 
     python bench.py [--gpus 1] [--steps K] [--warmup W]
 
 A step is one decode step of the scheduler loop that serving runs: the engine's step
 function over a batch of single tokens, token selection on the GPU and the copy of the
-chosen tokens to the host.  The default run decodes a batch of 8 requests whose contexts
-end at the model's context length, with random weights and uniform-random prompt ids.
-One JSON line is printed: decoded tokens a second (``value``), the 2,048-token prefill
-step (``prefill``), the decode step against the HBM roofline (``roofline``), decode at
-batch 1 and 64 with contexts that end at the context length, and the benchmark
-configuration's own decode points: prompts of 128 and 512 tokens with 128 output tokens at
-batch 1, 8 and 64 (``points``, tokens a second; ``points_roofline``, each point's fraction of
-the HBM roofline).
+chosen tokens to the host.  The default run decodes a batch of 8 requests at GPT-2 small
+shape whose contexts end at the model's context length, with uniform-random prompt ids.
+One JSON line is printed:
 
-    python bench.py --workload medium      GPT-2 medium shape: a Poisson stream of 256
-                                           requests (prompts 32-896, outputs 16-128),
-                                           continuous batching with prompt portions of 512
-    python bench.py --workload xl          GPT-2 XL shape: 64 requests of 768 + 256 tokens,
-                                           temperature 0.8, seed 7
+* ``value``: decoded tokens a second of those K steps; ``roofline``: the step against the HBM
+  roofline; ``prefill``: the step of 2 x 1,024 prompt tokens;
+* ``points`` / ``points_roofline``: decode at batch 1 and 64 with contexts that end at the
+  context length, and the benchmark configuration's own decode points (prompts of 128 and 512
+  tokens, 128 output tokens, batch 1, 8 and 64), tokens a second and fraction of the roofline;
+* ``points_fp32``: decode at batch 8 and the prefill step in true 32-bit;
+* ``points_long``: a configuration of the same layer sizes with 8,192 positions: decode at
+  batch 8 and 32 over contexts of 4,096 and 8,192, prefill of 2 x 4,096 tokens;
+* ``workloads``: the other two sizes of the benchmark, each in its own workload.
+  ``medium``: GPT-2 medium shape, 256 requests with prompts of 32-896 and outputs of 16-128
+  tokens through the continuous-batching scheduler with prompt portions of 512, arriving as
+  Poisson streams of three rates and as one burst; output tokens a second, time to first
+  token, time per output token and end-to-end time (mean, p50, p95, p99), the share of
+  iterations replayed from graphs, the flops of the stream against the peak, and one mixed
+  step's time on the host and on the GPU.  ``small_stream``: the same stream at GPT-2 small
+  shape, where the host has a third of the time per step.  ``xl``: GPT-2 XL shape, 64
+  requests of 768 + 256 tokens at temperature 0.8, seed 7: decoded tokens a second against the
+  roofline, prompt tokens a second.
 
-print one JSON line each about their own run (tokens a second, time to first token, time per
-output token, graphs recorded and dropped).
-
+    python bench.py --workload medium|small_stream|xl     one workload alone, one JSON line
+    python bench.py --prefill-only --steps K               the prefill step alone (for profiles)
     python bench.py --kernels [--shape small|medium|xl|all] [--only name,name]
 
-times every kernel of a decode step (1, 8 and 64 requests over 1,024 keys) and of the prefill
-step (2 x 1,024 tokens) alone, on weights that no cache holds (a graph of launches that rotate
-over copies of them, at least 25 launches untimed and 100 timed), and prints a table (to
-standard error) and one JSON line: microseconds, bytes, flops, and both as fractions of the
-published peaks and of two measured ones (a device copy and the library's 4096-cubed product).
+``--kernels`` times every kernel of a decode step (1, 8 and 64 requests over 1,024 keys) and of
+the prefill step (2 x 1,024 tokens) alone, on weights that no cache holds (a graph of launches
+that rotate over copies of them, at least 25 launches untimed and 100 timed), and prints a
+table (to standard error) and one JSON line: microseconds, bytes, flops, and both as fractions
+of the published peaks and of two measured ones (a device copy and the library's 4096-cubed
+product).
 """
 
 import argparse
@@ -49,6 +57,8 @@ SMALL = {
 }
 MEDIUM = dict(SMALL, n_layer=24, n_embd=1024, n_head=16, n_inner=4096)
 XL = dict(SMALL, n_layer=48, n_embd=1600, n_head=25, n_inner=6400)
+LONG = dict(SMALL, n_positions=8192)
+SHAPES = {"small": SMALL, "medium": MEDIUM, "xl": XL}
 PAGE_SIZE = 16
 PREFILL_TOKENS = 2048
 
@@ -60,7 +70,11 @@ def _random_prompt(generator, length, vocab):
     return torch.randint(0, vocab, (length,), generator=generator).numpy()
 
 
-def _build(dtype, max_requests, max_step_tokens, layers=None, shape=SMALL):
+def _build(dtype, max_requests, max_step_tokens, layers=None, shape=SMALL, pages=None):
+    """An engine over a model of ``shape`` with random weights (drawn on the GPU: the XL
+    shape's 1.5 billion take a second there), and what the weights occupy."""
+    import torch
+
     from pagedserve_amd.engine import Engine
     from pagedserve_amd.model import random_model
     from pagedserve_amd.sampling.sampler import Sampler
@@ -68,10 +82,17 @@ def _build(dtype, max_requests, max_step_tokens, layers=None, shape=SMALL):
     raw = dict(shape)
     if layers is not None:
         raw["n_layer"] = layers
-    model, config = random_model(raw, seed=0, dtype=dtype, device="cuda")
-    pages = max_requests * (config.n_positions // PAGE_SIZE) + 8
+    torch.cuda.synchronize()
+    before = torch.cuda.memory_allocated()
+    model, config = random_model(raw, seed=0, dtype=dtype, device="cuda", draw_on="cuda")
+    torch.cuda.synchronize()
+    torch.cuda.empty_cache()
+    resident = torch.cuda.memory_allocated() - before
+    if pages is None:
+        pages = max_requests * (config.n_positions // PAGE_SIZE) + 8
     engine = Engine(model, num_pages=pages, page_size=PAGE_SIZE, max_requests=max_requests,
                     max_step_tokens=max_step_tokens)
+    engine.weights_resident_bytes = resident
     return engine, Sampler("cuda", max_requests), config
 
 
@@ -149,20 +170,19 @@ def decode_point(engine, sampler, config, batch, prompt_len, output_tokens, warm
     return elapsed, mean_context
 
 
-def prefill_run(engine, config, reps=8, warmup=5, seed=1):
-    """Seconds per step of 2 x 1024 prompt tokens (logits at each prompt's last token), in the
-    steady state: the warm-up covers the steps that allocate buffers and record the layout's
-    graph."""
+def prefill_run(engine, config, reps=8, warmup=5, seed=1, prompts=2, length=PREFILL_TOKENS // 2):
+    """Seconds per step of ``prompts`` x ``length`` prompt tokens (logits at each prompt's last
+    token), in the steady state: the warm-up covers the steps that allocate buffers and record
+    the layout's graph."""
     import torch
 
     from pagedserve_amd.engine import StepEntry
 
     generator = torch.Generator().manual_seed(seed)
-    length = PREFILL_TOKENS // 2
     times = []
     for rep in range(reps + warmup):
         entries = [StepEntry(f"p{rep}_{i}", _random_prompt(generator, length, config.vocab_size),
-                             [length - 1]) for i in range(2)]
+                             [length - 1]) for i in range(prompts)]
         torch.cuda.synchronize()
         started = time.perf_counter()
         # on the engine's own stream, as the scheduler issues its steps: a caller on another
@@ -198,61 +218,162 @@ def decode_bytes(config, element_size, batch, mean_context):
     return matrices * element_size + vectors * 4 + cache
 
 
-def medium_workload(args):
-    """GPT-2 medium shape: a Poisson stream of 256 requests with uniform-random prompt lengths
-    32-896 and output lengths 16-128, continuous batching with prompt portions of 512."""
+def _fraction(config, element, batch, mean_context, seconds_per_step):
+    return round(decode_bytes(config, element, batch, mean_context) / seconds_per_step / 1e9 / HBM_GBPS, 4)
+
+
+def _ms(group):
+    return {key: (None if value is None else round(value * 1e3, 3)) for key, value in group.items()}
+
+
+def _shape_keys(config, shape):
+    return {"n_layer": config.n_layer, "n_layer_of_config": shape["n_layer"], "n_embd": config.n_embd,
+            "n_head": config.n_head, "n_inner": config.n_inner, "vocab_size": config.vocab_size,
+            "n_positions": config.n_positions, "page_size": PAGE_SIZE}
+
+
+# --------------------------------------------------------------------------------- streams
+def stream_requests(config, count, seed=0):
+    """``count`` requests with uniform-random prompt lengths 32-896 and output lengths 16-128."""
     import random
 
     import torch
 
-    from pagedserve_amd.engine import ContinuousBatchScheduler
-    from pagedserve_amd.engine.workload import TraceRequest, arrival_times, run_arrival_trace
+    from pagedserve_amd.engine.workload import TraceRequest
     from pagedserve_amd.sampling import SamplingParams
 
-    engine, sampler, config = _build(args.dtype, max_requests=64, max_step_tokens=PREFILL_TOKENS,
-                                     layers=args.layers, shape=MEDIUM)
-    scheduler = ContinuousBatchScheduler(engine, sampler, max_batch_size=64, eos_token_id=None,
-                                         scheduling_strategy="sarathi", prefill_chunk_size=512)
-    lengths = random.Random(0)
-    generator = torch.Generator().manual_seed(0)
+    lengths = random.Random(seed)
+    generator = torch.Generator().manual_seed(seed)
     requests = []
-    for _ in range(args.requests):
+    for _ in range(count):
         prompt, output = lengths.randint(32, 896), lengths.randint(16, 128)
         requests.append(TraceRequest(_random_prompt(generator, prompt, config.vocab_size), output,
                                      SamplingParams(max_new_tokens=output, ignore_eos=True)))
-    # the kernels' code is loaded by a few requests that are not part of the measurement
-    for request in requests[:2]:
-        scheduler.add_token_request(request.prompt_token_ids[:80], 4,
-                                    sampling=SamplingParams(max_new_tokens=4, ignore_eos=True))
-    scheduler.run_until_complete()
-    offsets = arrival_times(len(requests), args.request_rate, "poisson", seed=1234)
+    return requests
+
+
+def stream_run(engine, sampler, config, requests, rate, process, short, prompts_per_iteration=1):
+    """One pass of the requests through the continuous-batching scheduler (prompt portions of
+    512, up to 64 requests an iteration) with the given arrivals; a compact summary."""
+    import torch
+
+    from pagedserve_amd.engine import ContinuousBatchScheduler
+    from pagedserve_amd.engine.workload import arrival_times, run_arrival_trace
+
+    # an iteration's token budget: one portion of 512 beside up to 64 decoded tokens; with
+    # several prompts an iteration, the prompts share that budget
+    scheduler = ContinuousBatchScheduler(engine, sampler, max_batch_size=64, eos_token_id=None,
+                                         scheduling_strategy="sarathi", prefill_chunk_size=512,
+                                         max_prefill_requests=prompts_per_iteration,
+                                         max_num_batched_tokens=512 + 64)
+    before = engine.graph_summary()
+    offsets = arrival_times(len(requests), rate, process, seed=1234)
     summary = run_arrival_trace(scheduler, requests, offsets, synchronize=torch.cuda.synchronize)
     engine.cache.check_invariants()
-    graphs = engine.graph_summary()
-
-    def ms(group):
-        return {key: (None if value is None else round(value * 1e3, 3)) for key, value in group.items()}
-
+    after = engine.graph_summary()
+    flops = 0
+    for request, record in zip(requests, summary["records"]):
+        tokens = len(request.prompt_token_ids) + len(record.token_times)
+        flops += step_flops(config, [tokens], len(record.token_times))
+    iterations = max(summary["iterations"], 1)
     return {
-        "metric": "output tok/s of a Poisson stream of 256 requests (GPT-2 medium shape, prompt portions of 512)",
-        "value": round(summary["output_tokens_per_second"], 1), "unit": "tokens/s", "n_gpus": 1,
-        "higher_is_better": True, "dtype": "bf16" if args.dtype == "bfloat16" else "fp32",
-        "data": "synthetic (random weights, uniform-random prompt ids and lengths, seeded arrivals)",
-        "wall_s": round(summary["wall_seconds"], 3), "requests": summary["requests"],
-        "prompt_tokens": summary["prompt_tokens"], "output_tokens": summary["output_tokens"],
-        "total_tok_s": round(summary["total_tokens_per_second"], 1), "iterations": summary["iterations"],
+        "output_tok_s": round(summary["output_tokens_per_second"], 1),
+        "total_tok_s": round(summary["total_tokens_per_second"], 1),
+        "wall_s": round(summary["wall_seconds"], 3), "iterations": summary["iterations"],
+        "replayed": round((after["graph_replays"] - before["graph_replays"]) / iterations, 3),
+        "captures": after["captures"] - before["captures"], "evicted": after["evicted"] - before["evicted"],
+        "capture_ms": round((after["capture_seconds"] - before["capture_seconds"]) * 1e3, 1),
         "steps_run_ahead": scheduler.steps_run_ahead,
-        "ttft_ms": ms(summary["ttft_seconds"]), "tpot_ms": ms(summary["tpot_seconds"]),
-        "e2e_ms": ms(summary["e2e_seconds"]),
-        "graphs": {"kept": graphs["captured_graphs"], "captures": graphs["captures"],
-                   "evicted": graphs["evicted"], "capture_ms": round(graphs["capture_seconds"] * 1e3, 1),
-                   "replays": graphs["graph_replays"], "layouts_remembered": graphs["layouts_remembered"]},
-        "config": {"model": "gpt2-medium-shape", "n_layer": config.n_layer, "n_layer_of_config": MEDIUM["n_layer"],
-                   "n_embd": config.n_embd, "n_head": config.n_head, "n_inner": config.n_inner,
-                   "vocab_size": config.vocab_size, "n_positions": config.n_positions,
-                   "request_rate": args.request_rate, "arrivals": "poisson seed 1234", "strategy": "sarathi",
-                   "prefill_chunk_size": 512, "max_batch_size": 64, "page_size": PAGE_SIZE},
+        "of_peak_flops": round(flops / summary["wall_seconds"] / (PEAK_TFLOPS[short] * 1e12), 4),
+        "ttft_ms": _ms(summary["ttft_seconds"]), "tpot_ms": _ms(summary["tpot_seconds"]),
+        "e2e_ms": _ms(summary["e2e_seconds"]),
     }
+
+
+def mixed_step_times(engine, config, decodes=32, portion=512, context=300, reps=5):
+    """One mixed step (``decodes`` decoded tokens beside a prompt portion) issued kernel by
+    kernel and replayed from its graph: milliseconds that the host needs to issue it, and
+    milliseconds until the GPU is through with it."""
+    import torch
+
+    from pagedserve_amd.engine import StepEntry
+
+    generator = torch.Generator().manual_seed(5)
+    names = [f"mixed_d{i}" for i in range(decodes)]
+    for name in names:
+        engine.step([StepEntry(name, _random_prompt(generator, context, config.vocab_size), [context - 1])])
+    prompt = _random_prompt(generator, portion, config.vocab_size)
+
+    def one(rep):
+        entries = [StepEntry(name, [5], [0]) for name in names] + [StepEntry(f"mixed_p{rep}", prompt, [])]
+        torch.cuda.synchronize()
+        started = time.perf_counter()
+        with torch.cuda.stream(engine.stream):
+            engine.step(entries, greedy=True)
+        host = time.perf_counter() - started
+        torch.cuda.synchronize()
+        wall = time.perf_counter() - started
+        engine.finish(f"mixed_p{rep}")
+        return host, wall
+
+    graphs = engine.use_graphs
+    engine.use_graphs = False
+    direct = [one(rep) for rep in range(reps + 2)][2:]
+    engine.use_graphs = graphs
+    replayed = [one(rep) for rep in range(reps + 2, 2 * reps + 8)][-reps:]
+    for name in names:
+        engine.finish(name)
+
+    def mean(values):
+        return round(sum(values) / len(values) * 1e3, 3)
+
+    return {"tokens": decodes + portion, "decoded": decodes,
+            "direct_host_ms": mean([h for h, _ in direct]), "direct_ms": mean([w for _, w in direct]),
+            "replayed_host_ms": mean([h for h, _ in replayed]), "replayed_ms": mean([w for _, w in replayed])}
+
+
+def stream_workload(args, shape, name, rates):
+    """The Poisson streams and the burst of one shape."""
+    import torch
+
+    from pagedserve_amd.engine import ContinuousBatchScheduler
+    from pagedserve_amd.sampling import SamplingParams
+
+    short = "bf16" if args.dtype == "bfloat16" else "fp32"
+    engine, sampler, config = _build(args.dtype, max_requests=64, max_step_tokens=PREFILL_TOKENS,
+                                     layers=args.layers, shape=shape)
+    requests = stream_requests(config, args.requests)
+    # the kernels' code is loaded by a few requests that are not part of the measurement
+    warm = ContinuousBatchScheduler(engine, sampler, max_batch_size=64, eos_token_id=None)
+    for request in requests[:2]:
+        warm.add_token_request(request.prompt_token_ids[:80], 4,
+                               sampling=SamplingParams(max_new_tokens=4, ignore_eos=True))
+    warm.run_until_complete()
+    runs = {}
+    for rate in rates:
+        runs[f"poisson_{int(rate)}_per_s"] = stream_run(engine, sampler, config, requests, rate, "poisson", short)
+    runs["burst"] = stream_run(engine, sampler, config, requests, None, "burst", short)
+    # several prompts may share an iteration's 512 prompt tokens: the last portion of one
+    # prompt runs beside the first of the next instead of alone
+    runs["burst_prompts_share_an_iteration"] = stream_run(engine, sampler, config, requests, None, "burst",
+                                                         short, prompts_per_iteration=8)
+    mixed = mixed_step_times(engine, config)
+    best = max(run["output_tok_s"] for key, run in runs.items() if "share" not in key)
+    record = {
+        "metric": f"output tok/s of streams of {args.requests} requests (GPT-2 {name} shape, prompts 32-896, "
+                  "outputs 16-128, prompt portions of 512, up to 64 requests an iteration)",
+        "value": best, "unit": "tokens/s", "higher_is_better": True, "dtype": short,
+        "data": "synthetic (random weights, uniform-random prompt ids and lengths, seeded arrivals)",
+        "requests": args.requests, "prompt_tokens": sum(len(r.prompt_token_ids) for r in requests),
+        "output_tokens": sum(r.max_new_tokens for r in requests),
+        "weights_resident_bytes": engine.weights_resident_bytes,
+        "runs": runs, "mixed_step": mixed,
+        "config": dict(_shape_keys(config, shape), model=f"gpt2-{name}-shape", strategy="sarathi",
+                       prefill_chunk_size=512, max_batch_size=64, arrivals="poisson seed 1234 / burst"),
+    }
+    del engine, sampler, warm
+    torch.cuda.empty_cache()
+    return record
 
 
 def xl_workload(args):
@@ -290,32 +411,75 @@ def xl_workload(args):
     wall = time.perf_counter() - started
     engine.cache.check_invariants()
     decode_tokens = batch * (output_len - 1)
+    short = "bf16" if args.dtype == "bfloat16" else "fp32"
     element = 2 if args.dtype == "bfloat16" else 4
     step_seconds = (wall - prefilled) / steps
     moved = decode_bytes(config, element, batch, prompt_len + output_len / 2.0)
+    prefill_flops = step_flops(config, [prompt_len] * batch, batch)
     graphs = engine.graph_summary()
-    return {
+    record = {
         "metric": "decode tok/s of 64 requests x (768 prompt + 256 output), temperature 0.8 seed 7 (GPT-2 XL shape)",
         "value": round(decode_tokens / (wall - prefilled), 1), "unit": "tokens/s", "n_gpus": 1,
-        "higher_is_better": True, "dtype": "bf16" if args.dtype == "bfloat16" else "fp32",
+        "higher_is_better": True, "dtype": short,
         "data": "synthetic (random weights, uniform-random prompt ids)",
         "wall_s": round(wall, 3), "prefill_s": round(prefilled, 3),
-        "prefill_tok_s": round(batch * prompt_len / prefilled, 1), "decode_steps": steps,
-        "ms_per_step": round(step_seconds * 1e3, 4),
+        "prefill_tok_s": round(batch * prompt_len / prefilled, 1),
+        "prefill_of_peak_flops": round(prefill_flops / prefilled / (PEAK_TFLOPS[short] * 1e12), 4),
+        "decode_steps": steps, "ms_per_step": round(step_seconds * 1e3, 4),
         "roofline": {"bound": "hbm", "achieved": round(moved / step_seconds / 1e9, 1), "peak": HBM_GBPS,
                      "unit": "GB/s", "frac": round(moved / step_seconds / 1e9 / HBM_GBPS, 4)},
+        "weights_resident_bytes": engine.weights_resident_bytes,
         "steps_run_ahead": scheduler.steps_run_ahead,
         "graphs": {"kept": graphs["captured_graphs"], "captures": graphs["captures"],
                    "evicted": graphs["evicted"], "capture_ms": round(graphs["capture_seconds"] * 1e3, 1)},
-        "config": {"model": "gpt2-xl-shape", "n_layer": config.n_layer, "n_layer_of_config": XL["n_layer"],
-                   "n_embd": config.n_embd, "n_head": config.n_head, "n_inner": config.n_inner,
-                   "vocab_size": config.vocab_size, "n_positions": config.n_positions, "global_batch": batch,
-                   "prompt_len": prompt_len, "output_len": output_len, "temperature": 0.8, "seed": 7,
-                   "page_size": PAGE_SIZE},
+        "config": dict(_shape_keys(config, XL), model="gpt2-xl-shape", global_batch=batch,
+                       prompt_len=prompt_len, output_len=output_len, temperature=0.8, seed=7),
     }
+    del engine, sampler, scheduler
+    torch.cuda.empty_cache()
+    return record
 
 
-SHAPES = {"small": SMALL, "medium": MEDIUM, "xl": XL}
+def long_points(args, short, element):
+    """The small layer sizes with 8,192 positions: decode over long contexts, a long prefill."""
+    import torch
+
+    engine, sampler, config = _build(args.dtype, max_requests=32, max_step_tokens=8192, layers=args.layers,
+                                     shape=LONG)
+    points = {}
+    for batch, context in ((8, 4096), (8, 8192), (32, 4096), (32, 8192)):
+        steps = 32
+        seconds, mean_context = decode_run(engine, sampler, config, batch, context, steps, 8, seed=context + batch)
+        points[f"decode_b{batch}_ctx{context}"] = {
+            "value": round(batch * steps / seconds, 1), "ms_per_step": round(seconds / steps * 1e3, 4),
+            "frac": _fraction(config, element, batch, mean_context, seconds / steps)}
+    seconds = prefill_run(engine, config, reps=4, warmup=4, prompts=2, length=4096)
+    flops = step_flops(config, [4096, 4096], 2)
+    points["prefill_2x4096"] = {"value": round(8192 / seconds, 1), "tokens": 8192, "ms": round(seconds * 1e3, 4),
+                                "frac": round(flops / seconds / (PEAK_TFLOPS[short] * 1e12), 4)}
+    points["n_positions"] = config.n_positions
+    del engine, sampler
+    torch.cuda.empty_cache()
+    return points
+
+
+def fp32_points(args):
+    """Decode at batch 8 and the prefill step in true 32-bit (no reduced-precision matrix mode)."""
+    import torch
+
+    engine, sampler, config = _build("float32", max_requests=8, max_step_tokens=PREFILL_TOKENS, layers=args.layers)
+    steps = 32
+    seconds, mean_context = decode_run(engine, sampler, config, 8, config.n_positions, steps, 8)
+    points = {"decode_b8": {"value": round(8 * steps / seconds, 1), "ms_per_step": round(seconds / steps * 1e3, 4),
+                            "frac": _fraction(config, 4, 8, mean_context, seconds / steps)}}
+    seconds = prefill_run(engine, config, reps=3, warmup=3)
+    flops = step_flops(config, [PREFILL_TOKENS // 2] * 2, 2)
+    points["prefill"] = {"value": round(PREFILL_TOKENS / seconds, 1), "tokens": PREFILL_TOKENS,
+                         "ms": round(seconds * 1e3, 4),
+                         "frac": round(flops / seconds / (PEAK_TFLOPS["fp32"] * 1e12), 4)}
+    del engine, sampler
+    torch.cuda.empty_cache()
+    return points
 
 
 def kernel_tables(args):
@@ -352,15 +516,19 @@ def main(argv=None):
     parser.add_argument("--batch", type=int, default=8)
     parser.add_argument("--dtype", default="bfloat16", choices=("bfloat16", "float32"))
     parser.add_argument("--layers", type=int, default=None, help="fewer layers than the configuration")
-    parser.add_argument("--no-points", action="store_true", help="skip batch 1 / 64 and prefill")
+    parser.add_argument("--no-points", action="store_true",
+                        help="only the decode step at --batch (no prefill, points or workloads)")
+    parser.add_argument("--no-workloads", action="store_true",
+                        help="skip the medium, small-stream and XL workloads and the 32-bit and long points")
     parser.add_argument("--prefill-only", action="store_true",
                         help="only the 2,048-token prefill step, --steps times (for profiles)")
-    parser.add_argument("--workload", choices=("small", "medium", "xl"), default="small",
-                        help="small: the decode / prefill record (default); medium: the Poisson "
-                             "stream at GPT-2 medium shape; xl: 64 x (768 + 256) at GPT-2 XL shape")
-    parser.add_argument("--requests", type=int, default=256, help="requests of --workload medium")
-    parser.add_argument("--request-rate", type=float, default=400.0,
-                        help="mean arrivals a second of --workload medium")
+    parser.add_argument("--workload", choices=("small", "medium", "small_stream", "xl"), default="small",
+                        help="small: the whole record (default); medium / small_stream: the streams at "
+                             "GPT-2 medium / small shape alone; xl: 64 x (768 + 256) at GPT-2 XL shape alone")
+    parser.add_argument("--requests", type=int, default=256, help="requests of the streams")
+    parser.add_argument("--request-rates", default=None,
+                        help="mean arrivals a second of the Poisson streams, comma-separated "
+                             "(default: 100,200,400 at medium shape, 300,600,1200 at small shape)")
     parser.add_argument("--kernels", action="store_true",
                         help="time every kernel of the decode and prefill steps alone (see above)")
     parser.add_argument("--shape", choices=("small", "medium", "xl", "all"), default="small",
@@ -379,9 +547,18 @@ def main(argv=None):
     if args.kernels:
         print(json.dumps(kernel_tables(args)), flush=True)
         return 0
-    if args.workload != "small":
-        record = medium_workload(args) if args.workload == "medium" else xl_workload(args)
-        print(json.dumps(record), flush=True)
+
+    def rates(default):
+        return [float(piece) for piece in args.request_rates.split(",")] if args.request_rates else default
+
+    if args.workload == "medium":
+        print(json.dumps(stream_workload(args, MEDIUM, "medium", rates([100.0, 200.0, 400.0]))), flush=True)
+        return 0
+    if args.workload == "small_stream":
+        print(json.dumps(stream_workload(args, SMALL, "small", rates([300.0, 600.0, 1200.0]))), flush=True)
+        return 0
+    if args.workload == "xl":
+        print(json.dumps(xl_workload(args)), flush=True)
         return 0
     short = "bf16" if args.dtype == "bfloat16" else "fp32"
     element = 2 if args.dtype == "bfloat16" else 4
@@ -415,6 +592,7 @@ def main(argv=None):
             "n_positions": config.n_positions, "global_batch": args.batch, "seq_len": context,
             "page_size": PAGE_SIZE, "activation": config.activation_function,
             "parallelism": "single-gpu", "hip_graphs": bool(engine.use_graphs),
+            "weights_resident_bytes": engine.weights_resident_bytes,
         },
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_GBPS,
                      "unit": "GB/s", "frac": round(achieved / HBM_GBPS, 4)},
@@ -427,24 +605,35 @@ def main(argv=None):
             "ms": round(seconds * 1e3, 4),
             "frac": round(flops / seconds / (PEAK_TFLOPS[short] * 1e12), 4)}
         points = {}
+        fractions = {}
         for batch in (1, 64):
             steps = min(args.steps, 64)
-            t, _ = decode_run(engine, sampler, config, batch, context, steps, min(args.warmup, 8),
-                              seed=batch)
+            t, mean_context = decode_run(engine, sampler, config, batch, context, steps, min(args.warmup, 8),
+                                         seed=batch)
             points[f"decode_b{batch}"] = round(batch * steps / t, 1)
+            fractions[f"decode_b{batch}"] = _fraction(config, element, batch, mean_context, t / steps)
         # the benchmark configuration's decode points: prompts of 128 and 512 tokens, 128
         # output tokens, at batch 1, 8 and 64
-        fractions = {}
         for prompt_len in (128, 512):
             for batch in (1, 8, 64):
                 t, mean_context = decode_point(engine, sampler, config, batch, prompt_len, 128,
                                                seed=prompt_len + batch)
                 name = f"p{prompt_len}_b{batch}"
                 points[name] = round(batch * 128 / t, 1)
-                fractions[name] = round(decode_bytes(config, element, batch, mean_context)
-                                        / (t / 128) / 1e9 / HBM_GBPS, 4)
+                fractions[name] = _fraction(config, element, batch, mean_context, t / 128)
         record["points"] = points
         record["points_roofline"] = fractions
+        if not args.no_workloads and args.dtype == "bfloat16":
+            del engine, sampler
+            torch.cuda.empty_cache()
+            record["points_long"] = long_points(args, short, element)
+            record["points_fp32"] = fp32_points(args)
+            args.requests = min(args.requests, 256)
+            record["workloads"] = {
+                "medium": stream_workload(args, MEDIUM, "medium", rates([100.0, 200.0, 400.0])),
+                "small_stream": stream_workload(args, SMALL, "small", rates([300.0, 600.0, 1200.0])),
+                "xl": xl_workload(args),
+            }
     print(json.dumps(record), flush=True)
     return 0
 

@@ -93,15 +93,17 @@ def ignorable(config: GPT2Config, name: str) -> bool:
     return config.tie_word_embeddings and name == "lm_head.weight"
 
 
-def random_tensors(config: GPT2Config, seed: int):
+def random_tensors(config: GPT2Config, seed: int, device="cpu"):
     """Checkpoint tensors of a random model: matrices and tables N(0, 0.02), the two
     projections into the residual stream N(0, 0.02 / sqrt(2 n_layer)), biases 0, norm
-    scales 1.  Drawn on the CPU from one seeded generator, in a fixed order."""
-    generator = torch.Generator(device="cpu").manual_seed(int(seed))
+    scales 1.  Drawn from one seeded generator in a fixed order, on the CPU unless another
+    device is named (a generator of another device draws other numbers: the CPU's are the ones
+    that a written folder holds)."""
+    generator = torch.Generator(device=device).manual_seed(int(seed))
     d, inner = config.n_embd, config.n_inner
 
     def normal(shape, std):
-        return torch.randn(shape, generator=generator, dtype=torch.float32) * std
+        return torch.randn(shape, generator=generator, dtype=torch.float32, device=device) * std
 
     residual_std = 0.02 / math.sqrt(2 * config.n_layer)
     tensors = {
@@ -110,20 +112,20 @@ def random_tensors(config: GPT2Config, seed: int):
     }
     for i in range(config.n_layer):
         h = f"h.{i}."
-        tensors[h + "ln_1.weight"] = torch.ones(d)
-        tensors[h + "ln_1.bias"] = torch.zeros(d)
+        tensors[h + "ln_1.weight"] = torch.ones(d, device=device)
+        tensors[h + "ln_1.bias"] = torch.zeros(d, device=device)
         tensors[h + "attn.c_attn.weight"] = normal((d, 3 * d), 0.02)
-        tensors[h + "attn.c_attn.bias"] = torch.zeros(3 * d)
+        tensors[h + "attn.c_attn.bias"] = torch.zeros(3 * d, device=device)
         tensors[h + "attn.c_proj.weight"] = normal((d, d), residual_std)
-        tensors[h + "attn.c_proj.bias"] = torch.zeros(d)
-        tensors[h + "ln_2.weight"] = torch.ones(d)
-        tensors[h + "ln_2.bias"] = torch.zeros(d)
+        tensors[h + "attn.c_proj.bias"] = torch.zeros(d, device=device)
+        tensors[h + "ln_2.weight"] = torch.ones(d, device=device)
+        tensors[h + "ln_2.bias"] = torch.zeros(d, device=device)
         tensors[h + "mlp.c_fc.weight"] = normal((d, inner), 0.02)
-        tensors[h + "mlp.c_fc.bias"] = torch.zeros(inner)
+        tensors[h + "mlp.c_fc.bias"] = torch.zeros(inner, device=device)
         tensors[h + "mlp.c_proj.weight"] = normal((inner, d), residual_std)
-        tensors[h + "mlp.c_proj.bias"] = torch.zeros(d)
-    tensors["ln_f.weight"] = torch.ones(d)
-    tensors["ln_f.bias"] = torch.zeros(d)
+        tensors[h + "mlp.c_proj.bias"] = torch.zeros(d, device=device)
+    tensors["ln_f.weight"] = torch.ones(d, device=device)
+    tensors["ln_f.bias"] = torch.zeros(d, device=device)
     if not config.tie_word_embeddings:
         tensors["lm_head.weight"] = normal((config.vocab_size, d), 0.02)
     return tensors

@@ -40,9 +40,14 @@ def load_model(folder, dtype="float32", device="cuda"):
     return model, config
 
 
-def random_model(config, seed=0, dtype="bfloat16", device="cuda"):
+def random_model(config, seed=0, dtype="bfloat16", device="cuda", draw_on=None):
     """A bound model with random weights of ``config`` (typed, or a raw config.json dict),
-    made in memory: the same draws, layouts and casts as writing a folder and loading it."""
+    made in memory: the same draws, layouts and casts as writing a folder and loading it.
+    ``draw_on``: a device on which the architecture's initialiser draws instead of the CPU, if
+    it takes one (seconds instead of a minute for billions of weights; the numbers then differ
+    from a written folder's, the distributions do not)."""
+    import inspect
+
     from ..weights.loader import target_dtype
 
     if isinstance(config, dict):
@@ -53,7 +58,10 @@ def random_model(config, seed=0, dtype="bfloat16", device="cuda"):
     spec = architecture.build_spec(config)
     engine_dtype = resolve_dtype(dtype)
     model = DecoderModel(spec, engine_dtype, device)
-    drawn = architecture.random_tensors(config, seed)
+    if draw_on is not None and "device" in inspect.signature(architecture.random_tensors).parameters:
+        drawn = architecture.random_tensors(config, seed, device=draw_on)
+    else:
+        drawn = architecture.random_tensors(config, seed)
     sources = architecture.weight_sources(config, spec)
     tensors = {}
     for target, param in model.parameters().items():
