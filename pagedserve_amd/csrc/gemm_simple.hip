@@ -7,6 +7,14 @@
 //
 // Tile: 64 x 64 outputs per 256-thread block, 16 k per stage through LDS, 4 x 4 outputs per
 // thread.  Any m, n, k and any row strides; loads are bounds-checked and zero-filled.
+//
+// Up to 16 rows of float (a decode step of the 32-bit path) take a second kernel: the tiled one
+// would run on n / 64 blocks that each walk the whole k in stages of 16, a few dozen blocks
+// bound by the latency of hundreds of dependent trips (8 rows x 2304 x 768: 70 us).  Here a
+// wave owns a few output columns, its lanes stride over k with 16-byte loads of the weights
+// (each read once, as the step's bytes are the weights') and of the rows (which the caches
+// hold), every lane sums its share in ascending k, and the lanes' sums are added in a fixed
+// tree: a row's result does not depend on the other rows here either.
 #include "common.h"
 #include "pagedserve_hip.h"
 
@@ -85,6 +93,94 @@ __global__ __launch_bounds__(256) void gemm_nt_simple_kernel(
   }
 }
 
+// MR: rows held in registers (m <= MR); COLS: output columns per wave
+template <int EPI, int MR, int COLS>
+__global__ __launch_bounds__(256) void gemm_nt_f32_rows_kernel(
+    const float* __restrict__ a, const float* __restrict__ w, const float* __restrict__ bias,
+    float* __restrict__ c, int m, int n, int k, int lda, int ldc) {
+  const int lane = threadIdx.x & 63;
+  const int wave = threadIdx.x >> 6;
+  const int col0 = (blockIdx.x * 4 + wave) * COLS;
+  if (col0 >= n) return;
+  const float* w_row[COLS];
+#pragma unroll
+  for (int j = 0; j < COLS; ++j) w_row[j] = w + (int64_t)(col0 + j < n ? col0 + j : n - 1) * k;
+  const float* a_row[MR];
+#pragma unroll
+  for (int r = 0; r < MR; ++r) a_row[r] = a + (int64_t)(r < m ? r : m - 1) * lda;
+  float acc[COLS][MR];
+#pragma unroll
+  for (int j = 0; j < COLS; ++j)
+#pragma unroll
+    for (int r = 0; r < MR; ++r) acc[j][r] = 0.f;
+  for (int k0 = lane * 4; k0 < k; k0 += 256) {
+    float4 wv[COLS];
+#pragma unroll
+    for (int j = 0; j < COLS; ++j) wv[j] = *reinterpret_cast<const float4*>(w_row[j] + k0);
+#pragma unroll
+    for (int r = 0; r < MR; ++r) {
+      const float4 av = *reinterpret_cast<const float4*>(a_row[r] + k0);
+#pragma unroll
+      for (int j = 0; j < COLS; ++j) {
+        acc[j][r] = fmaf(av.x, wv[j].x, acc[j][r]);
+        acc[j][r] = fmaf(av.y, wv[j].y, acc[j][r]);
+        acc[j][r] = fmaf(av.z, wv[j].z, acc[j][r]);
+        acc[j][r] = fmaf(av.w, wv[j].w, acc[j][r]);
+      }
+    }
+  }
+  // every lane receives every total; lane j * MR + r finishes output (row r, column col0 + j)
+  float mine = 0.f;
+#pragma unroll
+  for (int j = 0; j < COLS; ++j)
+#pragma unroll
+    for (int r = 0; r < MR; ++r) {
+      const float total = wave_sum(acc[j][r]);
+      if (lane == j * MR + r) mine = total;
+    }
+  static_assert(COLS * MR <= 64, "one output per lane");
+  const int j = lane / MR;
+  const int r = lane - j * MR;
+  const int col = col0 + j;
+  if (j >= COLS || r >= m || col >= n) return;
+  float v = mine;
+  if (bias != nullptr) v += bias[col];
+  v = apply_activation<EPI>(v);
+  float* dst = c + (int64_t)r * ldc + col;
+  if (EPI == PS_EPI_RESIDUAL) v += *dst;
+  *dst = v;
+}
+
+static bool rows_kernel_takes(const void* a, const void* w, int m, int k, int lda) {
+  return m >= 1 && m <= 16 && k % 4 == 0 && lda % 4 == 0 &&
+         (reinterpret_cast<uintptr_t>(a) & 15u) == 0 && (reinterpret_cast<uintptr_t>(w) & 15u) == 0;
+}
+
+static int launch_f32_rows(const void* a, const void* w, const float* bias, void* c, int m, int n,
+                           int k, int lda, int ldc, int epilogue, hipStream_t s) {
+#define PS_LAUNCH_FR(EPI, MR, COLS)                                                              \
+  hipLaunchKernelGGL((gemm_nt_f32_rows_kernel<EPI, MR, COLS>), dim3((n + 4 * COLS - 1) / (4 * COLS)), \
+                     dim3(256), 0, s, (const float*)a, (const float*)w, bias, (float*)c, m, n, k, \
+                     lda, ldc)
+#define PS_LAUNCH_FR_M(EPI)                      \
+  do {                                           \
+    if (m <= 4) PS_LAUNCH_FR(EPI, 4, 4);         \
+    else if (m <= 8) PS_LAUNCH_FR(EPI, 8, 4);    \
+    else PS_LAUNCH_FR(EPI, 16, 2);               \
+  } while (0)
+  switch (epilogue) {
+    case PS_EPI_NONE: PS_LAUNCH_FR_M(PS_EPI_NONE); break;
+    case PS_EPI_GELU_TANH: PS_LAUNCH_FR_M(PS_EPI_GELU_TANH); break;
+    case PS_EPI_GELU_ERF: PS_LAUNCH_FR_M(PS_EPI_GELU_ERF); break;
+    case PS_EPI_RESIDUAL: PS_LAUNCH_FR_M(PS_EPI_RESIDUAL); break;
+    default: ps_set_error("ps_gemm_nt: unknown epilogue %d", epilogue); return 1;
+  }
+#undef PS_LAUNCH_FR_M
+#undef PS_LAUNCH_FR
+  PS_CHECK_LAUNCH("ps_gemm_nt(float rows)");
+  return 0;
+}
+
 template <typename TIn, typename TOut>
 static int launch_simple(const void* a, const void* w, const float* bias, void* c, int m, int n,
                          int k, int lda, int ldc, int epilogue, hipStream_t s) {
@@ -107,6 +203,8 @@ static int launch_simple(const void* a, const void* w, const float* bias, void* 
 int ps_gemm_nt_simple(const void* a, const void* w, const float* bias, void* c, int m, int n,
                       int k, int lda, int ldc, int dtype, int c_dtype, int epilogue,
                       hipStream_t s) {
+  if (dtype == PS_F32 && c_dtype == PS_F32 && rows_kernel_takes(a, w, m, k, lda))
+    return launch_f32_rows(a, w, bias, c, m, n, k, lda, ldc, epilogue, s);
   if (dtype == PS_F32 && c_dtype == PS_F32)
     return launch_simple<float, float>(a, w, bias, c, m, n, k, lda, ldc, epilogue, s);
   if (dtype == PS_BF16 && c_dtype == PS_F32)

@@ -113,7 +113,10 @@ GEMM_SHAPES = [(1, 50, 64), (5, 1000, 96), (64, 2304, 768), (130, 70, 320), (33,
                # ragged last tile and a last k range of one step
                (33, 1290, 5184), (20, 1600, 6400),
                # few rows and very many columns: two tiles of columns per block, ragged end
-               (9, 16411, 320), (16, 20000, 768)]
+               (9, 16411, 320), (16, 20000, 768),
+               # few rows in float: a k shorter than one pass of a wave's lanes, a k that is a
+               # multiple of 4 only, columns that end inside a wave's share
+               (13, 41, 16), (3, 333, 60), (4, 101, 100), (16, 7, 1028)]
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
