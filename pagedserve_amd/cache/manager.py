@@ -39,9 +39,14 @@ class CacheGroupSpec:
     kv_heads: int
     head_dim: int
     window: int = 0  # 0: every earlier key stays visible
+    value_dim: int = 0  # head size of the values where it differs from the keys' (0: the same)
+
+    @property
+    def value_head_dim(self) -> int:
+        return self.value_dim or self.head_dim
 
     def geometry(self):
-        return (self.kv_heads, self.head_dim, self.window)
+        return (self.kv_heads, self.head_dim, self.window, self.value_head_dim)
 
 
 @dataclass(frozen=True)
@@ -153,9 +158,10 @@ class CacheManager:
         self.value_pools: List[Optional[torch.Tensor]] = []
         for group, pool in zip(self.groups, self.pools):
             if allocate_pools:
-                shape = (len(group.entries), pool.num_pages, group.kv_heads, page_size, group.head_dim)
-                self.key_pools.append(torch.empty(shape, dtype=dtype, device=self.device))
-                self.value_pools.append(torch.empty(shape, dtype=dtype, device=self.device))
+                shape = (len(group.entries), pool.num_pages, group.kv_heads, page_size)
+                self.key_pools.append(torch.empty(shape + (group.head_dim,), dtype=dtype, device=self.device))
+                self.value_pools.append(torch.empty(shape + (group.value_head_dim,), dtype=dtype,
+                                                    device=self.device))
             else:
                 self.key_pools.append(None)
                 self.value_pools.append(None)
@@ -181,7 +187,8 @@ class CacheManager:
         group = self.groups[group_index]
         element = torch.empty(0, dtype=self.dtype).element_size()
         # src/model/kv_manager.py:55-58
-        return 2 * len(group.entries) * group.kv_heads * self.page_size * group.head_dim * element
+        return (len(group.entries) * group.kv_heads * self.page_size
+                * (group.head_dim + group.value_head_dim) * element)
 
     def pages_for_length(self, group_index: int, length: int, longest_step: Optional[int] = None) -> int:
         """Most pages that one request of ``length`` tokens holds in a group at any
@@ -312,7 +319,8 @@ class CacheManager:
 
     # ------------------------------------------------------------------ views
     def entry_pools(self, entry: int):
-        """(keys, values) of one cache entry: ``[pages, kv_heads, page, head_dim]``."""
+        """(keys, values) of one cache entry: ``[pages, kv_heads, page, head_dim]`` (the values
+        with their own head size where the group names one)."""
         group_index, local = self.entry_location[entry]
         return self.key_pools[group_index][local], self.value_pools[group_index][local]
 

@@ -29,7 +29,8 @@ REFERENCE_MODEL = "reference"   # a preset that the architecture's registry entr
 def _bytes_per_page(model, page_size, dtype):
     groups, _ = model.cache_requirements()
     element = torch.empty(0, dtype=dtype).element_size()
-    return sum(2 * len(g.entries) * g.kv_heads * page_size * g.head_dim * element for g in groups)
+    return sum(len(g.entries) * g.kv_heads * page_size * (g.head_dim + g.value_head_dim) * element
+               for g in groups)
 
 
 def build_scheduler(model=REFERENCE_MODEL, scheduling_strategy=ORCA_STRATEGY, prefill_chunk_size=16,

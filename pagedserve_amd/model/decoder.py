@@ -101,13 +101,14 @@ class DecoderModel:
         for entry in sorted(self._entry_spec):
             spec = self._entry_spec[entry]
             if isinstance(spec, PagedKVSpec):
-                by_geometry.setdefault((spec.kv_heads, spec.head_dim, spec.window), []).append(entry)
+                by_geometry.setdefault((spec.kv_heads, spec.head_dim, spec.window, spec.value_dim),
+                                       []).append(entry)
             elif isinstance(spec, SlotStateSpec):
                 states.append(StateSpec(entry, tuple(spec.shape), spec.dtype))
             elif spec is not None:
                 raise TypeError(f"unknown cache spec {spec!r}")
-        groups = [CacheGroupSpec(tuple(entries), kv_heads, head_dim, window)
-                  for (kv_heads, head_dim, window), entries in by_geometry.items()]
+        groups = [CacheGroupSpec(tuple(entries), kv_heads, head_dim, window, value_dim)
+                  for (kv_heads, head_dim, window, value_dim), entries in by_geometry.items()]
         return groups, states
 
     def cache_views(self, cache) -> List[CacheView]:

@@ -40,6 +40,7 @@ class PagedKVSpec:
     kv_heads: int
     head_dim: int
     window: int = 0
+    value_dim: int = 0     # head size of the cached values where it is not the keys' (0: the same)
 
 
 @dataclass(frozen=True)
@@ -58,7 +59,7 @@ class CacheView:
     writes: bool
     group: Optional[int] = None                # index of the cache group (paged entries)
     k_pool: Optional[torch.Tensor] = None      # [pages, kv_heads, page, head_dim]
-    v_pool: Optional[torch.Tensor] = None
+    v_pool: Optional[torch.Tensor] = None      # [pages, kv_heads, page, value head size]
     state: Optional[torch.Tensor] = None       # [max_slots, ...]
 
 

@@ -258,3 +258,20 @@ def test_random_orders_keep_the_invariants(seed, window):
     manager.check_invariants()
     assert all(pool.num_free == pool.num_pages for pool in manager.pools)
     assert len(manager.free_slots) == 5
+
+
+def test_values_may_have_another_head_size_than_keys():
+    """A group whose values are narrower than its keys: the value pool has its own last
+    dimension, a page's bytes count both, and groups that differ only in that are different
+    groups."""
+    wide = CacheGroupSpec((0,), 2, 16, 0, value_dim=8)
+    same = CacheGroupSpec((1,), 2, 16)
+    assert wide.value_head_dim == 8 and same.value_head_dim == 16
+    assert wide.geometry() != same.geometry()
+    manager = CacheManager([wide, same], 5, 4, 2, torch.float32, "cpu")
+    keys, values = manager.entry_pools(0)
+    assert keys.shape == (5, 2, 4, 16) and values.shape == (5, 2, 4, 8)
+    keys, values = manager.entry_pools(1)
+    assert keys.shape == values.shape == (5, 2, 4, 16)
+    assert manager.bytes_per_page(0) == 2 * 4 * (16 + 8) * 4
+    assert manager.bytes_per_page(1) == 2 * 4 * (16 + 16) * 4

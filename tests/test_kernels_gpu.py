@@ -13,7 +13,11 @@ DTYPES = [torch.float32, torch.bfloat16]
 
 
 def _tol(dtype):
-    return (2e-5, 2e-5) if dtype == torch.float32 else (2e-2, 2e-2)
+    """(atol, rtol).  bfloat16: a result stored in bfloat16 is off by up to 2^-9 of itself (half a
+    unit in the last place), and inputs rounded the same way move a sum of k products by some
+    2^-9 of its terms' size; measured, the kernels here stay within 9e-4 + 9e-4 |expected| at
+    every shape of these tests, and the bound leaves five times that."""
+    return (2e-5, 2e-5) if dtype == torch.float32 else (5e-3, 5e-3)
 
 
 def _rand(shape, dtype, seed, scale=1.0):
@@ -408,7 +412,7 @@ def test_attention_far_key_stands_out():
                 page = int(tables[item, key // page_size])
                 expected = v_pool[page, head, key % page_size].float()
                 got = out[item, head * head_dim:(head + 1) * head_dim].float()
-                torch.testing.assert_close(got, expected, atol=2e-2, rtol=2e-2)
+                torch.testing.assert_close(got, expected, atol=5e-3, rtol=5e-3)
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
@@ -566,7 +570,7 @@ def test_attention_prefill_tiles(heads, kv_heads, head_dim, page_size, window):
     kernels.attention_prefill(q, k_pool, v_pool, out, dev(tile_item), dev(tile_q0), dev(cu), dev(totals),
                               tables, heads, scale, window=window)
     assert torch.isfinite(out.float()).all()
-    torch.testing.assert_close(out.double(), expected, atol=2e-2, rtol=2e-2)
+    torch.testing.assert_close(out.double(), expected, atol=5e-3, rtol=5e-3)
 
 
 def test_attention_prefill_far_key_and_causality():
@@ -593,7 +597,7 @@ def test_attention_prefill_far_key_and_causality():
                               dev([0, total]), dev([total]), tables, heads, head_dim ** -0.5)
     value = v_pool[page, 0, target % page_size].float()
     for row in (137, 138, 299):
-        torch.testing.assert_close(out[row].float(), value, atol=2e-2, rtol=2e-2)
+        torch.testing.assert_close(out[row].float(), value, atol=5e-3, rtol=5e-3)
     assert float((out[136].float() - value).abs().max()) > 0.3
 
 
@@ -717,7 +721,7 @@ def test_norm_product_scatters_keys_and_values(m):
     scratch = torch.empty((m, k), dtype=dtype, device="cuda")
     kernels.linear(kernels.PendingNorm(h, gamma, beta, 1e-5, False, scratch), w, bias, out, packed=packed,
                    scatter=(k_pool, v_pool, tok_item, tok_pos, tables, q_cols, kv_cols))
-    torch.testing.assert_close(out.float(), plain.float(), atol=4e-2, rtol=2e-2)
+    torch.testing.assert_close(out.float(), plain.float(), atol=1e-2, rtol=5e-3)
     kernels.kv_write(out[:, q_cols:q_cols + kv_cols], out[:, q_cols + kv_cols:], k_ref, v_ref, tok_item, tok_pos, tables)
     view = torch.int16
     assert torch.equal(k_pool.view(view), k_ref.view(view)) and torch.equal(v_pool.view(view), v_ref.view(view))
@@ -920,7 +924,7 @@ def test_linear_takes_the_wide_product_for_long_k():
     kernels.linear(x, w, bias, out, packed=packed,
                    scatter=(k_pool, v_pool, tok_item, tok_pos, tables, q_cols, kv_cols))
     expected = x.double() @ w.double().t() + bias.double()
-    torch.testing.assert_close(out.double(), expected, atol=4e-2, rtol=2e-2)
+    torch.testing.assert_close(out.double(), expected, atol=1e-2, rtol=5e-3)
     # the two kernels add the k tiles in the same order: the same bits
     assert torch.equal(out, plain)
     assert torch.equal(k_pool.view(torch.int16), k_ref.view(torch.int16))
@@ -958,13 +962,13 @@ def test_attention_records_merged_inside_the_output_projection(heads, kv_heads, 
     kernels.attention_merge_linear(partial, count, heads, head_dim, splits, w, packed, bias, residual)
     context = _attention_expected(q, k_pool, v_pool, tables, tok_item, tok_pos, heads, scale)
     expected = start[:count].double() + context.to(dtype).double() @ w.double().t() + bias.double()
-    torch.testing.assert_close(residual[:count].double(), expected, atol=2e-2, rtol=2e-2)
+    torch.testing.assert_close(residual[:count].double(), expected, atol=5e-4, rtol=5e-4)
     assert torch.equal(residual[count:], start[count:])
     for heads_per_block in (1, 2, 4):
         grouped = start.clone()
         kernels.attention_merge_linear(partial, count, heads, head_dim, splits, w, packed, bias, grouped,
                                        heads_per_block=heads_per_block)
-        torch.testing.assert_close(grouped[:count].double(), expected, atol=2e-2, rtol=2e-2)
+        torch.testing.assert_close(grouped[:count].double(), expected, atol=5e-4, rtol=5e-4)
         # the same products, summed in another order
         torch.testing.assert_close(grouped[:count], residual[:count], atol=1e-4, rtol=1e-4)
         assert torch.equal(grouped[count:], start[count:])
@@ -974,7 +978,7 @@ def test_attention_records_merged_inside_the_output_projection(heads, kv_heads, 
     kernels.attention_decode_partial(q, k_pool, v_pool, partial, tok_item, tok_pos, tables, heads, scale, splits,
                                      tok_list=chosen)
     kernels.attention_merge_linear(partial, count, heads, head_dim, splits, w, packed, bias, residual, tok_list=chosen)
-    torch.testing.assert_close(residual[:count].double(), expected, atol=2e-2, rtol=2e-2)
+    torch.testing.assert_close(residual[:count].double(), expected, atol=5e-4, rtol=5e-4)
     assert not kernels.merge_linear_supported(dtype, 17, head_dim, packed)
     assert not kernels.merge_linear_supported(dtype, count, 48, packed)
     assert not kernels.merge_linear_supported(torch.float32, count, head_dim, packed)
@@ -1034,7 +1038,7 @@ def test_head_product_leaves_the_choice_where_it_cannot_make_it():
         top = kernels.TopChoice(m, "cuda")
         _, chosen = kernels.linear(a, w, None, out, choose=(top, tokens))
         assert not chosen and (tokens == -7).all()
-        torch.testing.assert_close(out.double(), a.double() @ w.double().t(), atol=2e-2, rtol=2e-2)
+        torch.testing.assert_close(out.double(), a.double() @ w.double().t(), atol=2e-4, rtol=2e-4)
     with pytest.raises(kernels.KernelError, match="plain float output"):
         kernels.linear(a, w, None, out, epilogue="gelu_tanh", choose=(top, tokens))
 

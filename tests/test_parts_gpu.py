@@ -17,7 +17,8 @@ DTYPES = [torch.float32, torch.bfloat16]
 
 
 def _tol(dtype):
-    return 2e-5 if dtype == torch.float32 else 2e-2
+    # bfloat16: five times what the parts measure (see tests/test_kernels_gpu.py: _tol)
+    return 2e-5 if dtype == torch.float32 else 5e-3
 
 
 def _ctx(engine_like, requests):
