@@ -384,7 +384,9 @@ def xl_workload(args):
     from pagedserve_amd.engine import ContinuousBatchScheduler
     from pagedserve_amd.sampling import SamplingParams
 
-    engine, sampler, config = _build(args.dtype, max_requests=64, max_step_tokens=PREFILL_TOKENS,
+    # (prompts are prefilled 4,096 tokens a step: 184 k prompt tokens a second where steps of
+    # 2,048 give 141 k: the products fill the chip with whole rounds of tiles)
+    engine, sampler, config = _build(args.dtype, max_requests=64, max_step_tokens=2 * PREFILL_TOKENS,
                                      layers=args.layers, shape=XL)
     scheduler = ContinuousBatchScheduler(engine, sampler, max_batch_size=64, eos_token_id=None)
     generator = torch.Generator().manual_seed(0)
@@ -433,7 +435,8 @@ def xl_workload(args):
         "graphs": {"kept": graphs["captured_graphs"], "captures": graphs["captures"],
                    "evicted": graphs["evicted"], "capture_ms": round(graphs["capture_seconds"] * 1e3, 1)},
         "config": dict(_shape_keys(config, XL), model="gpt2-xl-shape", global_batch=batch,
-                       prompt_len=prompt_len, output_len=output_len, temperature=0.8, seed=7),
+                       prompt_len=prompt_len, output_len=output_len, temperature=0.8, seed=7,
+                       max_step_tokens=engine.max_step_tokens),
     }
     del engine, sampler, scheduler
     torch.cuda.empty_cache()

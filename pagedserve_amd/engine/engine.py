@@ -121,6 +121,9 @@ class Engine:
         # a part that looks at host values of a step cannot be replayed
         self.use_graphs = use_graphs and getattr(model, "graph_safe", False)
         self.max_graphs = 48     # recorded layouts kept; the least recently replayed goes first
+        # direct runs of a layout with a prompt portion before it is recorded (a decode layout
+        # is recorded at its second step)
+        self.record_after = 3
         self.max_layouts_remembered = 512
         self._graphs = {}        # key -> StepGraph
         self._graph_seen = {}     # layout -> steps that ran without a graph (buffers exist now)
@@ -532,7 +535,7 @@ class Engine:
         # at once and are recorded at their second step, others when they keep coming back.
         seen_key = graph_key + (logits.data_ptr(),)
         seen = self._graph_seen.get(seen_key, 0)
-        if seen < (1 if singles == ctx.tokens else 3):
+        if seen < (1 if singles == ctx.tokens else self.record_after):
             # (re-inserted at the end: the layouts that have not come back for longest go first)
             self._graph_seen.pop(seen_key, None)
             self._graph_seen[seen_key] = seen + 1
