@@ -140,14 +140,14 @@ class DecoderModel:
         ``self.tokens_chosen`` says whether it did."""
         self.tokens_chosen = False
         tokens = ctx.tokens
-        h = ctx.workspace.rows("residual", self.spec.width, torch.float32)[:tokens]
+        h = ctx.workspace.first_rows("residual", self.spec.width, torch.float32, tokens)
         self.embedding.forward(ctx, self.position.embedding_table(), h)
         for call, view in zip(self.spec.schedule, views):
             self.blocks[call.block].forward(h, ctx, view)
         wanted = logit_rows.numel()
         if wanted == 0:
             return logits_out[:0]
-        final = ctx.workspace.rows("final", self.spec.width, self.dtype)[:wanted]
+        final = ctx.workspace.first_rows("final", self.spec.width, self.dtype, wanted)
         normed = None
         if getattr(self.head, "accepts_pending_norm", False):
             normed = self.final_norm.pending(h, final, rows=logit_rows)

@@ -300,8 +300,26 @@ class TopChoice:
         self.ticket = torch.zeros((1 + TOP_SLOTS) * 64, dtype=torch.int32, device=device)
 
 
+_MEMO_LIMIT = 512
+
+
+def _memo_key(x, out, scatter, a_packed, choose):
+    """What may differ between two calls of one call site: the row count and the addresses of
+    the operands that are not the site's own (weights, bias, flags are)."""
+    if isinstance(x, PendingNorm):
+        key = (x.count, x.h.data_ptr(), _ptr(x.rows), x.scratch.data_ptr(), x.gamma.data_ptr(),
+               out.data_ptr())
+    else:
+        key = (x.shape[0], x.data_ptr(), x.stride(0), out.data_ptr(), a_packed)
+    if scatter is not None:
+        key += (scatter[0].data_ptr(), scatter[2].data_ptr(), scatter[3].data_ptr(), scatter[4].data_ptr())
+    if choose is not None:
+        key += (choose[1].data_ptr(),)
+    return key
+
+
 def linear(x, w, bias, out, epilogue="none", scatter=None, packed=None, a_packed=False,
-           packed_out=False, choose=None, scatter_only=False):
+           packed_out=False, choose=None, scatter_only=False, memo=None):
     """out = epilogue(x w^T + bias) where ``x`` is a tensor or a ``PendingNorm``.
 
     ``scatter = (k_pool, v_pool, tok_item, tok_pos, tables, q_cols, kv_cols)`` also stores the
@@ -319,7 +337,28 @@ def linear(x, w, bias, out, epilogue="none", scatter=None, packed=None, a_packed
     ``choose = (TopChoice, tokens)`` asks for ``tokens[r]`` = the column of the largest value of
     row ``r`` of a float ``out`` (the lowest on ties), as ``sample`` gives it without a
     temperature; the call then returns ``(out, chosen)``, and where ``chosen`` is False the
-    kernel that ran could not do it and ``tokens`` is untouched."""
+    kernel that ran could not do it and ``tokens`` is untouched.
+
+    ``memo``: a dict that belongs to ONE call site, whose ``w``, ``bias``, ``packed``, epilogue
+    and flags are the same on every call (a part's product).  The checked argument block of a
+    call is kept in it under the row count and the addresses of the other operands, and a call
+    that finds its block goes straight to the library: checking and filling the block costs
+    the host more than the launch, and a step that is not replayed from a graph issues four
+    such calls a layer.  Whoever binds other weights clears the dict."""
+    if memo is not None:
+        key = _memo_key(x, out, scatter, a_packed, choose)
+        kept = memo.get(key)
+        if kept is not None:
+            args, layout, done = kept
+            status = _BOUND["ps_linear"](ctypes.byref(args), _stream())
+            if status != 0:
+                raise KernelError(f"ps_linear failed ({status}): "
+                                  f"{load_library().ps_last_error().decode('utf-8', 'replace')}")
+            if packed_out:
+                return out, bool(layout.value)
+            if choose is not None:
+                return out, bool(done.value)
+            return out
     _check(w, "w", ndim=2)
     _check(out, "out", ndim=2)
     n, k = w.shape
@@ -432,6 +471,10 @@ def linear(x, w, bias, out, epilogue="none", scatter=None, packed=None, a_packed
     status = fn(ctypes.byref(args), _stream())
     if status != 0:
         raise KernelError(f"ps_linear failed ({status}): {lib.ps_last_error().decode('utf-8', 'replace')}")
+    if memo is not None:
+        if len(memo) >= _MEMO_LIMIT:
+            memo.clear()
+        memo[key] = (args, layout, done)     # (the block points at ``layout`` and ``done``)
     if packed_out:
         return out, bool(layout.value)
     if choose is not None:

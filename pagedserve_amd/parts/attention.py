@@ -46,6 +46,9 @@ class Attention(Mixer):
         self.q_cols = heads * head_dim
         self.kv_cols = kv_heads * head_dim
         self.position = None
+        self._columns = {}
+        # what ``kernels.linear`` keeps per call site and step shape (its ``memo``)
+        self._memo_qkv, self._memo_out = {}, {}
 
     def parameters(self):
         total = self.q_cols + 2 * self.kv_cols
@@ -66,6 +69,8 @@ class Attention(Mixer):
         # copies in the layout that the products of few rows (decode steps) read fastest
         self.qkv_packed = kernels.pack_decode_weight(self.qkv_weight)
         self.out_packed = kernels.pack_decode_weight(self.out_weight)
+        self._memo_qkv.clear()
+        self._memo_out.clear()
 
     def cache_spec(self):
         return PagedKVSpec(self.kv_heads, self.head_dim, self.window)
@@ -73,26 +78,33 @@ class Attention(Mixer):
     def forward(self, x, residual, ctx, cache):
         tokens = ctx.tokens
         total = self.q_cols + 2 * self.kv_cols
-        qkv = ctx.workspace.rows("qkv", total, self.dtype)[:tokens]
+        qkv = ctx.workspace.first_rows("qkv", total, self.dtype, tokens)
         tables = ctx.tables[cache.group]
-        q = qkv[:, :self.q_cols]
-        k = qkv[:, self.q_cols:self.q_cols + self.kv_cols]
-        v = qkv[:, self.q_cols + self.kv_cols:]
+        columns = self._columns.get(tokens)
+        if columns is None or columns[0] is not qkv:
+            # (the three column views of a step's rows, made once per row count)
+            if len(self._columns) > 1024:
+                self._columns.clear()
+            columns = self._columns[tokens] = (qkv, qkv[:, :self.q_cols],
+                                               qkv[:, self.q_cols:self.q_cols + self.kv_cols],
+                                               qkv[:, self.q_cols + self.kv_cols:])
+        _, q, k, v = columns
         rotates = self.position is not None and self.position.transforms_qk
         if cache.writes and not rotates:
             # keys and values go to their pages from the product's own epilogue
             kernels.linear(x, self.qkv_weight, self.qkv_bias, qkv,
                            scatter=(cache.k_pool, cache.v_pool, ctx.tok_item, ctx.positions, tables,
                                     self.q_cols, self.kv_cols), packed=self.qkv_packed,
-                           scatter_only=True)
+                           scatter_only=True, memo=self._memo_qkv)
         else:
-            kernels.linear(x, self.qkv_weight, self.qkv_bias, qkv, packed=self.qkv_packed)
+            kernels.linear(x, self.qkv_weight, self.qkv_bias, qkv, packed=self.qkv_packed,
+                           memo=self._memo_qkv)
             if rotates:
                 self.position.apply_to_qk(q, k, ctx)
             if cache.writes:
                 kernels.kv_write(k, v, cache.k_pool, cache.v_pool, ctx.tok_item, ctx.positions,
                                  tables)
-        context = ctx.workspace.rows("attn", self.q_cols, self.dtype)[:tokens]
+        context = ctx.workspace.first_rows("attn", self.q_cols, self.dtype, tokens)
         singles = ctx.single_tokens.numel() if ctx.single_tokens is not None else 0
         if not kernels.decode_supported(self.head_dim):
             # a head size that the split-KV kernel does not take: every token, decoded ones
@@ -145,7 +157,7 @@ class Attention(Mixer):
                                       ctx.positions, tables, self.heads, self.scale, self.window,
                                       tok_list=None if whole else ctx.portion_tokens)
         kernels.linear(context, self.out_weight, self.out_bias, residual, epilogue="residual",
-                       packed=self.out_packed)
+                       packed=self.out_packed, memo=self._memo_out)
 
     def _range_records(self, ctx):
         """Scratch for one record per (token, head, key range): always asked for at its largest

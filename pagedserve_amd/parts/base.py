@@ -162,6 +162,7 @@ class Workspace:
         # counts the buffers that were replaced by larger ones: whoever holds addresses
         # (recorded graphs) compares it with the value at the time of recording
         self.moved = 0
+        self._views: Dict[tuple, torch.Tensor] = {}
 
     def rows(self, name: str, columns: int, dtype: torch.dtype, max_rows: Optional[int] = None):
         key = (name, columns, dtype, max_rows or self.max_rows)
@@ -170,6 +171,18 @@ class Workspace:
             buffer = torch.empty((max_rows or self.max_rows, columns), dtype=dtype, device=self.device)
             self._buffers[key] = buffer
         return buffer
+
+    def first_rows(self, name: str, columns: int, dtype: torch.dtype, count: int):
+        """``rows(name, columns, dtype)[:count]``, the same tensor object every time: a step of a
+        layer asks for a handful of such views, and making a view costs the host as much as
+        half a kernel launch."""
+        key = (name, columns, dtype, count)
+        view = self._views.get(key)
+        if view is None:
+            if len(self._views) > 4096:
+                self._views.clear()
+            view = self._views[key] = self.rows(name, columns, dtype)[:count]
+        return view
 
     def flat(self, name: str, numel: int, dtype: torch.dtype):
         """A 1-D scratch buffer of at least ``numel`` elements; callers ask for their worst

@@ -35,7 +35,7 @@ class PreNormBlock:
 
     def _normed(self, norm, part, h, ctx):
         """Input of ``part``: the norm as a pending object if the part takes one, else rows."""
-        scratch = ctx.workspace.rows("normed", self.width, self.dtype)[:ctx.tokens]
+        scratch = ctx.workspace.first_rows("normed", self.width, self.dtype, ctx.tokens)
         if getattr(part, "accepts_pending_norm", False):
             pending = norm.pending(h, scratch)
             if pending is not None:

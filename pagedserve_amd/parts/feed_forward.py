@@ -25,6 +25,7 @@ class DenseFeedForward(FeedForward):
         self.inner = inner
         self.activation = activation
         self.bias = bias
+        self._memo_up, self._memo_down = {}, {}
 
     def parameters(self):
         params = {
@@ -44,13 +45,15 @@ class DenseFeedForward(FeedForward):
         # copies in the layout that the products of few rows (decode steps) read fastest
         self.up_packed = kernels.pack_decode_weight(self.up_weight)
         self.down_packed = kernels.pack_decode_weight(self.down_weight)
+        self._memo_up.clear()
+        self._memo_down.clear()
 
     def forward(self, x, residual, ctx):
-        hidden = ctx.workspace.rows("ffn", self.inner, self.dtype)[:ctx.tokens]
+        hidden = ctx.workspace.first_rows("ffn", self.inner, self.dtype, ctx.tokens)
         # (the hidden rows belong to these two calls alone: at 17 to 64 rows the first may leave
         # them in the order in which the second reads them)
         _, hidden_packed = kernels.linear(x, self.up_weight, self.up_bias, hidden,
                                           epilogue=self.activation, packed=self.up_packed,
-                                          packed_out=True)
+                                          packed_out=True, memo=self._memo_up)
         kernels.linear(hidden, self.down_weight, self.down_bias, residual, epilogue="residual",
-                       packed=self.down_packed, a_packed=hidden_packed)
+                       packed=self.down_packed, a_packed=hidden_packed, memo=self._memo_down)
