@@ -1049,3 +1049,51 @@ def test_the_tile_that_the_step_lists_is_the_kernels_own():
     from pagedserve_amd.ops import kernels
 
     assert kernels.prefill_limits() == (kernels.PREFILL_TILE, kernels.PREFILL_TABLE_MAX)
+
+
+def test_linear_memo_of_a_call_site():
+    """A call site's memo: the second call with the same row count and operand addresses goes
+    straight to the library and gives the bits of the checked call; other rows or another
+    buffer are other entries; the flags that the library reports (rows handed on in the packed
+    order) come back on a hit as well."""
+    from pagedserve_amd.ops import kernels
+
+    k, n = 768, 256
+    w = _rand((n, k), torch.bfloat16, 700, k ** -0.5)
+    bias = _rand((n,), torch.float32, 701)
+    packed = kernels.pack_decode_weight(w)
+    rows = torch.empty((64, k), dtype=torch.bfloat16, device="cuda")
+    out = torch.empty((64, n), dtype=torch.bfloat16, device="cuda")
+    memo = {}
+    for count in (8, 40, 8, 40, 8):
+        rows[:count] = _rand((count, k), torch.bfloat16, 702 + len(memo))
+        out.zero_()       # (rows handed on in the packed order leave the places of absent rows alone)
+        got, handed_on = kernels.linear(rows[:count], w, bias, out[:count], epilogue="gelu_tanh", packed=packed,
+                                        packed_out=True, memo=memo)
+        plain = torch.zeros((64, n), dtype=torch.bfloat16, device="cuda")
+        _, plain_handed_on = kernels.linear(rows[:count], w, bias, plain[:count], epilogue="gelu_tanh",
+                                            packed=packed, packed_out=True)
+        assert handed_on == plain_handed_on == (count > 16)
+        assert torch.equal(got.view(torch.int16), plain[:count].view(torch.int16))
+    assert len(memo) == 2
+    other = torch.zeros((64, n), dtype=torch.bfloat16, device="cuda")
+    kernels.linear(rows[:8], w, bias, other[:8], epilogue="gelu_tanh", packed=packed, packed_out=True, memo=memo)
+    assert len(memo) == 3 and torch.equal(other[:8].view(torch.int16), out[:8].view(torch.int16))
+    # a pending norm in front: keyed by the stream's rows, the row list and the scratch
+    h = _rand((64, k), torch.float32, 710)
+    gamma, beta = _rand((k,), torch.float32, 711), _rand((k,), torch.float32, 712)
+    scratch = torch.empty((64, k), dtype=torch.bfloat16, device="cuda")
+    memo = {}
+    results = []
+    for _ in range(2):
+        result = torch.empty((8, n), dtype=torch.bfloat16, device="cuda")
+        holder = out[:8]
+        kernels.linear(kernels.PendingNorm(h[:8], gamma, beta, 1e-5, False, scratch[:8]), w, bias, holder, memo=memo)
+        result.copy_(holder)
+        results.append(result)
+        if len(results) == 1:
+            h[:8] = _rand((8, k), torch.float32, 720)    # the same addresses, other values: a hit reads them
+    assert len(memo) == 1 and not torch.equal(results[0], results[1])
+    expected = F.layer_norm(h[:8].double(), (k,), gamma.double(), beta.double(), 1e-5)
+    expected = expected.to(torch.bfloat16).double() @ w.double().t() + bias.double()
+    torch.testing.assert_close(results[1].double(), expected, atol=5e-3, rtol=5e-3)
