@@ -217,6 +217,7 @@ class ContinuousBatchScheduler:
         self._tickets = 0
         self.steps_run_ahead = 0
         self._inflight: Optional[_Flight] = None
+        self._failed_ahead: Optional[Exception] = None   # raised by the next call of step()
 
     # ----------------------------------------------------------------- views
     @property
@@ -363,6 +364,9 @@ class ContinuousBatchScheduler:
             torch.cuda.set_stream(previous)
 
     def _iterate(self) -> Dict[int, int]:
+        if self._failed_ahead is not None:
+            error, self._failed_ahead = self._failed_ahead, None
+            raise error
         flight, self._inflight = self._inflight, None
         if flight is None:
             flight = self._take_off()
@@ -370,11 +374,13 @@ class ContinuousBatchScheduler:
                 return {}
         try:
             self._inflight = self._take_off_ahead(flight)
-        except Exception:
-            # the step ahead failed in a way that the ordinary start would not report: the
-            # iteration that is already running keeps its tokens and lands on the next call
-            self._inflight = flight
-            raise
+        except Exception as error:
+            # The step ahead failed in a way that the ordinary start would not report.  The
+            # iteration that is already running is not lost with it: it lands now and its
+            # tokens go to the caller; the error is raised by the next call, before anything
+            # else is started.
+            self._inflight = None
+            self._failed_ahead = error
         return self._land(flight)
 
     def _choose_on_device(self, receivers, ahead):
@@ -495,7 +501,7 @@ class ContinuousBatchScheduler:
         self.finished[request.request_id] = request
 
     def has_work(self) -> bool:
-        return bool(self._live) or self._inflight is not None
+        return bool(self._live) or self._inflight is not None or self._failed_ahead is not None
 
     def run_until_complete(self):
         while self.has_work():

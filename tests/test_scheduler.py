@@ -513,3 +513,40 @@ def test_python_entry_takes_the_reference_keyword_names():
     for backend in ("flash", "torch", "triton"):
         with pytest.raises(ValueError, match="Unknown decode attention backend.*'hip'"):
             build_scheduler(model_name="reference", decode_attention_backend=backend)
+
+
+def test_a_failing_step_ahead_loses_no_tokens():
+    """The iteration that is launched ahead fails with an error that is no refusal (a kernel's,
+    say): the iteration that was already running still lands, its tokens reach the caller, the
+    error comes out of the next call, and the loop goes on from there as if nothing had been
+    launched ahead."""
+
+    class BreaksOnce(ChoosingEngine):
+        def __init__(self):
+            super().__init__()
+            self.broken = False
+
+        def step(self, entries, greedy=False, draws=None):
+            if not self.broken and any(entry.carry is not None for entry in entries):
+                self.broken = True
+                raise RuntimeError("a launch failed")
+            return super().step(entries, greedy=greedy, draws=draws)
+
+    engine = BreaksOnce()
+    scheduler = ContinuousBatchScheduler(engine, ArgmaxSampler(), tokenizer=None, max_batch_size=4,
+                                         eos_token_id=None)
+    first = scheduler.add_token_request([3, 1, 4], 6)
+    second = scheduler.add_token_request([2, 7], 6)
+    streamed = {first: [], second: []}
+    raised = 0
+    while scheduler.has_work():
+        try:
+            for rid, token in scheduler.step().items():
+                streamed[rid].append(token)
+        except RuntimeError as error:
+            assert "a launch failed" in str(error)
+            raised += 1
+    assert raised == 1 and engine.broken
+    assert streamed[first] == expected_tokens([3, 1, 4], 6) == scheduler.finished[first].generated_token_ids
+    assert streamed[second] == expected_tokens([2, 7], 6) == scheduler.finished[second].generated_token_ids
+    assert not engine.cache.requests
