@@ -31,8 +31,9 @@ One JSON line is printed:
     python bench.py --prefill-only --steps K               the prefill step alone (for profiles)
     python bench.py --kernels [--shape small|medium|xl|all] [--only name,name]
 
-``--kernels`` times every kernel of a decode step (1, 8 and 64 requests over 1,024 keys) and of
-the prefill step (2 x 1,024 tokens) alone, on weights that no cache holds (a graph of launches
+``--kernels`` times every kernel of a decode step (1, 8 and 64 requests over 1,024 keys), of
+the prefill step (2 x 1,024 tokens) and of a mixed step (32 decoded tokens beside a portion of
+512) alone, on weights that no cache holds (a graph of launches
 that rotate over copies of them, at least 25 launches untimed and 100 timed), and prints a
 table (to standard error) and one JSON line: microseconds, bytes, flops, and both as fractions
 of the published peaks and of two measured ones (a device copy and the library's 4096-cubed
@@ -506,6 +507,11 @@ def kernel_tables(args):
             key = f"{name}_prefill_2x{PREFILL_TOKENS // 2}"
             tables[key] = table.prefill_table(raw, 2, PREFILL_TOKENS // 2, peaks, PAGE_SIZE, only)
             print(table.format_table(key, tables[key]), file=sys.stderr, flush=True)
+            if only is None:
+                # a step of the streams: 32 decoded tokens over 500 keys beside a portion of 512
+                key = f"{name}_mixed_32_decoded_ctx500_beside_512"
+                tables[key] = table.mixed_table(raw, 32, 500, 512, peaks, PAGE_SIZE)
+                print(table.format_table(key, tables[key]), file=sys.stderr, flush=True)
     return {"metric": "microseconds per kernel, weights from memory", "unit": "us", "dtype": "bf16",
             "published_peak": {"hbm_GBps": HBM_GBPS, "bf16_TFLOPs": PEAK_TFLOPS["bf16"]},
             "measured_peak": peaks, "tables": tables}

@@ -308,6 +308,91 @@ def prefill_table(raw, prompts, length, peaks, page_size=16, only=None):
     return out
 
 
+def mixed_table(raw, decodes, context, portion, peaks, page_size=16):
+    """The kernels of one layer of a mixed step: ``decodes`` decoded tokens over ``context`` keys
+    each beside one prompt portion of ``portion`` tokens (a new request's first)."""
+    shape = _Shape(raw)
+    d, inner, heads, head_dim = shape.d, shape.inner, shape.heads, shape.head_dim
+    dtype = torch.bfloat16
+    rows = decodes + portion
+    generator = torch.Generator(device="cuda").manual_seed(3)
+
+    def randn(*size, scale=1.0, kind=torch.float32):
+        return (torch.randn(*size, device="cuda", generator=generator) * scale).to(kind)
+
+    h = randn(rows, d)
+    gamma, beta = randn(d) * 0.1 + 1, randn(d) * 0.1
+    normed = torch.empty(rows, d, dtype=dtype, device="cuda")
+    qkv = randn(rows, 3 * d, kind=dtype)
+    context_rows = torch.empty(rows, d, dtype=dtype, device="cuda")
+    hidden = torch.empty(rows, inner, dtype=dtype, device="cuda")
+    items = decodes + 1
+    lengths = [context] * decodes + [portion]
+    pages_each = [-(-length // page_size) for length in lengths]
+    table_width = -(-shape.positions // page_size)
+    tables = torch.zeros(items, table_width, dtype=torch.int32, device="cuda")
+    first = 0
+    for item, count in enumerate(pages_each):
+        tables[item, :count] = torch.arange(first, first + count, dtype=torch.int32, device="cuda")
+        first += count
+    positions = torch.tensor([context - 1] * decodes + list(range(portion)), dtype=torch.int32, device="cuda")
+    tok_item = torch.tensor(list(range(decodes)) + [decodes] * portion, dtype=torch.int32, device="cuda")
+    cu_tokens = torch.tensor(list(range(decodes + 1)) + [rows], dtype=torch.int32, device="cuda")
+    kv_lens = torch.tensor(lengths, dtype=torch.int32, device="cuda")
+    single_tokens = torch.arange(decodes, dtype=torch.int32, device="cuda")
+    tile = kernels.PREFILL_TILE
+    starts = sorted(range(0, portion, tile), reverse=True)
+    tile_item = torch.full((len(starts),), decodes, dtype=torch.int32, device="cuda")
+    tile_q0 = torch.tensor(starts, dtype=torch.int32, device="cuda")
+    k_pool = randn(first, heads, page_size, head_dim, kind=dtype)
+    v_pool = randn(first, heads, page_size, head_dim, kind=dtype)
+    part = Attention(width=d, dtype=dtype, heads=heads, kv_heads=heads, head_dim=head_dim, scale=head_dim ** -0.5)
+    out = []
+
+    def product(name, n, k, call, seed, extra_bytes=0):
+        copies = _copies(n * k * 2, least=8, most=48)
+        weights, packed = _matrices(n, k, copies, seed)
+        bias = randn(n) * 0.1
+        us = graph_time(lambda i: call(weights[i], packed[i], bias), copies)
+        out.append(_row(name, us, n * k * 2 + extra_bytes, 2 * rows * n * k, peaks))
+        del weights, packed
+        torch.cuda.empty_cache()
+
+    us = graph_time(lambda i: kernels.norm(h, gamma, beta, shape.eps, normed), 8)
+    out.append(_row("norm", us, rows * d * 6, 0, peaks))
+    product("qkv+cache_write", 3 * d, d,
+            lambda w, wp, bias: kernels.linear(normed, w, bias, qkv, packed=wp, scatter_only=True,
+                                               scatter=(k_pool, v_pool, tok_item, positions, tables, d, d)),
+            31, extra_bytes=rows * d * 2 * 4)
+    q = qkv[:, :d]
+    splits, waves = part._splits(decodes, max(context, portion))
+    worst = (6 * kernels.compute_units() + rows * heads) * (head_dim + 2)
+    partial = torch.empty(worst, dtype=torch.float32, device="cuda")
+    us = graph_time(lambda i: kernels.attention_decode(
+        q, k_pool, v_pool, context_rows, tok_item, positions, tables, heads, part.scale, splits,
+        partial=partial if splits > 1 else None, waves=waves, tok_list=single_tokens), 8)
+    out.append(_row(f"attention of the decoded tokens ({splits} key ranges, {waves} waves)", us,
+                    2 * decodes * context * d * 2, 4 * decodes * context * d, peaks,
+                    launches=2 if splits > 1 else 1))
+    if kernels.prefill_supported(dtype, head_dim, table_width):
+        us = graph_time(lambda i: kernels.attention_prefill(
+            q, k_pool, v_pool, context_rows, tile_item, tile_q0, cu_tokens, kv_lens, tables, heads,
+            head_dim ** -0.5, max_kv_len=max(context, portion)), 8)
+        out.append(_row("attention of the portion (tiled, causal)", us, portion * d * 2 * 4,
+                        4 * d * (portion * (portion + 1) // 2), peaks))
+    product("out_proj+residual", d, d,
+            lambda w, wp, bias: kernels.linear(context_rows, w, bias, h, epilogue="residual", packed=wp),
+            32, extra_bytes=rows * d * (2 + 8))
+    product("fc+gelu", inner, d,
+            lambda w, wp, bias: kernels.linear(normed, w, bias, hidden, epilogue=shape.activation, packed=wp),
+            33, extra_bytes=rows * (d + inner) * 2)
+    product("proj+residual", d, inner,
+            lambda w, wp, bias: kernels.linear(hidden, w, bias, h, epilogue="residual", packed=wp),
+            34, extra_bytes=rows * (inner * 2 + d * 8))
+    torch.cuda.empty_cache()
+    return out
+
+
 def format_table(title, rows):
     lines = [title,
              f"  {'kernel':<52} {'us':>8} {'MB':>9} {'GB/s':>8} {'of 8 TB/s':>9} {'GFLOP':>8} {'TFLOP/s':>8} {'of 2.5 PF':>9}"]
