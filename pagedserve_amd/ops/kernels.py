@@ -344,7 +344,9 @@ def linear(x, w, bias, out, epilogue="none", scatter=None, packed=None, a_packed
     call is kept in it under the row count and the addresses of the other operands, and a call
     that finds its block goes straight to the library: checking and filling the block costs
     the host more than the launch, and a step that is not replayed from a graph issues four
-    such calls a layer.  Whoever binds other weights clears the dict."""
+    such calls a layer.  Whoever binds other weights clears the dict; and because a block also
+    holds the room behind the addresses (rows that a buffer has space for), a site keeps one
+    dict per set of buffers (``parts.base.site_memo``)."""
     if memo is not None:
         key = _memo_key(x, out, scatter, a_packed, choose)
         kept = memo.get(key)

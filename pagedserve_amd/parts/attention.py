@@ -4,7 +4,7 @@ import torch
 
 from ..ops import kernels
 from ..weights.loader import MATRIX, VECTOR, ParamSpec
-from .base import Mixer, PagedKVSpec
+from .base import Mixer, PagedKVSpec, site_memo
 from .registry import register_mixer
 
 
@@ -47,7 +47,7 @@ class Attention(Mixer):
         self.kv_cols = kv_heads * head_dim
         self.position = None
         self._columns = {}
-        # what ``kernels.linear`` keeps per call site and step shape (its ``memo``)
+        # what ``kernels.linear`` keeps per call site and step shape (its ``memo``), per workspace
         self._memo_qkv, self._memo_out = {}, {}
 
     def parameters(self):
@@ -95,10 +95,10 @@ class Attention(Mixer):
             kernels.linear(x, self.qkv_weight, self.qkv_bias, qkv,
                            scatter=(cache.k_pool, cache.v_pool, ctx.tok_item, ctx.positions, tables,
                                     self.q_cols, self.kv_cols), packed=self.qkv_packed,
-                           scatter_only=True, memo=self._memo_qkv)
+                           scatter_only=True, memo=site_memo(self._memo_qkv, ctx.workspace))
         else:
             kernels.linear(x, self.qkv_weight, self.qkv_bias, qkv, packed=self.qkv_packed,
-                           memo=self._memo_qkv)
+                           memo=site_memo(self._memo_qkv, ctx.workspace))
             if rotates:
                 self.position.apply_to_qk(q, k, ctx)
             if cache.writes:
@@ -157,7 +157,7 @@ class Attention(Mixer):
                                       ctx.positions, tables, self.heads, self.scale, self.window,
                                       tok_list=None if whole else ctx.portion_tokens)
         kernels.linear(context, self.out_weight, self.out_bias, residual, epilogue="residual",
-                       packed=self.out_packed, memo=self._memo_out)
+                       packed=self.out_packed, memo=site_memo(self._memo_out, ctx.workspace))
 
     def _range_records(self, ctx):
         """Scratch for one record per (token, head, key range): always asked for at its largest

@@ -25,6 +25,7 @@ Folding the residual sum into the part lets the last matrix product of a part ad
 in float in its own epilogue instead of a separate pass over the stream.
 """
 
+import itertools
 from dataclasses import dataclass
 from typing import Dict, List, Optional
 
@@ -147,6 +148,22 @@ class FeedForward(Part):
         raise NotImplementedError
 
 
+_WORKSPACE_SERIALS = itertools.count(1)
+
+
+def site_memo(store: dict, workspace) -> dict:
+    """The memo of one call site of ``kernels.linear`` for the buffers of one workspace.  A
+    memo holds addresses and the room behind them; another workspace may get the same
+    addresses with other room (the allocator hands freed memory out again), so every workspace
+    has memos of its own, told apart by a serial number that is never used twice."""
+    memo = store.get(workspace.serial)
+    if memo is None:
+        if len(store) >= 8:
+            store.clear()
+        memo = store[workspace.serial] = {}
+    return memo
+
+
 class Workspace:
     """Activation buffers that live as long as the engine.
 
@@ -162,6 +179,7 @@ class Workspace:
         # counts the buffers that were replaced by larger ones: whoever holds addresses
         # (recorded graphs) compares it with the value at the time of recording
         self.moved = 0
+        self.serial = next(_WORKSPACE_SERIALS)
         self._views: Dict[tuple, torch.Tensor] = {}
 
     def rows(self, name: str, columns: int, dtype: torch.dtype, max_rows: Optional[int] = None):

@@ -2,7 +2,7 @@
 
 from ..ops import kernels
 from ..weights.loader import MATRIX, VECTOR, ParamSpec
-from .base import FeedForward
+from .base import FeedForward, site_memo
 from .registry import register_feed_forward
 
 ACTIVATIONS = ("gelu_tanh", "gelu_erf")
@@ -54,6 +54,6 @@ class DenseFeedForward(FeedForward):
         # them in the order in which the second reads them)
         _, hidden_packed = kernels.linear(x, self.up_weight, self.up_bias, hidden,
                                           epilogue=self.activation, packed=self.up_packed,
-                                          packed_out=True, memo=self._memo_up)
+                                          packed_out=True, memo=site_memo(self._memo_up, ctx.workspace))
         kernels.linear(hidden, self.down_weight, self.down_bias, residual, epilogue="residual",
-                       packed=self.down_packed, a_packed=hidden_packed, memo=self._memo_down)
+                       packed=self.down_packed, a_packed=hidden_packed, memo=site_memo(self._memo_down, ctx.workspace))
