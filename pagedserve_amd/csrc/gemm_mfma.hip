@@ -474,8 +474,10 @@ __global__ __launch_bounds__(64 * SK_WAVES) void gemm_nt_skinny_kernel(
 }
 
 // ---------------------------------------------------------------- skinny with fused norm
-#define SN_MAX_K 1024              // one round of loads covers it: 4 waves x 4 steps x 64
-#define SN_STRIDE (SN_MAX_K + 8)   // LDS row stride in elements (16-byte aligned, skewed)
+#define SN_MAX_K 1792              // one round of loads covers it: 4 waves x 7 steps x 64
+// LDS row stride in elements (16-byte aligned, skewed by four banks a row); 16 rows of the
+// longest k with the partial sums stay under the 64 KB that a block may declare
+#define SN_STRIDE(UNROLL) (((UNROLL) <= 4 ? 1024 : (UNROLL) * SK_WAVES * 64) + 8)
 
 // NR: rows that a wave normalises (rows wave, wave + 4, ...: 4 NR >= m).  Rows of LDS beyond
 // them stay as they are: they only feed outputs that are never stored.
@@ -485,7 +487,8 @@ __global__ __launch_bounds__(64 * SK_WAVES) void gemm_nt_skinny_norm_kernel(
     TOut* __restrict__ c, int m, int n, int k, int ldc, KvScatter scatter,
     const bf16_t* __restrict__ wp) {
   __shared__ float partial[SK_WAVES][1][4][64];
-  __shared__ __attribute__((aligned(16))) bf16_t xs[16 * SN_STRIDE];
+  constexpr int STRIDE = SN_STRIDE(UNROLL);
+  __shared__ __attribute__((aligned(16))) bf16_t xs[16 * STRIDE];
   const int lane = threadIdx.x & 63;
   const int wave = threadIdx.x >> 6;
   const int n0 = blockIdx.x * 16;
@@ -598,7 +601,7 @@ __global__ __launch_bounds__(64 * SK_WAVES) void gemm_nt_skinny_norm_kernel(
           packed.x = pack2_bf16(y0, y1);
           packed.y = pack2_bf16(y2, y3);
         }
-        *reinterpret_cast<uint2*>(&xs[token * SN_STRIDE + 4 * lane + 256 * i]) = packed;
+        *reinterpret_cast<uint2*>(&xs[token * STRIDE + 4 * lane + 256 * i]) = packed;
       }
     }
   }
@@ -611,8 +614,8 @@ __global__ __launch_bounds__(64 * SK_WAVES) void gemm_nt_skinny_norm_kernel(
     const int ku = wave * 64 + u * SK_WAVES * 64;
     const int kk = ku + group * 16;
     uint4 x0 = zero, x1 = zero;
-    if (first[u]) x0 = *reinterpret_cast<const uint4*>(&xs[sub * SN_STRIDE + kk]);
-    if (second[u]) x1 = *reinterpret_cast<const uint4*>(&xs[sub * SN_STRIDE + kk + 8]);
+    if (first[u]) x0 = *reinterpret_cast<const uint4*>(&xs[sub * STRIDE + kk]);
+    if (second[u]) x1 = *reinterpret_cast<const uint4*>(&xs[sub * STRIDE + kk + 8]);
     const uint4 w0 = first[u] ? wf[u][0] : zero;
     const uint4 w1 = second[u] ? wf[u][1] : zero;
     acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(*reinterpret_cast<const bf16x8*>(&w0),
@@ -794,15 +797,16 @@ static int launch_skinny_norm(const NormPrologue& norm, const void* w, const flo
   if (k % 64 != 0) wp = nullptr;
   dim3 grid((n + 15) / 16);
   dim3 block(64 * SK_WAVES);
+  // steps of 64 k per wave: 3 for up to 768 (GPT-2's width), 4 for 1024, 5 for 1280, 7 for 1792
+#define PS_NORM_STEPS(EPI, NR, STEPS)                                                         \
+  hipLaunchKernelGGL((gemm_nt_skinny_norm_kernel<TOut, EPI, NR, STEPS>), grid, block, 0, s,   \
+                     norm, (const bf16_t*)w, bias, (TOut*)c, m, n, k, ldc, scatter, wp)
 #define PS_NORM_LAUNCH(EPI, NR)                                                               \
   do {                                                                                        \
-    if (k <= SK_WAVES * 3 * 64)                                                               \
-      hipLaunchKernelGGL((gemm_nt_skinny_norm_kernel<TOut, EPI, NR, 3>), grid, block, 0, s,   \
-                         norm, (const bf16_t*)w, bias, (TOut*)c, m, n, k, ldc, scatter, wp);  \
-    else                                                                                      \
-      hipLaunchKernelGGL((gemm_nt_skinny_norm_kernel<TOut, EPI, NR, SK_UNROLL>), grid, block, \
-                         0, s, norm, (const bf16_t*)w, bias, (TOut*)c, m, n, k, ldc, scatter, \
-                         wp);                                                                 \
+    if (k <= SK_WAVES * 3 * 64) PS_NORM_STEPS(EPI, NR, 3);                                    \
+    else if (k <= SK_WAVES * 4 * 64) PS_NORM_STEPS(EPI, NR, 4);                               \
+    else if (k <= SK_WAVES * 5 * 64) PS_NORM_STEPS(EPI, NR, 5);                               \
+    else PS_NORM_STEPS(EPI, NR, 7);                                                           \
   } while (0)
 #define PS_NORM_CASE(EPI)                                                                     \
   case EPI:                                                                                   \
@@ -820,6 +824,7 @@ static int launch_skinny_norm(const NormPrologue& norm, const void* w, const flo
   }
 #undef PS_NORM_CASE
 #undef PS_NORM_LAUNCH
+#undef PS_NORM_STEPS
   PS_CHECK_LAUNCH("ps_linear(skinny, fused norm)");
   return 0;
 }

@@ -603,11 +603,12 @@ def test_attention_prefill_far_key_and_causality():
 
 @pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("m,n,k", [(1, 48, 64), (8, 2304, 768), (16, 100, 1024), (13, 257, 96), (17, 192, 768), (5, 64, 1600), (200, 320, 96),
+                                   (12, 144, 1280), (16, 208, 1792), (9, 96, 1104), (16, 4800, 1600), (7, 80, 1800),
                                    (40, 2304, 768), (64, 3072, 768), (33, 100, 1024), (50, 8000, 64), (64, 16400, 64)])
 @pytest.mark.parametrize("epilogue", ["none", "gelu_tanh", "residual"])
 @pytest.mark.parametrize("rms", [False, True])
 def test_linear_with_pending_norm(dtype, m, n, k, epilogue, rms):
-    """Norm + product as one call: fused for bfloat16 with up to 16 rows, k <= 1024 and up to
+    """Norm + product as one call: fused for bfloat16 with up to 16 rows, k <= 1792 and up to
     8,192 columns, two launches otherwise (17 to 64 rows: the normed rows travel in the lanes'
     operand order); with and without a row gather."""
     from pagedserve_amd.ops import kernels
