@@ -481,25 +481,43 @@ __global__ __launch_bounds__(64 * SK_WAVES) void gemm_nt_skinny_kernel(
 
 // NR: rows that a wave normalises (rows wave, wave + 4, ...: 4 NR >= m).  Rows of LDS beyond
 // them stay as they are: they only feed outputs that are never stored.
-template <typename TOut, int EPI, int NR, int UNROLL>
+// NT: accumulator tiles of 16 columns per block.  A block owns `cols` consecutive columns
+// (16 with one tile; 17 to 32 with two, the second tile partly empty): with more tiles of 16
+// than compute units the columns are dealt out evenly instead, one block to a unit, because a
+// unit that gets a second block takes twice as long as the others (1600 k, 1 row: 4,096
+// columns 5.7 us, 4,800 columns as 300 tiles 9.0 us).
+template <typename TOut, int EPI, int NR, int UNROLL, int NT>
 __global__ __launch_bounds__(64 * SK_WAVES) void gemm_nt_skinny_norm_kernel(
     NormPrologue norm, const bf16_t* __restrict__ w, const float* __restrict__ bias,
     TOut* __restrict__ c, int m, int n, int k, int ldc, KvScatter scatter,
-    const bf16_t* __restrict__ wp) {
-  __shared__ float partial[SK_WAVES][1][4][64];
+    const bf16_t* __restrict__ wp, int cols) {
   constexpr int STRIDE = SN_STRIDE(UNROLL);
+  // with two tiles the partial sums take the place of the rows once these have been used:
+  // both together would pass the 64 KB that a block may declare
+  constexpr int OWN_PARTIAL = NT == 1 ? SK_WAVES * 4 * 64 : 1;
+  __shared__ float partial_own[OWN_PARTIAL];
   __shared__ __attribute__((aligned(16))) bf16_t xs[16 * STRIDE];
+  static_assert(NT <= 2 && NT * SK_WAVES * 4 * 64 * sizeof(float) <= 16 * STRIDE * sizeof(bf16_t), "partial sums fit");
+  float (*partial)[SK_WAVES][1][4][64] = reinterpret_cast<float (*)[SK_WAVES][1][4][64]>(
+      NT == 1 ? partial_own : reinterpret_cast<float*>(xs));
   const int lane = threadIdx.x & 63;
   const int wave = threadIdx.x >> 6;
-  const int n0 = blockIdx.x * 16;
+  const int n0 = blockIdx.x * cols;
+  const int n1 = n0 + cols < n ? n0 + cols : n;
   const int sub = lane & 15;
   const int group = lane >> 4;
-  const int w_row = n0 + sub < n ? n0 + sub : n - 1;
-  const bf16_t* w_ptr = w + (int64_t)w_row * k + group * 16;
-  if (wp != nullptr) w_ptr = wp + (int64_t)(n0 / 16) * (k / 64) * 1024 + lane * 8;   // packed copy
+  const bf16_t* w_ptr[NT];
+#pragma unroll
+  for (int t = 0; t < NT; ++t) {
+    const int w_row = n0 + t * 16 + sub < n1 ? n0 + t * 16 + sub : n1 - 1;
+    w_ptr[t] = w + (int64_t)w_row * k + group * 16;
+    // packed copy: row r is lane group * 16 + r % 16 of tile r / 16
+    if (wp != nullptr)
+      w_ptr[t] = wp + (int64_t)(w_row >> 4) * (k / 64) * 1024 + (group * 16 + (w_row & 15)) * 8;
+  }
   const uint4 zero = {0u, 0u, 0u, 0u};
 
-  uint4 wf[UNROLL][2];
+  uint4 wf[UNROLL][NT][2];
   bool first[UNROLL], second[UNROLL];
   // 1. rows wave, wave + 4, wave + 8, wave + 12: statistics and normalisation in registers
   //    (mean, centred values, biased variance, rsqrt(var + eps), scale, shift; reference:
@@ -549,8 +567,11 @@ __global__ __launch_bounds__(64 * SK_WAVES) void gemm_nt_skinny_norm_kernel(
       second[u] = kk + 8 < k;
       const int p0 = wp != nullptr ? (first[u] ? (ku / 64) * 1024 : 0) : (first[u] ? ku : -group * 16);
       const int p1 = wp != nullptr ? p0 + 512 : (second[u] ? ku + 8 : -group * 16);
-      wf[u][0] = *reinterpret_cast<const uint4*>(w_ptr + p0);
-      wf[u][1] = *reinterpret_cast<const uint4*>(w_ptr + p1);
+#pragma unroll
+      for (int t = 0; t < NT; ++t) {
+        wf[u][t][0] = *reinterpret_cast<const uint4*>(w_ptr[t] + p0);
+        wf[u][t][1] = *reinterpret_cast<const uint4*>(w_ptr[t] + p1);
+      }
     }
     // The rows of a wave go through every stage together (the sums of all, the means of all,
     // ...), so that the lane exchanges and the square root of one row run behind those of
@@ -608,7 +629,9 @@ __global__ __launch_bounds__(64 * SK_WAVES) void gemm_nt_skinny_norm_kernel(
   __syncthreads();
 
   // 3. the product: column operand from LDS
-  f32x4 acc = {0.f, 0.f, 0.f, 0.f};
+  f32x4 acc[NT];
+#pragma unroll
+  for (int t = 0; t < NT; ++t) acc[t] = f32x4{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
   for (int u = 0; u < UNROLL; ++u) {
     const int ku = wave * 64 + u * SK_WAVES * 64;
@@ -616,17 +639,26 @@ __global__ __launch_bounds__(64 * SK_WAVES) void gemm_nt_skinny_norm_kernel(
     uint4 x0 = zero, x1 = zero;
     if (first[u]) x0 = *reinterpret_cast<const uint4*>(&xs[sub * STRIDE + kk]);
     if (second[u]) x1 = *reinterpret_cast<const uint4*>(&xs[sub * STRIDE + kk + 8]);
-    const uint4 w0 = first[u] ? wf[u][0] : zero;
-    const uint4 w1 = second[u] ? wf[u][1] : zero;
-    acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(*reinterpret_cast<const bf16x8*>(&w0),
-                                                  *reinterpret_cast<const bf16x8*>(&x0), acc, 0, 0, 0);
-    acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(*reinterpret_cast<const bf16x8*>(&w1),
-                                                  *reinterpret_cast<const bf16x8*>(&x1), acc, 0, 0, 0);
-  }
 #pragma unroll
-  for (int i = 0; i < 4; ++i) partial[wave][0][i][lane] = acc[i];
+    for (int t = 0; t < NT; ++t) {
+      const uint4 w0 = first[u] ? wf[u][t][0] : zero;
+      const uint4 w1 = second[u] ? wf[u][t][1] : zero;
+      acc[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(*reinterpret_cast<const bf16x8*>(&w0),
+                                                       *reinterpret_cast<const bf16x8*>(&x0), acc[t], 0, 0, 0);
+      acc[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(*reinterpret_cast<const bf16x8*>(&w1),
+                                                       *reinterpret_cast<const bf16x8*>(&x1), acc[t], 0, 0, 0);
+    }
+  }
+  if (NT > 1) __syncthreads();   // every wave has read its rows: their place is free
+#pragma unroll
+  for (int t = 0; t < NT; ++t)
+#pragma unroll
+    for (int i = 0; i < 4; ++i) partial[t][wave][0][i][lane] = acc[t][i];
   __syncthreads();
-  skinny_epilogue<TOut, EPI, 1>(partial, bias, c, m, n, ldc, n0, 0, 0, 1, scatter);
+#pragma unroll
+  for (int t = 0; t < NT; ++t)
+    if (n0 + t * 16 < n1)
+      skinny_epilogue<TOut, EPI, 1>(partial[t], bias, c, m, n1, ldc, n0 + t * 16, 0, 0, 1, scatter);
 }
 
 // --------------------------------------------------------------------------------- host
@@ -795,12 +827,26 @@ static int launch_skinny_norm(const NormPrologue& norm, const void* w, const flo
                               int m, int n, int k, int ldc, int epilogue, const KvScatter& scatter,
                               const bf16_t* wp, hipStream_t s) {
   if (k % 64 != 0) wp = nullptr;
-  dim3 grid((n + 15) / 16);
+  // More tiles of 16 columns than compute units (up to twice as many): the columns are dealt
+  // out evenly, one block to a unit, each with a whole tile and a partly empty one.
+  const int tiles = (n + 15) / 16;
+  const int units = ps_compute_units();
+  const bool even = tiles > units && tiles <= 2 * units;
+  const int cols = even ? (n + units - 1) / units : 16;
+  // (read from the matrix itself: in the packed copy a line of 128 bytes holds rows of two
+  // blocks, which would fetch it twice; 1600 k, 4,800 columns, 1 row: 7.7 against 8.5 us)
+  if (even && cols % 16 != 0) wp = nullptr;
+  dim3 grid((n + cols - 1) / cols);
   dim3 block(64 * SK_WAVES);
   // steps of 64 k per wave: 3 for up to 768 (GPT-2's width), 4 for 1024, 5 for 1280, 7 for 1792
+#define PS_NORM_TILES(EPI, NR, STEPS, NT)                                                     \
+  hipLaunchKernelGGL((gemm_nt_skinny_norm_kernel<TOut, EPI, NR, STEPS, NT>), grid, block, 0,  \
+                     s, norm, (const bf16_t*)w, bias, (TOut*)c, m, n, k, ldc, scatter, wp, cols)
 #define PS_NORM_STEPS(EPI, NR, STEPS)                                                         \
-  hipLaunchKernelGGL((gemm_nt_skinny_norm_kernel<TOut, EPI, NR, STEPS>), grid, block, 0, s,   \
-                     norm, (const bf16_t*)w, bias, (TOut*)c, m, n, k, ldc, scatter, wp)
+  do {                                                                                        \
+    if (even) PS_NORM_TILES(EPI, NR, STEPS, 2);                                               \
+    else PS_NORM_TILES(EPI, NR, STEPS, 1);                                                    \
+  } while (0)
 #define PS_NORM_LAUNCH(EPI, NR)                                                               \
   do {                                                                                        \
     if (k <= SK_WAVES * 3 * 64) PS_NORM_STEPS(EPI, NR, 3);                                    \
@@ -825,6 +871,7 @@ static int launch_skinny_norm(const NormPrologue& norm, const void* w, const flo
 #undef PS_NORM_CASE
 #undef PS_NORM_LAUNCH
 #undef PS_NORM_STEPS
+#undef PS_NORM_TILES
   PS_CHECK_LAUNCH("ps_linear(skinny, fused norm)");
   return 0;
 }

@@ -604,6 +604,8 @@ def test_attention_prefill_far_key_and_causality():
 @pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("m,n,k", [(1, 48, 64), (8, 2304, 768), (16, 100, 1024), (13, 257, 96), (17, 192, 768), (5, 64, 1600), (200, 320, 96),
                                    (12, 144, 1280), (16, 208, 1792), (9, 96, 1104), (16, 4800, 1600), (7, 80, 1800),
+                                   (3, 4112, 64), (8, 6400, 1280), (13, 8192, 768), (5, 5000, 96), (11, 4700, 1024),
+                                   (40, 4800, 1600), (64, 8192, 768), (24, 4500, 320), (17, 4112, 1792),
                                    (40, 2304, 768), (64, 3072, 768), (33, 100, 1024), (50, 8000, 64), (64, 16400, 64)])
 @pytest.mark.parametrize("epilogue", ["none", "gelu_tanh", "residual"])
 @pytest.mark.parametrize("rms", [False, True])
@@ -693,15 +695,19 @@ def test_linear_scatters_keys_and_values(dtype, m, k, geometry):
     assert torch.equal(k_pool, k_ref) and torch.equal(v_pool, v_ref)
 
 
-@pytest.mark.parametrize("m", [8, 24, 64])
-def test_norm_product_scatters_keys_and_values(m):
+@pytest.mark.parametrize("m,geometry", [(8, (6, 3, 32, 8, 192)), (24, (6, 3, 32, 8, 192)), (64, (6, 3, 32, 8, 192)),
+                                        (5, (25, 25, 64, 16, 1600)), (16, (40, 20, 64, 16, 704)),
+                                        (64, (25, 25, 64, 16, 1600)), (37, (40, 20, 64, 16, 704))])
+def test_norm_product_scatters_keys_and_values(m, geometry):
     """Norm, [q | k | v] product and the store into the pages as one call (one launch up to 16
     rows): the output is that of the norm and the product one after the other (up to the
-    rounding of the normed rows), and the pages hold exactly the key and value columns of it."""
+    rounding of the normed rows), and the pages hold exactly the key and value columns of it.
+    (The last two have more tiles of 16 columns than compute units: their columns are dealt
+    out evenly over blocks of two tiles.)"""
     from pagedserve_amd.ops import kernels
 
     dtype = torch.bfloat16
-    heads, kv_heads, head_dim, page_size, k = 6, 3, 32, 8, 192
+    heads, kv_heads, head_dim, page_size, k = geometry
     q_cols, kv_cols = heads * head_dim, kv_heads * head_dim
     n = q_cols + 2 * kv_cols
     lens = [5 + index for index in range(m)]
@@ -755,7 +761,8 @@ def test_attention_decode_sixteen_waves(dtype):
 
 PACKED_SHAPES = [(1, 50, 64), (8, 768, 3072), (8, 2304, 768), (16, 3072, 768), (17, 768, 768), (5, 1000, 320),
                  (64, 2304, 768), (48, 100, 3072), (9, 16411, 320), (16, 330, 1600), (40, 400, 1600), (300, 1000, 320),
-                 (40, 1600, 6400), (33, 1290, 5184)]
+                 (40, 1600, 6400), (33, 1290, 5184), (8, 4800, 1600), (3, 5008, 128),
+                 (40, 4800, 1600), (64, 6400, 1280), (20, 4112, 64), (33, 5008, 192), (50, 8192, 832)]
 
 
 @pytest.mark.parametrize("m,n,k", PACKED_SHAPES)
