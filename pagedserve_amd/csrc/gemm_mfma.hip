@@ -509,11 +509,23 @@ static void launch_skinny_mb(const void* a, const void* w, const float* bias, vo
   } while (0)
   if (two_tiles && per >= 2) {
     // very many blocks (wide models): two tiles of columns per block halve what the blocks
-    // fetch of the rows of A, which at 17 to 64 rows is most of their traffic
-    grid.x = (n + 31) / 32;
-    if (per == 2) PS_LAUNCH_SKU(2, 2, 2);
-    else if (per == 3) PS_LAUNCH_SKU(3, 2, 2);
-    else PS_LAUNCH_SKU(4, 2, 2);
+    // fetch of the rows of A, which at 17 to 64 rows is most of their traffic; the range of k
+    // is one round of 2 to 5 steps per wave (chosen by the caller)
+    if constexpr (EPI == PS_EPI_RESIDUAL) {
+      grid.x = (n + 31) / 32;
+      const int steps = (k_chunk + SK_WAVES * 64 - 1) / (SK_WAVES * 64);
+#define PS_LAUNCH_TT(MB)                                                                       \
+  do {                                                                                         \
+    if (steps <= 2) PS_LAUNCH_SKU(MB, 2, 2);                                                   \
+    else if (steps == 3) PS_LAUNCH_SKU(MB, 2, 3);                                              \
+    else if (steps == 4) PS_LAUNCH_SKU(MB, 2, 4);                                              \
+    else PS_LAUNCH_SKU(MB, 2, 5);                                                              \
+  } while (0)
+      if (per == 2) PS_LAUNCH_TT(2);
+      else if (per == 3) PS_LAUNCH_TT(3);
+      else PS_LAUNCH_TT(4);
+#undef PS_LAUNCH_TT
+    }
   } else if (per <= 2 && k_splits == 1 && n >= 16 * 1024) {
     // the output head: two tiles of columns per block (also at 17 to 32 rows: 50,257 x 768 at
     // 17 rows takes 27 us with one tile per block)
@@ -551,12 +563,19 @@ static int launch_skinny(const void* a, const void* w, const float* bias, void* 
   k_chunk = (k_chunk + 255) / 256 * 256;
   k_splits = (k + k_chunk - 1) / k_chunk;
   // More rows than 16 and half as many blocks again as compute units: two column tiles per
-  // block and ranges of 640 k (64 x 1600 x 6400 with weights from memory: 13.6 us against
-  // 17.7; at 1024 x 4096 and below the single tile stays ahead).
+  // block, and ranges of k such that the blocks come to one per compute unit or just under
+  // (a unit with two blocks takes twice as long as one with one), each range one round of a
+  // wave's loads: 1280 k at 64 x 1600 x 6400 (250 blocks: 11.7 us with weights from memory,
+  // against 13.7 with ranges of 640 and 17.7 with one tile and ranges of 1024), 1024 at 64 x
+  // 1280 x 5120 (200 blocks: 10.7 against 13.2); at 1024 x 4096 and below the single tile
+  // stays ahead.
   const bool two_tiles = epilogue == PS_EPI_RESIDUAL && m > 16 && k_splits > 1 &&
                          (int64_t)((n + 15) / 16) * k_splits >= ps_compute_units() * 3 / 2;
   if (two_tiles) {
-    k_chunk = 640;
+    const int tiles32 = (n + 31) / 32;
+    const int wanted = ps_compute_units() / tiles32 > 1 ? ps_compute_units() / tiles32 : 1;
+    k_chunk = ((k + wanted - 1) / wanted + 255) / 256 * 256;
+    k_chunk = k_chunk < 512 ? 512 : (k_chunk > 1280 ? 1280 : k_chunk);
     k_splits = (k + k_chunk - 1) / k_chunk;
   }
 #define PS_SKINNY_CASE(EPI)                                                                      \
