@@ -11,6 +11,10 @@
 //
 // Four waves in a 2 x 2 arrangement; a wave owns WM x WN accumulators of 32 x 32
 // (v_mfma_f32_32x32x16_bf16, float accumulation), so a block makes 64 WM x 64 WN outputs.
+// With KW = 2 the two waves of a row of the arrangement share one accumulator of 32 columns
+// instead and take half of every k tile's steps each; their sums meet in LDS at the end.  A
+// block then makes 64 x 32 outputs: twice as many blocks for a product of up to 64 rows whose
+// tiles of 64 columns would leave most compute units without one.
 // Per k tile there is one wait (own loads of the next tile have landed; later tiles stay in
 // flight) and one barrier, placed before the tile's last k step so that three steps' products
 // are queued in the matrix core meanwhile; after it the stage that was multiplied before is
@@ -44,12 +48,13 @@ __device__ inline void wait_ahead_and_sync(int ahead) {
   else wait_loads_and_sync<(MOST >= 6 ? 6 : 0) * LOADS>();
 }
 
-template <int WM, int WN, int STAGES, typename TOut, int EPI>
+template <int WM, int WN, int STAGES, typename TOut, int EPI, int KW = 1>
 __global__ __launch_bounds__(256) void gemm_nt_bf16_tiled_kernel(
     const bf16_t* __restrict__ a, const bf16_t* __restrict__ w, const float* __restrict__ bias,
     TOut* __restrict__ c, int m, int n, int k, int lda, int ldc, int tiles_m, int tiles_n,
     int row_major, int k_splits, int k_chunk, KvScatter scatter) {
-  constexpr int BM = 64 * WM, BN = 64 * WN;
+  static_assert(KW == 1 || (KW == 2 && WM == 1 && WN == 1), "k halves go with one accumulator per wave");
+  constexpr int BM = 64 * WM, BN = 64 * WN / KW;
   constexpr int STAGE_BYTES = (BM + BN) * TB_ROW;
   constexpr int LOADS_A = BM / 32;   // load instructions per wave and stage (8 rows each)
   constexpr int LOADS_W = BN / 32;
@@ -62,7 +67,8 @@ __global__ __launch_bounds__(256) void gemm_nt_bf16_tiled_kernel(
   const int lane = tid & 63;
   const int wave = tid >> 6;
   const int wave_m = wave >> 1;
-  const int wave_n = wave & 1;
+  const int wave_n = KW == 1 ? wave & 1 : 0;
+  const int wave_k = KW == 1 ? 0 : wave & 1;     // which half of a k tile's steps
   // Consecutive block ids run on different XCDs, each with an L2 of its own: blocks are
   // renumbered so that every XCD works on a contiguous run of tiles.  A run walked along the
   // rows of C reads few rows of A and all of W, one walked down the columns few rows of W and
@@ -151,8 +157,9 @@ __global__ __launch_bounds__(256) void gemm_nt_bf16_tiled_kernel(
                    : "v"(stage + (uint32_t)(w_row + j * 32 * TB_ROW) + slot)
                    : "memory");
   };
-  constexpr int STEPS = TB_BK / 16;
+  constexpr int STEPS = TB_BK / 16 / KW;          // k steps of a tile that this wave multiplies
   static_assert(STEPS % 2 == 0, "the operand buffers alternate per step");
+  const int s0 = wave_k * STEPS;                  // the first of them
 
 #pragma unroll
   for (int d = 0; d < STAGES - 1; ++d)
@@ -162,14 +169,14 @@ __global__ __launch_bounds__(256) void gemm_nt_bf16_tiled_kernel(
     const int ahead = k_tiles - 1 < STAGES - 2 ? k_tiles - 1 : STAGES - 2;
     wait_ahead_and_sync<LOADS, STAGES - 2>(ahead);
   }
-  fetch(0, 0, fa[0], fw[0]);
+  fetch(0, s0, fa[0], fw[0]);
   for (int kt = 0; kt < k_tiles; ++kt) {
     // the stage of tile kt - 1 is free: every wave met the others after its last read of it
     if (kt + STAGES - 1 < k_tiles) issue(kt + STAGES - 1);
 #pragma unroll
     for (int s = 0; s < STEPS; ++s) {
       if (s + 1 < STEPS) {
-        fetch(kt, s + 1, fa[(s + 1) & 1], fw[(s + 1) & 1]);
+        fetch(kt, s0 + s + 1, fa[(s + 1) & 1], fw[(s + 1) & 1]);
         asm volatile("s_waitcnt lgkmcnt(%0)" ::"n"(READS) : "memory");   // step s has arrived
       } else if (kt + 1 < k_tiles) {
         // own reads of this tile are complete before the others may overwrite its stage
@@ -177,7 +184,7 @@ __global__ __launch_bounds__(256) void gemm_nt_bf16_tiled_kernel(
         // tiles kt + 2 .. kt + STAGES - 1 may stay in flight, as far as they exist
         const int last = k_tiles - 1 < kt + STAGES - 1 ? k_tiles - 1 : kt + STAGES - 1;
         wait_ahead_and_sync<LOADS, STAGES - 2>(last - (kt + 1));
-        fetch(kt + 1, 0, fa[0], fw[0]);
+        fetch(kt + 1, s0, fa[0], fw[0]);
       } else {
         asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
       }
@@ -199,8 +206,22 @@ __global__ __launch_bounds__(256) void gemm_nt_bf16_tiled_kernel(
 
   // ---- epilogue (gemm_bf16_common.h): each wave turns its accumulators through a region of
   // LDS of its own and stores rows in aligned pieces
-  static_assert(4 * 32 * (WN * 32 + 8) * 4 <= STAGES * STAGE_BYTES, "the epilogue reuses the stages");
+  static_assert(4 * 32 * (WN * 32 + 8) * 4 + (KW - 1) * 2 * 16 * 64 * 4 <= STAGES * STAGE_BYTES,
+                "the epilogue reuses the stages");
   wait_loads_and_sync<0>();                       // every wave is past its last operand reads
+  if (KW == 2) {
+    // the wave of the second k half hands its sums to the wave of the first, behind the
+    // regions that the epilogue uses
+    float* meet = reinterpret_cast<float*>(lds) + 4 * 32 * (WN * 32 + 8) + wave_m * 16 * 64;
+    if (wave_k == 1) {
+#pragma unroll
+      for (int e = 0; e < 16; ++e) meet[e * 64 + lane] = acc[0][0][e];
+    }
+    __syncthreads();
+    if (wave_k == 1) return;
+#pragma unroll
+    for (int e = 0; e < 16; ++e) acc[0][0][e] += meet[e * 64 + lane];
+  }
   store_wave_tile<WM, WN, TOut, EPI>(acc, reinterpret_cast<float*>(lds) + wave * 32 * (WN * 32 + 8),
                                      lane, m0 + wave_m * WM * 32, n0 + wave_n * WN * 32, m, n, ldc,
                                      c, bias, split, k_splits, scatter);
@@ -212,11 +233,11 @@ bool ps_gemm_nt_bf16_tiled_supported(const void* a, const void* w, int m, int k,
          (reinterpret_cast<uintptr_t>(a) & 15u) == 0 && (reinterpret_cast<uintptr_t>(w) & 15u) == 0;
 }
 
-template <int WM, int WN, int STAGES, typename TOut>
+template <int WM, int WN, int STAGES, typename TOut, int KW = 1>
 static int launch_variant(const void* a, const void* w, const float* bias, void* c, int m, int n,
                           int k, int lda, int ldc, int epilogue, const KvScatter& scatter,
                           hipStream_t s) {
-  constexpr int BM = 64 * WM, BN = 64 * WN;
+  constexpr int BM = 64 * WM, BN = 64 * WN / KW;
   const int tiles_m = (m + BM - 1) / BM;
   const int tiles_n = (n + BN - 1) / BN;
   // what one XCD's run of tiles fetches into its L2, in rows of k values
@@ -236,7 +257,7 @@ static int launch_variant(const void* a, const void* w, const float* bias, void*
   k_splits = (k + k_chunk - 1) / k_chunk;
   dim3 grid(tiles_m * tiles_n * k_splits);
 #define PS_LAUNCH_TB(EPI)                                                                     \
-  hipLaunchKernelGGL((gemm_nt_bf16_tiled_kernel<WM, WN, STAGES, TOut, EPI>), grid, dim3(256), 0, \
+  hipLaunchKernelGGL((gemm_nt_bf16_tiled_kernel<WM, WN, STAGES, TOut, EPI, KW>), grid, dim3(256), 0, \
                      s, (const bf16_t*)a, (const bf16_t*)w, bias, (TOut*)c, m, n, k, lda, ldc, \
                      tiles_m, tiles_n, row_major, k_splits, k_chunk, scatter)
   switch (epilogue) {
@@ -282,6 +303,14 @@ static int launch_tiled_bf16(const void* a, const void* w, const float* bias, vo
   // (64 x 4800 x 1600: 13.8 against 11.9 us; 3 % of the decode step at that width).
   const int64_t tiles_64 = (int64_t)((m + 63) / 64) * ((n + 63) / 64);
   const int k_tiles = k / TB_BK;
+  // Up to 64 rows and so few columns that tiles of 64 leave half of the units without a block
+  // (the QKV and first feed-forward products of a wide model's decode step): tiles of 32
+  // columns, twice the blocks, each fetching the rows and half as much of the matrix (64 x
+  // 4800 x 1600 with weights from memory: 10.6 against 11.4 us; 64 x 5120 x 1280: 9.4 against
+  // 10.4; a ring of six stages instead of four: 10.8).  The time hardly depends on the columns
+  // (8,192: 11.0 us): a block walks its 25 tiles of k one behind the other.
+  if (m <= 64 && 2 * tiles_64 <= units && k_tiles > 2)
+    return launch_variant<1, 1, 4, TOut, 2>(a, w, bias, c, m, n, k, lda, ldc, epilogue, scatter, s);
   if ((tiles_64 <= 2 * units && k_tiles > 2) || k >= 2048)
     return launch_variant<1, 1, 4, TOut>(a, w, bias, c, m, n, k, lda, ldc, epilogue, scatter, s);
   // up to three blocks per unit: three stages each (544 x 4096 x 1024: 15.9 against 18.2 us)

@@ -606,6 +606,7 @@ def test_attention_prefill_far_key_and_causality():
                                    (12, 144, 1280), (16, 208, 1792), (9, 96, 1104), (16, 4800, 1600), (7, 80, 1800),
                                    (3, 4112, 64), (8, 6400, 1280), (13, 8192, 768), (5, 5000, 96), (11, 4700, 1024),
                                    (40, 4800, 1600), (64, 8192, 768), (24, 4500, 320), (17, 4112, 1792),
+                                   (64, 6400, 1600), (33, 2000, 1280), (48, 100, 2048), (61, 72, 1088),
                                    (40, 2304, 768), (64, 3072, 768), (33, 100, 1024), (50, 8000, 64), (64, 16400, 64)])
 @pytest.mark.parametrize("epilogue", ["none", "gelu_tanh", "residual"])
 @pytest.mark.parametrize("rms", [False, True])
