@@ -12,9 +12,10 @@
 // Four waves in a 2 x 2 arrangement; a wave owns WM x WN accumulators of 32 x 32
 // (v_mfma_f32_32x32x16_bf16, float accumulation), so a block makes 64 WM x 64 WN outputs.
 // With KW = 2 the two waves of a row of the arrangement share one accumulator of 32 columns
-// instead and take half of every k tile's steps each; their sums meet in LDS at the end.  A
-// block then makes 64 x 32 outputs: twice as many blocks for a product of up to 64 rows whose
-// tiles of 64 columns would leave most compute units without one.
+// instead and take every other k tile each; the block meets once per pair of tiles, and the
+// two sums meet in LDS at the end.  A block then makes 64 x 32 outputs: twice as many blocks
+// for a product of up to 64 rows whose tiles of 64 columns would leave most compute units
+// without one, and half as many meetings along k, which is what such a lone block waits for.
 // Per k tile there is one wait (own loads of the next tile have landed; later tiles stay in
 // flight) and one barrier, placed before the tile's last k step so that three steps' products
 // are queued in the matrix core meanwhile; after it the stage that was multiplied before is
@@ -68,7 +69,7 @@ __global__ __launch_bounds__(256) void gemm_nt_bf16_tiled_kernel(
   const int wave = tid >> 6;
   const int wave_m = wave >> 1;
   const int wave_n = KW == 1 ? wave & 1 : 0;
-  const int wave_k = KW == 1 ? 0 : wave & 1;     // which half of a k tile's steps
+  const int wave_k = KW == 1 ? 0 : wave & 1;     // which tile of a pair of k tiles
   // Consecutive block ids run on different XCDs, each with an L2 of its own: blocks are
   // renumbered so that every XCD works on a contiguous run of tiles.  A run walked along the
   // rows of C reads few rows of A and all of W, one walked down the columns few rows of W and
@@ -157,50 +158,89 @@ __global__ __launch_bounds__(256) void gemm_nt_bf16_tiled_kernel(
                    : "v"(stage + (uint32_t)(w_row + j * 32 * TB_ROW) + slot)
                    : "memory");
   };
-  constexpr int STEPS = TB_BK / 16 / KW;          // k steps of a tile that this wave multiplies
+  constexpr int STEPS = TB_BK / 16;
   static_assert(STEPS % 2 == 0, "the operand buffers alternate per step");
-  const int s0 = wave_k * STEPS;                  // the first of them
 
+  if constexpr (KW == 2) {
+    // Tiles in pairs: tile 2 p belongs to the first wave of a row, tile 2 p + 1 to the second.
+    // The ring holds STAGES / 2 pairs.  Per pair: wait until its two tiles have landed (later
+    // ones stay in flight), meet the other waves (which are then past the pair before, so
+    // that pair's stages can be refilled), multiply the own tile's four steps.
+    static_assert(STAGES % 2 == 0 && STAGES >= 4, "the ring holds whole pairs");
+    constexpr int HELD = STAGES / 2;
+    const int pairs = (k_tiles + 1) / 2;
 #pragma unroll
-  for (int d = 0; d < STAGES - 1; ++d)
-    if (d < k_tiles) issue(d);
-  {
-    // tile 0 has landed; tiles 1 .. STAGES - 2 may stay in flight, as far as they exist
-    const int ahead = k_tiles - 1 < STAGES - 2 ? k_tiles - 1 : STAGES - 2;
-    wait_ahead_and_sync<LOADS, STAGES - 2>(ahead);
-  }
-  fetch(0, s0, fa[0], fw[0]);
-  for (int kt = 0; kt < k_tiles; ++kt) {
-    // the stage of tile kt - 1 is free: every wave met the others after its last read of it
-    if (kt + STAGES - 1 < k_tiles) issue(kt + STAGES - 1);
+    for (int d = 0; d < 2 * (HELD - 1); ++d)
+      if (d < k_tiles) issue(d);
+    for (int p = 0; p < pairs; ++p) {
+      const int issued = k_tiles < 2 * (p + HELD - 1) ? k_tiles : 2 * (p + HELD - 1);
+      wait_ahead_and_sync<LOADS, STAGES - 4>(issued - (2 * p + 2));
 #pragma unroll
-    for (int s = 0; s < STEPS; ++s) {
-      if (s + 1 < STEPS) {
-        fetch(kt, s0 + s + 1, fa[(s + 1) & 1], fw[(s + 1) & 1]);
-        asm volatile("s_waitcnt lgkmcnt(%0)" ::"n"(READS) : "memory");   // step s has arrived
-      } else if (kt + 1 < k_tiles) {
-        // own reads of this tile are complete before the others may overwrite its stage
-        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
-        // tiles kt + 2 .. kt + STAGES - 1 may stay in flight, as far as they exist
-        const int last = k_tiles - 1 < kt + STAGES - 1 ? k_tiles - 1 : kt + STAGES - 1;
-        wait_ahead_and_sync<LOADS, STAGES - 2>(last - (kt + 1));
-        fetch(kt + 1, s0, fa[0], fw[0]);
-      } else {
-        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+      for (int d = 0; d < 2; ++d)
+        if (2 * (p + HELD - 1) + d < k_tiles) issue(2 * (p + HELD - 1) + d);
+      const int kt = 2 * p + wave_k;
+      if (kt < k_tiles) {
+        // all four steps' operands are asked for at once and used as they arrive (reads come
+        // back in the order of issue): one trip to LDS per tile stands open, not one per step
+        tb_u32x4 ga[STEPS], gw[STEPS];
+#pragma unroll
+        for (int s = 0; s < STEPS; ++s) fetch(kt, s, &ga[s], &gw[s]);
+#pragma unroll
+        for (int s = 0; s < STEPS; ++s) {
+          if (s == 0) asm volatile("s_waitcnt lgkmcnt(%0)" ::"n"(READS * (STEPS - 1)) : "memory");
+          else if (s == 1) asm volatile("s_waitcnt lgkmcnt(%0)" ::"n"(READS * (STEPS - 2)) : "memory");
+          else if (s == 2) asm volatile("s_waitcnt lgkmcnt(%0)" ::"n"(READS * (STEPS - 3)) : "memory");
+          else asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+          asm volatile("" : "+v"(ga[s]));
+          asm volatile("" : "+v"(gw[s]));
+          acc[0][0] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(
+              *reinterpret_cast<const bf16x8*>(&ga[s]), *reinterpret_cast<const bf16x8*>(&gw[s]),
+              acc[0][0], 0, 0, 0);
+        }
       }
-      // the registers are used only behind the wait (the compiler does not know that the
-      // assembly above left them on their way)
-#pragma unroll
-      for (int i = 0; i < WM; ++i) asm volatile("" : "+v"(fa[s & 1][i]));
-#pragma unroll
-      for (int j = 0; j < WN; ++j) asm volatile("" : "+v"(fw[s & 1][j]));
-#pragma unroll
-      for (int i = 0; i < WM; ++i)
-#pragma unroll
-        for (int j = 0; j < WN; ++j)
-          acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(
-              *reinterpret_cast<const bf16x8*>(&fa[s & 1][i]),
-              *reinterpret_cast<const bf16x8*>(&fw[s & 1][j]), acc[i][j], 0, 0, 0);
+    }
+  } else {
+  #pragma unroll
+    for (int d = 0; d < STAGES - 1; ++d)
+      if (d < k_tiles) issue(d);
+    {
+      // tile 0 has landed; tiles 1 .. STAGES - 2 may stay in flight, as far as they exist
+      const int ahead = k_tiles - 1 < STAGES - 2 ? k_tiles - 1 : STAGES - 2;
+      wait_ahead_and_sync<LOADS, STAGES - 2>(ahead);
+    }
+    fetch(0, 0, fa[0], fw[0]);
+    for (int kt = 0; kt < k_tiles; ++kt) {
+      // the stage of tile kt - 1 is free: every wave met the others after its last read of it
+      if (kt + STAGES - 1 < k_tiles) issue(kt + STAGES - 1);
+  #pragma unroll
+      for (int s = 0; s < STEPS; ++s) {
+        if (s + 1 < STEPS) {
+          fetch(kt, s + 1, fa[(s + 1) & 1], fw[(s + 1) & 1]);
+          asm volatile("s_waitcnt lgkmcnt(%0)" ::"n"(READS) : "memory");   // step s has arrived
+        } else if (kt + 1 < k_tiles) {
+          // own reads of this tile are complete before the others may overwrite its stage
+          asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+          // tiles kt + 2 .. kt + STAGES - 1 may stay in flight, as far as they exist
+          const int last = k_tiles - 1 < kt + STAGES - 1 ? k_tiles - 1 : kt + STAGES - 1;
+          wait_ahead_and_sync<LOADS, STAGES - 2>(last - (kt + 1));
+          fetch(kt + 1, 0, fa[0], fw[0]);
+        } else {
+          asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+        }
+        // the registers are used only behind the wait (the compiler does not know that the
+        // assembly above left them on their way)
+  #pragma unroll
+        for (int i = 0; i < WM; ++i) asm volatile("" : "+v"(fa[s & 1][i]));
+  #pragma unroll
+        for (int j = 0; j < WN; ++j) asm volatile("" : "+v"(fw[s & 1][j]));
+  #pragma unroll
+        for (int i = 0; i < WM; ++i)
+  #pragma unroll
+          for (int j = 0; j < WN; ++j)
+            acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(
+                *reinterpret_cast<const bf16x8*>(&fa[s & 1][i]),
+                *reinterpret_cast<const bf16x8*>(&fw[s & 1][j]), acc[i][j], 0, 0, 0);
+      }
     }
   }
 
@@ -210,7 +250,7 @@ __global__ __launch_bounds__(256) void gemm_nt_bf16_tiled_kernel(
                 "the epilogue reuses the stages");
   wait_loads_and_sync<0>();                       // every wave is past its last operand reads
   if (KW == 2) {
-    // the wave of the second k half hands its sums to the wave of the first, behind the
+    // the wave of the odd k tiles hands its sums to the wave of the even ones, behind the
     // regions that the epilogue uses
     float* meet = reinterpret_cast<float*>(lds) + 4 * 32 * (WN * 32 + 8) + wave_m * 16 * 64;
     if (wave_k == 1) {
@@ -305,12 +345,15 @@ static int launch_tiled_bf16(const void* a, const void* w, const float* bias, vo
   const int k_tiles = k / TB_BK;
   // Up to 64 rows and so few columns that tiles of 64 leave half of the units without a block
   // (the QKV and first feed-forward products of a wide model's decode step): tiles of 32
-  // columns, twice the blocks, each fetching the rows and half as much of the matrix (64 x
-  // 4800 x 1600 with weights from memory: 10.6 against 11.4 us; 64 x 5120 x 1280: 9.4 against
-  // 10.4; a ring of six stages instead of four: 10.8).  The time hardly depends on the columns
-  // (8,192: 11.0 us): a block walks its 25 tiles of k one behind the other.
+  // columns, twice the blocks, each fetching the rows and half as much of the matrix, and the
+  // two waves of a row taking every other k tile (64 x 4800 x 1600 with weights from memory:
+  // 9.9 against 11.4 us; 64 x 5120 x 1280: 8.9 against 10.4).  Six stages: two pairs of tiles
+  // in flight while one is multiplied (four stages 13.5 us, eight 9.8).  What remains is what a
+  // compute unit takes in: 307 KB per block at 55 KB/us beside 4.4 us that do not depend on k
+  // (the time hardly depends on the columns: 8,192 take 10.4 us); asking for a tile's four
+  // steps of operands at once instead of one step ahead changes nothing.
   if (m <= 64 && 2 * tiles_64 <= units && k_tiles > 2)
-    return launch_variant<1, 1, 4, TOut, 2>(a, w, bias, c, m, n, k, lda, ldc, epilogue, scatter, s);
+    return launch_variant<1, 1, 6, TOut, 2>(a, w, bias, c, m, n, k, lda, ldc, epilogue, scatter, s);
   if ((tiles_64 <= 2 * units && k_tiles > 2) || k >= 2048)
     return launch_variant<1, 1, 4, TOut>(a, w, bias, c, m, n, k, lda, ldc, epilogue, scatter, s);
   // up to three blocks per unit: three stages each (544 x 4096 x 1024: 15.9 against 18.2 us)
