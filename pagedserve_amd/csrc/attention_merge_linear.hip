@@ -25,10 +25,10 @@ typedef __attribute__((__vector_size__(4 * sizeof(float)))) float f32x4_t;
 
 // STEPS: head_dim / 64; PARTS: lanes that share the ranges of a row; GROUP: heads per block, one
 // wave each, whose results are summed through LDS before they are added to the residual rows.
-// Float atomic adds on a few rows are performed at some 15 per nanosecond on this chip, however
-// many blocks issue them (measured: 24 blocks adding 8 rows of 768 floats each take 10 us, 48
-// take 17): with a wave per head, 12 heads adding into 8 rows of 768 were 74,000 atomic adds and
-// most of this kernel's time.  Four heads to a block leave a quarter of them.
+// (The adds of the blocks of one column tile meet at that tile's addresses, other tiles are
+// elsewhere: spread like that, float atomic adds run at 75 to 90 per nanosecond, and the 74,000
+// of 12 heads at 8 rows of 768 take under a microsecond.  Four heads to a block are chosen by
+// what was measured, below.)
 template <int STEPS, int PARTS, int GROUP>
 __global__ __launch_bounds__(64 * GROUP) void attention_merge_linear_kernel(
     const float* __restrict__ partial, const int* __restrict__ tok_list, int count, int heads,
