@@ -105,6 +105,38 @@ def test_long_contexts_decode_in_ranges(tmp_path, dtype):
     engine.cache.check_invariants()
 
 
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("width,heads,inner,live", [(1600, 25, 6400, 12), (1600, 25, 6400, 40), (1280, 20, 5120, 64),
+                                                   (1536, 24, 7680, 33)])
+def test_wide_layers_with_many_decoded_tokens_a_step(tmp_path, dtype, width, heads, inner, live):
+    """Two layers of GPT-2 large and XL widths with 12 to 64 requests live at once: the decode
+    steps take the products' paths for 9 to 16 and for 17 to 64 rows over a k beyond 1,024 (the
+    norm inside the product with its columns dealt out evenly, tiles of 64 x 32, two column
+    tiles with ranges of k chosen by the number of blocks), which the three-request traces of
+    the real sizes above never reach."""
+    from pagedserve_amd.engine import Engine
+    from pagedserve_amd.model import load_model
+
+    config = {"architectures": ["GPT2LMHeadModel"], "model_type": "gpt2", "layer_norm_epsilon": 1e-5,
+              "activation_function": "gelu_new", "tie_word_embeddings": True, "n_layer": 2, "n_embd": width,
+              "n_head": heads, "n_inner": inner, "vocab_size": 1000, "n_positions": 128}
+    folder = str(tmp_path / "wide")
+    helpers.write_folder(folder, config, helpers.lively_tensors(config, 70 + live))
+    requests = {f"w{i}": helpers.random_tokens(14 + (i * 7) % 23, config["vocab_size"], 1200 + i)
+                for i in range(live + 6)}
+    reference = helpers.plain_logits_of_many(folder, requests, bfloat16=dtype == "bfloat16", device="cuda")
+    model, _ = load_model(folder, dtype=dtype)
+    steps = helpers.trace_mixed(requests, max_live=live, portion=(9, 4, 17, 2), decode_tail=12, seed=live)
+    most = max(sum(1 for entry in step["entries"] if len(entry["tokens"]) == 1) for step in steps)
+    assert most >= min(live, 17) - 5, most      # steps of that many single tokens do occur
+    pages = -(-helpers.live_token_budget(steps, round_to=16) // 16)
+    engine = Engine(model, num_pages=pages, page_size=16, max_requests=live, max_step_tokens=1024)
+    rows = helpers.replay_in_process(engine, steps)
+    error, scale, where = helpers.max_error(rows, reference)
+    assert error <= helpers.TOLERANCE[dtype] * scale, (dtype, width, live, error, scale, where)
+    engine.cache.check_invariants()
+
+
 @pytest.mark.parametrize("seed", [1, 2, 3])
 def test_random_configurations_in_32_bit(tmp_path, seed):
     """Eight configurations drawn at random for each seed (1 to 25 heads of 4 to 256 dimensions,
