@@ -178,7 +178,8 @@ class Attention(Mixer):
         the other path would cut 130 to 250 keys into two ranges and merge them with a launch
         of its own (1 to 4 requests over 20 to 250 keys: 5 % of the step, 8 requests 2 %).
         About three blocks of four waves per compute unit, never more ranges than the keys of
-        the longest request can feed."""
+        the longest request can feed; and not where the projection's blocks would read more
+        than 12 MB of records between them (wide models)."""
         visible = max_kv_len if self.window <= 0 else min(max_kv_len, self.window)
         pairs = count * self.heads
         units = kernels.compute_units()
@@ -186,7 +187,17 @@ class Attention(Mixer):
         if pairs > units * 3 // 4 or (most < 3 and 2 * pairs > units):
             return 0
         wanted = max(1, -(-3 * units // pairs))
-        return min(most, wanted, 64)
+        splits = min(most, wanted, 64)
+        # Every block of 16 output columns merges the records of its head again: together they
+        # read the records as often as the projection has column tiles, which grows with the
+        # square of the heads.  Beyond some 12 MB of that the other path is ahead (decode steps
+        # over 1,024 keys, merged against not: 8 requests of 16 heads, 12.3 MB, 0.837 against
+        # 0.821 ms; 4 of 25 heads, 21 MB, 2.089 against 1.995; under it 4 requests of 16 heads
+        # 0.724 against 0.771, 2 of 25 heads 1.903 against 1.951, 16 of 12 heads 2 % ahead).
+        tiles = -(-self.width // 16)
+        if tiles * pairs * splits * (self.head_dim + 2) * 4 > 12_000_000:
+            return 0
+        return splits
 
     def _splits(self, count: int, max_kv_len: int):
         """(ranges per request, waves per block) of the decode kernel, by the number of (token,

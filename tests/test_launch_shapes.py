@@ -10,6 +10,7 @@ from pagedserve_amd.parts.attention import Attention
 def _part(heads, head_dim=64, window=0):
     part = Attention.__new__(Attention)
     part.heads, part.head_dim, part.window = heads, head_dim, window
+    part.width = heads * head_dim
     return part
 
 
@@ -50,5 +51,10 @@ def test_documented_cases(monkeypatch):
     # where the keys feed three ranges
     assert part._merged_splits(8, 200) == 2 and part._merged_splits(1, 20) == 1
     assert part._merged_splits(16, 200) == 0 and part._merged_splits(16, 1024) == 4
+    # wide models: not where the projection's blocks would read the records too often
+    assert _part(16)._merged_splits(4, 1024) == 8 and _part(16)._merged_splits(8, 1024) == 0
+    assert _part(16)._merged_splits(8, 400) == 4 and _part(16)._merged_splits(12, 400) == 0
+    assert _part(25)._merged_splits(2, 1024) == 8 and _part(25)._merged_splits(4, 1024) == 0
+    assert _part(25)._merged_splits(4, 400) == 4
     # a window bounds the keys that a query sees
     assert _part(12, window=256)._splits(32, 8192) == (1, 4)
