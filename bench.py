@@ -76,7 +76,7 @@ def _build(dtype, max_requests, max_step_tokens, layers=None, shape=SMALL, pages
     shape's 1.5 billion take a second there), and what the weights occupy."""
     import torch
 
-    from pagedserve_amd.engine import Engine
+    from pagedserve_amd.engine import Engine, hostgc
     from pagedserve_amd.model import random_model
     from pagedserve_amd.sampling.sampler import Sampler
 
@@ -94,6 +94,9 @@ def _build(dtype, max_requests, max_step_tokens, layers=None, shape=SMALL, pages
     engine = Engine(model, num_pages=pages, page_size=PAGE_SIZE, max_requests=max_requests,
                     max_step_tokens=max_step_tokens)
     engine.weights_resident_bytes = resident
+    # (as the entry points do once an engine stands: the collector does not walk the model and
+    # the modules again in the middle of a timed step)
+    hostgc.settle()
     return engine, Sampler("cuda", max_requests), config
 
 

@@ -343,16 +343,20 @@ static int launch_tiled_bf16(const void* a, const void* w, const float* bias, vo
   // (64 x 4800 x 1600: 13.8 against 11.9 us; 3 % of the decode step at that width).
   const int64_t tiles_64 = (int64_t)((m + 63) / 64) * ((n + 63) / 64);
   const int k_tiles = k / TB_BK;
-  // Up to 64 rows and so few columns that tiles of 64 leave half of the units without a block
-  // (the QKV and first feed-forward products of a wide model's decode step): tiles of 32
-  // columns, twice the blocks, each fetching the rows and half as much of the matrix, and the
-  // two waves of a row taking every other k tile (64 x 4800 x 1600 with weights from memory:
-  // 9.9 against 11.4 us; 64 x 5120 x 1280: 8.9 against 10.4).  Six stages: two pairs of tiles
-  // in flight while one is multiplied (four stages 13.5 us, eight 9.8).  What remains is what a
-  // compute unit takes in: 307 KB per block at 55 KB/us beside 4.4 us that do not depend on k
-  // (the time hardly depends on the columns: 8,192 take 10.4 us); asking for a tile's four
-  // steps of operands at once instead of one step ahead changes nothing.
-  if (m <= 64 && 2 * tiles_64 <= units && k_tiles > 2)
+  // So few tiles of 64 x 64 that half of the units would be without a block (the QKV and first
+  // feed-forward products of a wide model's decode step; the products with few columns of a
+  // step that mixes a prompt portion with decoded tokens): tiles of 32 columns, twice the
+  // blocks, each fetching the rows and half as much of the matrix, and the two waves of a row
+  // taking every other k tile (64 x 4800 x 1600 with weights from memory: 9.9 against 11.4 us;
+  // 64 x 5120 x 1280: 8.9 against 10.4; 544 x 768 x 3072: 14.7 against 17.1; 544 x 768 x 768: 6.2
+  // against 7.0; 544 x 1024 x 4096, 288 blocks: 20.7 against 22.0; with a short k more blocks than
+  // units lose instead: 200 x 2304 x 768 on 288 blocks 7.2 against 6.8).  Six stages: two pairs of
+  // tiles in flight while one is multiplied (four stages 13.5 us, eight 9.8).  What remains is
+  // what a compute unit takes in: 307 KB per block at 55 KB/us beside 4.4 us that do not depend
+  // on k (the time hardly depends on the columns: 8,192 take 10.4 us); asking for a tile's four
+  // steps of operands at once instead of one step ahead changes nothing, and eight waves on a
+  // tile of 64 x 64, four for the even and four for the odd k tiles, gain a third of this.
+  if ((2 * tiles_64 <= units || (k >= 2048 && 16 * tiles_64 <= 9 * units)) && k_tiles > 2)
     return launch_variant<1, 1, 6, TOut, 2>(a, w, bias, c, m, n, k, lda, ldc, epilogue, scatter, s);
   if ((tiles_64 <= 2 * units && k_tiles > 2) || k >= 2048)
     return launch_variant<1, 1, 4, TOut>(a, w, bias, c, m, n, k, lda, ldc, epilogue, scatter, s);

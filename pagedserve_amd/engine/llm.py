@@ -16,6 +16,7 @@ from ..config.base import read_config_json
 from ..config.registry import find_preset
 from ..model.loading import load_model, random_model, resolve_dtype
 from ..sampling.params import SamplingParams
+from . import hostgc
 from .engine import Engine
 from .scheduler import ORCA_STRATEGY, ContinuousBatchScheduler
 from .tokenizer import load_tokenizer
@@ -111,6 +112,7 @@ def build_scheduler(model=REFERENCE_MODEL, scheduling_strategy=ORCA_STRATEGY, pr
         scheduling_strategy=scheduling_strategy, prefill_chunk_size=prefill_chunk_size,
         max_num_batched_tokens=step_tokens, max_prefill_requests=max_prefill_requests)
     scheduler.model_config = config
+    hostgc.settle()
     return scheduler
 
 

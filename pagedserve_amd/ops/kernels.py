@@ -301,6 +301,13 @@ class TopChoice:
 
 
 _MEMO_LIMIT = 512
+# What a memoized call keeps is the bytes of its argument block, nothing that the garbage
+# collector has to walk (a stream of requests leaves tens of thousands of blocks behind; as
+# ctypes structures with two result integers each they made a full collection take 90 ms, in
+# the middle of a step).  The two result integers that a block points at are these, shared by
+# all memoized calls: a call's results are read before the next call is made.
+_MEMO_LAYOUT = c_int(0)
+_MEMO_DONE = c_int(0)
 
 
 def _memo_key(x, out, scatter, a_packed, choose):
@@ -351,15 +358,15 @@ def linear(x, w, bias, out, epilogue="none", scatter=None, packed=None, a_packed
         key = _memo_key(x, out, scatter, a_packed, choose)
         kept = memo.get(key)
         if kept is not None:
-            args, layout, done = kept
-            status = _BOUND["ps_linear"](ctypes.byref(args), _stream())
+            # (the library reads the block and writes through the pointers in it only)
+            status = _BOUND["ps_linear_bytes"](kept, _stream())
             if status != 0:
                 raise KernelError(f"ps_linear failed ({status}): "
                                   f"{load_library().ps_last_error().decode('utf-8', 'replace')}")
             if packed_out:
-                return out, bool(layout.value)
+                return out, bool(_MEMO_LAYOUT.value)
             if choose is not None:
-                return out, bool(done.value)
+                return out, bool(_MEMO_DONE.value)
             return out
     _check(w, "w", ndim=2)
     _check(out, "out", ndim=2)
@@ -440,12 +447,12 @@ def linear(x, w, bias, out, epilogue="none", scatter=None, packed=None, a_packed
         args.head_dim, args.kv_heads = head_dim, kv_heads
         args.page_size, args.num_pages = page_size, pages
         args.scatter_only = 1 if scatter_only else 0
-    layout = c_int(0)
+    layout = _MEMO_LAYOUT if memo is not None else c_int(0)
     if packed_out:
         args.c_packed_request = 1
         args.c_rows = _row_capacity(out, n)
         args.c_layout = ctypes.pointer(layout)
-    done = c_int(0)
+    done = _MEMO_DONE if memo is not None else c_int(0)
     if choose is not None:
         top, tokens = choose
         _check(tokens, "tokens", torch.int32, 1)
@@ -470,13 +477,19 @@ def linear(x, w, bias, out, epilogue="none", scatter=None, packed=None, a_packed
         fn.argtypes = [ctypes.POINTER(_LinearArgs), c_void_p]
         fn.restype = c_int
         _BOUND["ps_linear"] = fn
+        # the same entry point taking the block as a bytes object (a second function object:
+        # argument types belong to the object, not to the symbol)
+        from_bytes = lib["ps_linear"]
+        from_bytes.argtypes = [ctypes.c_char_p, c_void_p]
+        from_bytes.restype = c_int
+        _BOUND["ps_linear_bytes"] = from_bytes
     status = fn(ctypes.byref(args), _stream())
     if status != 0:
         raise KernelError(f"ps_linear failed ({status}): {lib.ps_last_error().decode('utf-8', 'replace')}")
     if memo is not None:
         if len(memo) >= _MEMO_LIMIT:
             memo.clear()
-        memo[key] = (args, layout, done)     # (the block points at ``layout`` and ``done``)
+        memo[key] = bytes(args)
     if packed_out:
         return out, bool(layout.value)
     if choose is not None:

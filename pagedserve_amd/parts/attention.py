@@ -46,7 +46,6 @@ class Attention(Mixer):
         self.q_cols = heads * head_dim
         self.kv_cols = kv_heads * head_dim
         self.position = None
-        self._columns = {}
         # what ``kernels.linear`` keeps per call site and step shape (its ``memo``), per workspace
         self._memo_qkv, self._memo_out = {}, {}
 
@@ -78,17 +77,10 @@ class Attention(Mixer):
     def forward(self, x, residual, ctx, cache):
         tokens = ctx.tokens
         total = self.q_cols + 2 * self.kv_cols
-        qkv = ctx.workspace.first_rows("qkv", total, self.dtype, tokens)
+        # (the step's rows and their three column views, made once per row count for all layers)
+        qkv, q, k, v = ctx.workspace.column_views("qkv", total, self.dtype, tokens,
+                                                  (self.q_cols, self.kv_cols, self.kv_cols))
         tables = ctx.tables[cache.group]
-        columns = self._columns.get(tokens)
-        if columns is None or columns[0] is not qkv:
-            # (the three column views of a step's rows, made once per row count)
-            if len(self._columns) > 1024:
-                self._columns.clear()
-            columns = self._columns[tokens] = (qkv, qkv[:, :self.q_cols],
-                                               qkv[:, self.q_cols:self.q_cols + self.kv_cols],
-                                               qkv[:, self.q_cols + self.kv_cols:])
-        _, q, k, v = columns
         rotates = self.position is not None and self.position.transforms_qk
         if cache.writes and not rotates:
             # keys and values go to their pages from the product's own epilogue

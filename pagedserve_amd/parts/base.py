@@ -202,6 +202,23 @@ class Workspace:
             view = self._views[key] = self.rows(name, columns, dtype)[:count]
         return view
 
+    def column_views(self, name: str, columns: int, dtype: torch.dtype, count: int, cuts: tuple):
+        """``first_rows(name, columns, dtype, count)`` and its pieces along the columns (``cuts``:
+        the widths of the pieces), the same tensor objects every time and for every layer that
+        asks with the same sizes."""
+        key = (name, columns, dtype, count, cuts)
+        views = self._views.get(key)
+        if views is None:
+            if len(self._views) > 4096:
+                self._views.clear()
+            whole = self.first_rows(name, columns, dtype, count)
+            pieces, begin = [whole], 0
+            for width in cuts:
+                pieces.append(whole[:, begin:begin + width])
+                begin += width
+            views = self._views[key] = tuple(pieces)
+        return views
+
     def flat(self, name: str, numel: int, dtype: torch.dtype):
         """A 1-D scratch buffer of at least ``numel`` elements; callers ask for their worst
         case so that it is allocated once."""
