@@ -41,18 +41,25 @@ __global__ __launch_bounds__(64 * SK_WAVES) void gemm_nt_skinny_norm_kernel(
       NT == 1 ? partial_own : reinterpret_cast<float*>(xs));
   const int lane = threadIdx.x & 63;
   const int wave = threadIdx.x >> 6;
-  const int n0 = blockIdx.x * cols;
-  const int n1 = n0 + cols < n ? n0 + cols : n;
+  // (one tile: always 16 columns from a multiple of 16, and the addresses are as simple as that)
+  const int n0 = NT == 1 ? blockIdx.x * 16 : blockIdx.x * cols;
+  const int n1 = NT == 1 ? n : (n0 + cols < n ? n0 + cols : n);
   const int sub = lane & 15;
   const int group = lane >> 4;
   const bf16_t* w_ptr[NT];
+  if (NT == 1) {
+    const int w_row = n0 + sub < n ? n0 + sub : n - 1;
+    w_ptr[0] = w + (int64_t)w_row * k + group * 16;
+    if (wp != nullptr) w_ptr[0] = wp + (int64_t)(n0 / 16) * (k / 64) * 1024 + lane * 8;   // packed copy
+  } else {
 #pragma unroll
-  for (int t = 0; t < NT; ++t) {
-    const int w_row = n0 + t * 16 + sub < n1 ? n0 + t * 16 + sub : n1 - 1;
-    w_ptr[t] = w + (int64_t)w_row * k + group * 16;
-    // packed copy: row r is lane group * 16 + r % 16 of tile r / 16
-    if (wp != nullptr)
-      w_ptr[t] = wp + (int64_t)(w_row >> 4) * (k / 64) * 1024 + (group * 16 + (w_row & 15)) * 8;
+    for (int t = 0; t < NT; ++t) {
+      const int w_row = n0 + t * 16 + sub < n1 ? n0 + t * 16 + sub : n1 - 1;
+      w_ptr[t] = w + (int64_t)w_row * k + group * 16;
+      // packed copy: row r is lane group * 16 + r % 16 of tile r / 16
+      if (wp != nullptr)
+        w_ptr[t] = wp + (int64_t)(w_row >> 4) * (k / 64) * 1024 + (group * 16 + (w_row & 15)) * 8;
+    }
   }
   const uint4 zero = {0u, 0u, 0u, 0u};
 
