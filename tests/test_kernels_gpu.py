@@ -1103,6 +1103,10 @@ def test_linear_memo_of_a_call_site():
         if len(results) == 1:
             h[:8] = _rand((8, k), torch.float32, 720)    # the same addresses, other values: a hit reads them
     assert len(memo) == 1 and not torch.equal(results[0], results[1])
+    # what is kept per call is nothing that the garbage collector has to walk (a stream of
+    # requests leaves tens of thousands of entries behind)
+    import gc
+    assert all(type(kept) is bytes and not gc.is_tracked(kept) for kept in memo.values())
     expected = F.layer_norm(h[:8].double(), (k,), gamma.double(), beta.double(), 1e-5)
     expected = expected.to(torch.bfloat16).double() @ w.double().t() + bias.double()
     torch.testing.assert_close(results[1].double(), expected, atol=5e-3, rtol=5e-3)
