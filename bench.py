@@ -174,7 +174,7 @@ def decode_point(engine, sampler, config, batch, prompt_len, output_tokens, warm
     return elapsed, mean_context
 
 
-def prefill_run(engine, config, reps=8, warmup=5, seed=1, prompts=2, length=PREFILL_TOKENS // 2):
+def prefill_run(engine, config, reps=8, warmup=None, seed=1, prompts=2, length=PREFILL_TOKENS // 2):
     """Seconds per step of ``prompts`` x ``length`` prompt tokens (logits at each prompt's last
     token), in the steady state: the warm-up covers the steps that allocate buffers and record
     the layout's graph."""
@@ -184,6 +184,8 @@ def prefill_run(engine, config, reps=8, warmup=5, seed=1, prompts=2, length=PREF
 
     generator = torch.Generator().manual_seed(seed)
     times = []
+    # (a layout with a prompt portion is recorded once it has come back ``record_after`` times)
+    warmup = max(warmup or 0, engine.record_after + 2 if engine.use_graphs else 3)
     for rep in range(reps + warmup):
         entries = [StepEntry(f"p{rep}_{i}", _random_prompt(generator, length, config.vocab_size),
                              [length - 1]) for i in range(prompts)]
@@ -324,7 +326,8 @@ def mixed_step_times(engine, config, decodes=32, portion=512, context=300, reps=
     engine.use_graphs = False
     direct = [one(rep) for rep in range(reps + 2)][2:]
     engine.use_graphs = graphs
-    replayed = [one(rep) for rep in range(reps + 2, 2 * reps + 8)][-reps:]
+    # (the layout is recorded once it has come back ``record_after`` times)
+    replayed = [one(rep) for rep in range(reps + 2, 2 * reps + 4 + engine.record_after)][-reps:]
     for name in names:
         engine.finish(name)
 

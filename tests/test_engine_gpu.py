@@ -193,6 +193,7 @@ def test_graph_replay_of_mixed_steps(folders, references, dtype):
     requests = _requests("B", config)
     model, _ = load_model(folder, dtype=dtype)
     engine = Engine(model, num_pages=30, page_size=page_size, max_requests=4, max_step_tokens=128)
+    engine.record_after = 3       # (the default waits for many more returns)
     rows = {}
 
     def run(entries):
@@ -317,6 +318,7 @@ def test_more_layouts_than_recorded_graphs_are_kept(folders, references, dtype):
     model, _ = load_model(folder, dtype=dtype)
     engine = Engine(model, num_pages=40, page_size=page_size, max_requests=4, max_step_tokens=128)
     engine.max_graphs = 3
+    engine.record_after = 3
     rows = {}
 
     def run(entries):
