@@ -492,6 +492,7 @@ static void launch_skinny_mb(const void* a, const void* w, const float* bias, vo
   // with its rows on four blocks, 6.2 us on one)
   int z = 3 * ps_compute_units() / grid_xy;
   z = z < 1 ? 1 : (z > row_blocks ? row_blocks : z);
+  if (z < (row_blocks + 3) / 4) z = (row_blocks + 3) / 4;   // (a block holds at most four accumulators of 16 rows)
   const int per = (row_blocks + z - 1) / z;
   dim3 grid((n + 15) / 16, k_splits, (row_blocks + per - 1) / per);
   dim3 block(64 * SK_WAVES);
@@ -604,7 +605,18 @@ static int launch_skinny(const void* a, const void* w, const float* bias, void* 
 // added in place (residual epilogue), which keeps every block at one round.
 bool ps_gemm_nt_mfma_skinny(const void* a, const void* w, int m, int n, int k, int lda, int dtype,
                             int epilogue) {
-  if (dtype != PS_BF16 || m > 64) return false;
+  if (dtype != PS_BF16) return false;
+  // Somewhat more rows with the residual epilogue (the projections of a step that mixes a
+  // short prompt portion with decoded tokens): ranges of k over blocks and atomic adds still
+  // beat the tiled kernel's few blocks walking a long k, until the adds and the rows that every
+  // block fetches outweigh it (rows x columns, with weights from memory: 128 x 768 x 3072 9.3
+  // against 14.7 us, 224 rows 12.3 against 14.5, 256 rows 15.8; 128 x 1024 x 4096 11.7 against
+  // 16.6, 192 rows 16.7 against 18.3; 128 x 1600 x 6400 21.3 against 27.2, 160 rows 27.5 against
+  // 26.9; with a short k 128 x 768 x 768 4.6 against 5.8, 192 x 1024 x 1024 6.5 against 6.8, 96 x
+  // 1600 x 1600 9.2 against 9.3, 112 rows 10.6 against 9.4).
+  if (m > 64)
+    return epilogue == PS_EPI_RESIDUAL && m <= 224 && n < 64 * 256 &&
+           (int64_t)m * n <= (k >= 2048 ? 200000 : 160000);
   const bool skinny_k = n < 64 * 256 && (epilogue == PS_EPI_RESIDUAL || k <= 1024 || m <= 16);
   return skinny_k || !ps_gemm_nt_bf16_tiled_supported(a, w, m, k, lda);
 }
