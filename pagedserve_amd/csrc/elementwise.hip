@@ -156,6 +156,54 @@ __global__ __launch_bounds__(256) void norm_wave_kernel(
   }
 }
 
+// norm_row_kernel: one block of four waves per row, the row held in registers (width <= 256 *
+// VPT), the two sums met through LDS.  For few wide rows (a decode step of a wide model): a
+// wave alone would hold 25 values per lane at 1,600 columns and ask for them one after the
+// other, four waves ask for 7 each.
+template <typename T, bool RMS, int VPT>
+__global__ __launch_bounds__(256) void norm_row_kernel(
+    const float* __restrict__ x, const int* __restrict__ rows, const float* __restrict__ gamma,
+    const float* __restrict__ beta, T* __restrict__ out, int width, float eps, int packed) {
+  __shared__ float scratch[16];
+  const int r = blockIdx.x;
+  const float* src = x + (int64_t)(rows ? rows[r] : r) * width;
+  float v[VPT], g[VPT], b[VPT];
+#pragma unroll
+  for (int i = 0; i < VPT; ++i) {
+    const int col = threadIdx.x + i * 256;
+    const int safe = col < width ? col : width - 1;
+    v[i] = src[safe];
+    g[i] = gamma[safe];
+    b[i] = (!RMS && beta != nullptr) ? beta[safe] : 0.f;
+  }
+  float sum = 0.f;
+#pragma unroll
+  for (int i = 0; i < VPT; ++i) {
+    if ((int)threadIdx.x + i * 256 >= width) v[i] = 0.f;
+    sum += v[i];
+  }
+  float mean = 0.f;
+  if (!RMS) mean = block_sum(sum, scratch) / (float)width;
+  float sq = 0.f;
+#pragma unroll
+  for (int i = 0; i < VPT; ++i) {
+    const int col = threadIdx.x + i * 256;
+    const float c = col < width ? v[i] - mean : 0.f;
+    v[i] = c;
+    sq += c * c;
+  }
+  const float inv_std = 1.0f / sqrtf(block_sum(sq, scratch) / (float)width + eps);
+  T* dst = out + (int64_t)r * width;
+#pragma unroll
+  for (int i = 0; i < VPT; ++i) {
+    const int col = threadIdx.x + i * 256;
+    if (col >= width) continue;
+    const T y = from_float<T>(v[i] * inv_std * g[i] + b[i]);
+    if (packed) out[packed_offset(r, col, width)] = y;
+    else dst[col] = y;
+  }
+}
+
 template <typename T, bool RMS>
 __global__ void norm_block_kernel(const float* __restrict__ x, const int* __restrict__ rows,
                                   const float* __restrict__ gamma, const float* __restrict__ beta,
@@ -189,6 +237,16 @@ static void launch_norm(const float* x, const int* rows, const float* gamma, con
                         void* out, int n_rows, int width, float eps, int packed, hipStream_t s) {
   const int per_lane = (width + 63) / 64;
   const dim3 grid((n_rows + 3) / 4);
+  if (n_rows <= 64 && per_lane > 12 && per_lane <= 32) {
+    // few wide rows: a block of four waves per row
+#define PS_LAUNCH_NR(VPT)                                                                          \
+  hipLaunchKernelGGL((norm_row_kernel<T, RMS, VPT>), dim3(n_rows), dim3(256), 0, s, x, rows, gamma, \
+                     beta, (T*)out, width, eps, packed)
+    if (per_lane <= 16) PS_LAUNCH_NR(4);
+    else PS_LAUNCH_NR(8);
+#undef PS_LAUNCH_NR
+    return;
+  }
 #define PS_LAUNCH_NW(VPT)                                                                       \
   hipLaunchKernelGGL((norm_wave_kernel<T, RMS, VPT>), grid, dim3(256), 0, s, x, rows, gamma, beta, \
                      (T*)out, n_rows, width, eps, packed)
