@@ -1,8 +1,10 @@
 // Tiled paged attention for prompt portions on the matrix cores (bfloat16).
 //
-// One block per (tile of 64 queries of one request, head).  Its 2 KS waves are arranged as
-// 2 x KS: a wave owns 32 consecutive queries and every KS-th run of 32 keys, with an
-// online-softmax state of its own; the KS states of a query are merged through LDS at the end.
+// One block per (tile of 32 QW queries of one request, head), QW = 2 or 1.  Its QW KS waves are
+// arranged as QW x KS: a wave owns 32 consecutive queries and every KS-th run of 32 keys, with
+// an online-softmax state of its own; the KS states of a query are merged through LDS at the
+// end.  (Tiles of 32 queries are for steps whose tiles of 64 would leave half of the compute
+// units without a block: a prompt portion beside decoded tokens.)
 // A request's longest tile decides how long the launch takes, and splitting its keys over
 // waves shortens exactly that.  Keys and values are visited 32 KS at a time through the
 // request's block table, from the first key any query of the tile may see to the tile's last
@@ -39,7 +41,7 @@ typedef __attribute__((__vector_size__(16 * sizeof(float)))) float f32x16;
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
 
-#define AP_QUERIES 64      // queries per block
+#define AP_QUERIES 64      // queries per block (32 with QW = 1)
 #define AP_TABLE_MAX 2048  // block-table entries that a tile may need
 
 typedef const __attribute__((address_space(1))) void* ap_global_ptr;
@@ -50,8 +52,8 @@ __device__ inline void ap_wait_loads_and_sync() {
   asm volatile("s_waitcnt vmcnt(%0)\n\ts_barrier" ::"n"(PENDING) : "memory");
 }
 
-template <int NDB, int KS>  // head_dim / 16; waves along the keys
-__global__ __launch_bounds__(128 * KS) void attention_prefill_kernel(
+template <int NDB, int KS, int QW = 2>  // head_dim / 16; waves along the keys; waves along the queries
+__global__ __launch_bounds__(64 * QW * KS) void attention_prefill_kernel(
     const bf16_t* __restrict__ q, int64_t q_stride, const bf16_t* __restrict__ k_pool,
     const bf16_t* __restrict__ v_pool, bf16_t* __restrict__ out, int64_t out_stride,
     const int* __restrict__ tile_item, const int* __restrict__ tile_q0,
@@ -63,25 +65,27 @@ __global__ __launch_bounds__(128 * KS) void attention_prefill_kernel(
   constexpr int CH = HD / 8;                     // 16-byte pieces per row
   constexpr int SPREAD = ROW <= 256 ? 256 / ROW : 1;   // keys that share one pass over the banks
   constexpr int AP_KEYS = 32 * KS;               // keys per tile
-  constexpr int AP_WAVES = 2 * KS;
+  constexpr int AP_WAVES = QW * KS;
+  constexpr int QUERIES = 32 * QW;               // queries per block
+  static_assert(QW == 1 || QW == 2, "one or two waves along the queries");
   constexpr int TILE_BYTES = AP_KEYS * ROW;
   constexpr int STAGE_BYTES = 2 * TILE_BYTES;    // K tile, then V tile
   // The ring may take 96 KB; with four waves along the keys 64 KB, so that two such blocks
   // share a compute unit: the grids that take them have up to three blocks for two units, and
   // with one block per unit a third of them would wait for a second round (2 x 1,024 tokens of
   // 12 heads: 1.5 us less per launch).
-  constexpr int FIT = (KS >= 4 ? 65536 : 98304) / STAGE_BYTES;
+  constexpr int FIT = (KS >= 4 && QW == 2 ? 65536 : 98304) / STAGE_BYTES;
   constexpr int STAGES = FIT >= 4 ? 4 : (FIT >= 2 ? FIT : 2);
   static_assert(NDB <= 8 || STAGES == 2, "head sizes beyond 128 rely on a ring of two stages");
   constexpr int INSTRUCTIONS = KS * NDB;         // load instructions per operand and stage
   // every wave issues the same number of loads (the counter of loads in flight is per wave):
   // where they do not divide evenly the last ones are issued twice
-  constexpr int PER_OPERAND = (NDB + 1) / 2;
+  constexpr int PER_OPERAND = (NDB + QW - 1) / QW;
   constexpr int LOADS = 2 * PER_OPERAND;
   constexpr int NDB32 = (NDB + 1) / 2;           // blocks of 32 head dimensions
   static_assert(LOADS * 2 < 64, "the load counter has six bits");
   // the states that the waves merge at the end lie where the stages were
-  constexpr int MERGE_BYTES = (AP_WAVES - 2) * 64 * (NDB32 * 16 + 2) * 4;
+  constexpr int MERGE_BYTES = (AP_WAVES - QW) * 64 * (NDB32 * 16 + 2) * 4;
   constexpr int LDS_BYTES = STAGES * STAGE_BYTES > MERGE_BYTES ? STAGES * STAGE_BYTES : MERGE_BYTES;
   __shared__ __attribute__((aligned(1024))) unsigned char stages[LDS_BYTES];
   __shared__ int s_table[AP_TABLE_MAX];
@@ -89,8 +93,8 @@ __global__ __launch_bounds__(128 * KS) void attention_prefill_kernel(
   const int tid = threadIdx.x;
   const int lane = tid & 63;
   const int wave = tid >> 6;
-  const int wave_q = wave & 1;   // which 32 queries
-  const int wave_k = wave >> 1;  // which run of 32 keys of every tile
+  const int wave_q = wave % QW;  // which 32 queries
+  const int wave_k = wave / QW;  // which run of 32 keys of every tile
   const int sub = lane & 31;     // query of this lane within the wave; key or dimension row
   const int half = lane >> 5;    // which half of a step's reduction dimension
   const int head = blockIdx.x;
@@ -113,7 +117,7 @@ __global__ __launch_bounds__(128 * KS) void attention_prefill_kernel(
   const int wave_last_q = q0 + wave_q * 32 + 31 < count ? q0 + wave_q * 32 + 31 : count - 1;
   const int wave_last = start + wave_last_q;
   const bool wave_active = q0 + wave_q * 32 < count;
-  const int tile_last_q = q0 + AP_QUERIES - 1 < count ? q0 + AP_QUERIES - 1 : count - 1;
+  const int tile_last_q = q0 + QUERIES - 1 < count ? q0 + QUERIES - 1 : count - 1;
   const int key_end = start + tile_last_q + 1;
   int key_begin = 0;
   if (window > 0 && start + q0 - window + 1 > 0) key_begin = start + q0 - window + 1;
@@ -121,7 +125,7 @@ __global__ __launch_bounds__(128 * KS) void attention_prefill_kernel(
   // the block-table entries of keys key_begin .. key_end - 1
   const int first_logical = page_shift >= 0 ? (key_begin >> page_shift) : key_begin / page_size;
   const int last_logical = page_shift >= 0 ? ((key_end - 1) >> page_shift) : (key_end - 1) / page_size;
-  for (int i = tid; i <= last_logical - first_logical && i < AP_TABLE_MAX; i += 128 * KS) {
+  for (int i = tid; i <= last_logical - first_logical && i < AP_TABLE_MAX; i += 64 * QW * KS) {
     const int logical = first_logical + i;
     const int page = logical < table_width ? table[logical] : 0;
     s_table[i] = (page >= 0 && page < num_pages) ? page : 0;   // never an address outside the pool
@@ -371,11 +375,11 @@ __global__ __launch_bounds__(128 * KS) void attention_prefill_kernel(
   // accumulators of waves with the same queries have the same layout, so lane meets lane.
   if (KS > 1) {
     constexpr int STATE = NDB32 * 16 + 2;      // floats per lane
-    static_assert((AP_WAVES - 2) * 64 * STATE * 4 == MERGE_BYTES, "the merge reuses the stages");
+    static_assert((AP_WAVES - QW) * 64 * STATE * 4 == MERGE_BYTES, "the merge reuses the stages");
     ap_wait_loads_and_sync<0>();               // every wave is past its last operand reads
     float* states = reinterpret_cast<float*>(stages);
     if (wave_k > 0) {
-      float* mine = states + ((wave_k - 1) * 2 + wave_q) * 64 * STATE + lane;
+      float* mine = states + ((wave_k - 1) * QW + wave_q) * 64 * STATE + lane;
       mine[0] = m;
       mine[64] = l;
 #pragma unroll
@@ -387,7 +391,7 @@ __global__ __launch_bounds__(128 * KS) void attention_prefill_kernel(
     if (wave_k > 0) return;
 #pragma unroll 1
     for (int other = 1; other < KS; ++other) {
-      const float* theirs = states + ((other - 1) * 2 + wave_q) * 64 * STATE + lane;
+      const float* theirs = states + ((other - 1) * QW + wave_q) * 64 * STATE + lane;
       const float m_o = theirs[0];
       const float l_o = theirs[64];
       const float m_n = fmaxf(m, m_o);
@@ -423,6 +427,7 @@ __global__ __launch_bounds__(128 * KS) void attention_prefill_kernel(
 
 // What the host has to know of this file's constants to list a step's tiles.
 extern "C" int ps_attention_prefill_query_tile(void) { return AP_QUERIES; }
+extern "C" int ps_attention_prefill_small_tile(void) { return AP_QUERIES / 2; }
 extern "C" int ps_attention_prefill_table_max(void) { return AP_TABLE_MAX; }
 
 extern "C" int ps_attention_prefill(const void* q, int64_t q_stride, const void* k_pool,
@@ -431,7 +436,7 @@ extern "C" int ps_attention_prefill(const void* q, int64_t q_stride, const void*
                                     const int* cu_tokens, const int* kv_lens, const int* tables,
                                     int table_width, int heads, int kv_heads, int head_dim,
                                     int page_size, int num_pages, float scale, int window,
-                                    int max_kv_len, int dtype, void* stream) {
+                                    int max_kv_len, int query_tile, int dtype, void* stream) {
   PS_REQUIRE(tiles >= 0 && heads > 0 && kv_heads > 0 && page_size > 0 && num_pages > 0 &&
                  table_width > 0,
              "ps_attention_prefill: bad sizes");
@@ -441,6 +446,9 @@ extern "C" int ps_attention_prefill(const void* q, int64_t q_stride, const void*
   PS_REQUIRE(head_dim > 0 && head_dim % 16 == 0 && head_dim <= 256,
              "ps_attention_prefill: head_dim %d must be a multiple of 16 up to 256", head_dim);
   PS_REQUIRE(window >= 0 && tiles <= 65535, "ps_attention_prefill: bad window or too many tiles (%d)", tiles);
+  PS_REQUIRE(query_tile == AP_QUERIES || (query_tile == AP_QUERIES / 2 && head_dim <= 128),
+             "ps_attention_prefill: tiles of %d or (head sizes up to 128) %d queries, not %d", AP_QUERIES,
+             AP_QUERIES / 2, query_tile);
   PS_REQUIRE(scale > 0.f, "ps_attention_prefill: the score scale must be positive, got %g", scale);
   PS_REQUIRE(table_width <= AP_TABLE_MAX,
              "ps_attention_prefill: block tables of %d pages exceed the %d that a tile keeps",
@@ -462,6 +470,28 @@ extern "C" int ps_attention_prefill(const void* q, int64_t q_stride, const void*
   // with many, smaller blocks that share a unit balance better.
   const bool wide = (int64_t)tiles * heads <= ps_compute_units() * 3 / 2 &&
                     (max_kv_len <= 0 || max_kv_len >= 512);
+  // tiles of 32 queries: one wave along the queries, four along the keys (two such blocks
+  // share a compute unit)
+#define PS_LAUNCH_AP_SMALL(NDB)                                                                 \
+  hipLaunchKernelGGL((attention_prefill_kernel<NDB, 4, 1>), grid, dim3(256), 0, s,              \
+                     (const bf16_t*)q, q_stride, (const bf16_t*)k_pool, (const bf16_t*)v_pool,  \
+                     (bf16_t*)out, out_stride, tile_item, tile_q0, cu_tokens, kv_lens, tables,  \
+                     table_width, heads, kv_heads, page_size, page_shift, num_pages, scale, window)
+  if (query_tile != AP_QUERIES) {
+    switch (head_dim / 16) {
+      case 1: PS_LAUNCH_AP_SMALL(1); break;
+      case 2: PS_LAUNCH_AP_SMALL(2); break;
+      case 3: PS_LAUNCH_AP_SMALL(3); break;
+      case 4: PS_LAUNCH_AP_SMALL(4); break;
+      case 5: PS_LAUNCH_AP_SMALL(5); break;
+      case 6: PS_LAUNCH_AP_SMALL(6); break;
+      case 7: PS_LAUNCH_AP_SMALL(7); break;
+      default: PS_LAUNCH_AP_SMALL(8); break;
+    }
+    PS_CHECK_LAUNCH("ps_attention_prefill");
+    return 0;
+  }
+#undef PS_LAUNCH_AP_SMALL
 #define PS_LAUNCH_AP(NDB)                                                                       \
   do {                                                                                          \
     if (wide)                                                                                   \

@@ -178,16 +178,20 @@ int ps_attention_decode_static(const void* q, int64_t q_stride, const void* k_po
 // tile_item[i]; cu_tokens and kv_lens describe the step's items.  Blocks start in the order of
 // the list (all heads of tile 0, then of tile 1, ...): list the tiles that see the most keys first.
 // max_kv_len: no query sees more keys than that (0: unknown); it only steers the launch shape.
+// query_tile: the queries per tile that the list was cut for: ps_attention_prefill_query_tile(),
+// or, for head sizes up to 128, ps_attention_prefill_small_tile() (steps with so few tiles that
+// the larger ones would leave compute units without a block).
 int ps_attention_prefill(const void* q, int64_t q_stride, const void* k_pool, const void* v_pool,
                          void* out, int64_t out_stride, const int* tile_item, const int* tile_q0,
                          int tiles, const int* cu_tokens, const int* kv_lens, const int* tables,
                          int table_width, int heads, int kv_heads, int head_dim, int page_size,
-                         int num_pages, float scale, int window, int max_kv_len, int dtype,
-                         void* stream);
+                         int num_pages, float scale, int window, int max_kv_len, int query_tile,
+                         int dtype, void* stream);
 
-// The two constants of that kernel that a caller builds its index arrays by: queries per tile,
-// and the widest block table (entries per item) that it takes.
+// The constants of that kernel that a caller builds its index arrays by: queries per tile (of
+// the two sizes), and the widest block table (entries per item) that it takes.
 int ps_attention_prefill_query_tile(void);
+int ps_attention_prefill_small_tile(void);
 int ps_attention_prefill_table_max(void);
 
 // tokens[r] = argmax (inv_temperature[r] == 0) or a draw from softmax(logits * inv_temperature[r])

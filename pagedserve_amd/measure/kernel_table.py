@@ -341,6 +341,8 @@ def mixed_table(raw, decodes, context, portion, peaks, page_size=16):
     kv_lens = torch.tensor(lengths, dtype=torch.int32, device="cuda")
     single_tokens = torch.arange(decodes, dtype=torch.int32, device="cuda")
     tile = kernels.PREFILL_TILE
+    if kernels.prefill_small_tile_pays(heads, head_dim, -(-portion // tile)):
+        tile = kernels.PREFILL_SMALL_TILE   # as the attention part chooses
     starts = sorted(range(0, portion, tile), reverse=True)
     tile_item = torch.full((len(starts),), decodes, dtype=torch.int32, device="cuda")
     tile_q0 = torch.tensor(starts, dtype=torch.int32, device="cuda")
@@ -377,8 +379,8 @@ def mixed_table(raw, decodes, context, portion, peaks, page_size=16):
     if kernels.prefill_supported(dtype, head_dim, table_width):
         us = graph_time(lambda i: kernels.attention_prefill(
             q, k_pool, v_pool, context_rows, tile_item, tile_q0, cu_tokens, kv_lens, tables, heads,
-            head_dim ** -0.5, max_kv_len=max(context, portion)), 8)
-        out.append(_row("attention of the portion (tiled, causal)", us, portion * d * 2 * 4,
+            head_dim ** -0.5, max_kv_len=max(context, portion), query_tile=tile), 8)
+        out.append(_row(f"attention of the portion (tiles of {tile}, causal)", us, portion * d * 2 * 4,
                         4 * d * (portion * (portion + 1) // 2), peaks))
     product("out_proj+residual", d, d,
             lambda w, wp, bias: kernels.linear(context_rows, w, bias, h, epilogue="residual", packed=wp),

@@ -50,9 +50,14 @@ class DecoderModel:
             self.blocks.append(arrangement(width=spec.width, dtype=dtype, parts=parts))
         self.final_norm = build_part(NORMS, "norm", spec.final_norm, **common)
         # Queries of a prompt portion are handed to the mixers in tiles; each mixer says which
-        # size its kernel takes, and the step lists the tiles once per size that is asked for.
-        self.query_tiles = tuple(sorted({int(block.mixer.query_tile) for block in self.blocks
-                                         if getattr(block.mixer, "query_tile", None)}))
+        # size (or sizes) its kernel takes, and the step lists the tiles once per size that is
+        # asked for.
+        sizes = set()
+        for block in self.blocks:
+            asked = getattr(block.mixer, "query_tile", None)
+            if asked:
+                sizes.update(int(size) for size in (asked if isinstance(asked, (tuple, list)) else (asked,)))
+        self.query_tiles = tuple(sorted(sizes))
         # the mixer of the call that writes a cache entry decides what the entry holds
         self._entry_spec = {}
         for call in spec.schedule:

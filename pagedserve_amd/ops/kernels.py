@@ -42,7 +42,7 @@ _SIGNATURES = {
                                   c_void_p, c_void_p, c_int64, c_int, c_int, c_void_p],
     "ps_attention_prefill": [c_void_p, c_int64, c_void_p, c_void_p, c_void_p, c_int64, c_void_p,
                              c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int,
-                             c_int, c_int, c_int, c_float, c_int, c_int, c_int, c_void_p],
+                             c_int, c_int, c_int, c_float, c_int, c_int, c_int, c_int, c_void_p],
     "ps_sample": [c_void_p, c_int64, c_void_p, c_void_p, c_void_p, c_int, c_int, c_void_p],
 }
 
@@ -674,6 +674,7 @@ def attention_merge_linear(partial, count, heads, head_dim, splits, w, packed, b
 
 
 PREFILL_TILE = 64          # queries per block of the tiled prefill kernel
+PREFILL_SMALL_TILE = 32    # and of its variant for steps with few tiles (head sizes up to 128)
 PREFILL_TABLE_MAX = 2048   # block-table entries of an item that it keeps in LDS
 _PREFILL_CHECKED = False
 
@@ -686,13 +687,21 @@ def prefill_limits():
     return lib.ps_attention_prefill_query_tile(), lib.ps_attention_prefill_table_max()
 
 
+def prefill_small_tile():
+    """Queries per tile of the variant for few tiles, as the loaded library was built."""
+    lib = load_library()
+    lib.ps_attention_prefill_small_tile.restype = c_int
+    return lib.ps_attention_prefill_small_tile()
+
+
 def _check_prefill_constants():
     global _PREFILL_CHECKED
     if not _PREFILL_CHECKED:
-        if prefill_limits() != (PREFILL_TILE, PREFILL_TABLE_MAX):
+        built = prefill_limits() + (prefill_small_tile(),)
+        if built != (PREFILL_TILE, PREFILL_TABLE_MAX, PREFILL_SMALL_TILE):
             raise KernelError(f"attention_prefill: this module lists queries in tiles of {PREFILL_TILE} "
-                              f"and tables of up to {PREFILL_TABLE_MAX}, the library was built for "
-                              f"{prefill_limits()}; rebuild the library")
+                              f"or {PREFILL_SMALL_TILE} and tables of up to {PREFILL_TABLE_MAX}, the "
+                              f"library was built for {built}; rebuild the library")
         _PREFILL_CHECKED = True
 
 
@@ -703,10 +712,18 @@ def prefill_supported(dtype, head_dim, table_width=0) -> bool:
             and table_width <= PREFILL_TABLE_MAX)
 
 
+def prefill_small_tile_pays(heads, head_dim, tiles) -> bool:
+    """Whether ``tiles`` tiles of 64 queries of ``heads`` heads leave so many compute units
+    without a block (half of them or more) that tiles of 32 queries are the better cut: a
+    prompt portion of some hundred tokens beside decoded ones."""
+    return head_dim <= 128 and 2 * heads * tiles <= compute_units()
+
+
 def attention_prefill(q, k_pool, v_pool, out, tile_item, tile_q0, cu_tokens, kv_lens, tables,
-                      heads, scale, window=0, max_kv_len=0):
-    """Attention of items with several tokens, 64 queries per block, on the matrix cores.
-    Blocks start in the order of the tile list: the tiles that see the most keys belong first.
+                      heads, scale, window=0, max_kv_len=0, query_tile=PREFILL_TILE):
+    """Attention of items with several tokens, ``query_tile`` (64 or 32) queries per block, on
+    the matrix cores.  Blocks start in the order of the tile list, which is cut for that size:
+    the tiles that see the most keys belong first.
     ``max_kv_len`` (no query sees more keys; 0 = unknown) only steers the launch shape."""
     _check_prefill_constants()
     _check(q, "q", torch.bfloat16, 2)
@@ -731,7 +748,7 @@ def attention_prefill(q, k_pool, v_pool, out, tile_item, tile_q0, cu_tokens, kv_
           out.data_ptr(), out_stride, tile_item.data_ptr(), tile_q0.data_ptr(), tiles,
           cu_tokens.data_ptr(), kv_lens.data_ptr(), tables.data_ptr(), tables.shape[1], heads,
           kv_heads, head_dim, page_size, pages, float(scale), int(window), int(max_kv_len),
-          dtype_code(q.dtype), _stream())
+          int(query_tile), dtype_code(q.dtype), _stream())
     return out
 
 

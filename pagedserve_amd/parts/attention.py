@@ -25,9 +25,9 @@ class Attention(Mixer):
 
     accepts_pending_norm = True
 
-    # the step's index arrays list the queries of a prompt portion in tiles of this size (the
-    # tiled kernel's; ``kernels.attention_prefill`` checks it against the library's)
-    query_tile = kernels.PREFILL_TILE
+    # the step's index arrays list the queries of a prompt portion in tiles of these sizes (the
+    # tiled kernel's two; ``kernels.attention_prefill`` checks them against the library's)
+    query_tile = (kernels.PREFILL_TILE, kernels.PREFILL_SMALL_TILE)
 
     def __init__(self, width: int, dtype, heads: int, kv_heads: int, head_dim: int, scale: float,
                  window: int = 0, bias: bool = True):
@@ -139,11 +139,15 @@ class Attention(Mixer):
                                      tok_list=None if singles == tokens else ctx.single_tokens)
         whole = singles == 0
         if singles < tokens and kernels.prefill_supported(self.dtype, self.head_dim, tables.shape[1]):
-            tile_item, tile_q0 = ctx.query_tiles[self.query_tile]
+            size = kernels.PREFILL_TILE
+            tile_item, tile_q0 = ctx.query_tiles[size]
+            if kernels.prefill_small_tile_pays(self.heads, self.head_dim, tile_item.numel()):
+                size = kernels.PREFILL_SMALL_TILE
+                tile_item, tile_q0 = ctx.query_tiles[size]
             kernels.attention_prefill(q, cache.k_pool, cache.v_pool, context, tile_item,
                                       tile_q0, ctx.cu_tokens, ctx.kv_lens, tables,
                                       self.heads, self.scale, self.window,
-                                      max_kv_len=ctx.max_kv_len)
+                                      max_kv_len=ctx.max_kv_len, query_tile=size)
         elif singles < tokens:
             kernels.attention_rowwise(q, cache.k_pool, cache.v_pool, context, ctx.tok_item,
                                       ctx.positions, tables, self.heads, self.scale, self.window,

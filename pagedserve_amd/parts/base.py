@@ -268,8 +268,8 @@ class StepContext:
     single_tokens: Optional[torch.Tensor] = None   # int32: step indices of one-token items
     portion_tokens: Optional[torch.Tensor] = None  # int32: step indices of all other tokens
     max_positions: int = 0
-    # For every tile size that a mixer asked for (``Mixer.query_tile``): the queries of the
-    # items with several tokens, cut into tiles of that many.  size -> (int32 item of each tile,
+    # For every tile size that a mixer asked for (``Mixer.query_tile``, one size or several):
+    # the queries of the items with several tokens, cut into tiles of that many.  size -> (int32 item of each tile,
     # int32 first query of the tile within its item), the tiles that see the most keys first.
     query_tiles: Optional[Dict[int, tuple]] = None
     token_src: Optional[torch.Tensor] = None       # int32 [T]: >= 0: the token is carried_tokens[src]

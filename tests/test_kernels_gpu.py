@@ -531,9 +531,11 @@ def test_kernels_refuse_bad_sizes():
                                                                 # head sizes beyond 128: blocks of four waves only
                                                                 (2, 1, 256, 16), (3, 3, 192, 8), (2, 2, 144, 12), (12, 4, 160, 16), (1, 1, 208, 16)])
 @pytest.mark.parametrize("window", [0, 37])
-def test_attention_prefill_tiles(heads, kv_heads, head_dim, page_size, window):
+@pytest.mark.parametrize("tile", [64, 32])
+def test_attention_prefill_tiles(heads, kv_heads, head_dim, page_size, window, tile):
     """The tiled kernel against float64 attention over the gathered pages (every head size in
-    steps of 16 up to 128 in both arrangements of waves, larger ones in the one they have: the
+    steps of 16 up to 128 in both arrangements of waves and with tiles of 32 queries, larger
+    ones in the one arrangement they have, and refused with the small tiles: the
     kernel reads LDS by assembly into registers that the compiler must leave alone until the
     wait, which a run of every variant checks): fresh prompts and later portions of many
     lengths in one launch (1 < count, portions that start inside a page, more than one tile,
@@ -557,7 +559,7 @@ def test_attention_prefill_tiles(heads, kv_heads, head_dim, page_size, window):
         tok_item += [index] * new
         tok_pos += list(range(past, past + new))
         cu.append(cu[-1] + new)
-        for q0 in range(0, new, 64):
+        for q0 in range(0, new, tile):
             tile_item.append(index)
             tile_q0.append(q0)
 
@@ -565,15 +567,21 @@ def test_attention_prefill_tiles(heads, kv_heads, head_dim, page_size, window):
         return torch.tensor(values, dtype=torch.int32, device="cuda")
 
     scale = head_dim ** -0.5
-    expected = _attention_expected(q, k_pool, v_pool, tables, tok_item, tok_pos, heads, scale, window)
     out = torch.full_like(q, float("nan"))
+    if tile != kernels.PREFILL_TILE and head_dim > 128:
+        with pytest.raises(kernels.KernelError, match="head sizes up to 128"):
+            kernels.attention_prefill(q, k_pool, v_pool, out, dev(tile_item), dev(tile_q0), dev(cu),
+                                      dev(totals), tables, heads, scale, window=window, query_tile=tile)
+        return
+    expected = _attention_expected(q, k_pool, v_pool, tables, tok_item, tok_pos, heads, scale, window)
     kernels.attention_prefill(q, k_pool, v_pool, out, dev(tile_item), dev(tile_q0), dev(cu), dev(totals),
-                              tables, heads, scale, window=window)
+                              tables, heads, scale, window=window, query_tile=tile)
     assert torch.isfinite(out.float()).all()
     torch.testing.assert_close(out.double(), expected, atol=5e-3, rtol=5e-3)
 
 
-def test_attention_prefill_far_key_and_causality():
+@pytest.mark.parametrize("tile", [64, 32])
+def test_attention_prefill_far_key_and_causality(tile):
     """One early key is made to dominate for late queries only if they may see it; the query
     just before it must not feel it (a mask off by one would)."""
     from pagedserve_amd.ops import kernels
@@ -593,8 +601,10 @@ def test_attention_prefill_far_key_and_causality():
     def dev(values):
         return torch.tensor(values, dtype=torch.int32, device="cuda")
 
-    kernels.attention_prefill(q, k_pool, v_pool, out, dev([0, 0, 0, 0, 0]), dev([0, 64, 128, 192, 256]),
-                              dev([0, total]), dev([total]), tables, heads, head_dim ** -0.5)
+    starts = list(range(0, total, tile))
+    kernels.attention_prefill(q, k_pool, v_pool, out, dev([0] * len(starts)), dev(starts),
+                              dev([0, total]), dev([total]), tables, heads, head_dim ** -0.5,
+                              query_tile=tile)
     value = v_pool[page, 0, target % page_size].float()
     for row in (137, 138, 299):
         torch.testing.assert_close(out[row].float(), value, atol=5e-3, rtol=5e-3)
@@ -1061,6 +1071,7 @@ def test_the_tile_that_the_step_lists_is_the_kernels_own():
     from pagedserve_amd.ops import kernels
 
     assert kernels.prefill_limits() == (kernels.PREFILL_TILE, kernels.PREFILL_TABLE_MAX)
+    assert kernels.prefill_small_tile() == kernels.PREFILL_SMALL_TILE
 
 
 def test_linear_memo_of_a_call_site():
