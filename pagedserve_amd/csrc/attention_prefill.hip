@@ -1,10 +1,13 @@
 // Tiled paged attention for prompt portions on the matrix cores (bfloat16).
 //
-// One block per (tile of 32 QW queries of one request, head), QW = 2 or 1.  Its QW KS waves are
-// arranged as QW x KS: a wave owns 32 consecutive queries and every KS-th run of 32 keys, with
-// an online-softmax state of its own; the KS states of a query are merged through LDS at the
-// end.  (Tiles of 32 queries are for steps whose tiles of 64 would leave half of the compute
-// units without a block: a prompt portion beside decoded tokens.)
+// One block per (tile of 32 QW queries of one request, head), QW = 2, 1 or 4.  Its QW KS waves
+// are arranged as QW x KS: a wave owns 32 consecutive queries and, of every tile of keys, KR
+// runs of 32 keys, with an online-softmax state of its own; the KS states of a query are merged
+// through LDS at the end.  (Tiles of 32 queries are for steps whose tiles of 64 would leave
+// half of the compute units without a block: a prompt portion beside decoded tokens.  Tiles of
+// 128 queries, four waves that each take all 64 keys of a tile, are for long prompts: what
+// bounds the tiles of 64 there is what a compute unit takes in, 16 KB of keys and values per
+// 4,096 scores, and what a wave does per tile beside the scores; both are halved.)
 // A request's longest tile decides how long the launch takes, and splitting its keys over
 // waves shortens exactly that.  Keys and values are visited 32 KS at a time through the
 // request's block table, from the first key any query of the tile may see to the tile's last
@@ -41,8 +44,9 @@ typedef __attribute__((__vector_size__(16 * sizeof(float)))) float f32x16;
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
 
-#define AP_QUERIES 64      // queries per block (32 with QW = 1)
+#define AP_QUERIES 64      // queries per block (32 with QW = 1, 128 with QW = 4)
 #define AP_TABLE_MAX 2048  // block-table entries that a tile may need
+#define AP_LARGE_HEAD_DIM 64   // largest head size of the blocks of 128 queries
 
 typedef const __attribute__((address_space(1))) void* ap_global_ptr;
 typedef __attribute__((address_space(3))) void* ap_lds_ptr;
@@ -52,7 +56,8 @@ __device__ inline void ap_wait_loads_and_sync() {
   asm volatile("s_waitcnt vmcnt(%0)\n\ts_barrier" ::"n"(PENDING) : "memory");
 }
 
-template <int NDB, int KS, int QW = 2>  // head_dim / 16; waves along the keys; waves along the queries
+// head_dim / 16; waves along the keys; waves along the queries; runs of 32 keys per wave and tile
+template <int NDB, int KS, int QW = 2, int KR = 1>
 __global__ __launch_bounds__(64 * QW * KS) void attention_prefill_kernel(
     const bf16_t* __restrict__ q, int64_t q_stride, const bf16_t* __restrict__ k_pool,
     const bf16_t* __restrict__ v_pool, bf16_t* __restrict__ out, int64_t out_stride,
@@ -64,23 +69,25 @@ __global__ __launch_bounds__(64 * QW * KS) void attention_prefill_kernel(
   constexpr int ROW = HD * 2;                    // bytes of one key in a tile
   constexpr int CH = HD / 8;                     // 16-byte pieces per row
   constexpr int SPREAD = ROW <= 256 ? 256 / ROW : 1;   // keys that share one pass over the banks
-  constexpr int AP_KEYS = 32 * KS;               // keys per tile
+  constexpr int WAVE_KEYS = 32 * KR;             // keys of a wave per tile
+  constexpr int AP_KEYS = WAVE_KEYS * KS;        // keys per tile
   constexpr int AP_WAVES = QW * KS;
   constexpr int QUERIES = 32 * QW;               // queries per block
-  static_assert(QW == 1 || QW == 2, "one or two waves along the queries");
+  static_assert(QW == 1 || QW == 2 || QW == 4, "one, two or four waves along the queries");
+  static_assert(KR == 1 || KR == 2, "one or two runs of keys per wave");
   constexpr int TILE_BYTES = AP_KEYS * ROW;
   constexpr int STAGE_BYTES = 2 * TILE_BYTES;    // K tile, then V tile
   // The ring may take 96 KB; with four waves along the keys 64 KB, so that two such blocks
   // share a compute unit: the grids that take them have up to three blocks for two units, and
   // with one block per unit a third of them would wait for a second round (2 x 1,024 tokens of
   // 12 heads: 1.5 us less per launch).
-  constexpr int FIT = (KS >= 4 && QW == 2 ? 65536 : 98304) / STAGE_BYTES;
+  constexpr int FIT = ((KS >= 4 && QW == 2) || QW == 4 ? 65536 : 98304) / STAGE_BYTES;
   constexpr int STAGES = FIT >= 4 ? 4 : (FIT >= 2 ? FIT : 2);
   static_assert(NDB <= 8 || STAGES == 2, "head sizes beyond 128 rely on a ring of two stages");
-  constexpr int INSTRUCTIONS = KS * NDB;         // load instructions per operand and stage
+  constexpr int INSTRUCTIONS = KS * KR * NDB;    // load instructions per operand and stage
   // every wave issues the same number of loads (the counter of loads in flight is per wave):
   // where they do not divide evenly the last ones are issued twice
-  constexpr int PER_OPERAND = (NDB + QW - 1) / QW;
+  constexpr int PER_OPERAND = (INSTRUCTIONS + AP_WAVES - 1) / AP_WAVES;
   constexpr int LOADS = 2 * PER_OPERAND;
   constexpr int NDB32 = (NDB + 1) / 2;           // blocks of 32 head dimensions
   static_assert(LOADS * 2 < 64, "the load counter has six bits");
@@ -88,11 +95,11 @@ __global__ __launch_bounds__(64 * QW * KS) void attention_prefill_kernel(
   constexpr int MERGE_BYTES = (AP_WAVES - QW) * 64 * (NDB32 * 16 + 2) * 4;
   constexpr int LDS_BYTES = STAGES * STAGE_BYTES > MERGE_BYTES ? STAGES * STAGE_BYTES : MERGE_BYTES;
   __shared__ __attribute__((aligned(1024))) unsigned char stages[LDS_BYTES];
-  __shared__ int s_table[AP_TABLE_MAX];
+  __shared__ uint32_t s_table[AP_TABLE_MAX];
 
   const int tid = threadIdx.x;
   const int lane = tid & 63;
-  const int wave = tid >> 6;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);   // the same in every lane: scalar
   const int wave_q = wave % QW;  // which 32 queries
   const int wave_k = wave / QW;  // which run of 32 keys of every tile
   const int sub = lane & 31;     // query of this lane within the wave; key or dimension row
@@ -125,10 +132,16 @@ __global__ __launch_bounds__(64 * QW * KS) void attention_prefill_kernel(
   // the block-table entries of keys key_begin .. key_end - 1
   const int first_logical = page_shift >= 0 ? (key_begin >> page_shift) : key_begin / page_size;
   const int last_logical = page_shift >= 0 ? ((key_end - 1) >> page_shift) : (key_end - 1) / page_size;
+  // kept as the number of the page's first key row of this head within the pool (a row: one
+  // key's HD values; the host checks that the pool has fewer than 2^32 of them), so that a
+  // load's address is one multiplication away
+  const uint32_t page_rows = (uint32_t)kv_heads * (uint32_t)page_size;
+  const uint32_t head_rows = (uint32_t)kv_head * (uint32_t)page_size;
   for (int i = tid; i <= last_logical - first_logical && i < AP_TABLE_MAX; i += 64 * QW * KS) {
     const int logical = first_logical + i;
-    const int page = logical < table_width ? table[logical] : 0;
-    s_table[i] = (page >= 0 && page < num_pages) ? page : 0;   // never an address outside the pool
+    int page = logical < table_width ? table[logical] : 0;
+    page = (page >= 0 && page < num_pages) ? page : 0;         // never an address outside the pool
+    s_table[i] = (uint32_t)page * page_rows + head_rows;
   }
 
   // queries as column operand of the first product: lane (query sub, dims step*16 + half*8 ..)
@@ -156,23 +169,30 @@ __global__ __launch_bounds__(64 * QW * KS) void attention_prefill_kernel(
     load_key[j] = key_local;
     load_piece[j] = (slot + CH - (key_local / SPREAD) % CH) % CH;
   }
-  const int head_offset = kv_head * page_size * HD;   // inside a page: fits an int
-  const int64_t page_elems = (int64_t)kv_heads * page_size * HD;
-  int load_fixed[PER_OPERAND];
-#pragma unroll
-  for (int j = 0; j < PER_OPERAND; ++j) load_fixed[j] = head_offset + load_piece[j] * 8;
+  const int page_mask = page_size - 1;                // where the page size is a power of two
   auto issue = [&](int tile_number, int k0) {
     unsigned char* stage = stages + (tile_number % STAGES) * STAGE_BYTES;
+    // the rows first (their table entries are then on their way together), then the loads
+    uint32_t row[PER_OPERAND];
 #pragma unroll
     for (int j = 0; j < PER_OPERAND; ++j) {
       // keys outside the tile's visible range are fetched from a visible key instead: they
       // are masked below, and whatever lies in pages that were given back is never read
       int key = k0 + load_key[j];
       key = key < key_begin ? key_begin : (key >= key_end ? key_end - 1 : key);
-      const int logical = page_shift >= 0 ? (key >> page_shift) : key / page_size;
-      const int page = s_table[logical - first_logical];
-      const int64_t offset =
-          (int64_t)page * page_elems + (load_fixed[j] + (key - logical * page_size) * HD);
+      int logical, within;
+      if (page_shift >= 0) {
+        logical = key >> page_shift;
+        within = key & page_mask;
+      } else {
+        logical = key / page_size;
+        within = key - logical * page_size;
+      }
+      row[j] = s_table[logical - first_logical] + (uint32_t)within;
+    }
+#pragma unroll
+    for (int j = 0; j < PER_OPERAND; ++j) {
+      const uint64_t offset = (uint64_t)row[j] * (uint32_t)HD + (uint32_t)(load_piece[j] * 8);
       const int number = wave * PER_OPERAND + j < INSTRUCTIONS ? wave * PER_OPERAND + j : INSTRUCTIONS - 1;
       const int dst = number * 1024;
       __builtin_amdgcn_global_load_lds((ap_global_ptr)(k_pool + offset), (ap_lds_ptr)(stage + dst),
@@ -193,25 +213,28 @@ __global__ __launch_bounds__(64 * QW * KS) void attention_prefill_kernel(
     for (int e = 0; e < 16; ++e) acc[db][e] = 0.f;
 
   // ---- operand addresses inside a tile
-  // K row operand: lane (key sub, half) reads piece 2*step + half of key wave_k*32 + sub
-  int k_off[NDB];
-  {
-    const int key_local = wave_k * 32 + sub;
+  // K row operand: lane (key sub, half) reads piece 2*step + half of key sub of each of the
+  // wave's runs of 32 keys
+  int k_off[KR][NDB];
+#pragma unroll
+  for (int r = 0; r < KR; ++r) {
+    const int key_local = wave_k * WAVE_KEYS + r * 32 + sub;
     const int turn = (key_local / SPREAD) % CH;
 #pragma unroll
     for (int step = 0; step < NDB; ++step)
-      k_off[step] = key_local * ROW + ((2 * step + half + turn) % CH) * 16;
+      k_off[r][step] = key_local * ROW + ((2 * step + half + turn) % CH) * 16;
   }
   // V row operand through the transposing read: in the 16 lanes of group g = lane / 16, lane r
   // points at dimensions d0 + 4 (r % 4) .. + 3 of key base + half*4 + r / 4 (+ 8 for the second
   // read) and receives dimension d0 + r of four keys, d0 = db*32 + (g & 1) * 16.
-  int v_off[2][NDB32][2];
+  // (a run of 32 keys is two instructions' worth of 16)
+  int v_off[2 * KR][NDB32][2];
   {
     const int r16 = lane & 15;
-    const int v_dim = ((lane >> 4) & 1) * 16 + 4 * (r16 & 3);   // within the block of 32 dims
-    const int v_key = wave_k * 32 + half * 4 + (r16 >> 2);       // first run of 16 keys of the wave
+    const int v_dim = ((lane >> 4) & 1) * 16 + 4 * (r16 & 3);        // within the block of 32 dims
+    const int v_key = wave_k * WAVE_KEYS + half * 4 + (r16 >> 2);     // first 16 keys of the wave
 #pragma unroll
-    for (int run = 0; run < 2; ++run)
+    for (int run = 0; run < 2 * KR; ++run)
 #pragma unroll
       for (int db = 0; db < NDB32; ++db) {
         int dim = db * 32 + v_dim;
@@ -245,24 +268,26 @@ __global__ __launch_bounds__(64 * QW * KS) void attention_prefill_kernel(
     // the stage that the tile before this one lay in is free since the barrier: the tile that
     // is STAGES - 1 ahead is asked for at once
     if (t + STAGES - 1 < tiles) issue(t + STAGES - 1, k0 + (STAGES - 1) * AP_KEYS);
-    // this wave's run of 32 keys; it is skipped where no query of the wave can see it
-    const int kw = k0 + wave_k * 32;
+    // this wave's keys of the tile; they are skipped where no query of the wave can see them
+    const int kw = k0 + wave_k * WAVE_KEYS;
     const bool active = wave_active && kw <= wave_last && kw < key_end &&
-                        !(window > 0 && kw + 31 < wave_first - window + 1);
+                        !(window > 0 && kw + WAVE_KEYS - 1 < wave_first - window + 1);
     // S^T: element e is key (e/4)*8 + half*4 + e%4 of the run.  The operand reads are written
     // as assembly: the compiler would otherwise wait for every tile in flight before each.
     // The transposing reads of V are issued right behind them.
     const uint32_t stage_base =
         (uint32_t)(uintptr_t)(ap_lds_ptr)stages + (uint32_t)((t % STAGES) * STAGE_BYTES);
-    u32x4 kr[NDB];
-    u32x2 vr[2][NDB32][2];
+    u32x4 kr[KR][NDB];
+    u32x2 vr[2 * KR][NDB32][2];
     if (active) {
       if constexpr (NDB <= 8) {
 #pragma unroll
-        for (int step = 0; step < NDB; ++step)
-          asm volatile("ds_read_b128 %0, %1" : "=v"(kr[step]) : "v"(stage_base + k_off[step]) : "memory");
+        for (int r = 0; r < KR; ++r)
 #pragma unroll
-        for (int run = 0; run < 2; ++run)
+          for (int step = 0; step < NDB; ++step)
+            asm volatile("ds_read_b128 %0, %1" : "=v"(kr[r][step]) : "v"(stage_base + k_off[r][step]) : "memory");
+#pragma unroll
+        for (int run = 0; run < 2 * KR; ++run)
 #pragma unroll
           for (int db = 0; db < NDB32; ++db)
 #pragma unroll
@@ -279,11 +304,13 @@ __global__ __launch_bounds__(64 * QW * KS) void attention_prefill_kernel(
         // which costs nothing with a ring of two stages: none is in flight at this point).
         typedef short ap_i16x4 __attribute__((ext_vector_type(4)));
 #pragma unroll
-        for (int step = 0; step < NDB; ++step)
-          kr[step] = *reinterpret_cast<const __attribute__((address_space(3))) u32x4*>(
-              (uintptr_t)(stage_base + k_off[step]));
+        for (int r = 0; r < KR; ++r)
 #pragma unroll
-        for (int run = 0; run < 2; ++run)
+          for (int step = 0; step < NDB; ++step)
+            kr[r][step] = *reinterpret_cast<const __attribute__((address_space(3))) u32x4*>(
+                (uintptr_t)(stage_base + k_off[r][step]));
+#pragma unroll
+        for (int run = 0; run < 2 * KR; ++run)
 #pragma unroll
           for (int db = 0; db < NDB32; ++db)
 #pragma unroll
@@ -298,34 +325,41 @@ __global__ __launch_bounds__(64 * QW * KS) void attention_prefill_kernel(
     // Everything read by assembly is waited for before the compiler's own code goes on (it
     // does not know that those registers are still on their way).
     asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
-    f32x16 s;
+    f32x16 s[KR];
     if (active) {
 #pragma unroll
-      for (int e = 0; e < 16; ++e) s[e] = 0.f;
+      for (int r = 0; r < KR; ++r) {
 #pragma unroll
-      for (int step = 0; step < NDB; ++step) {
-        asm volatile("" : "+v"(kr[step]));   // used only behind the wait
-        s = __builtin_amdgcn_mfma_f32_32x32x16_bf16(*reinterpret_cast<const bf16x8*>(&kr[step]),
-                                                  qf[step], s, 0, 0, 0);
+        for (int e = 0; e < 16; ++e) s[r][e] = 0.f;
+#pragma unroll
+        for (int step = 0; step < NDB; ++step) {
+          asm volatile("" : "+v"(kr[r][step]));   // used only behind the wait
+          s[r] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(*reinterpret_cast<const bf16x8*>(&kr[r][step]),
+                                                       qf[step], s[r], 0, 0, 0);
+        }
       }
     }
     if (!active) continue;
-    // the whole run is visible to every query of the wave: no mask
-    const bool masked = kw + 31 > wave_first || kw + 32 > key_end ||
+    // all of these keys are visible to every query of the wave: no mask
+    const bool masked = kw + WAVE_KEYS - 1 > wave_first || kw + WAVE_KEYS > key_end ||
                         (window > 0 && kw < wave_last - window + 1) || !q_valid;
     // scores stay unscaled until the exponential: p = 2^(s c - m), with m kept in scaled units
     float tile_max = -INFINITY;
     if (__builtin_amdgcn_readfirstlane(__any(masked) ? 1 : 0)) {
 #pragma unroll
-      for (int e = 0; e < 16; ++e) {
-        const int key = kw + (e >> 2) * 8 + half * 4 + (e & 3);
-        const bool visible = (key <= q_pos) & (window <= 0 || q_pos - key < window);
-        s[e] = visible ? s[e] : -INFINITY;
-        tile_max = fmaxf(tile_max, s[e]);
-      }
+      for (int r = 0; r < KR; ++r)
+#pragma unroll
+        for (int e = 0; e < 16; ++e) {
+          const int key = kw + r * 32 + (e >> 2) * 8 + half * 4 + (e & 3);
+          const bool visible = (key <= q_pos) & (window <= 0 || q_pos - key < window);
+          s[r][e] = visible ? s[r][e] : -INFINITY;
+          tile_max = fmaxf(tile_max, s[r][e]);
+        }
     } else {
 #pragma unroll
-      for (int e = 0; e < 16; ++e) tile_max = fmaxf(tile_max, s[e]);
+      for (int r = 0; r < KR; ++r)
+#pragma unroll
+        for (int e = 0; e < 16; ++e) tile_max = fmaxf(tile_max, s[r][e]);
     }
     tile_max = halves_max(tile_max) * scale_log2;   // scale > 0
     const float m_new = fmaxf(m, tile_max);
@@ -334,16 +368,20 @@ __global__ __launch_bounds__(64 * QW * KS) void attention_prefill_kernel(
     // products below run in any case.
     const float reference = (m_new == -INFINITY) ? 0.f : m_new;
     float tile_sum = 0.f;
-    uint32_t words[8];
+    u32x4 p[2 * KR];      // per 16 keys
 #pragma unroll
-    for (int e = 0; e < 16; e += 2) {
-      const float p0 = __builtin_amdgcn_exp2f(fmaf(s[e], scale_log2, -reference));
-      const float p1 = __builtin_amdgcn_exp2f(fmaf(s[e + 1], scale_log2, -reference));
-      tile_sum += p0 + p1;
-      words[e >> 1] = pack2_bf16(p0, p1);
+    for (int r = 0; r < KR; ++r) {
+      uint32_t words[8];
+#pragma unroll
+      for (int e = 0; e < 16; e += 2) {
+        const float p0 = __builtin_amdgcn_exp2f(fmaf(s[r][e], scale_log2, -reference));
+        const float p1 = __builtin_amdgcn_exp2f(fmaf(s[r][e + 1], scale_log2, -reference));
+        tile_sum += p0 + p1;
+        words[e >> 1] = pack2_bf16(p0, p1);
+      }
+      p[2 * r] = u32x4{words[0], words[1], words[2], words[3]};
+      p[2 * r + 1] = u32x4{words[4], words[5], words[6], words[7]};
     }
-    const u32x4 p_lo = {words[0], words[1], words[2], words[3]};
-    const u32x4 p_hi = {words[4], words[5], words[6], words[7]};
     tile_sum = halves_sum(tile_sum);
     // the running maximum rarely moves after the first tiles: rescale only where it did
     if (__builtin_amdgcn_readfirstlane(__any(m_new != m) ? 1 : 0)) {
@@ -360,14 +398,14 @@ __global__ __launch_bounds__(64 * QW * KS) void attention_prefill_kernel(
     // O^T += V^T P^T, 16 keys per instruction: slots 0..3 are keys base + half*4 + 0..3,
     // slots 4..7 keys base + 8 + half*4 + 0..3, in both operands
 #pragma unroll
-    for (int run = 0; run < 2; ++run)
+    for (int run = 0; run < 2 * KR; ++run)
 #pragma unroll
       for (int db = 0; db < NDB32; ++db) {
         asm volatile("" : "+v"(vr[run][db][0]), "+v"(vr[run][db][1]));   // used only behind the wait
         const u32x4 raw = {vr[run][db][0].x, vr[run][db][0].y, vr[run][db][1].x, vr[run][db][1].y};
         acc[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(
-            *reinterpret_cast<const bf16x8*>(&raw),
-            *reinterpret_cast<const bf16x8*>(run == 0 ? &p_lo : &p_hi), acc[db], 0, 0, 0);
+            *reinterpret_cast<const bf16x8*>(&raw), *reinterpret_cast<const bf16x8*>(&p[run]),
+            acc[db], 0, 0, 0);
       }
   }
 
@@ -428,6 +466,8 @@ __global__ __launch_bounds__(64 * QW * KS) void attention_prefill_kernel(
 // What the host has to know of this file's constants to list a step's tiles.
 extern "C" int ps_attention_prefill_query_tile(void) { return AP_QUERIES; }
 extern "C" int ps_attention_prefill_small_tile(void) { return AP_QUERIES / 2; }
+extern "C" int ps_attention_prefill_large_tile(void) { return AP_QUERIES * 2; }
+extern "C" int ps_attention_prefill_large_tile_head_dim(void) { return AP_LARGE_HEAD_DIM; }
 extern "C" int ps_attention_prefill_table_max(void) { return AP_TABLE_MAX; }
 
 extern "C" int ps_attention_prefill(const void* q, int64_t q_stride, const void* k_pool,
@@ -446,9 +486,13 @@ extern "C" int ps_attention_prefill(const void* q, int64_t q_stride, const void*
   PS_REQUIRE(head_dim > 0 && head_dim % 16 == 0 && head_dim <= 256,
              "ps_attention_prefill: head_dim %d must be a multiple of 16 up to 256", head_dim);
   PS_REQUIRE(window >= 0 && tiles <= 65535, "ps_attention_prefill: bad window or too many tiles (%d)", tiles);
-  PS_REQUIRE(query_tile == AP_QUERIES || (query_tile == AP_QUERIES / 2 && head_dim <= 128),
-             "ps_attention_prefill: tiles of %d or (head sizes up to 128) %d queries, not %d", AP_QUERIES,
-             AP_QUERIES / 2, query_tile);
+  PS_REQUIRE(query_tile == AP_QUERIES || (query_tile == AP_QUERIES / 2 && head_dim <= 128) ||
+                 (query_tile == AP_QUERIES * 2 && head_dim <= AP_LARGE_HEAD_DIM),
+             "ps_attention_prefill: tiles of %d, (head sizes up to 128) %d or (head sizes up to %d) %d "
+             "queries, not %d", AP_QUERIES, AP_QUERIES / 2, AP_LARGE_HEAD_DIM, AP_QUERIES * 2, query_tile);
+  PS_REQUIRE((int64_t)num_pages * kv_heads * page_size < ((int64_t)1 << 32),
+             "ps_attention_prefill: a pool of %d pages x %d heads x %d keys has 2^32 key rows or more",
+             num_pages, kv_heads, page_size);
   PS_REQUIRE(scale > 0.f, "ps_attention_prefill: the score scale must be positive, got %g", scale);
   PS_REQUIRE(table_width <= AP_TABLE_MAX,
              "ps_attention_prefill: block tables of %d pages exceed the %d that a tile keeps",
@@ -477,6 +521,26 @@ extern "C" int ps_attention_prefill(const void* q, int64_t q_stride, const void*
                      (const bf16_t*)q, q_stride, (const bf16_t*)k_pool, (const bf16_t*)v_pool,  \
                      (bf16_t*)out, out_stride, tile_item, tile_q0, cu_tokens, kv_lens, tables,  \
                      table_width, heads, kv_heads, page_size, page_shift, num_pages, scale, window)
+  // tiles of 128 queries: four waves along the queries, each with all 64 keys of a tile: a
+  // block takes in half as many keys and values per score, and a wave's work per tile that
+  // does not depend on the scores (addresses, waits, checks) is spread over twice as many
+#define PS_LAUNCH_AP_LARGE_TILE(NDB)                                                            \
+  hipLaunchKernelGGL((attention_prefill_kernel<NDB, 1, 4, 2>), grid, dim3(256), 0, s,           \
+                     (const bf16_t*)q, q_stride, (const bf16_t*)k_pool, (const bf16_t*)v_pool,  \
+                     (bf16_t*)out, out_stride, tile_item, tile_q0, cu_tokens, kv_lens, tables,  \
+                     table_width, heads, kv_heads, page_size, page_shift, num_pages, scale, window)
+  if (query_tile == AP_QUERIES * 2) {
+    static_assert(AP_LARGE_HEAD_DIM == 64, "the cases below");
+    switch (head_dim / 16) {
+      case 1: PS_LAUNCH_AP_LARGE_TILE(1); break;
+      case 2: PS_LAUNCH_AP_LARGE_TILE(2); break;
+      case 3: PS_LAUNCH_AP_LARGE_TILE(3); break;
+      default: PS_LAUNCH_AP_LARGE_TILE(4); break;
+    }
+    PS_CHECK_LAUNCH("ps_attention_prefill");
+    return 0;
+  }
+#undef PS_LAUNCH_AP_LARGE_TILE
   if (query_tile != AP_QUERIES) {
     switch (head_dim / 16) {
       case 1: PS_LAUNCH_AP_SMALL(1); break;

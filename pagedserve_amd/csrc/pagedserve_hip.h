@@ -180,7 +180,9 @@ int ps_attention_decode_static(const void* q, int64_t q_stride, const void* k_po
 // max_kv_len: no query sees more keys than that (0: unknown); it only steers the launch shape.
 // query_tile: the queries per tile that the list was cut for: ps_attention_prefill_query_tile(),
 // or, for head sizes up to 128, ps_attention_prefill_small_tile() (steps with so few tiles that
-// the larger ones would leave compute units without a block).
+// the larger ones would leave compute units without a block), or, for head sizes up to
+// ps_attention_prefill_large_tile_head_dim(), ps_attention_prefill_large_tile() (long prompts:
+// a block then takes in half as many keys and values per score).
 int ps_attention_prefill(const void* q, int64_t q_stride, const void* k_pool, const void* v_pool,
                          void* out, int64_t out_stride, const int* tile_item, const int* tile_q0,
                          int tiles, const int* cu_tokens, const int* kv_lens, const int* tables,
@@ -192,6 +194,8 @@ int ps_attention_prefill(const void* q, int64_t q_stride, const void* k_pool, co
 // the two sizes), and the widest block table (entries per item) that it takes.
 int ps_attention_prefill_query_tile(void);
 int ps_attention_prefill_small_tile(void);
+int ps_attention_prefill_large_tile(void);
+int ps_attention_prefill_large_tile_head_dim(void);
 int ps_attention_prefill_table_max(void);
 
 // tokens[r] = argmax (inv_temperature[r] == 0) or a draw from softmax(logits * inv_temperature[r])

@@ -259,6 +259,8 @@ def prefill_table(raw, prompts, length, peaks, page_size=16, only=None):
     cu_tokens = torch.arange(prompts + 1, dtype=torch.int32, device="cuda") * length
     kv_lens = torch.full((prompts,), length, dtype=torch.int32, device="cuda")
     tile = kernels.PREFILL_TILE
+    if kernels.prefill_large_tile_pays(heads, head_dim, prompts * -(-length // kernels.PREFILL_LARGE_TILE)):
+        tile = kernels.PREFILL_LARGE_TILE   # as the attention part chooses
     starts = list(range(0, length, tile))
     order = sorted(((item, q0) for item in range(prompts) for q0 in starts), key=lambda t: -t[1])
     tile_item = torch.tensor([t[0] for t in order], dtype=torch.int32, device="cuda")
@@ -292,9 +294,9 @@ def prefill_table(raw, prompts, length, peaks, page_size=16, only=None):
         q = qkv[:, :d]
         us = graph_time(lambda i: kernels.attention_prefill(
             q, k_pool, v_pool, context_rows, tile_item, tile_q0, cu_tokens, kv_lens, tables, heads,
-            head_dim ** -0.5, max_kv_len=length), 8)
+            head_dim ** -0.5, max_kv_len=length, query_tile=tile), 8)
         flops = prompts * 4 * d * (length * (length + 1) // 2)
-        out.append(_row("attention (tiled, causal)", us, rows * d * 2 * 4, flops, peaks))
+        out.append(_row(f"attention (tiles of {tile}, causal)", us, rows * d * 2 * 4, flops, peaks))
     product("out_proj+residual", d, d,
             lambda w, wp, bias: kernels.linear(context_rows, w, bias, h, epilogue="residual", packed=wp),
             22, extra_bytes=rows * d * (2 + 8))

@@ -675,6 +675,8 @@ def attention_merge_linear(partial, count, heads, head_dim, splits, w, packed, b
 
 PREFILL_TILE = 64          # queries per block of the tiled prefill kernel
 PREFILL_SMALL_TILE = 32    # and of its variant for steps with few tiles (head sizes up to 128)
+PREFILL_LARGE_TILE = 128   # and of its variant for long prompts (head sizes up to 64)
+PREFILL_LARGE_TILE_HEAD_DIM = 64
 PREFILL_TABLE_MAX = 2048   # block-table entries of an item that it keeps in LDS
 _PREFILL_CHECKED = False
 
@@ -694,14 +696,25 @@ def prefill_small_tile():
     return lib.ps_attention_prefill_small_tile()
 
 
+def prefill_large_tile():
+    """(queries per tile, largest head size) of the variant for long prompts, as the loaded
+    library was built."""
+    lib = load_library()
+    lib.ps_attention_prefill_large_tile.restype = c_int
+    lib.ps_attention_prefill_large_tile_head_dim.restype = c_int
+    return lib.ps_attention_prefill_large_tile(), lib.ps_attention_prefill_large_tile_head_dim()
+
+
 def _check_prefill_constants():
     global _PREFILL_CHECKED
     if not _PREFILL_CHECKED:
-        built = prefill_limits() + (prefill_small_tile(),)
-        if built != (PREFILL_TILE, PREFILL_TABLE_MAX, PREFILL_SMALL_TILE):
-            raise KernelError(f"attention_prefill: this module lists queries in tiles of {PREFILL_TILE} "
-                              f"or {PREFILL_SMALL_TILE} and tables of up to {PREFILL_TABLE_MAX}, the "
-                              f"library was built for {built}; rebuild the library")
+        built = prefill_limits() + (prefill_small_tile(),) + prefill_large_tile()
+        if built != (PREFILL_TILE, PREFILL_TABLE_MAX, PREFILL_SMALL_TILE, PREFILL_LARGE_TILE,
+                     PREFILL_LARGE_TILE_HEAD_DIM):
+            raise KernelError(f"attention_prefill: this module lists queries in tiles of {PREFILL_TILE}, "
+                              f"{PREFILL_SMALL_TILE} or {PREFILL_LARGE_TILE} (head sizes up to "
+                              f"{PREFILL_LARGE_TILE_HEAD_DIM}) and tables of up to {PREFILL_TABLE_MAX}, "
+                              f"the library was built for {built}; rebuild the library")
         _PREFILL_CHECKED = True
 
 
@@ -719,10 +732,19 @@ def prefill_small_tile_pays(heads, head_dim, tiles) -> bool:
     return head_dim <= 128 and 2 * heads * tiles <= compute_units()
 
 
+def prefill_large_tile_pays(heads, head_dim, large_tiles) -> bool:
+    """Whether ``large_tiles`` tiles of 128 queries of ``heads`` heads are the better cut: from
+    three blocks per compute unit on (two are resident at a time), measured: 2 x 4,096 tokens of
+    12 heads, 768 blocks, 90 against 118 us; 4 x 1,024 of 25 heads, 800 blocks, 36 against 45;
+    4 x 1,024 of 16 heads, 512 blocks, level; 2 x 2,048 of 12 heads, 384 blocks, 46 against 37:
+    with fewer blocks the one that sees the most keys decides, and it is longer."""
+    return head_dim <= PREFILL_LARGE_TILE_HEAD_DIM and heads * large_tiles >= 3 * compute_units()
+
+
 def attention_prefill(q, k_pool, v_pool, out, tile_item, tile_q0, cu_tokens, kv_lens, tables,
                       heads, scale, window=0, max_kv_len=0, query_tile=PREFILL_TILE):
-    """Attention of items with several tokens, ``query_tile`` (64 or 32) queries per block, on
-    the matrix cores.  Blocks start in the order of the tile list, which is cut for that size:
+    """Attention of items with several tokens, ``query_tile`` (64, 32 or 128) queries per block,
+    on the matrix cores.  Blocks start in the order of the tile list, which is cut for that size:
     the tiles that see the most keys belong first.
     ``max_kv_len`` (no query sees more keys; 0 = unknown) only steers the launch shape."""
     _check_prefill_constants()

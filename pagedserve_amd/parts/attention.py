@@ -26,8 +26,8 @@ class Attention(Mixer):
     accepts_pending_norm = True
 
     # the step's index arrays list the queries of a prompt portion in tiles of these sizes (the
-    # tiled kernel's two; ``kernels.attention_prefill`` checks them against the library's)
-    query_tile = (kernels.PREFILL_TILE, kernels.PREFILL_SMALL_TILE)
+    # tiled kernel's three; ``kernels.attention_prefill`` checks them against the library's)
+    query_tile = (kernels.PREFILL_TILE, kernels.PREFILL_SMALL_TILE, kernels.PREFILL_LARGE_TILE)
 
     def __init__(self, width: int, dtype, heads: int, kv_heads: int, head_dim: int, scale: float,
                  window: int = 0, bias: bool = True):
@@ -143,6 +143,10 @@ class Attention(Mixer):
             tile_item, tile_q0 = ctx.query_tiles[size]
             if kernels.prefill_small_tile_pays(self.heads, self.head_dim, tile_item.numel()):
                 size = kernels.PREFILL_SMALL_TILE
+                tile_item, tile_q0 = ctx.query_tiles[size]
+            elif kernels.prefill_large_tile_pays(self.heads, self.head_dim,
+                                                 ctx.query_tiles[kernels.PREFILL_LARGE_TILE][0].numel()):
+                size = kernels.PREFILL_LARGE_TILE
                 tile_item, tile_q0 = ctx.query_tiles[size]
             kernels.attention_prefill(q, cache.k_pool, cache.v_pool, context, tile_item,
                                       tile_q0, ctx.cu_tokens, ctx.kv_lens, tables,

@@ -531,11 +531,12 @@ def test_kernels_refuse_bad_sizes():
                                                                 # head sizes beyond 128: blocks of four waves only
                                                                 (2, 1, 256, 16), (3, 3, 192, 8), (2, 2, 144, 12), (12, 4, 160, 16), (1, 1, 208, 16)])
 @pytest.mark.parametrize("window", [0, 37])
-@pytest.mark.parametrize("tile", [64, 32])
+@pytest.mark.parametrize("tile", [64, 32, 128])
 def test_attention_prefill_tiles(heads, kv_heads, head_dim, page_size, window, tile):
     """The tiled kernel against float64 attention over the gathered pages (every head size in
-    steps of 16 up to 128 in both arrangements of waves and with tiles of 32 queries, larger
-    ones in the one arrangement they have, and refused with the small tiles: the
+    steps of 16 up to 128 in both arrangements of waves and with tiles of 32 queries, up to 64
+    also with tiles of 128, larger ones in the one arrangement they have, and refused with
+    the other tiles: the
     kernel reads LDS by assembly into registers that the compiler must leave alone until the
     wait, which a run of every variant checks): fresh prompts and later portions of many
     lengths in one launch (1 < count, portions that start inside a page, more than one tile,
@@ -568,8 +569,9 @@ def test_attention_prefill_tiles(heads, kv_heads, head_dim, page_size, window, t
 
     scale = head_dim ** -0.5
     out = torch.full_like(q, float("nan"))
-    if tile != kernels.PREFILL_TILE and head_dim > 128:
-        with pytest.raises(kernels.KernelError, match="head sizes up to 128"):
+    if tile != kernels.PREFILL_TILE and head_dim > (128 if tile == kernels.PREFILL_SMALL_TILE
+                                                     else kernels.PREFILL_LARGE_TILE_HEAD_DIM):
+        with pytest.raises(kernels.KernelError, match="head sizes up to"):
             kernels.attention_prefill(q, k_pool, v_pool, out, dev(tile_item), dev(tile_q0), dev(cu),
                                       dev(totals), tables, heads, scale, window=window, query_tile=tile)
         return
@@ -580,7 +582,7 @@ def test_attention_prefill_tiles(heads, kv_heads, head_dim, page_size, window, t
     torch.testing.assert_close(out.double(), expected, atol=5e-3, rtol=5e-3)
 
 
-@pytest.mark.parametrize("tile", [64, 32])
+@pytest.mark.parametrize("tile", [64, 32, 128])
 def test_attention_prefill_far_key_and_causality(tile):
     """One early key is made to dominate for late queries only if they may see it; the query
     just before it must not feel it (a mask off by one would)."""
@@ -1072,6 +1074,7 @@ def test_the_tile_that_the_step_lists_is_the_kernels_own():
 
     assert kernels.prefill_limits() == (kernels.PREFILL_TILE, kernels.PREFILL_TABLE_MAX)
     assert kernels.prefill_small_tile() == kernels.PREFILL_SMALL_TILE
+    assert kernels.prefill_large_tile() == (kernels.PREFILL_LARGE_TILE, kernels.PREFILL_LARGE_TILE_HEAD_DIM)
 
 
 def test_linear_memo_of_a_call_site():

@@ -617,7 +617,7 @@ def test_mixers_may_ask_for_query_tiles_of_different_sizes(tmp_path):
     spec = dataclasses.replace(base, blocks=(base.blocks[0],
                                              base.blocks[1].with_part("mixer", PartSpec.make("toy_tiles"))))
     model = DecoderModel(spec, torch.bfloat16, "cuda")
-    assert model.query_tiles == (24, kernels.PREFILL_SMALL_TILE, kernels.PREFILL_TILE)
+    assert model.query_tiles == (24, kernels.PREFILL_SMALL_TILE, kernels.PREFILL_TILE, kernels.PREFILL_LARGE_TILE)
     from pagedserve_amd.weights import load_parameters
 
     sources = {k: v for k, v in arch.weight_sources(typed, base).items()
