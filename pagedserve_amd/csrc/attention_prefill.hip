@@ -322,9 +322,12 @@ __global__ __launch_bounds__(64 * QW * KS) void attention_prefill_kernel(
             }
       }
     }
-    // Everything read by assembly is waited for before the compiler's own code goes on (it
-    // does not know that those registers are still on their way).
-    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+    // The compiler does not know that the registers read by assembly are still on their way:
+    // it touches them only behind the statements that name them again, each of which stands
+    // behind a wait.  Reads come back in the order of issue: here the keys have arrived, the
+    // values may still be in flight while the scores are made and weighed.
+    constexpr int V_READS = 4 * NDB32 * KR;
+    asm volatile("s_waitcnt lgkmcnt(%0)" ::"n"(NDB <= 8 ? (V_READS < 15 ? V_READS : 15) : 0) : "memory");
     f32x16 s[KR];
     if (active) {
 #pragma unroll
@@ -397,6 +400,7 @@ __global__ __launch_bounds__(64 * QW * KS) void attention_prefill_kernel(
 
     // O^T += V^T P^T, 16 keys per instruction: slots 0..3 are keys base + half*4 + 0..3,
     // slots 4..7 keys base + 8 + half*4 + 0..3, in both operands
+    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");   // the values have arrived
 #pragma unroll
     for (int run = 0; run < 2 * KR; ++run)
 #pragma unroll
