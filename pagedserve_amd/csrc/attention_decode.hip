@@ -118,7 +118,7 @@ __global__ __launch_bounds__(64 * AD_WAVES) void attention_decode_kernel(
   const int t = tok_list ? tok_list[n] : n;
   const int kv_head = head / (heads / kv_heads);
   const int lane = threadIdx.x & 63;
-  const int wave = threadIdx.x >> 6;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);   // the same in every lane: scalar
   const int group = lane / LPK;
   const int dim0 = (lane % LPK) * 8;
   const bool has_dims = dim0 < head_dim;

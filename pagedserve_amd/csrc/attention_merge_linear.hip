@@ -40,7 +40,7 @@ __global__ __launch_bounds__(64 * GROUP) void attention_merge_linear_kernel(
   constexpr int HEAD_DIM = STEPS * 64;
   constexpr int STRIDE = HEAD_DIM + 2;
   const int lane = threadIdx.x & 63;
-  const int wave = threadIdx.x >> 6;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);   // the same in every lane: scalar
   const int column = lane & 15;        // column of the matrix-core operand: a row of the step
   const int group = lane >> 4;         // which 16 of every 64 head dimensions
   // (a wave beyond the last head works on a copy of the last head and adds nothing)

@@ -76,7 +76,7 @@ __global__ __launch_bounds__(256) void gemm_nt_tiled_kernel(
 
   const int tid = threadIdx.x;
   const int lane = tid & 63;
-  const int wave = tid >> 6;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);   // the same in every lane: scalar
   const int wave_m = wave >> 1;
   const int wave_n = wave & 1;
   // Consecutive block ids run on different XCDs, each with an L2 of its own.  Blocks are
@@ -320,7 +320,7 @@ __global__ __launch_bounds__(64 * SK_WAVES) void gemm_nt_skinny_kernel(
   // as the weights themselves.
   __shared__ float partial[NT][SK_WAVES][MB][4][64];
   const int lane = threadIdx.x & 63;
-  const int wave = threadIdx.x >> 6;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);   // the same in every lane: scalar
   const int n0 = blockIdx.x * 16 * NT;
   const int split = blockIdx.y;
   const int row0 = blockIdx.z * (MB * 16);

@@ -66,7 +66,7 @@ __global__ __launch_bounds__(256) void gemm_nt_bf16_tiled_kernel(
 
   const int tid = threadIdx.x;
   const int lane = tid & 63;
-  const int wave = tid >> 6;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);   // the same in every lane: scalar
   const int wave_m = wave >> 1;
   const int wave_n = KW == 1 ? wave & 1 : 0;
   const int wave_k = KW == 1 ? 0 : wave & 1;     // which tile of a pair of k tiles

@@ -60,7 +60,7 @@ __global__ __launch_bounds__(256) void gemm_nt_bf16_wide_kernel(
 
   const int tid = threadIdx.x;
   const int lane = tid & 63;
-  const int wave = tid >> 6;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);   // the same in every lane: scalar
   // every XCD works on a contiguous run of tiles (see gemm_tiled_bf16.hip)
   const int blocks = gridDim.x;
   const int per_xcd = blocks / 8;
