@@ -28,7 +28,7 @@ One JSON line is printed:
   roofline, prompt tokens a second.
 
     python bench.py --workload medium|small_stream|xl     one workload alone, one JSON line
-    python bench.py --prefill-only --steps K               the prefill step alone (for profiles)
+    python bench.py --prefill-only --steps K [--prefill-length L]   the prefill step of 2 x L tokens alone (for profiles)
     python bench.py --kernels [--shape small|medium|xl|all] [--only name,name]
 
 ``--kernels`` times every kernel of a decode step (1, 8 and 64 requests over 1,024 keys), of
@@ -537,6 +537,9 @@ def main(argv=None):
                         help="skip the medium, small-stream and XL workloads and the 32-bit and long points")
     parser.add_argument("--prefill-only", action="store_true",
                         help="only the 2,048-token prefill step, --steps times (for profiles)")
+    parser.add_argument("--prefill-length", type=int, default=PREFILL_TOKENS // 2,
+                        help="--prefill-only: tokens of each of the two prompts (beyond the small shape's "
+                             "positions the configuration of points_long is used)")
     parser.add_argument("--workload", choices=("small", "medium", "small_stream", "xl"), default="small",
                         help="small: the whole record (default); medium / small_stream: the streams at "
                              "GPT-2 medium / small shape alone; xl: 64 x (768 + 256) at GPT-2 XL shape alone")
@@ -577,17 +580,22 @@ def main(argv=None):
         return 0
     short = "bf16" if args.dtype == "bfloat16" else "fp32"
     element = 2 if args.dtype == "bfloat16" else 4
-    engine, sampler, config = _build(args.dtype, max_requests=64, max_step_tokens=PREFILL_TOKENS,
-                                     layers=args.layers)
-    context = config.n_positions
     if args.prefill_only:
-        seconds = prefill_run(engine, config, reps=args.steps, warmup=max(min(args.warmup, 8), 5))
-        flops = step_flops(config, [PREFILL_TOKENS // 2] * 2, 2)
+        length = args.prefill_length
+        long = 2 * length > PREFILL_TOKENS
+        engine, sampler, config = _build(args.dtype, max_requests=64, max_step_tokens=max(PREFILL_TOKENS, 2 * length),
+                                         layers=args.layers, shape=LONG if long else SMALL)
+        seconds = prefill_run(engine, config, reps=args.steps, warmup=max(min(args.warmup, 8), 5),
+                              prompts=2, length=length)
+        flops = step_flops(config, [length] * 2, 2)
         print(json.dumps({"prefill": {
-            "value": round(PREFILL_TOKENS / seconds, 1), "tokens": PREFILL_TOKENS,
+            "value": round(2 * length / seconds, 1), "tokens": 2 * length,
             "ms": round(seconds * 1e3, 4),
             "frac": round(flops / seconds / (PEAK_TFLOPS[short] * 1e12), 4)}}), flush=True)
         return 0
+    engine, sampler, config = _build(args.dtype, max_requests=64, max_step_tokens=PREFILL_TOKENS,
+                                     layers=args.layers)
+    context = config.n_positions
     elapsed, mean_context = decode_run(engine, sampler, config, args.batch, context, args.steps,
                                        args.warmup)
     ms_per_step = elapsed / args.steps * 1e3
