@@ -58,3 +58,23 @@ def test_documented_cases(monkeypatch):
     assert _part(25)._merged_splits(4, 400) == 4
     # a window bounds the keys that a query sees
     assert _part(12, window=256)._splits(32, 8192) == (1, 4)
+
+
+def test_query_tiles_of_the_prefill_attention(monkeypatch):
+    """Which of the tiled kernel's three tile sizes a step takes: 32 queries while tiles of 64
+    leave half of the compute units without a block, 128 from three blocks per unit on (head
+    sizes up to 64), 64 otherwise; never both of the special ones."""
+    monkeypatch.setattr(kernels, "compute_units", lambda: 256)
+    small, large = kernels.prefill_small_tile_pays, kernels.prefill_large_tile_pays
+    # a portion of 512 tokens beside decoded ones: 8 tiles of 64, 4 of 128
+    assert small(12, 64, 8) and small(16, 64, 8) and not small(25, 64, 8)
+    assert not large(12, 64, 4) and not large(25, 64, 4)
+    # the prefill step of 2 x 1,024 tokens stays with tiles of 64 at every GPT-2 shape
+    for heads in (12, 16, 25):
+        assert not small(heads, 64, 32) and not large(heads, 64, 16)
+    # long prompts
+    assert large(12, 64, 64) and large(25, 64, 32) and large(16, 64, 48) and not large(16, 64, 47)
+    assert not large(12, 128, 64) and not large(12, 80, 640) and not small(1, 144, 1)
+    for heads in (1, 3, 12, 25, 64):
+        for tiles in range(1, 400):
+            assert not (small(heads, 64, tiles) and large(heads, 64, -(-tiles // 2)))
