@@ -397,11 +397,13 @@ def xl_workload(args):
                                      layers=args.layers, shape=XL)
     scheduler = ContinuousBatchScheduler(engine, sampler, max_batch_size=64, eos_token_id=None)
     generator = torch.Generator().manual_seed(0)
-    for _ in range(2):
-        scheduler.add_token_request(_random_prompt(generator, 80, config.vocab_size), 4,
+    prompt_len, output_len, batch = 768, 256, 64
+    # (untimed: a few requests of the same shape, among them one whole prefill step, so that
+    # every kernel that the measurement launches has been loaded once)
+    for _ in range(7):
+        scheduler.add_token_request(_random_prompt(generator, prompt_len, config.vocab_size), 4,
                                     sampling=SamplingParams(max_new_tokens=4, temperature=0.8, seed=7, ignore_eos=True))
     scheduler.run_until_complete()
-    prompt_len, output_len, batch = 768, 256, 64
     for _ in range(batch):
         scheduler.add_token_request(
             _random_prompt(generator, prompt_len, config.vocab_size), output_len,

@@ -81,7 +81,7 @@ __global__ __launch_bounds__(64 * QW * KS) void attention_prefill_kernel(
   // share a compute unit: the grids that take them have up to three blocks for two units, and
   // with one block per unit a third of them would wait for a second round (2 x 1,024 tokens of
   // 12 heads: 1.5 us less per launch).
-  constexpr int FIT = ((KS >= 4 && QW == 2) || QW == 4 ? 65536 : 98304) / STAGE_BYTES;
+  constexpr int FIT = (KS == 2 && QW == 2 && NDB <= 4 ? 32768 : ((KS >= 4 && QW == 2) || QW == 4 ? 65536 : 98304)) / STAGE_BYTES;
   constexpr int STAGES = FIT >= 4 ? 4 : (FIT >= 2 ? FIT : 2);
   static_assert(NDB <= 8 || STAGES == 2, "head sizes beyond 128 rely on a ring of two stages");
   constexpr int INSTRUCTIONS = KS * KR * NDB;    // load instructions per operand and stage
@@ -259,6 +259,126 @@ __global__ __launch_bounds__(64 * QW * KS) void attention_prefill_kernel(
   for (int d = 0; d < STAGES - 1; ++d)
     if (d < tiles) issue(d, k_first + d * AP_KEYS);
 
+  // ---- the parts of an iteration
+  typedef u32x4 KeyRegs[KR][NDB];
+  typedef u32x2 ValueRegs[2 * KR][NDB32][2];
+  constexpr int V_READS = 4 * NDB32 * KR;
+  auto wave_keys = [&](int t) { return k_first + t * AP_KEYS + wave_k * WAVE_KEYS; };
+  // a wave's keys of a tile are skipped where no query of the wave can see them
+  auto sees = [&](int kw) {
+    return wave_active && kw <= wave_last && kw < key_end &&
+           !(window > 0 && kw + WAVE_KEYS - 1 < wave_first - window + 1);
+  };
+  auto stage_of = [&](int t) {
+    return (uint32_t)(uintptr_t)(ap_lds_ptr)stages + (uint32_t)((t % STAGES) * STAGE_BYTES);
+  };
+  // S^T: element e is key (e/4)*8 + half*4 + e%4 of the run.  The operand reads are written
+  // as assembly: the compiler would otherwise wait for every tile in flight before each.
+  auto read_keys = [&](uint32_t stage_base, KeyRegs& kr) {
+#pragma unroll
+    for (int r = 0; r < KR; ++r)
+#pragma unroll
+      for (int step = 0; step < NDB; ++step)
+        asm volatile("ds_read_b128 %0, %1" : "=v"(kr[r][step]) : "v"(stage_base + k_off[r][step]) : "memory");
+  };
+  auto read_values = [&](uint32_t stage_base, ValueRegs& vr) {
+#pragma unroll
+    for (int run = 0; run < 2 * KR; ++run)
+#pragma unroll
+      for (int db = 0; db < NDB32; ++db)
+#pragma unroll
+        for (int second = 0; second < 2; ++second)
+          asm volatile("ds_read_b64_tr_b16 %0, %1"
+                       : "=v"(vr[run][db][second])
+                       : "v"(stage_base + v_off[run][db][second])
+                       : "memory");
+  };
+  auto scores = [&](KeyRegs& kr, f32x16 (&s)[KR]) {
+#pragma unroll
+    for (int r = 0; r < KR; ++r) {
+#pragma unroll
+      for (int e = 0; e < 16; ++e) s[r][e] = 0.f;
+#pragma unroll
+      for (int step = 0; step < NDB; ++step) {
+        asm volatile("" : "+v"(kr[r][step]));   // used only behind the wait
+        s[r] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(*reinterpret_cast<const bf16x8*>(&kr[r][step]),
+                                                     qf[step], s[r], 0, 0, 0);
+      }
+    }
+  };
+  // softmax of a wave's scores of one tile and the second product (the values' reads may
+  // still be in flight when it starts)
+  auto weigh = [&](const int kw, f32x16 (&s)[KR], ValueRegs& vr) {
+    // all of these keys are visible to every query of the wave: no mask
+      const bool masked = kw + WAVE_KEYS - 1 > wave_first || kw + WAVE_KEYS > key_end ||
+                          (window > 0 && kw < wave_last - window + 1) || !q_valid;
+      // scores stay unscaled until the exponential: p = 2^(s c - m), with m kept in scaled units
+      float tile_max = -INFINITY;
+      if (__builtin_amdgcn_readfirstlane(__any(masked) ? 1 : 0)) {
+#pragma unroll
+        for (int r = 0; r < KR; ++r)
+#pragma unroll
+          for (int e = 0; e < 16; ++e) {
+            const int key = kw + r * 32 + (e >> 2) * 8 + half * 4 + (e & 3);
+            const bool visible = (key <= q_pos) & (window <= 0 || q_pos - key < window);
+            s[r][e] = visible ? s[r][e] : -INFINITY;
+            tile_max = fmaxf(tile_max, s[r][e]);
+          }
+      } else {
+#pragma unroll
+        for (int r = 0; r < KR; ++r)
+#pragma unroll
+          for (int e = 0; e < 16; ++e) tile_max = fmaxf(tile_max, s[r][e]);
+      }
+      tile_max = halves_max(tile_max) * scale_log2;   // scale > 0
+      const float m_new = fmaxf(m, tile_max);
+      // A query that has seen nothing yet (m_new = -inf) takes 0 as its reference: its scores
+      // are all -inf and their exponentials 0.  Other lanes of the wave may differ, so the
+      // products below run in any case.
+      const float reference = (m_new == -INFINITY) ? 0.f : m_new;
+      float tile_sum = 0.f;
+      u32x4 p[2 * KR];      // per 16 keys
+#pragma unroll
+      for (int r = 0; r < KR; ++r) {
+        uint32_t words[8];
+#pragma unroll
+        for (int e = 0; e < 16; e += 2) {
+          const float p0 = __builtin_amdgcn_exp2f(fmaf(s[r][e], scale_log2, -reference));
+          const float p1 = __builtin_amdgcn_exp2f(fmaf(s[r][e + 1], scale_log2, -reference));
+          tile_sum += p0 + p1;
+          words[e >> 1] = pack2_bf16(p0, p1);
+        }
+        p[2 * r] = u32x4{words[0], words[1], words[2], words[3]};
+        p[2 * r + 1] = u32x4{words[4], words[5], words[6], words[7]};
+      }
+      tile_sum = halves_sum(tile_sum);
+      // the running maximum rarely moves after the first tiles: rescale only where it did
+      if (__builtin_amdgcn_readfirstlane(__any(m_new != m) ? 1 : 0)) {
+        const float correction = (m == -INFINITY) ? 0.f : __builtin_amdgcn_exp2f(m - reference);
+        l *= correction;
+#pragma unroll
+        for (int db = 0; db < NDB32; ++db)
+#pragma unroll
+          for (int e = 0; e < 16; ++e) acc[db][e] *= correction;
+        m = m_new;
+      }
+      l += tile_sum;
+
+      // O^T += V^T P^T, 16 keys per instruction: slots 0..3 are keys base + half*4 + 0..3,
+      // slots 4..7 keys base + 8 + half*4 + 0..3, in both operands
+      asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");   // the values have arrived
+#pragma unroll
+      for (int run = 0; run < 2 * KR; ++run)
+#pragma unroll
+        for (int db = 0; db < NDB32; ++db) {
+          asm volatile("" : "+v"(vr[run][db][0]), "+v"(vr[run][db][1]));   // used only behind the wait
+          const u32x4 raw = {vr[run][db][0].x, vr[run][db][0].y, vr[run][db][1].x, vr[run][db][1].y};
+          acc[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(
+              *reinterpret_cast<const bf16x8*>(&raw), *reinterpret_cast<const bf16x8*>(&p[run]),
+              acc[db], 0, 0, 0);
+        }
+  };
+
   for (int t = 0; t < tiles; ++t) {
     const int k0 = k_first + t * AP_KEYS;
     const int ahead = tiles - 1 - t < STAGES - 2 ? tiles - 1 - t : STAGES - 2;
@@ -268,149 +388,49 @@ __global__ __launch_bounds__(64 * QW * KS) void attention_prefill_kernel(
     // the stage that the tile before this one lay in is free since the barrier: the tile that
     // is STAGES - 1 ahead is asked for at once
     if (t + STAGES - 1 < tiles) issue(t + STAGES - 1, k0 + (STAGES - 1) * AP_KEYS);
-    // this wave's keys of the tile; they are skipped where no query of the wave can see them
-    const int kw = k0 + wave_k * WAVE_KEYS;
-    const bool active = wave_active && kw <= wave_last && kw < key_end &&
-                        !(window > 0 && kw + WAVE_KEYS - 1 < wave_first - window + 1);
-    // S^T: element e is key (e/4)*8 + half*4 + e%4 of the run.  The operand reads are written
-    // as assembly: the compiler would otherwise wait for every tile in flight before each.
-    // The transposing reads of V are issued right behind them.
-    const uint32_t stage_base =
-        (uint32_t)(uintptr_t)(ap_lds_ptr)stages + (uint32_t)((t % STAGES) * STAGE_BYTES);
-    u32x4 kr[KR][NDB];
-    u32x2 vr[2 * KR][NDB32][2];
-    if (active) {
-      if constexpr (NDB <= 8) {
-#pragma unroll
-        for (int r = 0; r < KR; ++r)
-#pragma unroll
-          for (int step = 0; step < NDB; ++step)
-            asm volatile("ds_read_b128 %0, %1" : "=v"(kr[r][step]) : "v"(stage_base + k_off[r][step]) : "memory");
-#pragma unroll
-        for (int run = 0; run < 2 * KR; ++run)
-#pragma unroll
-          for (int db = 0; db < NDB32; ++db)
-#pragma unroll
-            for (int second = 0; second < 2; ++second)
-              asm volatile("ds_read_b64_tr_b16 %0, %1"
-                           : "=v"(vr[run][db][second])
-                           : "v"(stage_base + v_off[run][db][second])
-                           : "memory");
-      } else {
-        // Head sizes beyond 128 need more registers than a wave's 256 vector registers: the
-        // compiler then moves values to the accumulation registers where it sees fit, also a
-        // register that an assembly read above has not yet filled.  Here the reads are the
-        // compiler's own (it waits for them itself, and for every load in flight before them,
-        // which costs nothing with a ring of two stages: none is in flight at this point).
-        typedef short ap_i16x4 __attribute__((ext_vector_type(4)));
-#pragma unroll
-        for (int r = 0; r < KR; ++r)
-#pragma unroll
-          for (int step = 0; step < NDB; ++step)
-            kr[r][step] = *reinterpret_cast<const __attribute__((address_space(3))) u32x4*>(
-                (uintptr_t)(stage_base + k_off[r][step]));
-#pragma unroll
-        for (int run = 0; run < 2 * KR; ++run)
-#pragma unroll
-          for (int db = 0; db < NDB32; ++db)
-#pragma unroll
-            for (int second = 0; second < 2; ++second) {
-              const ap_i16x4 raw = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
-                  reinterpret_cast<__attribute__((address_space(3))) ap_i16x4*>(
-                      (uintptr_t)(stage_base + v_off[run][db][second])));
-              vr[run][db][second] = *reinterpret_cast<const u32x2*>(&raw);
-            }
-      }
-    }
-    // The compiler does not know that the registers read by assembly are still on their way:
-    // it touches them only behind the statements that name them again, each of which stands
-    // behind a wait.  Reads come back in the order of issue: here the keys have arrived, the
-    // values may still be in flight while the scores are made and weighed.
-    constexpr int V_READS = 4 * NDB32 * KR;
-    asm volatile("s_waitcnt lgkmcnt(%0)" ::"n"(NDB <= 8 ? (V_READS < 15 ? V_READS : 15) : 0) : "memory");
-    f32x16 s[KR];
-    if (active) {
-#pragma unroll
-      for (int r = 0; r < KR; ++r) {
-#pragma unroll
-        for (int e = 0; e < 16; ++e) s[r][e] = 0.f;
-#pragma unroll
-        for (int step = 0; step < NDB; ++step) {
-          asm volatile("" : "+v"(kr[r][step]));   // used only behind the wait
-          s[r] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(*reinterpret_cast<const bf16x8*>(&kr[r][step]),
-                                                       qf[step], s[r], 0, 0, 0);
-        }
-      }
-    }
-    if (!active) continue;
-    // all of these keys are visible to every query of the wave: no mask
-    const bool masked = kw + WAVE_KEYS - 1 > wave_first || kw + WAVE_KEYS > key_end ||
-                        (window > 0 && kw < wave_last - window + 1) || !q_valid;
-    // scores stay unscaled until the exponential: p = 2^(s c - m), with m kept in scaled units
-    float tile_max = -INFINITY;
-    if (__builtin_amdgcn_readfirstlane(__any(masked) ? 1 : 0)) {
-#pragma unroll
-      for (int r = 0; r < KR; ++r)
-#pragma unroll
-        for (int e = 0; e < 16; ++e) {
-          const int key = kw + r * 32 + (e >> 2) * 8 + half * 4 + (e & 3);
-          const bool visible = (key <= q_pos) & (window <= 0 || q_pos - key < window);
-          s[r][e] = visible ? s[r][e] : -INFINITY;
-          tile_max = fmaxf(tile_max, s[r][e]);
-        }
+    const int kw = wave_keys(t);
+    if (!sees(kw)) continue;
+    const uint32_t stage_base = stage_of(t);
+    KeyRegs kr;
+    ValueRegs vr;
+    if constexpr (NDB <= 8) {
+      // the transposing reads of V are issued right behind the keys'
+      read_keys(stage_base, kr);
+      read_values(stage_base, vr);
+      // The compiler does not know that the registers read by assembly are still on their
+      // way: it touches them only behind the statements that name them again, each of which
+      // stands behind a wait on the same straight path.  Reads come back in the order of
+      // issue: here the keys have arrived, the values may still be in flight while the scores
+      // are made and weighed.
+      asm volatile("s_waitcnt lgkmcnt(%0)" ::"n"(V_READS < 15 ? V_READS : 15) : "memory");
     } else {
+      // Head sizes beyond 128 need more registers than a wave's 256 vector registers: the
+      // compiler then moves values to the accumulation registers where it sees fit, also a
+      // register that an assembly read above has not yet filled.  Here the reads are the
+      // compiler's own (it waits for them itself, and for every load in flight before them,
+      // which costs nothing with a ring of two stages: none is in flight at this point).
+      typedef short ap_i16x4 __attribute__((ext_vector_type(4)));
 #pragma unroll
       for (int r = 0; r < KR; ++r)
 #pragma unroll
-        for (int e = 0; e < 16; ++e) tile_max = fmaxf(tile_max, s[r][e]);
+        for (int step = 0; step < NDB; ++step)
+          kr[r][step] = *reinterpret_cast<const __attribute__((address_space(3))) u32x4*>(
+              (uintptr_t)(stage_base + k_off[r][step]));
+#pragma unroll
+      for (int run = 0; run < 2 * KR; ++run)
+#pragma unroll
+        for (int db = 0; db < NDB32; ++db)
+#pragma unroll
+          for (int second = 0; second < 2; ++second) {
+            const ap_i16x4 raw = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
+                reinterpret_cast<__attribute__((address_space(3))) ap_i16x4*>(
+                    (uintptr_t)(stage_base + v_off[run][db][second])));
+            vr[run][db][second] = *reinterpret_cast<const u32x2*>(&raw);
+          }
     }
-    tile_max = halves_max(tile_max) * scale_log2;   // scale > 0
-    const float m_new = fmaxf(m, tile_max);
-    // A query that has seen nothing yet (m_new = -inf) takes 0 as its reference: its scores
-    // are all -inf and their exponentials 0.  Other lanes of the wave may differ, so the
-    // products below run in any case.
-    const float reference = (m_new == -INFINITY) ? 0.f : m_new;
-    float tile_sum = 0.f;
-    u32x4 p[2 * KR];      // per 16 keys
-#pragma unroll
-    for (int r = 0; r < KR; ++r) {
-      uint32_t words[8];
-#pragma unroll
-      for (int e = 0; e < 16; e += 2) {
-        const float p0 = __builtin_amdgcn_exp2f(fmaf(s[r][e], scale_log2, -reference));
-        const float p1 = __builtin_amdgcn_exp2f(fmaf(s[r][e + 1], scale_log2, -reference));
-        tile_sum += p0 + p1;
-        words[e >> 1] = pack2_bf16(p0, p1);
-      }
-      p[2 * r] = u32x4{words[0], words[1], words[2], words[3]};
-      p[2 * r + 1] = u32x4{words[4], words[5], words[6], words[7]};
-    }
-    tile_sum = halves_sum(tile_sum);
-    // the running maximum rarely moves after the first tiles: rescale only where it did
-    if (__builtin_amdgcn_readfirstlane(__any(m_new != m) ? 1 : 0)) {
-      const float correction = (m == -INFINITY) ? 0.f : __builtin_amdgcn_exp2f(m - reference);
-      l *= correction;
-#pragma unroll
-      for (int db = 0; db < NDB32; ++db)
-#pragma unroll
-        for (int e = 0; e < 16; ++e) acc[db][e] *= correction;
-      m = m_new;
-    }
-    l += tile_sum;
-
-    // O^T += V^T P^T, 16 keys per instruction: slots 0..3 are keys base + half*4 + 0..3,
-    // slots 4..7 keys base + 8 + half*4 + 0..3, in both operands
-    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");   // the values have arrived
-#pragma unroll
-    for (int run = 0; run < 2 * KR; ++run)
-#pragma unroll
-      for (int db = 0; db < NDB32; ++db) {
-        asm volatile("" : "+v"(vr[run][db][0]), "+v"(vr[run][db][1]));   // used only behind the wait
-        const u32x4 raw = {vr[run][db][0].x, vr[run][db][0].y, vr[run][db][1].x, vr[run][db][1].y};
-        acc[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(
-            *reinterpret_cast<const bf16x8*>(&raw), *reinterpret_cast<const bf16x8*>(&p[run]),
-            acc[db], 0, 0, 0);
-      }
+    f32x16 s[KR];
+    scores(kr, s);
+    weigh(kw, s, vr);
   }
 
   // ---- the KS states of a query are merged by the wave with the first run of keys.  The

@@ -259,7 +259,7 @@ def prefill_table(raw, prompts, length, peaks, page_size=16, only=None):
     cu_tokens = torch.arange(prompts + 1, dtype=torch.int32, device="cuda") * length
     kv_lens = torch.full((prompts,), length, dtype=torch.int32, device="cuda")
     tile = kernels.PREFILL_TILE
-    if kernels.prefill_large_tile_pays(heads, head_dim, prompts * -(-length // kernels.PREFILL_LARGE_TILE)):
+    if kernels.prefill_large_tile_pays(heads, head_dim, prompts * -(-length // kernels.PREFILL_LARGE_TILE), length):
         tile = kernels.PREFILL_LARGE_TILE   # as the attention part chooses
     starts = list(range(0, length, tile))
     order = sorted(((item, q0) for item in range(prompts) for q0 in starts), key=lambda t: -t[1])

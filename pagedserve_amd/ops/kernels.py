@@ -732,13 +732,17 @@ def prefill_small_tile_pays(heads, head_dim, tiles) -> bool:
     return head_dim <= 128 and 2 * heads * tiles <= compute_units()
 
 
-def prefill_large_tile_pays(heads, head_dim, large_tiles) -> bool:
+def prefill_large_tile_pays(heads, head_dim, large_tiles, max_kv_len=0) -> bool:
     """Whether ``large_tiles`` tiles of 128 queries of ``heads`` heads are the better cut: from
-    three blocks per compute unit on (two are resident at a time), measured: 2 x 4,096 tokens of
-    12 heads, 768 blocks, 90 against 118 us; 4 x 1,024 of 25 heads, 800 blocks, 36 against 45;
-    4 x 1,024 of 16 heads, 512 blocks, level; 2 x 2,048 of 12 heads, 384 blocks, 46 against 37:
-    with fewer blocks the one that sees the most keys decides, and it is longer."""
-    return head_dim <= PREFILL_LARGE_TILE_HEAD_DIM and heads * large_tiles >= 3 * compute_units()
+    three blocks per compute unit on (two are resident at a time; with fewer the block that
+    sees the most keys decides, and it is twice as long) and where a request holds 2,048 keys
+    or more (``max_kv_len``: no query sees more; 0 = unknown).  Measured against the tiles of
+    64, four of whose blocks share a compute unit: 2 x 4,096 tokens of 12 heads, 768 blocks, 86
+    against 97 us; 2 x 4,096 of 25 heads 178 against 202; 2 x 3,072 of 25 heads 107 against 117;
+    4 x 2,048 of 12 heads 57 against 59; but 4 x 1,024 of 25 heads, 800 blocks, 35 against 33; 16 x
+    512 of 12 heads 24 against 22; 2 x 3,072 of 12 heads, 576 blocks, 65 against 56."""
+    return (head_dim <= PREFILL_LARGE_TILE_HEAD_DIM and heads * large_tiles >= 3 * compute_units()
+            and (max_kv_len <= 0 or max_kv_len >= 2048))
 
 
 def attention_prefill(q, k_pool, v_pool, out, tile_item, tile_q0, cu_tokens, kv_lens, tables,

@@ -145,7 +145,8 @@ class Attention(Mixer):
                 size = kernels.PREFILL_SMALL_TILE
                 tile_item, tile_q0 = ctx.query_tiles[size]
             elif kernels.prefill_large_tile_pays(self.heads, self.head_dim,
-                                                 ctx.query_tiles[kernels.PREFILL_LARGE_TILE][0].numel()):
+                                                 ctx.query_tiles[kernels.PREFILL_LARGE_TILE][0].numel(),
+                                                 ctx.max_kv_len):
                 size = kernels.PREFILL_LARGE_TILE
                 tile_item, tile_q0 = ctx.query_tiles[size]
             kernels.attention_prefill(q, cache.k_pool, cache.v_pool, context, tile_item,

@@ -74,6 +74,7 @@ def test_query_tiles_of_the_prefill_attention(monkeypatch):
         assert not small(heads, 64, 32) and not large(heads, 64, 16)
     # long prompts
     assert large(12, 64, 64) and large(25, 64, 32) and large(16, 64, 48) and not large(16, 64, 47)
+    assert large(12, 64, 64, 4096) and large(12, 64, 64, 2048) and not large(25, 64, 48, 1024)
     assert not large(12, 128, 64) and not large(12, 80, 640) and not small(1, 144, 1)
     for heads in (1, 3, 12, 25, 64):
         for tiles in range(1, 400):

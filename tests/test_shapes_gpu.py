@@ -138,34 +138,36 @@ def test_wide_layers_with_many_decoded_tokens_a_step(tmp_path, dtype, width, hea
 
 
 def test_long_prompts_take_tiles_of_128_queries(tmp_path):
-    """A step with so many (head, tile) pairs that the attention part cuts the prompts' queries
-    into tiles of 128 (64 heads of 16 dimensions, three portions of 520 to 780 tokens, two of
-    them behind cached prefixes that end inside a page and inside a tile): every position's
-    logits against the plain implementation, and the window of the second layer's keys is
-    not involved (GPT-2 has none).  The steps before it run the tiles of 64 and of 32."""
+    """A step with so many (head, tile) pairs over so many keys that the attention part cuts
+    the prompts' queries into tiles of 128 (32 heads of 16 dimensions, three portions of 1,840
+    to 2,100 tokens, two of them behind cached prefixes that end inside a page and inside a
+    tile): every position's logits against the plain implementation.  The step before it runs
+    the tiles of 64 and of 32."""
     from pagedserve_amd.engine import Engine
     from pagedserve_amd.model import load_model
     from pagedserve_amd.ops import kernels
 
+    length = 2100
     config = {"architectures": ["GPT2LMHeadModel"], "model_type": "gpt2", "layer_norm_epsilon": 1e-5,
-              "activation_function": "gelu_new", "tie_word_embeddings": True, "n_layer": 2, "n_embd": 1024,
-              "n_head": 64, "n_inner": 256, "vocab_size": 333, "n_positions": 800}
+              "activation_function": "gelu_new", "tie_word_embeddings": True, "n_layer": 2, "n_embd": 512,
+              "n_head": 32, "n_inner": 256, "vocab_size": 333, "n_positions": 2304}
     folder = str(tmp_path / "many_heads")
     helpers.write_folder(folder, config, helpers.lively_tensors(config, 83))
-    requests = {name: helpers.random_tokens(780, config["vocab_size"], 1300 + i) for i, name in enumerate("abc")}
+    requests = {name: helpers.random_tokens(length, config["vocab_size"], 1300 + i) for i, name in enumerate("abc")}
     reference = helpers.plain_logits_of_many(folder, requests, bfloat16=True, device="cuda")
     cuts = {"a": 100, "b": 260}
     first = [{"id": rid, "tokens": requests[rid][:cut], "want": list(range(cut))} for rid, cut in cuts.items()]
-    second = [{"id": rid, "tokens": requests[rid][cuts.get(rid, 0):], "want": list(range(780 - cuts.get(rid, 0)))}
-              for rid in "abc"]
+    second = [{"id": rid, "tokens": requests[rid][cuts.get(rid, 0):],
+               "want": list(range(length - cuts.get(rid, 0)))} for rid in "abc"]
     steps = [{"step": 0, "entries": first, "end": []}, {"step": 1, "entries": second, "end": list("abc")}]
     large = sum(-(-len(entry["tokens"]) // kernels.PREFILL_LARGE_TILE) for entry in second)
-    assert kernels.prefill_large_tile_pays(config["n_head"], 16, large)
-    assert not kernels.prefill_large_tile_pays(config["n_head"], 16, 4)
+    assert kernels.prefill_large_tile_pays(config["n_head"], 16, large, config["n_positions"])
+    assert not kernels.prefill_large_tile_pays(config["n_head"], 16, 4, config["n_positions"])
+    assert not kernels.prefill_large_tile_pays(config["n_head"], 16, large, 1024)
     model, _ = load_model(folder, dtype="bfloat16")
-    engine = Engine(model, num_pages=3 * 49 + 2, page_size=16, max_requests=4, max_step_tokens=2048)
+    engine = Engine(model, num_pages=3 * 132 + 2, page_size=16, max_requests=4, max_step_tokens=6144)
     rows = helpers.replay_in_process(engine, steps)
-    assert len(rows) == 3 * 780
+    assert len(rows) == 3 * length
     error, scale, where = helpers.max_error(rows, reference)
     assert error <= helpers.TOLERANCE["bfloat16"] * scale, (error, scale, where)
     engine.cache.check_invariants()
