@@ -77,10 +77,14 @@ __global__ __launch_bounds__(64 * QW * KS) void attention_prefill_kernel(
   static_assert(KR == 1 || KR == 2, "one or two runs of keys per wave");
   constexpr int TILE_BYTES = AP_KEYS * ROW;
   constexpr int STAGE_BYTES = 2 * TILE_BYTES;    // K tile, then V tile
-  // The ring may take 96 KB; with four waves along the keys 64 KB, so that two such blocks
-  // share a compute unit: the grids that take them have up to three blocks for two units, and
-  // with one block per unit a third of them would wait for a second round (2 x 1,024 tokens of
-  // 12 heads: 1.5 us less per launch).
+  // The ring may take 96 KB; with four waves along the keys (and with blocks of 128 queries)
+  // 64 KB, so that two such blocks share a compute unit: the grids that take them have up to
+  // three blocks for two units, and with one block per unit a third of them would wait for a
+  // second round (2 x 1,024 tokens of 12 heads: 1.5 us less per launch).  The blocks of four
+  // waves and 64 queries, which long prompts take by the thousand, get 32 KB at head sizes up
+  // to 64, two stages: four of them then share a compute unit, four waves to a SIMD (their
+  // 126 registers allow it), and what one wave waits for another fills (2 x 4,096 tokens of
+  // 12 heads: 97 against 114 us with a ring of four stages and two blocks to a unit).
   constexpr int FIT = (KS == 2 && QW == 2 && NDB <= 4 ? 32768 : ((KS >= 4 && QW == 2) || QW == 4 ? 65536 : 98304)) / STAGE_BYTES;
   constexpr int STAGES = FIT >= 4 ? 4 : (FIT >= 2 ? FIT : 2);
   static_assert(NDB <= 8 || STAGES == 2, "head sizes beyond 128 rely on a ring of two stages");
