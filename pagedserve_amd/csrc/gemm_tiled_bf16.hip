@@ -217,15 +217,17 @@ __global__ __launch_bounds__(256) void gemm_nt_bf16_tiled_kernel(
         if (s + 1 < STEPS) {
           fetch(kt, s + 1, fa[(s + 1) & 1], fw[(s + 1) & 1]);
           asm volatile("s_waitcnt lgkmcnt(%0)" ::"n"(READS) : "memory");   // step s has arrived
-        } else if (kt + 1 < k_tiles) {
-          // own reads of this tile are complete before the others may overwrite its stage
-          asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
-          // tiles kt + 2 .. kt + STAGES - 1 may stay in flight, as far as they exist
-          const int last = k_tiles - 1 < kt + STAGES - 1 ? k_tiles - 1 : kt + STAGES - 1;
-          wait_ahead_and_sync<LOADS, STAGES - 2>(last - (kt + 1));
-          fetch(kt + 1, 0, fa[0], fw[0]);
         } else {
+          // own reads of this tile are complete before the others may overwrite its stage
+          // (one wait for both cases, ahead of the branch: the last step's operands are then
+          // complete on every path that leads to their product)
           asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+          if (kt + 1 < k_tiles) {
+            // tiles kt + 2 .. kt + STAGES - 1 may stay in flight, as far as they exist
+            const int last = k_tiles - 1 < kt + STAGES - 1 ? k_tiles - 1 : kt + STAGES - 1;
+            wait_ahead_and_sync<LOADS, STAGES - 2>(last - (kt + 1));
+            fetch(kt + 1, 0, fa[0], fw[0]);
+          }
         }
         // the registers are used only behind the wait (the compiler does not know that the
         // assembly above left them on their way)
@@ -248,7 +250,9 @@ __global__ __launch_bounds__(256) void gemm_nt_bf16_tiled_kernel(
   // LDS of its own and stores rows in aligned pieces
   static_assert(4 * 32 * (WN * 32 + 8) * 4 + (KW - 1) * 2 * 16 * 64 * 4 <= STAGES * STAGE_BYTES,
                 "the epilogue reuses the stages");
-  wait_loads_and_sync<0>();                       // every wave is past its last operand reads
+  // every wave is past its last operand reads (and no assembly read is on its way any more,
+  // whichever way the loop was left)
+  asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)\n\ts_barrier" ::: "memory");
   if (KW == 2) {
     // the wave of the odd k tiles hands its sums to the wave of the even ones, behind the
     // regions that the epilogue uses

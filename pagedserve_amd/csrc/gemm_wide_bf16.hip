@@ -221,8 +221,9 @@ __global__ __launch_bounds__(256) void gemm_nt_bf16_wide_kernel(
       if (kt + 4 < k_tiles) run_tile(kt + 4, std::integral_constant<int, 4 % GW_STAGES>{}, std::false_type{});
   }
 
-  // ---- epilogue: every wave is past its last operand reads before LDS is reused
-  gw_wait_loads_and_sync<0>();
+  // ---- epilogue: every wave is past its last operand reads before LDS is reused (and no
+  // assembly read is on its way any more, whichever way the loops were left)
+  asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)\n\ts_barrier" ::: "memory");
   store_wave_tile<WM, GW_WN, TOut, EPI>(
       acc, reinterpret_cast<float*>(lds) + wave * 32 * (GW_WN * 32 + 8), lane, m0,
       n0 + wave * (GW_WN * 32), m, n, ldc, c, bias, 0, 1, scatter);

@@ -1,5 +1,6 @@
-"""The tiled prefill attention reads its operands from LDS by inline assembly and waits for
-them itself.  The compiler's assembly of every variant is checked for instructions that touch
+"""The tiled prefill attention and the tiled and wide matrix products read their operands from
+LDS by inline assembly and wait for them themselves.  The compiler's assembly of every variant
+is checked for instructions that touch
 a register between the read that fills it and the wait that covers it (`assembly_reads.py`),
 and the check itself is pinned on two hand-written fragments.  Runs where hipcc is found."""
 
@@ -52,21 +53,27 @@ def test_the_check_tells_a_copy_before_the_wait_from_one_behind_it():
     assert assembly_reads.registers_touched_in_flight(own, "_Z4test") == {"_Z4testv": []}
 
 
-def test_no_variant_of_the_prefill_attention_touches_a_register_in_flight(tmp_path):
+@pytest.mark.parametrize("name,prefix,least", [
+    ("attention_prefill.hip", "_Z24attention_prefill_kernel", 30),   # every head size in its arrangements of waves
+    ("gemm_tiled_bf16.hip", "_Z25gemm_nt_bf16_tiled_kernel", 60),    # tile shapes x ring depths x outputs x epilogues
+    ("gemm_wide_bf16.hip", "_Z24gemm_nt_bf16_wide_kernel", 16),
+])
+def test_no_kernel_touches_a_register_in_flight(tmp_path, name, prefix, least):
+    """The three sources that read LDS by assembly, compiled to assembly with the library's own
+    flags: no variant of their kernels names a register between its read and its wait."""
     from pagedserve_amd.ops import library
 
     hipcc = os.environ.get("HIPCC") or shutil.which("hipcc") or "/opt/rocm/bin/hipcc"
     if not os.path.exists(hipcc):
         pytest.skip("hipcc was not found")
-    name = "attention_prefill.hip"
-    output = os.path.join(str(tmp_path), "attention_prefill.s")
+    output = os.path.join(str(tmp_path), name.replace(".hip", ".s"))
     command = ([hipcc] + library.HIPCC_FLAGS + library.EXTRA_FLAGS.get(name, [])
                + ["-I", library.SOURCE_DIR, "-S", "--cuda-device-only",
                   os.path.join(library.SOURCE_DIR, name), "-o", output])
     done = subprocess.run(command, capture_output=True, text=True)
     assert done.returncode == 0, done.stderr[-2000:]
     with open(output) as handle:
-        found = assembly_reads.registers_touched_in_flight(handle.read(), "_Z24attention_prefill_kernel")
-    assert len(found) >= 30, sorted(found)       # every head size in its arrangements of waves
+        found = assembly_reads.registers_touched_in_flight(handle.read(), prefix)
+    assert len(found) >= least, sorted(found)
     dirty = {kernel: problems[:3] for kernel, problems in found.items() if problems}
     assert not dirty, dirty
