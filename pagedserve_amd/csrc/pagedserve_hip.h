@@ -190,6 +190,21 @@ int ps_attention_prefill(const void* q, int64_t q_stride, const void* k_pool, co
                          int num_pages, float scale, int window, int max_kv_len, int query_tile,
                          int dtype, void* stream);
 
+// Both of the above in one launch, for a step that has items of one token (tok_list lists the
+// `singles` tokens; tok_item and tok_pos are indexed by token as in ps_attention_decode, which
+// this computes with one range of keys) and items of several (tiles of
+// ps_attention_prefill_query_tile() queries as in ps_attention_prefill): blocks of both kinds
+// share the compute units, where two launches would leave most of them waiting twice.
+// bfloat16 and head sizes of 16 to 64 in steps of 16 (ps_attention_mixed_supported).
+int ps_attention_mixed_supported(int dtype, int head_dim, int table_width);
+int ps_attention_mixed(const void* q, int64_t q_stride, const void* k_pool, const void* v_pool,
+                       void* out, int64_t out_stride, const int* tok_list, int singles,
+                       const int* tok_item, const int* tok_pos, const int* tile_item,
+                       const int* tile_q0, int tiles, const int* cu_tokens, const int* kv_lens,
+                       const int* tables, int table_width, int heads, int kv_heads, int head_dim,
+                       int page_size, int num_pages, float scale, int window, int dtype,
+                       void* stream);
+
 // The constants of that kernel that a caller builds its index arrays by: queries per tile (of
 // the two sizes), and the widest block table (entries per item) that it takes.
 int ps_attention_prefill_query_tile(void);

@@ -43,6 +43,9 @@ _SIGNATURES = {
     "ps_attention_prefill": [c_void_p, c_int64, c_void_p, c_void_p, c_void_p, c_int64, c_void_p,
                              c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int,
                              c_int, c_int, c_int, c_float, c_int, c_int, c_int, c_int, c_void_p],
+    "ps_attention_mixed": [c_void_p, c_int64, c_void_p, c_void_p, c_void_p, c_int64, c_void_p, c_int,
+                           c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_void_p,
+                           c_int, c_int, c_int, c_int, c_int, c_int, c_float, c_int, c_int, c_void_p],
     "ps_sample": [c_void_p, c_int64, c_void_p, c_void_p, c_void_p, c_int, c_int, c_void_p],
 }
 
@@ -775,6 +778,50 @@ def attention_prefill(q, k_pool, v_pool, out, tile_item, tile_q0, cu_tokens, kv_
           cu_tokens.data_ptr(), kv_lens.data_ptr(), tables.data_ptr(), tables.shape[1], heads,
           kv_heads, head_dim, page_size, pages, float(scale), int(window), int(max_kv_len),
           int(query_tile), dtype_code(q.dtype), _stream())
+    return out
+
+
+def mixed_supported(dtype, head_dim, table_width=0) -> bool:
+    """Whether one launch can take a step's one-token items and its items of several tokens
+    together (``attention_mixed``): bfloat16, head sizes of 16 to 64 in steps of 16."""
+    return (dtype == torch.bfloat16 and head_dim % 16 == 0 and 16 <= head_dim <= 64
+            and table_width <= PREFILL_TABLE_MAX)
+
+
+def attention_mixed(q, k_pool, v_pool, out, tok_list, tok_item, positions, tile_item, tile_q0,
+                    cu_tokens, kv_lens, tables, heads, scale, window=0):
+    """The attention of a step that mixes decoded tokens with prompt portions, in one launch:
+    the tokens listed in ``tok_list`` (the step's one-token items) as ``attention_decode`` with
+    one range of keys computes them, the tiles of 64 queries listed in ``tile_item`` /
+    ``tile_q0`` as ``attention_prefill`` does; blocks of both kinds share the compute units."""
+    _check_prefill_constants()
+    _check(q, "q", torch.bfloat16, 2)
+    _check(out, "out", torch.bfloat16, 2)
+    pages, kv_heads, page_size, head_dim = _check_pools(k_pool, v_pool, q.dtype)
+    q_stride = _rows(q, "q")
+    out_stride = _rows(out, "out")
+    if q.shape[1] != heads * head_dim or out.shape != q.shape:
+        raise KernelError("attention_mixed: q/out rows must hold heads x head_dim values")
+    for name, tensor in (("tok_list", tok_list), ("tok_item", tok_item), ("positions", positions),
+                         ("tile_item", tile_item), ("tile_q0", tile_q0), ("cu_tokens", cu_tokens),
+                         ("kv_lens", kv_lens)):
+        _check(tensor, name, torch.int32, 1)
+        if not tensor.is_contiguous():
+            raise KernelError(f"attention_mixed: {name} must be contiguous")
+    _check(tables, "tables", torch.int32, 2)
+    tiles = tile_item.numel()
+    items = kv_lens.numel()
+    tokens = q.shape[0]
+    if tile_q0.numel() != tiles or cu_tokens.numel() != items + 1 or tables.shape[0] != items \
+            or not tables.is_contiguous() or tok_item.numel() != tokens or positions.numel() != tokens \
+            or tok_list.numel() > tokens:
+        raise KernelError("attention_mixed: inconsistent token, tile or item arrays")
+    _call("ps_attention_mixed", q.data_ptr(), q_stride, k_pool.data_ptr(), v_pool.data_ptr(),
+          out.data_ptr(), out_stride, tok_list.data_ptr(), tok_list.numel(), tok_item.data_ptr(),
+          positions.data_ptr(), tile_item.data_ptr(), tile_q0.data_ptr(), tiles,
+          cu_tokens.data_ptr(), kv_lens.data_ptr(), tables.data_ptr(), tables.shape[1], heads,
+          kv_heads, head_dim, page_size, pages, float(scale), int(window), dtype_code(q.dtype),
+          _stream())
     return out
 
 

@@ -37,6 +37,7 @@ HIPCC_FLAGS = [
 # accumulation registers; the skinny decode products are better off without.
 EXTRA_FLAGS = {
     "attention_prefill.hip": ["-mllvm", "-amdgpu-mfma-vgpr-form"],
+    "attention_mixed.hip": ["-mllvm", "-amdgpu-mfma-vgpr-form"],
     "gemm_tiled_bf16.hip": ["-mllvm", "-amdgpu-mfma-vgpr-form"],
 }
 

@@ -25,6 +25,10 @@ class Attention(Mixer):
 
     accepts_pending_norm = True
 
+    # decoded tokens and prompt portions of one step in one attention launch where the kernel
+    # takes the shape (``kernels.attention_mixed``)
+    fuse_mixed = True
+
     # the step's index arrays list the queries of a prompt portion in tiles of these sizes (the
     # tiled kernel's three; ``kernels.attention_prefill`` checks them against the library's)
     query_tile = (kernels.PREFILL_TILE, kernels.PREFILL_SMALL_TILE, kernels.PREFILL_LARGE_TILE)
@@ -117,6 +121,21 @@ class Attention(Mixer):
             kernels.attention_merge_linear(partial, singles, self.heads, self.head_dim, splits,
                                            self.out_weight, self.out_packed, self.out_bias, residual)
             return
+        tiled = singles < tokens and kernels.prefill_supported(self.dtype, self.head_dim, tables.shape[1])
+        if singles and tiled and self.fuse_mixed and kernels.mixed_supported(self.dtype, self.head_dim,
+                                                                            tables.shape[1]) \
+                and self._splits(singles, ctx.max_kv_len) == (1, 4):
+            # decoded tokens beside prompt portions: one launch whose blocks are of both kinds
+            tile_item, tile_q0 = ctx.query_tiles[kernels.PREFILL_TILE]
+            if not kernels.prefill_large_tile_pays(self.heads, self.head_dim,
+                                                   ctx.query_tiles[kernels.PREFILL_LARGE_TILE][0].numel(),
+                                                   ctx.max_kv_len):
+                kernels.attention_mixed(q, cache.k_pool, cache.v_pool, context, ctx.single_tokens,
+                                        ctx.tok_item, ctx.positions, tile_item, tile_q0, ctx.cu_tokens,
+                                        ctx.kv_lens, tables, self.heads, self.scale, self.window)
+                kernels.linear(context, self.out_weight, self.out_bias, residual, epilogue="residual",
+                               packed=self.out_packed, memo=site_memo(self._memo_out, ctx.workspace))
+                return
         if singles:
             # one-token items: keys of a request are cut into ranges so that few requests
             # still fill the chip
@@ -138,7 +157,7 @@ class Attention(Mixer):
                                      partial=partial, window=self.window, waves=waves,
                                      tok_list=None if singles == tokens else ctx.single_tokens)
         whole = singles == 0
-        if singles < tokens and kernels.prefill_supported(self.dtype, self.head_dim, tables.shape[1]):
+        if tiled:
             size = kernels.PREFILL_TILE
             tile_item, tile_q0 = ctx.query_tiles[size]
             if kernels.prefill_small_tile_pays(self.heads, self.head_dim, tile_item.numel()):

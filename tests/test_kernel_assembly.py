@@ -55,11 +55,12 @@ def test_the_check_tells_a_copy_before_the_wait_from_one_behind_it():
 
 @pytest.mark.parametrize("name,prefix,least", [
     ("attention_prefill.hip", "_Z24attention_prefill_kernel", 30),   # every head size in its arrangements of waves
+    ("attention_mixed.hip", "_Z22attention_mixed_kernel", 8),         # four head sizes x two kinds of loads
     ("gemm_tiled_bf16.hip", "_Z25gemm_nt_bf16_tiled_kernel", 60),    # tile shapes x ring depths x outputs x epilogues
     ("gemm_wide_bf16.hip", "_Z24gemm_nt_bf16_wide_kernel", 16),
 ])
 def test_no_kernel_touches_a_register_in_flight(tmp_path, name, prefix, least):
-    """The three sources that read LDS by assembly, compiled to assembly with the library's own
+    """The sources that read LDS by assembly, compiled to assembly with the library's own
     flags: no variant of their kernels names a register between its read and its wait."""
     from pagedserve_amd.ops import library
 

@@ -582,6 +582,68 @@ def test_attention_prefill_tiles(heads, kv_heads, head_dim, page_size, window, t
     torch.testing.assert_close(out.double(), expected, atol=5e-3, rtol=5e-3)
 
 
+@pytest.mark.parametrize("heads,kv_heads,head_dim,page_size", [(12, 12, 64, 16), (4, 4, 16, 8), (6, 2, 48, 16), (25, 25, 64, 16),
+                                                                (3, 1, 32, 12), (16, 4, 64, 5)])
+@pytest.mark.parametrize("window", [0, 37])
+def test_attention_mixed_is_both_kernels_in_one_launch(heads, kv_heads, head_dim, page_size, window):
+    """One launch for the one-token items and the items of several tokens of a step, listed in
+    any order among each other: every row against float64 attention over the gathered pages,
+    and bit for bit what the two kernels give that it is made of (the decode kernel with one
+    range of keys, the tiled kernel with tiles of 64 queries where it takes its four-wave
+    blocks).  NaN lies behind every request's last key and in the pages that nobody owns."""
+    from pagedserve_amd.ops import kernels
+
+    dtype = torch.bfloat16
+    # (cached before the step, tokens of the step)
+    items = [(130, 1), (0, 70), (15, 1), (511, 1), (30, 200), (0, 1), (63, 3), (250, 1), (17, 130), (99, 1)]
+    totals = [past + new for past, new in items]
+    k_pool, v_pool, tables = _paged_fixture(dtype, totals, kv_heads, head_dim, page_size, 71)
+    for index, total in enumerate(totals):
+        if total % page_size:
+            last = int(tables[index, total // page_size])
+            k_pool[last, :, total % page_size:] = float("nan")
+            v_pool[last, :, total % page_size:] = float("nan")
+    tokens = sum(new for _, new in items)
+    q = _rand((tokens, heads * head_dim), dtype, 72)
+    tok_item, tok_pos, singles, tile_item, tile_q0, cu = [], [], [], [], [], [0]
+    for index, (past, new) in enumerate(items):
+        if new == 1:
+            singles.append(len(tok_item))
+        else:
+            for q0 in range(0, new, kernels.PREFILL_TILE):
+                tile_item.append(index)
+                tile_q0.append(q0)
+        tok_item += [index] * new
+        tok_pos += list(range(past, past + new))
+        cu.append(cu[-1] + new)
+
+    def dev(values):
+        return torch.tensor(values, dtype=torch.int32, device="cuda")
+
+    scale = head_dim ** -0.5
+    assert kernels.mixed_supported(dtype, head_dim, tables.shape[1])
+    out = torch.full_like(q, float("nan"))
+    kernels.attention_mixed(q, k_pool, v_pool, out, dev(singles), dev(tok_item), dev(tok_pos), dev(tile_item),
+                            dev(tile_q0), dev(cu), dev(totals), tables, heads, scale, window=window)
+    assert torch.isfinite(out.float()).all()
+    expected = _attention_expected(q, k_pool, v_pool, tables, tok_item, tok_pos, heads, scale, window)
+    torch.testing.assert_close(out.double(), expected, atol=5e-3, rtol=5e-3)
+    # the same blocks launched kind by kind (max_kv_len below 512: the tiled kernel's blocks of
+    # four waves, which are the ones that the common launch runs)
+    apart = torch.full_like(q, float("nan"))
+    kernels.attention_decode(q, k_pool, v_pool, apart, dev(tok_item), dev(tok_pos), tables, heads, scale, 1,
+                             window=window, waves=4, tok_list=dev(singles))
+    kernels.attention_prefill(q, k_pool, v_pool, apart, dev(tile_item), dev(tile_q0), dev(cu), dev(totals),
+                              tables, heads, scale, window=window, max_kv_len=256)
+    assert torch.equal(out, apart)
+    with pytest.raises(kernels.KernelError, match="launch the two kernels"):
+        wide = torch.zeros(4, 2 * 128, dtype=dtype, device="cuda")
+        pool = torch.zeros(4, 2, page_size, 128, dtype=dtype, device="cuda")
+        kernels.attention_mixed(wide, pool, pool, wide.clone(), dev([0]), dev([0, 1, 1, 1]), dev([0, 0, 1, 2]),
+                                dev([1]), dev([0]), dev([0, 1, 4]), dev([1, 3]),
+                                torch.zeros(2, 2, dtype=torch.int32, device="cuda"), 2, 0.1)
+
+
 @pytest.mark.parametrize("tile", [64, 32, 128])
 def test_attention_prefill_far_key_and_causality(tile):
     """One early key is made to dominate for late queries only if they may see it; the query
