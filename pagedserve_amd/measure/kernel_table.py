@@ -372,17 +372,31 @@ def mixed_table(raw, decodes, context, portion, peaks, page_size=16):
     splits, waves = part._splits(decodes, max(context, portion))
     worst = (6 * kernels.compute_units() + rows * heads) * (head_dim + 2)
     partial = torch.empty(worst, dtype=torch.float32, device="cuda")
+    fused = (part.fuse_mixed and kernels.mixed_supported(dtype, head_dim, table_width)
+             and (splits, waves) == (1, 4))
+    if fused:
+        # as the attention part runs them: both kinds of block in one launch (tiles of 64)
+        starts64 = sorted(range(0, portion, kernels.PREFILL_TILE), reverse=True)
+        item64 = torch.full((len(starts64),), decodes, dtype=torch.int32, device="cuda")
+        q064 = torch.tensor(starts64, dtype=torch.int32, device="cuda")
+        us = graph_time(lambda i: kernels.attention_mixed(
+            q, k_pool, v_pool, context_rows, single_tokens, tok_item, positions, item64, q064, cu_tokens,
+            kv_lens, tables, heads, part.scale), 8)
+        out.append(_row("attention (decoded tokens and portion in one launch)", us,
+                        2 * decodes * context * d * 2 + portion * d * 2 * 4,
+                        4 * decodes * context * d + 4 * d * (portion * (portion + 1) // 2), peaks))
     us = graph_time(lambda i: kernels.attention_decode(
         q, k_pool, v_pool, context_rows, tok_item, positions, tables, heads, part.scale, splits,
         partial=partial if splits > 1 else None, waves=waves, tok_list=single_tokens), 8)
-    out.append(_row(f"attention of the decoded tokens ({splits} key ranges, {waves} waves)", us,
+    apart = " (apart: not part of the step)" if fused else ""
+    out.append(_row(f"attention of the decoded tokens ({splits} key ranges, {waves} waves){apart}", us,
                     2 * decodes * context * d * 2, 4 * decodes * context * d, peaks,
                     launches=2 if splits > 1 else 1))
     if kernels.prefill_supported(dtype, head_dim, table_width):
         us = graph_time(lambda i: kernels.attention_prefill(
             q, k_pool, v_pool, context_rows, tile_item, tile_q0, cu_tokens, kv_lens, tables, heads,
             head_dim ** -0.5, max_kv_len=max(context, portion), query_tile=tile), 8)
-        out.append(_row(f"attention of the portion (tiles of {tile}, causal)", us, portion * d * 2 * 4,
+        out.append(_row(f"attention of the portion (tiles of {tile}, causal){apart}", us, portion * d * 2 * 4,
                         4 * d * (portion * (portion + 1) // 2), peaks))
     product("out_proj+residual", d, d,
             lambda w, wp, bias: kernels.linear(context_rows, w, bias, h, epilogue="residual", packed=wp),
