@@ -122,20 +122,15 @@ class Attention(Mixer):
                                            self.out_weight, self.out_packed, self.out_bias, residual)
             return
         tiled = singles < tokens and kernels.prefill_supported(self.dtype, self.head_dim, tables.shape[1])
-        if singles and tiled and self.fuse_mixed and kernels.mixed_supported(self.dtype, self.head_dim,
-                                                                            tables.shape[1]) \
-                and self._splits(singles, ctx.max_kv_len) == (1, 4):
+        if singles and tiled and self._one_launch(singles, ctx, tables):
             # decoded tokens beside prompt portions: one launch whose blocks are of both kinds
             tile_item, tile_q0 = ctx.query_tiles[kernels.PREFILL_TILE]
-            if not kernels.prefill_large_tile_pays(self.heads, self.head_dim,
-                                                   ctx.query_tiles[kernels.PREFILL_LARGE_TILE][0].numel(),
-                                                   ctx.max_kv_len):
-                kernels.attention_mixed(q, cache.k_pool, cache.v_pool, context, ctx.single_tokens,
-                                        ctx.tok_item, ctx.positions, tile_item, tile_q0, ctx.cu_tokens,
-                                        ctx.kv_lens, tables, self.heads, self.scale, self.window)
-                kernels.linear(context, self.out_weight, self.out_bias, residual, epilogue="residual",
-                               packed=self.out_packed, memo=site_memo(self._memo_out, ctx.workspace))
-                return
+            kernels.attention_mixed(q, cache.k_pool, cache.v_pool, context, ctx.single_tokens,
+                                    ctx.tok_item, ctx.positions, tile_item, tile_q0, ctx.cu_tokens,
+                                    ctx.kv_lens, tables, self.heads, self.scale, self.window)
+            kernels.linear(context, self.out_weight, self.out_bias, residual, epilogue="residual",
+                           packed=self.out_packed, memo=site_memo(self._memo_out, ctx.workspace))
+            return
         if singles:
             # one-token items: keys of a request are cut into ranges so that few requests
             # still fill the chip
@@ -178,6 +173,18 @@ class Attention(Mixer):
                                       tok_list=None if whole else ctx.portion_tokens)
         kernels.linear(context, self.out_weight, self.out_bias, residual, epilogue="residual",
                        packed=self.out_packed, memo=site_memo(self._memo_out, ctx.workspace))
+
+    def _one_launch(self, singles: int, ctx, tables) -> bool:
+        """Whether a step's one-token items and its items of several tokens go to the kernel
+        that runs both kinds of block in one grid: where it takes the shape, where the decoded
+        tokens would get one four-wave block per head each anyway (the blocks it runs), and
+        where the prompts are not so long that tiles of 128 queries are the better cut."""
+        if not (self.fuse_mixed and kernels.mixed_supported(self.dtype, self.head_dim, tables.shape[1])):
+            return False
+        if self._splits(singles, ctx.max_kv_len) != (1, 4):
+            return False
+        large_tiles = ctx.query_tiles[kernels.PREFILL_LARGE_TILE][0].numel()
+        return not kernels.prefill_large_tile_pays(self.heads, self.head_dim, large_tiles, ctx.max_kv_len)
 
     def _range_records(self, ctx):
         """Scratch for one record per (token, head, key range): always asked for at its largest
