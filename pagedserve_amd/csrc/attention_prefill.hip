@@ -86,11 +86,12 @@ extern "C" int ps_attention_prefill(const void* q, int64_t q_stride, const void*
   }
   hipStream_t s = (hipStream_t)stream;
   dim3 grid(heads, tiles);
-  // With few blocks (up to three for two compute units: 2 x 1,024 tokens of 12 heads measured
-  // 1 % of the step ahead) each takes a compute unit for itself, and four waves along the keys
-  // shorten the longest block (if the caller knows of no long context, that does not pay);
-  // with many, smaller blocks that share a unit balance better.
-  const bool wide = (int64_t)tiles * heads <= ps_compute_units() * 3 / 2 &&
+  // With few blocks, up to two per compute unit, which hold them all at once (128 registers and
+  // 72 KB of LDS each), four waves along the keys shorten the longest block (2 x 1,024 tokens of
+  // 12 heads, 384 blocks: 16.6 against 18.6 us; of 16 heads, 512 blocks: 17.3 against 18.7; 3 x
+  // 1,024 of 12 heads, 576 blocks: level; 768 blocks: 24.5 against 20.6).  If the caller knows of
+  // no long context that does not pay; with many, smaller blocks balance better.
+  const bool wide = (int64_t)tiles * heads <= ps_compute_units() * 2 &&
                     (max_kv_len <= 0 || max_kv_len >= 512);
   // tiles of 32 queries: one wave along the queries, four along the keys (two such blocks
   // share a compute unit)

@@ -64,8 +64,8 @@ __device__ __forceinline__ void attention_prefill_block(
   constexpr int STAGE_BYTES = 2 * TILE_BYTES;    // K tile, then V tile
   // The ring may take 96 KB; with four waves along the keys (and with blocks of 128 queries)
   // 64 KB, so that two such blocks share a compute unit: the grids that take them have up to
-  // three blocks for two units, and with one block per unit a third of them would wait for a
-  // second round (2 x 1,024 tokens of 12 heads: 1.5 us less per launch).  The blocks of four
+  // two blocks per unit, and with one block per unit half of them would wait for a second
+  // round (2 x 1,024 tokens of 12 heads: 1.5 us less per launch).  The blocks of four
   // waves and 64 queries, which long prompts take by the thousand, get 32 KB at head sizes up
   // to 64, two stages: four of them then share a compute unit, four waves to a SIMD (their
   // 126 registers allow it), and what one wave waits for another fills (2 x 4,096 tokens of
