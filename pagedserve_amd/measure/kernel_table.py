@@ -373,7 +373,7 @@ def mixed_table(raw, decodes, context, portion, peaks, page_size=16):
     worst = (6 * kernels.compute_units() + rows * heads) * (head_dim + 2)
     partial = torch.empty(worst, dtype=torch.float32, device="cuda")
     fused = (part.fuse_mixed and kernels.mixed_supported(dtype, head_dim, table_width)
-             and (splits, waves) == (1, 4))
+             and not (4 * decodes * heads < kernels.compute_units() and max(context, portion) > 512))
     if fused:
         # as the attention part runs them: both kinds of block in one launch (tiles of 64)
         starts64 = sorted(range(0, portion, kernels.PREFILL_TILE), reverse=True)

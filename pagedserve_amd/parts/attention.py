@@ -176,12 +176,20 @@ class Attention(Mixer):
 
     def _one_launch(self, singles: int, ctx, tables) -> bool:
         """Whether a step's one-token items and its items of several tokens go to the kernel
-        that runs both kinds of block in one grid: where it takes the shape, where the decoded
-        tokens would get one four-wave block per head each anyway (the blocks it runs), and
-        where the prompts are not so long that tiles of 128 queries are the better cut."""
+        that runs both kinds of block in one grid: where it takes the shape, where the prompts
+        are not so long that tiles of 128 queries are the better cut, and not where a handful
+        of tokens is decoded over long contexts.  Its decode blocks are of four waves over all
+        keys of a request, also where the decode kernel alone would run ranges or blocks of
+        sixteen waves: beside the tiles' blocks they are not what the launch waits for (a
+        portion of 512 beside 8 tokens over 900 keys: the step 0.978 against 1.005 ms at GPT-2
+        small shape, 16 over 300 keys 0.90 against 0.99, 24 over 600 keys 0.97 against 1.08; at
+        medium shape 16 over 900 keys 2.24 against 2.34), unless they are so few that their
+        eight rounds of loads are (2 and 4 tokens over 900 keys: 0.956 against 0.946 and 0.974
+        against 0.958 ms)."""
         if not (self.fuse_mixed and kernels.mixed_supported(self.dtype, self.head_dim, tables.shape[1])):
             return False
-        if self._splits(singles, ctx.max_kv_len) != (1, 4):
+        visible = ctx.max_kv_len if self.window <= 0 else min(ctx.max_kv_len, self.window)
+        if 4 * singles * self.heads < kernels.compute_units() and visible > 512:
             return False
         large_tiles = ctx.query_tiles[kernels.PREFILL_LARGE_TILE][0].numel()
         return not kernels.prefill_large_tile_pays(self.heads, self.head_dim, large_tiles, ctx.max_kv_len)

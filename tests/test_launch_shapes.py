@@ -79,3 +79,43 @@ def test_query_tiles_of_the_prefill_attention(monkeypatch):
     for heads in (1, 3, 12, 25, 64):
         for tiles in range(1, 400):
             assert not (small(heads, 64, tiles) and large(heads, 64, -(-tiles // 2)))
+
+
+def test_one_attention_launch_for_mixed_steps(monkeypatch):
+    """Decoded tokens and prompt portions of a step share one attention launch where the kernel
+    takes the shape, except a handful of tokens over long contexts and prompts long enough for
+    tiles of 128 queries."""
+    import types
+
+    import torch
+
+    monkeypatch.setattr(kernels, "compute_units", lambda: 256)
+
+    class Count:
+        def __init__(self, count):
+            self.count = count
+
+        def numel(self):
+            return self.count
+
+    def ctx(max_kv_len, large_tiles=4):
+        return types.SimpleNamespace(max_kv_len=max_kv_len,
+                                     query_tiles={kernels.PREFILL_LARGE_TILE: (Count(large_tiles), None)})
+
+    tables = types.SimpleNamespace(shape=(8, 64))
+    part = _part(12)
+    part.dtype, part.fuse_mixed = torch.bfloat16, True
+    assert part._one_launch(32, ctx(1024), tables) and part._one_launch(8, ctx(1024), tables)
+    assert part._one_launch(6, ctx(1024), tables) and not part._one_launch(5, ctx(1024), tables)
+    assert part._one_launch(2, ctx(512), tables) and not part._one_launch(2, ctx(1024), tables)
+    assert not part._one_launch(32, ctx(4096, large_tiles=64), tables)      # long prompts: tiles of 128
+    windowed = _part(12, window=256)
+    windowed.dtype, windowed.fuse_mixed = torch.bfloat16, True
+    assert windowed._one_launch(2, ctx(1024), tables)                       # a window bounds the keys
+    for other in (_part(12, head_dim=128), _part(12, head_dim=40)):
+        other.dtype, other.fuse_mixed = torch.bfloat16, True
+        assert not other._one_launch(32, ctx(1024), tables)
+    part.dtype = torch.float32
+    assert not part._one_launch(32, ctx(1024), tables)
+    part.dtype, part.fuse_mixed = torch.bfloat16, False
+    assert not part._one_launch(32, ctx(1024), tables)
