@@ -749,11 +749,22 @@ def prefill_large_tile_pays(heads, head_dim, large_tiles, max_kv_len=0) -> bool:
 
 
 def attention_prefill(q, k_pool, v_pool, out, tile_item, tile_q0, cu_tokens, kv_lens, tables,
-                      heads, scale, window=0, max_kv_len=0, query_tile=PREFILL_TILE):
+                      heads, scale, window=0, max_kv_len=0, query_tile=PREFILL_TILE, memo=None):
     """Attention of items with several tokens, ``query_tile`` (64, 32 or 128) queries per block,
     on the matrix cores.  Blocks start in the order of the tile list, which is cut for that size:
     the tiles that see the most keys belong first.
-    ``max_kv_len`` (no query sees more keys; 0 = unknown) only steers the launch shape."""
+    ``max_kv_len`` (no query sees more keys; 0 = unknown) only steers the launch shape.
+    ``memo``: as in ``attention_mixed``."""
+    key = None
+    if memo is not None:
+        key = (q.data_ptr(), q.shape[0], out.data_ptr(), k_pool.data_ptr(), v_pool.data_ptr(),
+               tile_item.data_ptr(), tile_item.numel(), tile_q0.data_ptr(), cu_tokens.data_ptr(),
+               cu_tokens.numel(), kv_lens.data_ptr(), tables.data_ptr(), tables.shape[1], heads, scale,
+               window, max_kv_len, query_tile)
+        kept = memo.get(key)
+        if kept is not None:
+            _call("ps_attention_prefill", *kept, _stream())
+            return out
     _check_prefill_constants()
     _check(q, "q", torch.bfloat16, 2)
     _check(out, "out", torch.bfloat16, 2)
@@ -773,11 +784,12 @@ def attention_prefill(q, k_pool, v_pool, out, tile_item, tile_q0, cu_tokens, kv_
     if tile_q0.numel() != tiles or cu_tokens.numel() != items + 1 or tables.shape[0] != items \
             or not tables.is_contiguous():
         raise KernelError("attention_prefill: inconsistent tile or item arrays")
-    _call("ps_attention_prefill", q.data_ptr(), q_stride, k_pool.data_ptr(), v_pool.data_ptr(),
-          out.data_ptr(), out_stride, tile_item.data_ptr(), tile_q0.data_ptr(), tiles,
-          cu_tokens.data_ptr(), kv_lens.data_ptr(), tables.data_ptr(), tables.shape[1], heads,
-          kv_heads, head_dim, page_size, pages, float(scale), int(window), int(max_kv_len),
-          int(query_tile), dtype_code(q.dtype), _stream())
+    _kept_call("ps_attention_prefill", memo, key,
+               (q.data_ptr(), q_stride, k_pool.data_ptr(), v_pool.data_ptr(),
+                out.data_ptr(), out_stride, tile_item.data_ptr(), tile_q0.data_ptr(), tiles,
+                cu_tokens.data_ptr(), kv_lens.data_ptr(), tables.data_ptr(), tables.shape[1], heads,
+                kv_heads, head_dim, page_size, pages, float(scale), int(window), int(max_kv_len),
+                int(query_tile), dtype_code(q.dtype)))
     return out
 
 
@@ -788,12 +800,36 @@ def mixed_supported(dtype, head_dim, table_width=0) -> bool:
             and table_width <= PREFILL_TABLE_MAX)
 
 
+def _kept_call(name, memo, key, args):
+    """Calls ``name`` with ``args`` and keeps them under ``key``: the next call of this site
+    with the same addresses and counts skips the checks that led to them (a step that is not
+    replayed from a graph is issued by the host at the GPU's own pace, and the checks of an
+    attention call take as long as three launches)."""
+    _call(name, *args, _stream())
+    if memo is not None:
+        if len(memo) >= 256:
+            memo.clear()
+        memo[key] = args
+
+
 def attention_mixed(q, k_pool, v_pool, out, tok_list, tok_item, positions, tile_item, tile_q0,
-                    cu_tokens, kv_lens, tables, heads, scale, window=0):
+                    cu_tokens, kv_lens, tables, heads, scale, window=0, memo=None):
     """The attention of a step that mixes decoded tokens with prompt portions, in one launch:
     the tokens listed in ``tok_list`` (the step's one-token items) as ``attention_decode`` with
     one range of keys computes them, the tiles of 64 queries listed in ``tile_item`` /
-    ``tile_q0`` as ``attention_prefill`` does; blocks of both kinds share the compute units."""
+    ``tile_q0`` as ``attention_prefill`` does; blocks of both kinds share the compute units.
+    ``memo`` (a dict of the call site, for the buffers of one workspace): what a checked call
+    handed to the library, by the operands' addresses and counts."""
+    key = None
+    if memo is not None:
+        key = (q.data_ptr(), q.shape[0], out.data_ptr(), k_pool.data_ptr(), v_pool.data_ptr(),
+               tok_list.data_ptr(), tok_list.numel(), tok_item.data_ptr(), positions.data_ptr(),
+               tile_item.data_ptr(), tile_item.numel(), tile_q0.data_ptr(), cu_tokens.data_ptr(),
+               cu_tokens.numel(), kv_lens.data_ptr(), tables.data_ptr(), tables.shape[1], heads, scale, window)
+        kept = memo.get(key)
+        if kept is not None:
+            _call("ps_attention_mixed", *kept, _stream())
+            return out
     _check_prefill_constants()
     _check(q, "q", torch.bfloat16, 2)
     _check(out, "out", torch.bfloat16, 2)
@@ -816,12 +852,12 @@ def attention_mixed(q, k_pool, v_pool, out, tok_list, tok_item, positions, tile_
             or not tables.is_contiguous() or tok_item.numel() != tokens or positions.numel() != tokens \
             or tok_list.numel() > tokens:
         raise KernelError("attention_mixed: inconsistent token, tile or item arrays")
-    _call("ps_attention_mixed", q.data_ptr(), q_stride, k_pool.data_ptr(), v_pool.data_ptr(),
-          out.data_ptr(), out_stride, tok_list.data_ptr(), tok_list.numel(), tok_item.data_ptr(),
-          positions.data_ptr(), tile_item.data_ptr(), tile_q0.data_ptr(), tiles,
-          cu_tokens.data_ptr(), kv_lens.data_ptr(), tables.data_ptr(), tables.shape[1], heads,
-          kv_heads, head_dim, page_size, pages, float(scale), int(window), dtype_code(q.dtype),
-          _stream())
+    _kept_call("ps_attention_mixed", memo, key,
+               (q.data_ptr(), q_stride, k_pool.data_ptr(), v_pool.data_ptr(),
+                out.data_ptr(), out_stride, tok_list.data_ptr(), tok_list.numel(), tok_item.data_ptr(),
+                positions.data_ptr(), tile_item.data_ptr(), tile_q0.data_ptr(), tiles,
+                cu_tokens.data_ptr(), kv_lens.data_ptr(), tables.data_ptr(), tables.shape[1], heads,
+                kv_heads, head_dim, page_size, pages, float(scale), int(window), dtype_code(q.dtype)))
     return out
 
 

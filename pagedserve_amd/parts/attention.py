@@ -51,7 +51,7 @@ class Attention(Mixer):
         self.kv_cols = kv_heads * head_dim
         self.position = None
         # what ``kernels.linear`` keeps per call site and step shape (its ``memo``), per workspace
-        self._memo_qkv, self._memo_out = {}, {}
+        self._memo_qkv, self._memo_out, self._memo_attention = {}, {}, {}
 
     def parameters(self):
         total = self.q_cols + 2 * self.kv_cols
@@ -74,6 +74,7 @@ class Attention(Mixer):
         self.out_packed = kernels.pack_decode_weight(self.out_weight)
         self._memo_qkv.clear()
         self._memo_out.clear()
+        self._memo_attention.clear()
 
     def cache_spec(self):
         return PagedKVSpec(self.kv_heads, self.head_dim, self.window)
@@ -127,7 +128,8 @@ class Attention(Mixer):
             tile_item, tile_q0 = ctx.query_tiles[kernels.PREFILL_TILE]
             kernels.attention_mixed(q, cache.k_pool, cache.v_pool, context, ctx.single_tokens,
                                     ctx.tok_item, ctx.positions, tile_item, tile_q0, ctx.cu_tokens,
-                                    ctx.kv_lens, tables, self.heads, self.scale, self.window)
+                                    ctx.kv_lens, tables, self.heads, self.scale, self.window,
+                                    memo=site_memo(self._memo_attention, ctx.workspace))
             kernels.linear(context, self.out_weight, self.out_bias, residual, epilogue="residual",
                            packed=self.out_packed, memo=site_memo(self._memo_out, ctx.workspace))
             return
@@ -166,7 +168,8 @@ class Attention(Mixer):
             kernels.attention_prefill(q, cache.k_pool, cache.v_pool, context, tile_item,
                                       tile_q0, ctx.cu_tokens, ctx.kv_lens, tables,
                                       self.heads, self.scale, self.window,
-                                      max_kv_len=ctx.max_kv_len, query_tile=size)
+                                      max_kv_len=ctx.max_kv_len, query_tile=size,
+                                      memo=site_memo(self._memo_attention, ctx.workspace))
         elif singles < tokens:
             kernels.attention_rowwise(q, cache.k_pool, cache.v_pool, context, ctx.tok_item,
                                       ctx.positions, tables, self.heads, self.scale, self.window,

@@ -636,6 +636,15 @@ def test_attention_mixed_is_both_kernels_in_one_launch(heads, kv_heads, head_dim
     kernels.attention_prefill(q, k_pool, v_pool, apart, dev(tile_item), dev(tile_q0), dev(cu), dev(totals),
                               tables, heads, scale, window=window, max_kv_len=256)
     assert torch.equal(out, apart)
+    # a call site's memo: the second call with the same addresses goes straight to the library
+    memo = {}
+    first, second = torch.zeros_like(q), torch.zeros_like(q)
+    lists = (dev(singles), dev(tok_item), dev(tok_pos), dev(tile_item), dev(tile_q0), dev(cu), dev(totals))
+    for target in (first, first, second):
+        target.zero_()
+        kernels.attention_mixed(q, k_pool, v_pool, target, *lists, tables, heads, scale, window=window, memo=memo)
+        assert torch.equal(target, out)
+    assert len(memo) == 2 and all(type(kept) is tuple for kept in memo.values())
     with pytest.raises(kernels.KernelError, match="launch the two kernels"):
         wide = torch.zeros(4, 2 * 128, dtype=dtype, device="cuda")
         pool = torch.zeros(4, 2, page_size, 128, dtype=dtype, device="cuda")
