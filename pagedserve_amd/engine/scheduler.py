@@ -28,13 +28,16 @@ than ``max_batch_size``.  The decoding requests of an iteration are then those t
 served least recently, so that every one advances at the same rate; the reference always
 takes the lowest ids (``:165-166``), and the others starve until those finish.
 
-**Running ahead.**  While every running request decodes and nobody waits, the
-iteration after the current one is launched before the current one's tokens have reached
-the host: its entries say "the token that the last step chose for row r" instead of a token
-id, and the host's work for an iteration overlaps the GPU's work for the next.  A request
-that ends by length is known beforehand and left out; one that ends at the end token has one
-token too many computed, which is dropped.  The tokens that a request receives are the same
-either way.
+**Running ahead.**  Where the engine chooses the tokens on the device, the iteration after
+the current one is chosen and launched before the current one's tokens have reached the
+host: everything that decides its work is known without them (how far every prompt has come,
+who decodes, who ends by length and gives its pages back, whose turn it is), and a decoding
+request's entry says "the token that the last step chose for row r" instead of a token id.
+So the host's work for an iteration (choosing, packing, launching) overlaps the GPU's work for
+the one before, prompt portions included.  One that ends at the end token has one token too
+many computed, which is dropped, and its pages come back an iteration later.  The tokens that
+a request receives are the same either way, and without end tokens so is every iteration's
+work.
 """
 
 from dataclasses import dataclass, field
@@ -68,11 +71,16 @@ class RequestState:
     prefill_cursor: int = 0                     # prompt tokens that are cached
     finish_reason: Optional[str] = None
     last_served: int = -1                       # ticket of its last turn; tickets grow with time
+    # row of the running iteration's chosen tokens that holds the token the next decode step
+    # brings, while that token has not reached the host
+    carry_row: Optional[int] = None
+    ending: Optional[str] = None                # "length": the token on its way is the last one
+    released: bool = False                      # pages, slot and promise have gone back
     prompt_array: Optional[object] = field(default=None, repr=False)   # the prompt as an int64 array
 
     @property
     def is_prefilling(self) -> bool:
-        return self.pending_token_id is None
+        return self.pending_token_id is None and self.carry_row is None
 
     @property
     def prompt_left(self) -> int:
@@ -171,7 +179,9 @@ class _Flight:
     chosen: list              # (request, number of tokens)
     receivers: list           # requests that get a token from it, in the order of the logits rows
     output: object
-    can_carry: bool           # every row is a decoded token chosen on the device
+    can_carry: bool           # its tokens are chosen on the device (or it chooses none)
+    advanced: bool = False    # its requests have been moved on (all but the tokens' values)
+    deliveries: list = field(default_factory=list)   # (request, row of its token)
 
 
 class ContinuousBatchScheduler:
@@ -342,6 +352,9 @@ class ContinuousBatchScheduler:
                 else:
                     tokens = request.prompt_token_ids[start:start + size]
                 entries.append(StepEntry(request.request_id, tokens, want))
+            elif request.carry_row is not None:
+                # the token is still on the device: row ``carry_row`` of the last step's choices
+                entries.append(StepEntry(request.request_id, [0], [0], carry=request.carry_row))
             else:
                 entries.append(StepEntry(request.request_id, [request.pending_token_id], [0]))
         return entries
@@ -383,7 +396,7 @@ class ContinuousBatchScheduler:
             self._failed_ahead = error
         return self._land(flight)
 
-    def _choose_on_device(self, receivers, ahead):
+    def _choose_on_device(self, receivers):
         """How the engine should pick the tokens of ``receivers``: keyword arguments of
         ``engine.step``.  Greedy rows are picked inside the step (one launch less, and part of
         a decode step's graph); with temperatures each row gets ``(1 / temperature, uniform
@@ -394,16 +407,18 @@ class ContinuousBatchScheduler:
             return {"greedy": True}
         if not getattr(self.engine, "supports_draws", False):
             return {}
-        # ``ahead`` = 1 when the request's last token is still on its way to the host
+        # a request whose last token is still on its way to the host draws its next but one
         return {"draws": [(0.0 if r.sampling.temperature == 0 else 1.0 / r.sampling.temperature,
-                           uniform_for(r.seed, r.request_id, len(r.generated_token_ids) + ahead))
+                           uniform_for(r.seed, r.request_id,
+                                       len(r.generated_token_ids) + (r.carry_row is not None)))
                           for r in receivers]}
 
-    def _take_off(self) -> Optional[_Flight]:
-        """Choose an iteration's work, promise pages to its newcomers, start it on the GPU."""
+    def _take_off(self, ahead: bool = False) -> Optional[_Flight]:
+        """Choose an iteration's work, promise pages to its newcomers, start it on the GPU.
+        ``ahead``: the iteration before it still runs, and nothing to choose is no error."""
         chosen = self.select_requests()
         if not chosen:
-            if self._live:
+            if self._live and not ahead:
                 raise RuntimeError("No request can be scheduled with the available KV memory")
             return None
         newcomers = [request for request, _ in chosen if not request.reserved_blocks]
@@ -411,7 +426,7 @@ class ContinuousBatchScheduler:
             self.ledger.promise(request)
         entries = self.build_step_entries(chosen)
         receivers = [request for (request, _), entry in zip(chosen, entries) if entry.want]
-        how = self._choose_on_device(receivers, 0)
+        how = self._choose_on_device(receivers)
         try:
             output = self.engine.step(entries, **how)
         except Exception:
@@ -420,42 +435,61 @@ class ContinuousBatchScheduler:
             for request in newcomers:
                 self.ledger.withdraw(request)
             raise
-        only_decodes = all(not request.is_prefilling for request, _ in chosen)
-        return _Flight(chosen, receivers, output, bool(how) and only_decodes)
+        if receivers:
+            on_device = bool(how) and getattr(output, "host_tokens", None) is not None
+        else:
+            # no token to wait for; only an engine that chooses tokens lets the next iteration
+            # carry them on
+            on_device = bool(getattr(self.engine, "supports_draws", False))
+        return _Flight(chosen, receivers, output, on_device)
 
     def _take_off_ahead(self, flight) -> Optional[_Flight]:
-        """Start the iteration after ``flight`` before ``flight``'s tokens are known, if it is
-        certain which requests it holds: all of ``flight``'s that do not end by length, each
-        carrying on the token that ``flight`` chooses for it."""
-        if (not self.run_ahead or not flight.can_carry
-                or getattr(flight.output, "host_tokens", None) is None):
+        """Start the iteration after ``flight`` before ``flight``'s tokens are known: its
+        requests are moved on first (all but the tokens' values), then the next iteration is
+        chosen as ever; a request whose token is on its way carries it on from the device."""
+        if not self.run_ahead or not flight.can_carry:
             return None
-        if any(request.is_prefilling for request in self._live.values()):
-            return None         # a prompt waits: the next iteration is chosen in the ordinary way
-        if len(self._live) != len(flight.chosen):
-            return None         # a request sat ``flight`` out, or has just ended
-        chosen, entries = [], []
-        for row, (request, _) in enumerate(flight.chosen):
-            if request.finish_reason is not None:
-                continue        # ended at the end token while ``flight`` was already running
-            if len(request.generated_token_ids) + 2 > request.max_new_tokens:
-                continue        # ``flight`` brings its last token
-            chosen.append((request, 1))
-            entries.append(StepEntry(request.request_id, [0], [0], carry=row))
-        if not chosen:
-            return None
-        receivers = [request for request, _ in chosen]
+        self._advance(flight)
         try:
-            output = self.engine.step(entries, **self._choose_on_device(receivers, 1))
+            ahead = self._take_off(ahead=True)
         except ValueError:
             return None         # the ordinary start of the next iteration reports it
-        self.steps_run_ahead += 1
-        return _Flight(chosen, receivers, output, True)
+        if ahead is not None:
+            self.steps_run_ahead += 1
+        return ahead
+
+    def _advance(self, flight):
+        """What a started iteration changes whatever tokens it chooses: prompts have come
+        further, the receivers have a token on its way (``flight.deliveries``), those for whom
+        it is the last by length give back what they hold, and everybody has had a turn."""
+        flight.advanced = True
+        rows = {id(request): row for row, request in enumerate(flight.receivers)}
+        served = []
+        for request, size in flight.chosen:
+            if request.finish_reason is not None:
+                continue        # ended at the end token after this iteration had been started ahead
+            served.append(request)
+            if request.is_prefilling:
+                request.prefill_cursor += size
+                if request.prompt_left:
+                    continue
+            row = rows[id(request)]
+            request.carry_row = row
+            flight.deliveries.append((request, row))
+            if len(request.generated_token_ids) + 1 >= request.max_new_tokens:
+                request.ending = "length"
+                self._release(request)
+        # those that had waited longest for this turn are also first in line for the next one
+        for request in sorted(served, key=lambda request: (request.last_served, request.request_id)):
+            request.last_served = self._tickets
+            self._tickets += 1
 
     def _tokens_of(self, flight) -> List[int]:
         output = flight.output
         if output.logits.shape[0] != len(flight.receivers):
             raise RuntimeError("the engine returned a wrong number of logits rows")
+        if not flight.receivers:
+            return []
         if getattr(output, "tokens", None) is None:
             receivers = flight.receivers
             return self.sampler.sample(
@@ -464,40 +498,40 @@ class ContinuousBatchScheduler:
         return output.token_list() if hasattr(output, "token_list") else output.tokens.tolist()
 
     def _land(self, flight) -> Dict[int, int]:
-        """Read the tokens of a started iteration and move its requests on."""
-        tokens = dict(zip((id(request) for request in flight.receivers), self._tokens_of(flight)))
+        """Read the tokens of a started iteration and hand them to its requests."""
+        if not flight.advanced:
+            self._advance(flight)
+        tokens = self._tokens_of(flight)
         emitted = {}
-        served = []
-        for request, size in flight.chosen:
+        for request, row in flight.deliveries:
             if request.finish_reason is not None:
-                continue        # ended after this iteration had been started ahead: its token is dropped
-            served.append(request)
-            if request.is_prefilling:
-                request.prefill_cursor += size
-                if request.prompt_left:
-                    continue
-            token = int(tokens[id(request)])
+                continue        # (cannot happen: a delivery is made once, and before any later one)
+            token = int(tokens[row])
             request.generated_token_ids.append(token)
             request.pending_token_id = token
+            request.carry_row = None
             emitted[request.request_id] = token
             if (token == self.eos_token_id and self.eos_token_id is not None
                     and not request.sampling.ignore_eos):
                 self._retire(request, "stop")
-            elif len(request.generated_token_ids) >= request.max_new_tokens:
-                self._retire(request, "length")
-        # those that had waited longest for this turn are also first in line for the next one
-        for request in sorted(served, key=lambda request: (request.last_served, request.request_id)):
-            request.last_served = self._tickets
-            self._tickets += 1
+            elif request.ending is not None:
+                self._retire(request, request.ending)
         self.iterations += 1
         return emitted
 
-    def _retire(self, request, reason):
-        """The request is over: pages, slot and promise go back."""
-        request.finish_reason = reason
+    def _release(self, request):
+        """Pages, slot and promise go back; the request takes part in nothing from here on."""
+        if request.released:
+            return
+        request.released = True
         del self._live[request.request_id]
         self.engine.finish(request.request_id)
         self.ledger.withdraw(request)
+
+    def _retire(self, request, reason):
+        """The request is over and its last token is with it."""
+        request.finish_reason = reason
+        self._release(request)
         self.finished[request.request_id] = request
 
     def has_work(self) -> bool:

@@ -2,6 +2,7 @@
 the cache bookkeeping of the real engine and returns made-up logits."""
 
 import random
+from collections import Counter
 from types import SimpleNamespace
 
 import pytest
@@ -304,12 +305,16 @@ class ChoosingEngine(FakeEngine):
         self.most_outstanding = 0
 
     def step(self, entries, greedy=False, draws=None):
-        assert greedy or draws is not None
+        wanted = sum(len(entry.want) for entry in entries)
+        assert greedy or draws is not None or not wanted
         for entry in entries:
             if entry.carry is not None:
                 assert len(entry.tokens) == 1 and 0 <= entry.carry < len(self.last_tokens)
                 entry.tokens = [self.last_tokens[entry.carry]]
         output = super().step(entries)
+        if not wanted:
+            self.last_tokens = []       # as the engine: nothing to carry on from this step
+            return output
         tokens = output.logits.argmax(-1)
         self.last_tokens = tokens.tolist()
         self.outstanding += 1
@@ -328,10 +333,10 @@ class ChoosingEngine(FakeEngine):
 
 @pytest.mark.parametrize("run_ahead", [False, True])
 def test_running_ahead_decisions(run_ahead):
-    """While all requests decode and nobody waits, the next iteration is launched before the
-    last one's tokens are read: requests that end by length are left out of it, one that meets
-    the end token gets its extra token dropped, a newcomer stops it until its prompt is in.
-    Tokens and finish reasons are those of the step-by-step run."""
+    """The next iteration is launched before the last one's tokens are read: requests that end
+    by length are left out of it, one that meets the end token gets its extra token dropped, a
+    newcomer's prompt runs beside the tokens that are carried on.  Tokens and finish reasons
+    are those of the step-by-step run."""
     end_token = expected_tokens([3, 1, 4], 9)[5]
     prompts = {"a": [3, 1, 4], "b": [2, 7], "c": [9, 9, 9, 9], "late": [5, 6]}
     budgets = {"a": 9, "b": 4, "c": 12, "late": 6}
@@ -363,6 +368,109 @@ def test_running_ahead_decisions(run_ahead):
             assert len(step) <= 4
     else:
         assert scheduler.steps_run_ahead == 0 and engine.most_outstanding == 1
+
+
+def _burst(run_ahead, strategy, seed, end_token=None):
+    """A burst of requests on so few pages that newcomers wait for others to end, fewer turns
+    than decoding requests, prompts cut into portions: (scheduler, engine, expected tokens)."""
+    rng = random.Random(seed)
+    engine = ChoosingEngine(pages=rng.choice([14, 24]), page_size=4, max_requests=6, max_step_tokens=32)
+    scheduler = ContinuousBatchScheduler(
+        engine, ArgmaxSampler(), tokenizer=None, scheduling_strategy=strategy,
+        max_batch_size=rng.choice([3, 6]), prefill_chunk_size=rng.choice([2, 5, 16]),
+        max_num_batched_tokens=rng.choice([8, 32]), max_prefill_requests=rng.choice([1, 3]),
+        eos_token_id=end_token, run_ahead=run_ahead)
+    expected = {}
+    for _ in range(14):
+        prompt = [rng.randrange(VOCAB - 1) for _ in range(rng.randint(1, 20))]
+        count = rng.randint(1, 12)
+        free_run = expected_tokens(prompt, count)
+        cut = free_run.index(end_token) + 1 if end_token in free_run else count
+        expected[scheduler.add_token_request(prompt, max_new_tokens=count)] = free_run[:cut]
+    return scheduler, engine, expected
+
+
+@pytest.mark.parametrize("strategy", [ORCA_STRATEGY, SARATHI_STRATEGY])
+@pytest.mark.parametrize("seed", range(6))
+def test_running_ahead_changes_no_iteration(strategy, seed):
+    """With nothing ending at an end token, everything that decides an iteration's work is
+    known before the tokens of the one before it are: launched ahead or not, the engine sees
+    the same steps with the same tokens (prompt portions, turns, newcomers that take the
+    pages of requests that have just ended by length), and every step but the first is
+    launched while its predecessor's tokens are still on their way."""
+    runs = {}
+    for run_ahead in (False, True):
+        scheduler, engine, expected = _burst(run_ahead, strategy, seed)
+        streamed = {}
+        while scheduler.has_work():
+            for rid, token in scheduler.step().items():
+                streamed.setdefault(rid, []).append(token)
+            engine.cache.check_invariants()
+        assert streamed == expected
+        assert {rid: r.generated_token_ids for rid, r in scheduler.finished.items()} == expected
+        assert all(r.finish_reason == "length" for r in scheduler.finished.values())
+        assert scheduler.reserved_blocks == [0] and not engine.cache.requests
+        runs[run_ahead] = (engine.steps, scheduler.iterations)
+        if run_ahead:
+            assert scheduler.steps_run_ahead == len(engine.steps) - 1
+            assert engine.most_outstanding == 2
+        else:
+            assert scheduler.steps_run_ahead == 0 and engine.most_outstanding == 1
+    assert runs[True] == runs[False]
+    assert any(len(tokens) > 1 for step in runs[True][0][1:] for _, tokens, _ in step)   # prompts ran ahead too
+
+
+@pytest.mark.parametrize("strategy", [ORCA_STRATEGY, SARATHI_STRATEGY])
+@pytest.mark.parametrize("seed", range(6))
+def test_running_ahead_with_end_tokens(strategy, seed):
+    """A request that meets the end token is known to have ended one iteration late: the
+    token computed for it meanwhile is dropped, its pages go back then, and every request
+    still receives exactly the tokens of the step-by-step run."""
+    free_runs = _burst(False, strategy, seed)[2]
+    # the token that cuts the most requests short
+    end_token = Counter(token for run in free_runs.values() for token in set(run[:-1])).most_common(1)[0][0]
+    ended_early = 0
+    for run_ahead in (False, True):
+        scheduler, engine, expected = _burst(run_ahead, strategy, seed, end_token=end_token)
+        streamed = {}
+        while scheduler.has_work():
+            for rid, token in scheduler.step().items():
+                streamed.setdefault(rid, []).append(token)
+            engine.cache.check_invariants()
+        assert streamed == expected
+        assert {rid: r.generated_token_ids for rid, r in scheduler.finished.items()} == expected
+        for rid, request in scheduler.finished.items():
+            stopped = expected[rid][-1] == end_token
+            assert request.finish_reason == ("stop" if stopped else "length")
+            ended_early += stopped and len(expected[rid]) < request.max_new_tokens
+        assert scheduler.reserved_blocks == [0] and not engine.cache.requests
+    assert ended_early >= 2
+
+
+def test_arrivals_while_running_ahead():
+    """Requests that arrive between iterations join the next one that is chosen, beside tokens
+    that are carried on; outputs are exact."""
+    for seed in range(5):
+        rng = random.Random(100 + seed)
+        engine = ChoosingEngine(pages=rng.choice([12, 20, 64]), page_size=4, max_requests=6, max_step_tokens=32)
+        scheduler = ContinuousBatchScheduler(
+            engine, ArgmaxSampler(), tokenizer=None,
+            scheduling_strategy=rng.choice([ORCA_STRATEGY, SARATHI_STRATEGY]),
+            max_batch_size=rng.choice([2, 4, 6]), prefill_chunk_size=rng.choice([1, 3, 8]),
+            max_num_batched_tokens=rng.choice([8, 32]), eos_token_id=None)
+        expected = {}
+        pending = 25
+        while pending or scheduler.has_work():
+            if pending and rng.random() < 0.5:
+                prompt = [rng.randrange(VOCAB) for _ in range(rng.randint(1, 20))]
+                count = rng.randint(1, 12)
+                expected[scheduler.add_token_request(prompt, max_new_tokens=count)] = expected_tokens(prompt, count)
+                pending -= 1
+            if scheduler.has_work():
+                scheduler.step()
+        assert {rid: r.generated_token_ids for rid, r in scheduler.finished.items()} == expected
+        assert scheduler.reserved_blocks == [0] and not engine.cache.requests
+        assert scheduler.steps_run_ahead > scheduler.iterations // 2 and engine.most_outstanding == 2
 
 
 @pytest.mark.parametrize("strategy", [ORCA_STRATEGY, SARATHI_STRATEGY])
