@@ -314,22 +314,63 @@ _MEMO_DONE = c_int(0)
 
 
 def _memo_key(x, out, scatter, a_packed, choose):
-    """What may differ between two calls of one call site: the row count and the addresses of
-    the operands that are not the site's own (weights, bias, flags are)."""
+    """What may differ between two calls of one call site, in two parts: the row count and
+    the addresses of the step's buffers and index arrays, which the same call site of another
+    layer meets too, and the addresses that tell the site's own operands apart where it may be
+    called with several (its norm's parameters; the cache pools, of which a block that runs
+    twice in a step has two pairs).  Weights, bias and flags are the site's own and in neither."""
     if isinstance(x, PendingNorm):
-        key = (x.count, x.h.data_ptr(), _ptr(x.rows), x.scratch.data_ptr(), x.gamma.data_ptr(),
-               out.data_ptr())
+        step = (x.count, x.h.data_ptr(), _ptr(x.rows), x.scratch.data_ptr(), out.data_ptr())
+        site = (x.gamma.data_ptr(),)
     else:
-        key = (x.shape[0], x.data_ptr(), x.stride(0), out.data_ptr(), a_packed)
+        step = (x.shape[0], x.data_ptr(), x.stride(0), out.data_ptr(), a_packed)
+        site = ()
     if scatter is not None:
-        key += (scatter[0].data_ptr(), scatter[2].data_ptr(), scatter[3].data_ptr(), scatter[4].data_ptr())
+        step += (scatter[2].data_ptr(), scatter[3].data_ptr(), scatter[4].data_ptr())
+        site += (scatter[0].data_ptr(), scatter[1].data_ptr())
     if choose is not None:
-        key += (choose[1].data_ptr(),)
-    return key
+        step += (choose[1].data_ptr(),)
+    return step, site
+
+
+def _field_ranges(names):
+    return tuple((getattr(_LinearArgs, name).offset,
+                  getattr(_LinearArgs, name).offset + getattr(_LinearArgs, name).size) for name in names)
+
+
+# The fields of an argument block by who decides them.  The site's own: its weights and bias,
+# equal on every call, and the norm parameters and pools that the call was made with (the second
+# part of ``_memo_key``).  The step's: equal for the same call site of every layer within a step
+# (the layers share the workspace and the index arrays).  All others are sizes, codes and flags.
+_SITE_FIELDS = ("w", "bias", "gamma", "beta", "k_pool", "v_pool", "w_packed")
+_STEP_FIELDS = ("a", "c", "m", "lda", "ldc", "norm_h", "norm_rows", "norm_out", "tok_item", "tok_pos",
+                "tables", "table_width", "a_packed", "c_rows", "norm_out_rows", "c_layout",
+                "top_tokens", "top_keys", "top_ticket", "top_done")
+_SITE_RANGES = _field_ranges(_SITE_FIELDS)
+_SIZE_RANGES = _field_ranges(name for name, _ in _LinearArgs._fields_
+                             if name not in _SITE_FIELDS and name not in _STEP_FIELDS)
+_NULL = bytes(ctypes.sizeof(c_void_p))
+
+
+def _sibling_block(sibling: bytes, own: bytes):
+    """The argument block of this site for a step whose block for the same call site of another
+    layer is ``sibling`` (checked in this step, same buffers and index arrays), from ``own``, a
+    checked block of this site for other rows: the step's fields of the one with the site's
+    fields of the other.  None where the two sites do not agree in every size, code and flag,
+    or in which of their own operands they have at all."""
+    for begin, end in _SIZE_RANGES:
+        if sibling[begin:end] != own[begin:end]:
+            return None
+    block = bytearray(sibling)
+    for begin, end in _SITE_RANGES:
+        if (sibling[begin:end] == _NULL) != (own[begin:end] == _NULL):
+            return None
+        block[begin:end] = own[begin:end]
+    return bytes(block)
 
 
 def linear(x, w, bias, out, epilogue="none", scatter=None, packed=None, a_packed=False,
-           packed_out=False, choose=None, scatter_only=False, memo=None):
+           packed_out=False, choose=None, scatter_only=False, memo=None, shared=None):
     """out = epilogue(x w^T + bias) where ``x`` is a tensor or a ``PendingNorm``.
 
     ``scatter = (k_pool, v_pool, tok_item, tok_pos, tables, q_cols, kv_cols)`` also stores the
@@ -356,10 +397,29 @@ def linear(x, w, bias, out, epilogue="none", scatter=None, packed=None, a_packed
     the host more than the launch, and a step that is not replayed from a graph issues four
     such calls a layer.  Whoever binds other weights clears the dict; and because a block also
     holds the room behind the addresses (rows that a buffer has space for), a site keeps one
-    dict per set of buffers (``parts.base.site_memo``)."""
+    dict per set of buffers (``parts.base.site_memo``).
+
+    ``shared``: a dict that lives for ONE step and is handed to the calls of all layers.  A
+    step with a row count that a site has not seen finds nothing in the site's memo; but the
+    same call site of the layer before has just had its block checked for the very same
+    buffers and index arrays, and left it here.  This site's block is then that one with the
+    site's own operands (weights, bias, norm parameters, pools) taken from a block that this
+    site was checked with for the same norm parameters and pools, provided the two agree in
+    every size, code and flag: one check per step instead of one per layer."""
     if memo is not None:
-        key = _memo_key(x, out, scatter, a_packed, choose)
+        step_key, site_key = _memo_key(x, out, scatter, a_packed, choose)
+        key = step_key + site_key
         kept = memo.get(key)
+        if kept is None and shared is not None:
+            # (a checked block of this site with these very norm parameters and pools)
+            sibling, own = shared.get(step_key), memo.get(("site",) + site_key)
+            if sibling is not None and own is not None:
+                kept = _sibling_block(sibling, own)
+                if kept is not None:
+                    if len(memo) >= _MEMO_LIMIT:
+                        memo.clear()
+                        memo[("site",) + site_key] = own
+                    memo[key] = kept
         if kept is not None:
             # (the library reads the block and writes through the pointers in it only)
             status = _BOUND["ps_linear_bytes"](kept, _stream())
@@ -492,7 +552,9 @@ def linear(x, w, bias, out, epilogue="none", scatter=None, packed=None, a_packed
     if memo is not None:
         if len(memo) >= _MEMO_LIMIT:
             memo.clear()
-        memo[key] = bytes(args)
+        memo[key] = memo[("site",) + site_key] = bytes(args)
+        if shared is not None:
+            shared[step_key] = memo[key]
     if packed_out:
         return out, bool(layout.value)
     if choose is not None:
@@ -749,19 +811,21 @@ def prefill_large_tile_pays(heads, head_dim, large_tiles, max_kv_len=0) -> bool:
 
 
 def attention_prefill(q, k_pool, v_pool, out, tile_item, tile_q0, cu_tokens, kv_lens, tables,
-                      heads, scale, window=0, max_kv_len=0, query_tile=PREFILL_TILE, memo=None):
+                      heads, scale, window=0, max_kv_len=0, query_tile=PREFILL_TILE, memo=None,
+                      shared=None):
     """Attention of items with several tokens, ``query_tile`` (64, 32 or 128) queries per block,
     on the matrix cores.  Blocks start in the order of the tile list, which is cut for that size:
     the tiles that see the most keys belong first.
     ``max_kv_len`` (no query sees more keys; 0 = unknown) only steers the launch shape.
-    ``memo``: as in ``attention_mixed``."""
-    key = None
+    ``memo``, ``shared``: as in ``attention_mixed``."""
+    key = step_key = None
     if memo is not None:
-        key = (q.data_ptr(), q.shape[0], out.data_ptr(), k_pool.data_ptr(), v_pool.data_ptr(),
-               tile_item.data_ptr(), tile_item.numel(), tile_q0.data_ptr(), cu_tokens.data_ptr(),
-               cu_tokens.numel(), kv_lens.data_ptr(), tables.data_ptr(), tables.shape[1], heads, scale,
-               window, max_kv_len, query_tile)
-        kept = memo.get(key)
+        step_key = ("prefill", q.data_ptr(), q.shape[0], out.data_ptr(),
+                    tile_item.data_ptr(), tile_item.numel(), tile_q0.data_ptr(), cu_tokens.data_ptr(),
+                    cu_tokens.numel(), kv_lens.data_ptr(), tables.data_ptr(), tables.shape[1], heads, scale,
+                    window, max_kv_len, query_tile)
+        key = step_key + (k_pool.data_ptr(), v_pool.data_ptr())
+        kept = memo.get(key) or _sibling_call(memo, shared, key, step_key, k_pool, v_pool)
         if kept is not None:
             _call("ps_attention_prefill", *kept, _stream())
             return out
@@ -789,7 +853,8 @@ def attention_prefill(q, k_pool, v_pool, out, tile_item, tile_q0, cu_tokens, kv_
                 out.data_ptr(), out_stride, tile_item.data_ptr(), tile_q0.data_ptr(), tiles,
                 cu_tokens.data_ptr(), kv_lens.data_ptr(), tables.data_ptr(), tables.shape[1], heads,
                 kv_heads, head_dim, page_size, pages, float(scale), int(window), int(max_kv_len),
-                int(query_tile), dtype_code(q.dtype)))
+                int(query_tile), dtype_code(q.dtype)),
+               shared, step_key, (kv_heads, head_dim, page_size, pages, q.dtype))
     return out
 
 
@@ -800,33 +865,64 @@ def mixed_supported(dtype, head_dim, table_width=0) -> bool:
             and table_width <= PREFILL_TABLE_MAX)
 
 
-def _kept_call(name, memo, key, args):
+def _kept_call(name, memo, key, args, shared=None, step_key=None, pool_shape=None):
     """Calls ``name`` with ``args`` and keeps them under ``key``: the next call of this site
     with the same addresses and counts skips the checks that led to them (a step that is not
     replayed from a graph is issued by the host at the GPU's own pace, and the checks of an
-    attention call take as long as three launches)."""
+    attention call take as long as three launches).  ``shared`` (a dict that lives for one
+    step) gets them too, under the part of the key that the same call of the other layers
+    shares, with the pools' shape and type."""
     _call(name, *args, _stream())
     if memo is not None:
         if len(memo) >= 256:
             memo.clear()
         memo[key] = args
+        memo["site", args[2], args[3]] = pool_shape
+        if shared is not None:
+            shared[step_key] = (args, pool_shape)
+
+
+def _sibling_call(memo, shared, key, step_key, k_pool, v_pool):
+    """The arguments of an attention call whose checks the same call of another layer has
+    passed in this step (same queries' buffer, same index arrays), for this site's pools:
+    theirs with the two pool addresses replaced, if these are the pools that this site has been
+    checked with and of the other site's shape and type.  None otherwise."""
+    if shared is None:
+        return None
+    pools = (k_pool.data_ptr(), v_pool.data_ptr())
+    sibling, own = shared.get(step_key), memo.get(("site",) + pools)
+    if sibling is None or own is None:
+        return None
+    args, pool_shape = sibling
+    if own != pool_shape:
+        return None
+    args = args[:2] + pools + args[4:]
+    if len(memo) >= 256:
+        memo.clear()
+        memo[("site",) + pools] = own
+    memo[key] = args
+    return args
 
 
 def attention_mixed(q, k_pool, v_pool, out, tok_list, tok_item, positions, tile_item, tile_q0,
-                    cu_tokens, kv_lens, tables, heads, scale, window=0, memo=None):
+                    cu_tokens, kv_lens, tables, heads, scale, window=0, memo=None, shared=None):
     """The attention of a step that mixes decoded tokens with prompt portions, in one launch:
     the tokens listed in ``tok_list`` (the step's one-token items) as ``attention_decode`` with
     one range of keys computes them, the tiles of 64 queries listed in ``tile_item`` /
     ``tile_q0`` as ``attention_prefill`` does; blocks of both kinds share the compute units.
     ``memo`` (a dict of the call site, for the buffers of one workspace): what a checked call
-    handed to the library, by the operands' addresses and counts."""
-    key = None
+    handed to the library, by the operands' addresses and counts.  ``shared`` (a dict that
+    lives for one step, handed to the calls of all layers): what the same call of the layer
+    before was checked with in this step; only the pools differ, and a site whose pools have
+    been checked before takes the rest from there."""
+    key = step_key = None
     if memo is not None:
-        key = (q.data_ptr(), q.shape[0], out.data_ptr(), k_pool.data_ptr(), v_pool.data_ptr(),
-               tok_list.data_ptr(), tok_list.numel(), tok_item.data_ptr(), positions.data_ptr(),
-               tile_item.data_ptr(), tile_item.numel(), tile_q0.data_ptr(), cu_tokens.data_ptr(),
-               cu_tokens.numel(), kv_lens.data_ptr(), tables.data_ptr(), tables.shape[1], heads, scale, window)
-        kept = memo.get(key)
+        step_key = ("mixed", q.data_ptr(), q.shape[0], out.data_ptr(),
+                    tok_list.data_ptr(), tok_list.numel(), tok_item.data_ptr(), positions.data_ptr(),
+                    tile_item.data_ptr(), tile_item.numel(), tile_q0.data_ptr(), cu_tokens.data_ptr(),
+                    cu_tokens.numel(), kv_lens.data_ptr(), tables.data_ptr(), tables.shape[1], heads, scale, window)
+        key = step_key + (k_pool.data_ptr(), v_pool.data_ptr())
+        kept = memo.get(key) or _sibling_call(memo, shared, key, step_key, k_pool, v_pool)
         if kept is not None:
             _call("ps_attention_mixed", *kept, _stream())
             return out
@@ -857,7 +953,8 @@ def attention_mixed(q, k_pool, v_pool, out, tok_list, tok_item, positions, tile_
                 out.data_ptr(), out_stride, tok_list.data_ptr(), tok_list.numel(), tok_item.data_ptr(),
                 positions.data_ptr(), tile_item.data_ptr(), tile_q0.data_ptr(), tiles,
                 cu_tokens.data_ptr(), kv_lens.data_ptr(), tables.data_ptr(), tables.shape[1], heads,
-                kv_heads, head_dim, page_size, pages, float(scale), int(window), dtype_code(q.dtype)))
+                kv_heads, head_dim, page_size, pages, float(scale), int(window), dtype_code(q.dtype)),
+               shared, step_key, (kv_heads, head_dim, page_size, pages, q.dtype))
     return out
 
 

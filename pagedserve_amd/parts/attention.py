@@ -92,10 +92,12 @@ class Attention(Mixer):
             kernels.linear(x, self.qkv_weight, self.qkv_bias, qkv,
                            scatter=(cache.k_pool, cache.v_pool, ctx.tok_item, ctx.positions, tables,
                                     self.q_cols, self.kv_cols), packed=self.qkv_packed,
-                           scatter_only=True, memo=site_memo(self._memo_qkv, ctx.workspace))
+                           scatter_only=True, memo=site_memo(self._memo_qkv, ctx.workspace),
+                           shared=ctx.shared_calls)
         else:
             kernels.linear(x, self.qkv_weight, self.qkv_bias, qkv, packed=self.qkv_packed,
-                           memo=site_memo(self._memo_qkv, ctx.workspace))
+                           memo=site_memo(self._memo_qkv, ctx.workspace),
+                           shared=ctx.shared_calls)
             if rotates:
                 self.position.apply_to_qk(q, k, ctx)
             if cache.writes:
@@ -129,9 +131,11 @@ class Attention(Mixer):
             kernels.attention_mixed(q, cache.k_pool, cache.v_pool, context, ctx.single_tokens,
                                     ctx.tok_item, ctx.positions, tile_item, tile_q0, ctx.cu_tokens,
                                     ctx.kv_lens, tables, self.heads, self.scale, self.window,
-                                    memo=site_memo(self._memo_attention, ctx.workspace))
+                                    memo=site_memo(self._memo_attention, ctx.workspace),
+                                    shared=ctx.shared_calls)
             kernels.linear(context, self.out_weight, self.out_bias, residual, epilogue="residual",
-                           packed=self.out_packed, memo=site_memo(self._memo_out, ctx.workspace))
+                           packed=self.out_packed, memo=site_memo(self._memo_out, ctx.workspace),
+                       shared=ctx.shared_calls)
             return
         if singles:
             # one-token items: keys of a request are cut into ranges so that few requests
@@ -169,13 +173,15 @@ class Attention(Mixer):
                                       tile_q0, ctx.cu_tokens, ctx.kv_lens, tables,
                                       self.heads, self.scale, self.window,
                                       max_kv_len=ctx.max_kv_len, query_tile=size,
-                                      memo=site_memo(self._memo_attention, ctx.workspace))
+                                      memo=site_memo(self._memo_attention, ctx.workspace),
+                                      shared=ctx.shared_calls)
         elif singles < tokens:
             kernels.attention_rowwise(q, cache.k_pool, cache.v_pool, context, ctx.tok_item,
                                       ctx.positions, tables, self.heads, self.scale, self.window,
                                       tok_list=None if whole else ctx.portion_tokens)
         kernels.linear(context, self.out_weight, self.out_bias, residual, epilogue="residual",
-                       packed=self.out_packed, memo=site_memo(self._memo_out, ctx.workspace))
+                       packed=self.out_packed, memo=site_memo(self._memo_out, ctx.workspace),
+                       shared=ctx.shared_calls)
 
     def _one_launch(self, singles: int, ctx, tables) -> bool:
         """Whether a step's one-token items and its items of several tokens go to the kernel

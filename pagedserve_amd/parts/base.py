@@ -26,7 +26,7 @@ in float in its own epilogue instead of a separate pass over the stream.
 """
 
 import itertools
-from dataclasses import dataclass
+from dataclasses import dataclass, field
 from typing import Dict, List, Optional
 
 import torch
@@ -275,3 +275,6 @@ class StepContext:
     token_src: Optional[torch.Tensor] = None       # int32 [T]: >= 0: the token is carried_tokens[src]
     carried_tokens: Optional[torch.Tensor] = None  # int32: tokens that the last step chose
     extra: Optional[dict] = None
+    # what ``kernels.linear`` and the attention calls leave for the same call of the next layer
+    # (their ``shared``): lives for this step only
+    shared_calls: dict = field(default_factory=dict)

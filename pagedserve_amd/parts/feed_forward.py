@@ -54,6 +54,8 @@ class DenseFeedForward(FeedForward):
         # them in the order in which the second reads them)
         _, hidden_packed = kernels.linear(x, self.up_weight, self.up_bias, hidden,
                                           epilogue=self.activation, packed=self.up_packed,
-                                          packed_out=True, memo=site_memo(self._memo_up, ctx.workspace))
+                                          packed_out=True, memo=site_memo(self._memo_up, ctx.workspace),
+                                          shared=ctx.shared_calls)
         kernels.linear(hidden, self.down_weight, self.down_bias, residual, epilogue="residual",
-                       packed=self.down_packed, a_packed=hidden_packed, memo=site_memo(self._memo_down, ctx.workspace))
+                       packed=self.down_packed, a_packed=hidden_packed, memo=site_memo(self._memo_down, ctx.workspace),
+                       shared=ctx.shared_calls)

@@ -644,7 +644,42 @@ def test_attention_mixed_is_both_kernels_in_one_launch(heads, kv_heads, head_dim
         target.zero_()
         kernels.attention_mixed(q, k_pool, v_pool, target, *lists, tables, heads, scale, window=window, memo=memo)
         assert torch.equal(target, out)
-    assert len(memo) == 2 and all(type(kept) is tuple for kept in memo.values())
+    assert len(memo) == 2 + 1 and all(type(kept) is tuple for kept in memo.values())   # (+ the site's own entry)
+    # the same call of another layer (other pools) in a step whose index arrays are new to both:
+    # the first is checked, the second takes the first's arguments with its own pools
+    other_k, other_v = (k_pool * 0.5).contiguous(), (v_pool * 2.0).contiguous()
+    other_memo = {}
+    third = torch.zeros_like(q)
+    kernels.attention_mixed(q, other_k, other_v, third, *lists, tables, heads, scale, window=window, memo=other_memo)
+    expected_other = third.clone()
+    assert not torch.equal(expected_other, out)
+    new_lists = tuple(index.clone() for index in lists)
+    shared = {}
+    checks = []
+    real_check = kernels._check
+    kernels._check = lambda *args, **kwargs: (checks.append(args[1]), real_check(*args, **kwargs))[1]
+    try:
+        # (the layers of a step write to one buffer: the target is part of what they share)
+        first.zero_()
+        kernels.attention_mixed(q, k_pool, v_pool, first, *new_lists, tables, heads, scale, window=window,
+                                memo=memo, shared=shared)
+        assert checks and len(shared) == 1
+        own_pools = first.clone()
+        del checks[:]
+        first.zero_()
+        kernels.attention_mixed(q, other_k, other_v, first, *new_lists, tables, heads, scale, window=window,
+                                memo=other_memo, shared=shared)
+        assert not checks
+        other_pools = first.clone()
+        # pools that this site has not been checked with take the whole way
+        fresh_k = other_k.clone()
+        first.zero_()
+        kernels.attention_mixed(q, fresh_k, other_v, first, *new_lists, tables, heads, scale, window=window,
+                                memo=other_memo, shared=shared)
+        assert checks
+    finally:
+        kernels._check = real_check
+    assert torch.equal(own_pools, out) and torch.equal(other_pools, expected_other) and torch.equal(first, expected_other)
     with pytest.raises(kernels.KernelError, match="launch the two kernels"):
         wide = torch.zeros(4, 2 * 128, dtype=dtype, device="cuda")
         pool = torch.zeros(4, 2, page_size, 128, dtype=dtype, device="cuda")
@@ -1148,6 +1183,80 @@ def test_the_tile_that_the_step_lists_is_the_kernels_own():
     assert kernels.prefill_large_tile() == (kernels.PREFILL_LARGE_TILE, kernels.PREFILL_LARGE_TILE_HEAD_DIM)
 
 
+def test_linear_checks_shared_by_the_layers_of_a_step():
+    """The same call site of several layers in a step with a row count that none has seen: the
+    first layer's call is checked and leaves its argument block for the step; the others take
+    it with their own weights, bias and norm parameters from a block of their own, without a
+    check, and give the bits of a checked call.  Sites that differ in a size or in which
+    operands they have take the whole way."""
+    from pagedserve_amd.ops import kernels
+
+    k, n = 256, 192
+    rows = _rand((64, k), torch.bfloat16, 730)
+    h = _rand((64, k), torch.float32, 731)
+    scratch = torch.empty((64, k), dtype=torch.bfloat16, device="cuda")
+    out = torch.empty((64, n), dtype=torch.bfloat16, device="cuda")
+
+    def site(seed, columns=n, with_bias=True):
+        w = _rand((columns, k), torch.bfloat16, seed, k ** -0.5)
+        return dict(w=w, bias=_rand((columns,), torch.float32, seed + 1) if with_bias else None,
+                    packed=kernels.pack_decode_weight(w), gamma=_rand((k,), torch.float32, seed + 2),
+                    beta=_rand((k,), torch.float32, seed + 3), memo={}, norm_memo={})
+
+    def call(site_, count, shared=None, memo=True, normed=False, target=None):
+        target = out if target is None else target
+        target.zero_()
+        x = kernels.PendingNorm(h[:count], site_["gamma"], site_["beta"], 1e-5, False, scratch[:count]) \
+            if normed else rows[:count]
+        kept = site_["norm_memo" if normed else "memo"] if memo else None
+        kernels.linear(x, site_["w"], site_["bias"], target[:count, :site_["w"].shape[0]], epilogue="gelu_tanh",
+                       packed=site_["packed"], memo=kept, shared=shared)
+        return target[:count, :site_["w"].shape[0]].clone()
+
+    layers = [site(740), site(750), site(760)]
+    narrow, bare = site(770, columns=128), site(780, with_bias=False)
+    for normed in (False, True):
+        for each in layers + [narrow, bare]:
+            call(each, 8, normed=normed)              # every site has been checked once, at other rows
+        checks = []
+        real_check = kernels._check
+        kernels._check = lambda *args, **kwargs: (checks.append(args[1]), real_check(*args, **kwargs))[1]
+        try:
+            for count in (24, 40):
+                shared = {}
+                got = []
+                for index, each in enumerate(layers):
+                    del checks[:]
+                    got.append(call(each, count, shared, normed=normed))
+                    assert bool(checks) == (index == 0), (normed, count, index, checks)
+                for each in (narrow, bare):           # other sizes, no bias: nothing to take over
+                    del checks[:]
+                    got.append(call(each, count, shared, normed=normed))
+                    assert checks
+                # a second step of these rows finds every block in the site's own memo
+                del checks[:]
+                again = [call(each, count, {}, normed=normed) for each in layers + [narrow, bare]]
+                assert not checks
+                for each, result, repeated in zip(layers + [narrow, bare], got, again):
+                    plain = call(each, count, memo=False, normed=normed)
+                    assert torch.equal(result.view(torch.int16), plain.view(torch.int16))
+                    assert torch.equal(repeated.view(torch.int16), plain.view(torch.int16))
+                assert not torch.equal(got[0], got[1]) and not torch.equal(got[1], got[2])
+        finally:
+            kernels._check = real_check
+    # a site that is called with two sets of norm parameters (a block that runs twice in a step
+    # has two pairs of pools in the same way): each call takes what it was checked with
+    first, second = layers[0], dict(layers[0], gamma=layers[1]["gamma"], beta=layers[1]["beta"])
+    call(second, 8, normed=True)
+    shared = {}
+    call(layers[2], 56, shared, normed=True)
+    for each in (first, second, first):
+        got = call(each, 56, shared, normed=True)
+        plain = call(each, 56, memo=False, normed=True)
+        assert torch.equal(got.view(torch.int16), plain.view(torch.int16))
+    assert not torch.equal(call(first, 56, shared, normed=True), call(second, 56, shared, normed=True))
+
+
 def test_linear_memo_of_a_call_site():
     """A call site's memo: the second call with the same row count and operand addresses goes
     straight to the library and gives the bits of the checked call; other rows or another
@@ -1172,10 +1281,10 @@ def test_linear_memo_of_a_call_site():
                                             packed=packed, packed_out=True)
         assert handed_on == plain_handed_on == (count > 16)
         assert torch.equal(got.view(torch.int16), plain[:count].view(torch.int16))
-    assert len(memo) == 2
+    assert len(memo) == 2 + 1      # (+ "site": the last checked block, for steps that share checks)
     other = torch.zeros((64, n), dtype=torch.bfloat16, device="cuda")
     kernels.linear(rows[:8], w, bias, other[:8], epilogue="gelu_tanh", packed=packed, packed_out=True, memo=memo)
-    assert len(memo) == 3 and torch.equal(other[:8].view(torch.int16), out[:8].view(torch.int16))
+    assert len(memo) == 3 + 1 and torch.equal(other[:8].view(torch.int16), out[:8].view(torch.int16))
     # a pending norm in front: keyed by the stream's rows, the row list and the scratch
     h = _rand((64, k), torch.float32, 710)
     gamma, beta = _rand((k,), torch.float32, 711), _rand((k,), torch.float32, 712)
@@ -1190,7 +1299,7 @@ def test_linear_memo_of_a_call_site():
         results.append(result)
         if len(results) == 1:
             h[:8] = _rand((8, k), torch.float32, 720)    # the same addresses, other values: a hit reads them
-    assert len(memo) == 1 and not torch.equal(results[0], results[1])
+    assert len(memo) == 1 + 1 and not torch.equal(results[0], results[1])
     # what is kept per call is nothing that the garbage collector has to walk (a stream of
     # requests leaves tens of thousands of entries behind)
     import gc

@@ -119,3 +119,46 @@ def test_one_attention_launch_for_mixed_steps(monkeypatch):
     assert not part._one_launch(32, ctx(1024), tables)
     part.dtype, part.fuse_mixed = torch.bfloat16, False
     assert not part._one_launch(32, ctx(1024), tables)
+
+
+def test_argument_blocks_shared_between_the_layers_of_a_step():
+    """``kernels._sibling_block``: the block of the same call site of another layer, with this
+    site's own operands; nothing where the sites differ in a size or in the operands they have."""
+    import ctypes
+
+    names = [name for name, _ in kernels._LinearArgs._fields_]
+    assert set(kernels._SITE_FIELDS) | set(kernels._STEP_FIELDS) <= set(names)
+    assert not set(kernels._SITE_FIELDS) & set(kernels._STEP_FIELDS)
+
+    def block(**fields):
+        args = kernels._LinearArgs()
+        for name, value in fields.items():
+            setattr(args, name, value)
+        return bytes(args)
+
+    def read(data):
+        return kernels._LinearArgs.from_buffer_copy(data)
+
+    sizes = dict(n=192, k=256, epilogue=2, dtype=1, c_dtype=1, eps=1e-5, head_dim=64, q_cols=768)
+    own = block(w=0x1000, bias=0x2000, gamma=0x3000, k_pool=0x4000, v_pool=0x5000, w_packed=0x6000,
+                a=0x10, c=0x20, m=8, lda=256, ldc=192, tok_item=0x30, **sizes)
+    sibling = block(w=0x9000, bias=0xA000, gamma=0xB000, k_pool=0xC000, v_pool=0xD000, w_packed=0xE000,
+                    a=0x50, c=0x60, m=40, lda=512, ldc=384, tok_item=0x70, tables=0x80, table_width=64,
+                    norm_h=0x90, **sizes)
+    made = read(kernels._sibling_block(sibling, own))
+    assert (made.w, made.bias, made.gamma, made.k_pool, made.v_pool, made.w_packed) == \
+        (0x1000, 0x2000, 0x3000, 0x4000, 0x5000, 0x6000)
+    assert (made.a, made.c, made.m, made.lda, made.ldc, made.tok_item, made.tables, made.table_width,
+            made.norm_h) == (0x50, 0x60, 40, 512, 384, 0x70, 0x80, 64, 0x90)
+    assert (made.n, made.k, made.epilogue, made.head_dim, made.q_cols) == (192, 256, 2, 64, 768)
+    assert made.beta is None
+    for name, value in (("n", 128), ("k", 512), ("epilogue", 1), ("c_dtype", 2), ("eps", 1e-6),
+                        ("scatter_only", 1), ("page_size", 16), ("rms", 1), ("c_packed_request", 1)):
+        other = read(sibling)
+        setattr(other, name, value)
+        assert kernels._sibling_block(bytes(other), own) is None, name
+    for name in ("bias", "gamma", "w_packed", "k_pool"):
+        other = read(own)
+        setattr(other, name, None)                 # this site has no such operand, the other has
+        assert kernels._sibling_block(sibling, bytes(other)) is None, name
+    assert ctypes.sizeof(kernels._LinearArgs) == len(own)
