@@ -93,11 +93,15 @@ __global__ __launch_bounds__(256) void gemm_nt_simple_kernel(
   }
 }
 
-// MR: rows held in registers (m <= MR); COLS: output columns per wave
+// MR: rows held in registers (m <= MR); COLS: output columns per wave.  A lane walks k in
+// steps of 256 values and asks for 4 / COLS such steps of its COLS weight rows at once (four
+// 16-byte loads in flight whatever COLS is); the sums are formed in the order of k either way,
+// so the result does not depend on COLS.
 template <int EPI, int MR, int COLS>
 __global__ __launch_bounds__(256) void gemm_nt_f32_rows_kernel(
     const float* __restrict__ a, const float* __restrict__ w, const float* __restrict__ bias,
     float* __restrict__ c, int m, int n, int k, int lda, int ldc) {
+  constexpr int AHEAD = 4 / COLS;
   const int lane = threadIdx.x & 63;
   const int wave = threadIdx.x >> 6;
   const int col0 = (blockIdx.x * 4 + wave) * COLS;
@@ -113,19 +117,27 @@ __global__ __launch_bounds__(256) void gemm_nt_f32_rows_kernel(
   for (int j = 0; j < COLS; ++j)
 #pragma unroll
     for (int r = 0; r < MR; ++r) acc[j][r] = 0.f;
-  for (int k0 = lane * 4; k0 < k; k0 += 256) {
-    float4 wv[COLS];
+  for (int k0 = lane * 4; k0 < k; k0 += 256 * AHEAD) {
+    float4 wv[AHEAD][COLS];
 #pragma unroll
-    for (int j = 0; j < COLS; ++j) wv[j] = *reinterpret_cast<const float4*>(w_row[j] + k0);
+    for (int u = 0; u < AHEAD; ++u)
 #pragma unroll
-    for (int r = 0; r < MR; ++r) {
-      const float4 av = *reinterpret_cast<const float4*>(a_row[r] + k0);
+      for (int j = 0; j < COLS; ++j)
+        wv[u][j] = k0 + 256 * u < k ? *reinterpret_cast<const float4*>(w_row[j] + k0 + 256 * u)
+                                    : make_float4(0.f, 0.f, 0.f, 0.f);
 #pragma unroll
-      for (int j = 0; j < COLS; ++j) {
-        acc[j][r] = fmaf(av.x, wv[j].x, acc[j][r]);
-        acc[j][r] = fmaf(av.y, wv[j].y, acc[j][r]);
-        acc[j][r] = fmaf(av.z, wv[j].z, acc[j][r]);
-        acc[j][r] = fmaf(av.w, wv[j].w, acc[j][r]);
+    for (int u = 0; u < AHEAD; ++u) {
+      if (k0 + 256 * u >= k) break;
+#pragma unroll
+      for (int r = 0; r < MR; ++r) {
+        const float4 av = *reinterpret_cast<const float4*>(a_row[r] + k0 + 256 * u);
+#pragma unroll
+        for (int j = 0; j < COLS; ++j) {
+          acc[j][r] = fmaf(av.x, wv[u][j].x, acc[j][r]);
+          acc[j][r] = fmaf(av.y, wv[u][j].y, acc[j][r]);
+          acc[j][r] = fmaf(av.z, wv[u][j].z, acc[j][r]);
+          acc[j][r] = fmaf(av.w, wv[u][j].w, acc[j][r]);
+        }
       }
     }
   }
@@ -162,11 +174,25 @@ static int launch_f32_rows(const void* a, const void* w, const float* bias, void
   hipLaunchKernelGGL((gemm_nt_f32_rows_kernel<EPI, MR, COLS>), dim3((n + 4 * COLS - 1) / (4 * COLS)), \
                      dim3(256), 0, s, (const float*)a, (const float*)w, bias, (float*)c, m, n, k, \
                      lda, ldc)
-#define PS_LAUNCH_FR_M(EPI)                      \
-  do {                                           \
-    if (m <= 4) PS_LAUNCH_FR(EPI, 4, 4);         \
-    else if (m <= 8) PS_LAUNCH_FR(EPI, 8, 4);    \
-    else PS_LAUNCH_FR(EPI, 16, 2);               \
+  // Columns per wave by the blocks they leave: a block of four waves per compute unit counts
+  // for more than the reuse of the rows (8 x 768 x 3072 on 48 blocks of 4 columns a wave took
+  // 31 us, twelve trips to memory one after the other).
+  const int units = ps_compute_units();
+  const int cols = (n + 15) / 16 >= 3 * units / 4 ? 4 : (n + 7) / 8 >= 3 * units / 4 ? 2 : 1;
+#define PS_LAUNCH_FR_M(EPI)                                   \
+  do {                                                        \
+    if (m <= 4) {                                             \
+      if (cols == 4) PS_LAUNCH_FR(EPI, 4, 4);                 \
+      else if (cols == 2) PS_LAUNCH_FR(EPI, 4, 2);            \
+      else PS_LAUNCH_FR(EPI, 4, 1);                           \
+    } else if (m <= 8) {                                      \
+      if (cols == 4) PS_LAUNCH_FR(EPI, 8, 4);                 \
+      else if (cols == 2) PS_LAUNCH_FR(EPI, 8, 2);            \
+      else PS_LAUNCH_FR(EPI, 8, 1);                           \
+    } else {                                                  \
+      if (cols >= 2) PS_LAUNCH_FR(EPI, 16, 2);                \
+      else PS_LAUNCH_FR(EPI, 16, 1);                          \
+    }                                                         \
   } while (0)
   switch (epilogue) {
     case PS_EPI_NONE: PS_LAUNCH_FR_M(PS_EPI_NONE); break;

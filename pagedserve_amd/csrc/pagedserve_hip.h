@@ -120,6 +120,19 @@ int ps_attention_rowwise(const void* q, int64_t q_stride, const void* k_pool, co
                          int heads, int kv_heads, int head_dim, int page_size, int num_pages,
                          float scale, int window, int dtype, void* stream);
 
+// The same result in true 32-bit for the items of several tokens (prompt portions), a block
+// of four waves per (tile of ps_attention_tiled_f32_tile() queries, head): float pools, float
+// q and out, keys and values through LDS, scores by plain fused multiply-adds.  The tiles are
+// listed as for ps_attention_prefill (item and first query of each, cut at the tile size).
+// head_dim a multiple of 4 up to 128 (ps_attention_tiled_f32_supported); 16-byte aligned rows.
+int ps_attention_tiled_f32_supported(int head_dim);
+int ps_attention_tiled_f32_tile();
+int ps_attention_tiled_f32(const void* q, int64_t q_stride, const void* k_pool, const void* v_pool,
+                           void* out, int64_t out_stride, const int* tile_item, const int* tile_q0,
+                           int tiles, const int* cu_tokens, const int* kv_lens, const int* tables,
+                           int table_width, int heads, int kv_heads, int head_dim, int page_size,
+                           int num_pages, float scale, int window, void* stream);
+
 // The same result for single queries, with each token's keys cut into `splits` ranges that
 // run as separate blocks of `waves` (4 or 16) waves; `partial` is scratch of
 // count * heads * splits * (head_dim + 2) floats (unused when splits == 1).  head_dim is a

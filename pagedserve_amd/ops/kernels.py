@@ -40,6 +40,9 @@ _SIGNATURES = {
                                     c_int, c_int, c_float, c_int, c_int, c_int, c_int, c_void_p],
     "ps_attention_merge_linear": [c_void_p, c_int64, c_void_p, c_int, c_int, c_int, c_int, c_void_p,
                                   c_void_p, c_void_p, c_int64, c_int, c_int, c_void_p],
+    "ps_attention_tiled_f32": [c_void_p, c_int64, c_void_p, c_void_p, c_void_p, c_int64, c_void_p,
+                               c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int,
+                               c_int, c_int, c_int, c_float, c_int, c_void_p],
     "ps_attention_prefill": [c_void_p, c_int64, c_void_p, c_void_p, c_void_p, c_int64, c_void_p,
                              c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int,
                              c_int, c_int, c_int, c_float, c_int, c_int, c_int, c_int, c_void_p],
@@ -855,6 +858,55 @@ def attention_prefill(q, k_pool, v_pool, out, tile_item, tile_q0, cu_tokens, kv_
                 kv_heads, head_dim, page_size, pages, float(scale), int(window), int(max_kv_len),
                 int(query_tile), dtype_code(q.dtype)),
                shared, step_key, (kv_heads, head_dim, page_size, pages, q.dtype))
+    return out
+
+
+def tiled_f32_supported(dtype, head_dim) -> bool:
+    """Whether ``attention_tiled_f32`` takes the shape: float storage, head sizes that are
+    multiples of 4 up to 128."""
+    return dtype == torch.float32 and head_dim % 4 == 0 and 4 <= head_dim <= 128
+
+
+_TILED_F32_CHECKED = False
+
+
+def attention_tiled_f32(q, k_pool, v_pool, out, tile_item, tile_q0, cu_tokens, kv_lens, tables, heads,
+                        scale, window=0):
+    """Attention of items with several tokens in true 32-bit, ``PREFILL_TILE`` queries per
+    block: keys and values pass through LDS once per tile of queries instead of once per query
+    (``attention_rowwise``), scores and sums are plain float arithmetic.  The tile list is the
+    one of ``attention_prefill`` at that size."""
+    global _TILED_F32_CHECKED
+    if not _TILED_F32_CHECKED:
+        lib = load_library()
+        lib.ps_attention_tiled_f32_tile.restype = c_int
+        if lib.ps_attention_tiled_f32_tile() != PREFILL_TILE:
+            raise KernelError(f"the library's 32-bit tiled attention takes tiles of "
+                              f"{lib.ps_attention_tiled_f32_tile()} queries, this module lists tiles "
+                              f"of {PREFILL_TILE}; rebuild the library")
+        _TILED_F32_CHECKED = True
+    _check(q, "q", torch.float32, 2)
+    _check(out, "out", torch.float32, 2)
+    pages, kv_heads, page_size, head_dim = _check_pools(k_pool, v_pool, q.dtype)
+    q_stride = _rows(q, "q")
+    out_stride = _rows(out, "out")
+    if q.shape[1] != heads * head_dim or out.shape != q.shape:
+        raise KernelError("attention_tiled_f32: q/out rows must hold heads x head_dim values")
+    for name, tensor in (("tile_item", tile_item), ("tile_q0", tile_q0), ("cu_tokens", cu_tokens),
+                         ("kv_lens", kv_lens)):
+        _check(tensor, name, torch.int32, 1)
+        if not tensor.is_contiguous():
+            raise KernelError(f"attention_tiled_f32: {name} must be contiguous")
+    _check(tables, "tables", torch.int32, 2)
+    tiles = tile_item.numel()
+    items = kv_lens.numel()
+    if tile_q0.numel() != tiles or cu_tokens.numel() != items + 1 or tables.shape[0] != items \
+            or not tables.is_contiguous():
+        raise KernelError("attention_tiled_f32: inconsistent tile or item arrays")
+    _call("ps_attention_tiled_f32", q.data_ptr(), q_stride, k_pool.data_ptr(), v_pool.data_ptr(),
+          out.data_ptr(), out_stride, tile_item.data_ptr(), tile_q0.data_ptr(), tiles,
+          cu_tokens.data_ptr(), kv_lens.data_ptr(), tables.data_ptr(), tables.shape[1], heads,
+          kv_heads, head_dim, page_size, pages, float(scale), int(window), _stream())
     return out
 
 

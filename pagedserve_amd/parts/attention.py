@@ -175,6 +175,20 @@ class Attention(Mixer):
                                       max_kv_len=ctx.max_kv_len, query_tile=size,
                                       memo=site_memo(self._memo_attention, ctx.workspace),
                                       shared=ctx.shared_calls)
+        elif singles < tokens and kernels.tiled_f32_supported(self.dtype, self.head_dim):
+            # 32-bit: tiles of queries too, on plain float arithmetic.  The tiles hold the items
+            # of several tokens; one-token items that the split-KV kernel did not take (a head
+            # size that it refuses) go to the kernel that takes all sizes
+            tile_item, tile_q0 = ctx.query_tiles[kernels.PREFILL_TILE]
+            if tile_item.numel():
+                kernels.attention_tiled_f32(q, cache.k_pool, cache.v_pool, context, tile_item, tile_q0,
+                                            ctx.cu_tokens, ctx.kv_lens, tables, self.heads, self.scale,
+                                            self.window)
+            if not singles and ctx.single_tokens is not None and ctx.single_tokens.numel():
+                kernels.attention_rowwise(q, cache.k_pool, cache.v_pool, context, ctx.tok_item,
+                                          ctx.positions, tables, self.heads, self.scale, self.window,
+                                          tok_list=None if ctx.single_tokens.numel() == tokens
+                                          else ctx.single_tokens)
         elif singles < tokens:
             kernels.attention_rowwise(q, cache.k_pool, cache.v_pool, context, ctx.tok_item,
                                       ctx.positions, tables, self.heads, self.scale, self.window,

@@ -582,6 +582,79 @@ def test_attention_prefill_tiles(heads, kv_heads, head_dim, page_size, window, t
     torch.testing.assert_close(out.double(), expected, atol=5e-3, rtol=5e-3)
 
 
+@pytest.mark.parametrize("heads,kv_heads,head_dim,page_size", [(1, 1, 32, 16), (4, 4, 16, 8), (6, 2, 48, 16), (2, 2, 128, 4), (12, 12, 64, 16),
+                                                                (3, 1, 80, 12), (5, 5, 4, 3), (3, 3, 20, 5), (2, 1, 100, 16), (7, 7, 12, 1),
+                                                                (25, 25, 64, 16), (2, 2, 68, 8)])
+@pytest.mark.parametrize("window", [0, 37])
+def test_attention_tiled_f32(heads, kv_heads, head_dim, page_size, window):
+    """The 32-bit tiled kernel against float64 attention over the gathered pages, and against
+    the one-wave-per-token kernel that it stands in for: fresh prompts and later portions of
+    many lengths in one launch (portions that start inside a page, more than one tile, a tile's
+    last rows empty, two tokens), fragmented tables, NaN behind every request's last key, head
+    sizes that are multiples of 4 on both sides of 64; other head sizes are refused."""
+    from pagedserve_amd.ops import kernels
+
+    dtype = torch.float32
+    items = [(0, 2), (0, 64), (0, 65), (0, 200), (30, 23), (17, 130), (100, 16), (63, 3), (250, 70)]
+    totals = [past + new for past, new in items]
+    k_pool, v_pool, tables = _paged_fixture(dtype, totals, kv_heads, head_dim, page_size, 53)
+    for index, total in enumerate(totals):
+        if total % page_size:
+            last = int(tables[index, total // page_size])
+            k_pool[last, :, total % page_size:] = float("nan")
+            v_pool[last, :, total % page_size:] = float("nan")
+    tokens = sum(new for _, new in items)
+    q = _rand((tokens, heads * head_dim), dtype, 54)
+    tok_item, tok_pos, tile_item, tile_q0, cu = [], [], [], [], [0]
+    for index, (past, new) in enumerate(items):
+        tok_item += [index] * new
+        tok_pos += list(range(past, past + new))
+        cu.append(cu[-1] + new)
+        for q0 in range(0, new, kernels.PREFILL_TILE):
+            tile_item.append(index)
+            tile_q0.append(q0)
+
+    def dev(values):
+        return torch.tensor(values, dtype=torch.int32, device="cuda")
+
+    scale = head_dim ** -0.5
+    assert kernels.tiled_f32_supported(dtype, head_dim)
+    # the tiles in another order than the items': every block finds its own rows
+    order = list(reversed(range(len(tile_item))))
+    out = torch.full_like(q, float("nan"))
+    kernels.attention_tiled_f32(q, k_pool, v_pool, out, dev([tile_item[i] for i in order]),
+                                dev([tile_q0[i] for i in order]), dev(cu), dev(totals), tables, heads, scale,
+                                window=window)
+    assert torch.isfinite(out).all()
+    expected = _attention_expected(q, k_pool, v_pool, tables, tok_item, tok_pos, heads, scale, window)
+    torch.testing.assert_close(out.double(), expected, atol=3e-5, rtol=3e-5)
+    rowwise = torch.full_like(q, float("nan"))
+    kernels.attention_rowwise(q, k_pool, v_pool, rowwise, dev(tok_item), dev(tok_pos), tables, heads, scale,
+                              window=window)
+    torch.testing.assert_close(out, rowwise, atol=2e-5, rtol=2e-5)
+
+
+def test_attention_tiled_f32_refuses_what_it_cannot_take():
+    from pagedserve_amd.ops import kernels
+
+    assert not kernels.tiled_f32_supported(torch.float32, 6) and not kernels.tiled_f32_supported(torch.float32, 132)
+    assert not kernels.tiled_f32_supported(torch.bfloat16, 64)
+    index = torch.zeros(1, dtype=torch.int32, device="cuda")
+    cu = torch.tensor([0, 2], dtype=torch.int32, device="cuda")
+    lens = torch.tensor([2], dtype=torch.int32, device="cuda")
+    tables = torch.zeros((1, 4), dtype=torch.int32, device="cuda")
+    for head_dim in (6, 132):
+        q = torch.zeros((2, head_dim), device="cuda")
+        pool = torch.zeros((4, 1, 8, head_dim), device="cuda")
+        with pytest.raises(kernels.KernelError, match="multiple of 4 up to 128"):
+            kernels.attention_tiled_f32(q, pool, pool.clone(), torch.zeros_like(q), index, index, cu, lens, tables,
+                                        1, 1.0)
+    q = torch.zeros((2, 64), device="cuda", dtype=torch.bfloat16)
+    pool = torch.zeros((4, 1, 8, 64), device="cuda", dtype=torch.bfloat16)
+    with pytest.raises(kernels.KernelError):
+        kernels.attention_tiled_f32(q, pool, pool.clone(), torch.zeros_like(q), index, index, cu, lens, tables, 1, 1.0)
+
+
 @pytest.mark.parametrize("heads,kv_heads,head_dim,page_size", [(12, 12, 64, 16), (4, 4, 16, 8), (6, 2, 48, 16), (25, 25, 64, 16),
                                                                 (3, 1, 32, 12), (16, 4, 64, 5)])
 @pytest.mark.parametrize("window", [0, 37])
