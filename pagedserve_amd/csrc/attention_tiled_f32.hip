@@ -21,7 +21,7 @@
 #include "common.h"
 #include "pagedserve_hip.h"
 
-#define AF_TILE 64       // queries of a block, and keys of a round
+#define AF_TILE 64       // queries of a block, and keys per turn of its loop
 #define AF_MAX_DIM 128
 #define AF_P_STRIDE 68   // floats from row to row of the probabilities in LDS
 
@@ -42,7 +42,7 @@ __global__ __launch_bounds__(256) void attention_tiled_f32_kernel(
   __shared__ int64_t s_base[AF_TILE];   // first value of each key's row in the pools, or -1
 
   const int tid = threadIdx.x;
-  const int tx = tid & 15;    // keys tx + 16 j of a round; dimension groups tx + 16 v
+  const int tx = tid & 15;    // keys tx + 16 j of a turn of the loop; dimension groups tx + 16 v
   const int ty = tid >> 4;    // queries 4 ty + i of the tile
   const int tile_index = blockIdx.x / heads;
   const int head = blockIdx.x - tile_index * heads;
@@ -85,7 +85,7 @@ __global__ __launch_bounds__(256) void attention_tiled_f32_kernel(
   }
 
   for (int k0 = key_begin; k0 < key_end; k0 += AF_TILE) {
-    // (the round before has been read: the barrier at the end of the loop)
+    // (the 64 keys before have been read: the barrier at the end of the loop)
     if (tid < AF_TILE) {
       const int key = k0 + tid;
       int64_t base = -1;
